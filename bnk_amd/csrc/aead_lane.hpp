@@ -1,0 +1,138 @@
+// Per-lane ChaCha20-Poly1305 building blocks for gfx950.
+//
+// One lane owns one packet end to end: the 16-word ChaCha20 state and the
+// Poly1305 accumulator stay in VGPRs for the packet's whole life, there is no
+// cross-lane traffic and no LDS.  32-bit add/xor/rotate (v_alignbit_b32) for
+// ChaCha20; Poly1305 in radix 2^26 with v_mad_u64_u32 partial products.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace bnk {
+
+#define BNK_DEV __device__ __forceinline__
+
+BNK_DEV uint32_t rotl32(uint32_t v, int c) { return __builtin_rotateleft32(v, c); }
+
+#define BNK_QR(a, b, c, d)                          \
+    a += b; d ^= a; d = rotl32(d, 16);              \
+    c += d; b ^= c; b = rotl32(b, 12);              \
+    a += b; d ^= a; d = rotl32(d, 8);               \
+    c += d; b ^= c; b = rotl32(b, 7)
+
+// RFC 8439 section 2.3 with the WireGuard nonce: words 13..15 of the state
+// are 0, counter low, counter high.
+BNK_DEV void chacha_block(const uint32_t (&k)[8], uint32_t blk, uint32_t n1,
+                          uint32_t n2, uint32_t (&x)[16])
+{
+    x[0] = 0x61707865u; x[1] = 0x3320646eu; x[2] = 0x79622d32u; x[3] = 0x6b206574u;
+#pragma unroll
+    for (int i = 0; i < 8; i++) x[4 + i] = k[i];
+    x[12] = blk; x[13] = 0; x[14] = n1; x[15] = n2;
+#pragma unroll 1
+    for (int r = 0; r < 10; r++) {
+        BNK_QR(x[0], x[4], x[8], x[12]);
+        BNK_QR(x[1], x[5], x[9], x[13]);
+        BNK_QR(x[2], x[6], x[10], x[14]);
+        BNK_QR(x[3], x[7], x[11], x[15]);
+        BNK_QR(x[0], x[5], x[10], x[15]);
+        BNK_QR(x[1], x[6], x[11], x[12]);
+        BNK_QR(x[2], x[7], x[8], x[13]);
+        BNK_QR(x[3], x[4], x[9], x[14]);
+    }
+    x[0] += 0x61707865u; x[1] += 0x3320646eu; x[2] += 0x79622d32u; x[3] += 0x6b206574u;
+#pragma unroll
+    for (int i = 0; i < 8; i++) x[4 + i] += k[i];
+    x[12] += blk; x[14] += n1; x[15] += n2;
+}
+
+// Poly1305 (RFC 8439 section 2.5), radix 2^26.
+struct Poly26 {
+    uint32_t r0, r1, r2, r3, r4;
+    uint32_t s1, s2, s3, s4; // 5 * r
+    uint32_t h0, h1, h2, h3, h4;
+    uint32_t pad0, pad1, pad2, pad3;
+
+    // otk = first 8 words of ChaCha20 block 0
+    BNK_DEV void init(const uint32_t (&x)[16])
+    {
+        const uint32_t t0 = x[0] & 0x0fffffffu, t1 = x[1] & 0x0ffffffcu;
+        const uint32_t t2 = x[2] & 0x0ffffffcu, t3 = x[3] & 0x0ffffffcu;
+        r0 = t0 & 0x3ffffffu;
+        r1 = ((t0 >> 26) | (t1 << 6)) & 0x3ffffffu;
+        r2 = ((t1 >> 20) | (t2 << 12)) & 0x3ffffffu;
+        r3 = ((t2 >> 14) | (t3 << 18)) & 0x3ffffffu;
+        r4 = t3 >> 8;
+        s1 = r1 * 5; s2 = r2 * 5; s3 = r3 * 5; s4 = r4 * 5;
+        h0 = h1 = h2 = h3 = h4 = 0;
+        pad0 = x[4]; pad1 = x[5]; pad2 = x[6]; pad3 = x[7];
+    }
+
+    // One full 16-byte block (little-endian words w0..w3) with bit 128 set.
+    BNK_DEV void block(uint32_t w0, uint32_t w1, uint32_t w2, uint32_t w3)
+    {
+        const uint32_t a0 = h0 + (w0 & 0x3ffffffu);
+        const uint32_t a1 = h1 + (__builtin_amdgcn_alignbit(w1, w0, 26) & 0x3ffffffu);
+        const uint32_t a2 = h2 + (__builtin_amdgcn_alignbit(w2, w1, 20) & 0x3ffffffu);
+        const uint32_t a3 = h3 + (__builtin_amdgcn_alignbit(w3, w2, 14) & 0x3ffffffu);
+        const uint32_t a4 = h4 + ((w3 >> 8) | (1u << 24));
+
+        uint64_t d0 = (uint64_t)a0 * r0 + (uint64_t)a1 * s4 + (uint64_t)a2 * s3 +
+                      (uint64_t)a3 * s2 + (uint64_t)a4 * s1;
+        uint64_t d1 = (uint64_t)a0 * r1 + (uint64_t)a1 * r0 + (uint64_t)a2 * s4 +
+                      (uint64_t)a3 * s3 + (uint64_t)a4 * s2;
+        uint64_t d2 = (uint64_t)a0 * r2 + (uint64_t)a1 * r1 + (uint64_t)a2 * r0 +
+                      (uint64_t)a3 * s4 + (uint64_t)a4 * s3;
+        uint64_t d3 = (uint64_t)a0 * r3 + (uint64_t)a1 * r2 + (uint64_t)a2 * r1 +
+                      (uint64_t)a3 * r0 + (uint64_t)a4 * s4;
+        uint64_t d4 = (uint64_t)a0 * r4 + (uint64_t)a1 * r3 + (uint64_t)a2 * r2 +
+                      (uint64_t)a3 * r1 + (uint64_t)a4 * r0;
+
+        uint32_t c;
+        c = (uint32_t)(d0 >> 26); h0 = (uint32_t)d0 & 0x3ffffffu; d1 += c;
+        c = (uint32_t)(d1 >> 26); h1 = (uint32_t)d1 & 0x3ffffffu; d2 += c;
+        c = (uint32_t)(d2 >> 26); h2 = (uint32_t)d2 & 0x3ffffffu; d3 += c;
+        c = (uint32_t)(d3 >> 26); h3 = (uint32_t)d3 & 0x3ffffffu; d4 += c;
+        c = (uint32_t)(d4 >> 26); h4 = (uint32_t)d4 & 0x3ffffffu;
+        h0 += c * 5;
+        c = h0 >> 26; h0 &= 0x3ffffffu;
+        h1 += c;
+    }
+
+    // tag = ((h mod 2^130-5) + s) mod 2^128 as four little-endian words
+    BNK_DEV void finish(uint32_t (&tag)[4])
+    {
+        uint32_t c;
+        c = h1 >> 26; h1 &= 0x3ffffffu; h2 += c;
+        c = h2 >> 26; h2 &= 0x3ffffffu; h3 += c;
+        c = h3 >> 26; h3 &= 0x3ffffffu; h4 += c;
+        c = h4 >> 26; h4 &= 0x3ffffffu; h0 += c * 5;
+        c = h0 >> 26; h0 &= 0x3ffffffu; h1 += c;
+
+        // g = h + 5 - 2^130; keep g when it did not go negative (h >= p)
+        uint32_t g0 = h0 + 5; c = g0 >> 26; g0 &= 0x3ffffffu;
+        uint32_t g1 = h1 + c; c = g1 >> 26; g1 &= 0x3ffffffu;
+        uint32_t g2 = h2 + c; c = g2 >> 26; g2 &= 0x3ffffffu;
+        uint32_t g3 = h3 + c; c = g3 >> 26; g3 &= 0x3ffffffu;
+        uint32_t g4 = h4 + c - (1u << 26);
+        const uint32_t take_g = (g4 >> 31) - 1; // all ones when g4 >= 0
+        h0 = (h0 & ~take_g) | (g0 & take_g);
+        h1 = (h1 & ~take_g) | (g1 & take_g);
+        h2 = (h2 & ~take_g) | (g2 & take_g);
+        h3 = (h3 & ~take_g) | (g3 & take_g);
+        h4 = (h4 & ~take_g) | (g4 & take_g);
+
+        const uint32_t w0 = h0 | (h1 << 26);
+        const uint32_t w1 = (h1 >> 6) | (h2 << 20);
+        const uint32_t w2 = (h2 >> 12) | (h3 << 14);
+        const uint32_t w3 = (h3 >> 18) | (h4 << 8);
+        uint64_t f;
+        f = (uint64_t)w0 + pad0;             tag[0] = (uint32_t)f;
+        f = (uint64_t)w1 + pad1 + (f >> 32); tag[1] = (uint32_t)f;
+        f = (uint64_t)w2 + pad2 + (f >> 32); tag[2] = (uint32_t)f;
+        f = (uint64_t)w3 + pad3 + (f >> 32); tag[3] = (uint32_t)f;
+    }
+};
+
+} // namespace bnk

@@ -1,0 +1,501 @@
+// C ABI of libbnkhip.so (see include/bnkhip.h): argument checking, staging of
+// host batches through the context's device buffers, kernel launches.
+#include <string.h>
+
+#include <algorithm>
+#include <new>
+
+#include "ctx.hpp"
+#include "filter_host.hpp"
+
+using namespace bnk;
+
+namespace {
+
+thread_local std::string g_init_err;
+
+int fail(bnk_ctx *ctx, int code, const std::string &what)
+{
+    if (ctx) ctx->err = what;
+    else g_init_err = what;
+    return code;
+}
+
+int fail_hip(bnk_ctx *ctx, const char *what, hipError_t e)
+{
+    return fail(ctx, e == hipErrorOutOfMemory ? BNK_E_NOMEM : BNK_E_HIP,
+                std::string(what) + ": " + hipGetErrorString(e));
+}
+
+#define HIPCHK(ctx, expr)                                         \
+    do {                                                          \
+        hipError_t e_ = (expr);                                   \
+        if (e_ != hipSuccess) return fail_hip((ctx), #expr, e_);  \
+    } while (0)
+
+// Every entry point takes the context lock and makes the context's device
+// current for the calling thread.
+struct Guard {
+    std::unique_lock<std::mutex> lk;
+    int rc = BNK_OK;
+    explicit Guard(bnk_ctx *ctx)
+    {
+        if (!ctx) { rc = fail(nullptr, BNK_E_INVAL, "null context"); return; }
+        lk = std::unique_lock<std::mutex>(ctx->mu);
+        if (!ctx->alive) { rc = fail(ctx, BNK_E_STATE, "context is shut down"); return; }
+        hipError_t e = hipSetDevice(ctx->device);
+        if (e != hipSuccess) rc = fail_hip(ctx, "hipSetDevice", e);
+    }
+};
+
+inline uint64_t pkt_off(const bnk_batch *b, uint32_t i)
+{
+    return b->offsets ? b->offsets[i] : (uint64_t)i * b->stride;
+}
+
+struct Span {
+    uint64_t lo = UINT64_MAX, hi = 0;
+    void add(uint64_t a, uint64_t b) { lo = std::min(lo, a); hi = std::max(hi, b); }
+    uint64_t size() const { return hi > lo ? hi - lo : 0; }
+};
+
+// Checks that packet i of a host batch occupies [off, off + len + delta)
+// inside the arena and accumulates the touched span.  lens come from `src`
+// (the input batch) because an output batch only carries a layout.
+int scan_host_layout(bnk_ctx *ctx, const bnk_batch *lay, const bnk_batch *src, int delta,
+                     Span *span, const char *name)
+{
+    const uint32_t n = src->n;
+    for (uint32_t i = 0; i < n; i++) {
+        const uint64_t off = pkt_off(lay, i);
+        int64_t len = (int64_t)(src->lens ? src->lens[i] : src->len) + delta;
+        if (len < 0) len = 0;
+        if (off > lay->bytes || (uint64_t)len > lay->bytes - off)
+            return fail(ctx, BNK_E_INVAL, std::string(name) + ": packet " + std::to_string(i) +
+                                              " lies outside the arena");
+        span->add(off, off + (uint64_t)len);
+    }
+    return BNK_OK;
+}
+
+int check_batch_common(bnk_ctx *ctx, const bnk_batch *b, const char *name)
+{
+    if (!b) return fail(ctx, BNK_E_INVAL, std::string(name) + ": null batch");
+    if (b->mem != BNK_MEM_HOST && b->mem != BNK_MEM_DEVICE)
+        return fail(ctx, BNK_E_INVAL, std::string(name) + ": bad mem kind");
+    if (b->n && !b->base) return fail(ctx, BNK_E_INVAL, std::string(name) + ": null arena");
+    return BNK_OK;
+}
+
+// Host-resident view of a batch staged on the device.
+struct Staged {
+    uint8_t *d_in = nullptr, *d_out = nullptr;
+    const uint64_t *d_in_off = nullptr, *d_out_off = nullptr;
+    const uint32_t *d_lens = nullptr, *d_peer = nullptr;
+    const uint64_t *d_counters = nullptr;
+    Span sin, sout;
+    bool in_place = false;
+};
+
+bool same_layout(const bnk_batch *a, const bnk_batch *b)
+{
+    if (a->base != b->base) return false;
+    if (a->offsets || b->offsets) return a->offsets == b->offsets;
+    return a->stride == b->stride;
+}
+
+// Copies the rebased offsets of `lay` into pinned staging at `slot` and
+// queues the upload.
+int upload_offsets(bnk_ctx *ctx, const bnk_batch *lay, uint32_t n, uint64_t lo, DevBuf *dst,
+                   size_t pin_off, const uint64_t **out)
+{
+    if (!lay->offsets) { *out = nullptr; return BNK_OK; }
+    HIPCHK(ctx, dst->reserve((size_t)n * 8));
+    uint64_t *h = reinterpret_cast<uint64_t *>(ctx->pin.as<uint8_t>() + pin_off);
+    for (uint32_t i = 0; i < n; i++) h[i] = lay->offsets[i] - lo;
+    HIPCHK(ctx, hipMemcpyAsync(dst->p, h, (size_t)n * 8, hipMemcpyHostToDevice, ctx->stream));
+    *out = dst->as<uint64_t>();
+    return BNK_OK;
+}
+
+// Stages a host input batch (and the layout of its output batch) on the
+// device.  in_delta/out_delta adjust the per-packet byte counts: seal writes
+// len + 16, open writes len - 16.
+int stage_host(bnk_ctx *ctx, const bnk_batch *in, const bnk_batch *out, int out_delta,
+               uint32_t n_keys, Staged *st)
+{
+    const uint32_t n = in->n;
+    int rc = scan_host_layout(ctx, in, in, 0, &st->sin, "in");
+    if (rc) return rc;
+    rc = scan_host_layout(ctx, out, in, out_delta, &st->sout, "out");
+    if (rc) return rc;
+    if (in->peer)
+        for (uint32_t i = 0; i < n; i++)
+            if (in->peer[i] >= n_keys)
+                return fail(ctx, BNK_E_RANGE, "peer index " + std::to_string(in->peer[i]) +
+                                                  " beyond the key table");
+    // pinned staging for the two rebased offset arrays
+    HIPCHK(ctx, ctx->pin.reserve((size_t)n * 16 + 64));
+
+    st->in_place = same_layout(in, out);
+    if (st->in_place) {
+        Span u = st->sin;
+        u.add(st->sout.lo, st->sout.hi);
+        st->sin = st->sout = u;
+    }
+    HIPCHK(ctx, ctx->in_arena.reserve(st->sin.size() + 16));
+    st->d_in = ctx->in_arena.as<uint8_t>();
+    HIPCHK(ctx, hipMemcpyAsync(st->d_in, (const uint8_t *)in->base + st->sin.lo, st->sin.size(),
+                               hipMemcpyHostToDevice, ctx->stream));
+    if (st->in_place) {
+        st->d_out = st->d_in;
+    } else {
+        HIPCHK(ctx, ctx->out_arena.reserve(st->sout.size() + 16));
+        st->d_out = ctx->out_arena.as<uint8_t>();
+        // bytes between packets of the output arena must survive the round
+        // trip, so the device copy starts from the host's content
+        HIPCHK(ctx, hipMemcpyAsync(st->d_out, (const uint8_t *)out->base + st->sout.lo,
+                                   st->sout.size(), hipMemcpyHostToDevice, ctx->stream));
+    }
+    rc = upload_offsets(ctx, in, n, st->sin.lo, &ctx->off_in, 0, &st->d_in_off);
+    if (rc) return rc;
+    if (st->in_place) {
+        st->d_out_off = st->d_in_off;
+    } else {
+        rc = upload_offsets(ctx, out, n, st->sout.lo, &ctx->off_out, (size_t)n * 8, &st->d_out_off);
+        if (rc) return rc;
+    }
+    if (in->lens) {
+        HIPCHK(ctx, ctx->lens.reserve((size_t)n * 4));
+        HIPCHK(ctx, hipMemcpyAsync(ctx->lens.p, in->lens, (size_t)n * 4, hipMemcpyHostToDevice,
+                                   ctx->stream));
+        st->d_lens = ctx->lens.as<uint32_t>();
+    }
+    if (in->peer) {
+        HIPCHK(ctx, ctx->peer.reserve((size_t)n * 4));
+        HIPCHK(ctx, hipMemcpyAsync(ctx->peer.p, in->peer, (size_t)n * 4, hipMemcpyHostToDevice,
+                                   ctx->stream));
+        st->d_peer = ctx->peer.as<uint32_t>();
+    }
+    if (in->counters) {
+        HIPCHK(ctx, ctx->counters.reserve((size_t)n * 8));
+        HIPCHK(ctx, hipMemcpyAsync(ctx->counters.p, in->counters, (size_t)n * 8,
+                                   hipMemcpyHostToDevice, ctx->stream));
+        st->d_counters = ctx->counters.as<uint64_t>();
+    }
+    return BNK_OK;
+}
+
+// Lanes of a wave should run the same number of ChaCha20 blocks: when lengths
+// vary, hand packets to lanes in length order.
+int maybe_sort(bnk_ctx *ctx, const uint32_t *d_lens, uint32_t n, uint32_t tag_bytes,
+               const uint32_t **order)
+{
+    *order = nullptr;
+    if (!d_lens || n <= 64) return BNK_OK;
+    HIPCHK(ctx, ctx->order.reserve((size_t)n * 4));
+    HIPCHK(ctx, ctx->hist.reserve(LEN_BINS * 4));
+    HIPCHK(ctx, ctx->cursor.reserve(LEN_BINS * 4));
+    HIPCHK(ctx, launch_length_sort(d_lens, n, tag_bytes, ctx->order.as<uint32_t>(),
+                                   ctx->hist.as<uint32_t>(), ctx->cursor.as<uint32_t>(),
+                                   ctx->stream));
+    *order = ctx->order.as<uint32_t>();
+    return BNK_OK;
+}
+
+// Reads and clears the device status word; the stream must be idle.
+int take_status(bnk_ctx *ctx, uint32_t *status)
+{
+    HIPCHK(ctx, hipMemcpyAsync(status, ctx->d_status, 4, hipMemcpyDeviceToHost, ctx->stream));
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    if (*status) HIPCHK(ctx, launch_fill_u32(ctx->d_status, 1, 0, ctx->stream));
+    return BNK_OK;
+}
+
+int aead_batch(bnk_ctx *ctx, bool open, const bnk_batch *in, const bnk_batch *out,
+               uint8_t *verdict)
+{
+    int rc = check_batch_common(ctx, in, "in");
+    if (rc) return rc;
+    rc = check_batch_common(ctx, out, "out");
+    if (rc) return rc;
+    if (in->mem != out->mem) return fail(ctx, BNK_E_INVAL, "in and out must use the same mem kind");
+    const uint32_t n = in->n;
+    if (n == 0) return BNK_OK;
+    if (open && !verdict) return fail(ctx, BNK_E_INVAL, "null verdict array");
+    const int which = open ? BNK_KEYS_RECV : BNK_KEYS_SEND;
+    if (!ctx->d_keys[which] || ctx->n_keys[which] == 0)
+        return fail(ctx, BNK_E_STATE, open ? "no receive keys loaded" : "no send keys loaded");
+    if (!in->peer && ctx->n_keys[which] < 1) return fail(ctx, BNK_E_RANGE, "empty key table");
+
+    AeadArgs a{};
+    a.keys = ctx->d_keys[which];
+    a.n_peers = ctx->n_keys[which];
+    a.status = ctx->d_status;
+    a.counter0 = in->counter0;
+    a.n = n;
+    a.in_stride = in->stride;
+    a.out_stride = out->stride;
+    a.len = in->len;
+
+    if (in->mem == BNK_MEM_DEVICE) {
+        // Device batches cannot be walked on the host; check what is uniform.
+        if (!in->offsets && !in->lens &&
+            ((uint64_t)(n - 1) * in->stride + in->len > in->bytes))
+            return fail(ctx, BNK_E_INVAL, "in: uniform layout exceeds the arena");
+        if (!out->offsets && !in->lens) {
+            const int64_t ol = (int64_t)in->len + (open ? -16 : 16);
+            if ((uint64_t)(n - 1) * out->stride + (uint64_t)std::max<int64_t>(ol, 0) > out->bytes)
+                return fail(ctx, BNK_E_INVAL, "out: uniform layout exceeds the arena");
+        }
+        a.in = (const uint8_t *)in->base;
+        a.out = (uint8_t *)out->base;
+        a.in_off = in->offsets;
+        a.out_off = out->offsets;
+        a.lens = in->lens;
+        a.peer = in->peer;
+        a.counters = in->counters;
+        a.verdict = verdict;
+        rc = maybe_sort(ctx, a.lens, n, open ? 16 : 0, &a.order);
+        if (rc) return rc;
+        HIPCHK(ctx, open ? launch_aead_open(a, ctx->stream) : launch_aead_seal(a, ctx->stream));
+        return BNK_OK;
+    }
+
+    Staged st;
+    rc = stage_host(ctx, in, out, open ? -16 : 16, ctx->n_keys[which], &st);
+    if (rc) return rc;
+    a.in = st.d_in;
+    a.out = st.d_out;
+    a.in_off = st.d_in_off;
+    a.out_off = st.d_out_off;
+    a.lens = st.d_lens;
+    a.peer = st.d_peer;
+    a.counters = st.d_counters;
+    if (open) {
+        HIPCHK(ctx, ctx->verdict.reserve(n));
+        a.verdict = ctx->verdict.as<uint8_t>();
+    }
+    rc = maybe_sort(ctx, a.lens, n, open ? 16 : 0, &a.order);
+    if (rc) return rc;
+    HIPCHK(ctx, open ? launch_aead_open(a, ctx->stream) : launch_aead_seal(a, ctx->stream));
+    HIPCHK(ctx, hipMemcpyAsync((uint8_t *)out->base + st.sout.lo, st.d_out, st.sout.size(),
+                               hipMemcpyDeviceToHost, ctx->stream));
+    if (open)
+        HIPCHK(ctx, hipMemcpyAsync(verdict, a.verdict, n, hipMemcpyDeviceToHost, ctx->stream));
+    uint32_t status = 0;
+    rc = take_status(ctx, &status);
+    if (rc) return rc;
+    if (status & STATUS_PEER_RANGE) return fail(ctx, BNK_E_RANGE, "peer index beyond the key table");
+    return BNK_OK;
+}
+
+} // namespace
+
+extern "C" {
+
+int bnk_init(int device_ordinal, bnk_ctx **out)
+{
+    if (!out) return fail(nullptr, BNK_E_INVAL, "null out pointer");
+    *out = nullptr;
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count <= 0)
+        return fail(nullptr, BNK_E_NODEV, std::string("no HIP device: ") +
+                                              (e != hipSuccess ? hipGetErrorString(e) : "count is 0"));
+    if (device_ordinal < 0 || device_ordinal >= count)
+        return fail(nullptr, BNK_E_NODEV, "device ordinal out of range");
+    hipDeviceProp_t prop;
+    e = hipGetDeviceProperties(&prop, device_ordinal);
+    if (e != hipSuccess) return fail_hip(nullptr, "hipGetDeviceProperties", e);
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(nullptr, BNK_E_NODEV,
+                    std::string("device is ") + prop.gcnArchName + ", this library is built for gfx950");
+    bnk_ctx *ctx = new (std::nothrow) bnk_ctx;
+    if (!ctx) return fail(nullptr, BNK_E_NOMEM, "out of host memory");
+    ctx->device = device_ordinal;
+    auto bail = [&](const char *what, hipError_t err) {
+        int rc = fail_hip(nullptr, what, err);
+        ctx->alive = true;
+        bnk_shutdown(ctx);
+        return rc;
+    };
+    if ((e = hipSetDevice(device_ordinal)) != hipSuccess) return bail("hipSetDevice", e);
+    if ((e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking)) != hipSuccess)
+        return bail("hipStreamCreate", e);
+    if ((e = hipEventCreate(&ctx->ev0)) != hipSuccess) return bail("hipEventCreate", e);
+    if ((e = hipEventCreate(&ctx->ev1)) != hipSuccess) return bail("hipEventCreate", e);
+    if ((e = hipMalloc((void **)&ctx->d_status, 256)) != hipSuccess) return bail("hipMalloc", e);
+    if ((e = launch_fill_u32(ctx->d_status, 64, 0, ctx->stream)) != hipSuccess)
+        return bail("status clear", e);
+    ctx->filter = filter_create();
+    if (!ctx->filter) return bail("filter state", hipErrorOutOfMemory);
+    if ((e = hipStreamSynchronize(ctx->stream)) != hipSuccess) return bail("hipStreamSynchronize", e);
+    ctx->alive = true;
+    *out = ctx;
+    return BNK_OK;
+}
+
+void bnk_shutdown(bnk_ctx *ctx)
+{
+    if (!ctx) return;
+    {
+        std::lock_guard<std::mutex> lk(ctx->mu);
+        if (!ctx->alive) return;
+        ctx->alive = false;
+        (void)hipSetDevice(ctx->device);
+        if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+        for (DevBuf *b : {&ctx->in_arena, &ctx->out_arena, &ctx->off_in, &ctx->off_out, &ctx->lens,
+                          &ctx->peer, &ctx->counters, &ctx->verdict, &ctx->order, &ctx->hist,
+                          &ctx->cursor, &ctx->misc})
+            b->release();
+        ctx->pin.release();
+        for (int w = 0; w < 2; w++)
+            if (ctx->d_keys[w]) (void)hipFree(ctx->d_keys[w]);
+        if (ctx->d_status) (void)hipFree(ctx->d_status);
+        if (ctx->filter) filter_destroy(ctx->filter);
+        if (ctx->ev0) (void)hipEventDestroy(ctx->ev0);
+        if (ctx->ev1) (void)hipEventDestroy(ctx->ev1);
+        if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
+    }
+    delete ctx;
+}
+
+const char *bnk_last_error(bnk_ctx *ctx) { return ctx ? ctx->err.c_str() : g_init_err.c_str(); }
+
+int bnk_ring_alloc(bnk_ctx *ctx, size_t bytes, void **host_pinned)
+{
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    if (!host_pinned || bytes == 0) return fail(ctx, BNK_E_INVAL, "bad ring request");
+    HIPCHK(ctx, hipHostMalloc(host_pinned, bytes, hipHostMallocDefault));
+    return BNK_OK;
+}
+
+int bnk_ring_free(bnk_ctx *ctx, void *host_pinned)
+{
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    if (!host_pinned) return BNK_OK;
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    HIPCHK(ctx, hipHostFree(host_pinned));
+    return BNK_OK;
+}
+
+int bnk_dev_alloc(bnk_ctx *ctx, size_t bytes, void **dev)
+{
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    if (!dev || bytes == 0) return fail(ctx, BNK_E_INVAL, "bad device allocation request");
+    HIPCHK(ctx, hipMalloc(dev, bytes));
+    return BNK_OK;
+}
+
+int bnk_dev_free(bnk_ctx *ctx, void *dev)
+{
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    if (!dev) return BNK_OK;
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    HIPCHK(ctx, hipFree(dev));
+    return BNK_OK;
+}
+
+int bnk_copy_to_device(bnk_ctx *ctx, void *dev, const void *host, size_t bytes)
+{
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    if (bytes == 0) return BNK_OK;
+    if (!dev || !host) return fail(ctx, BNK_E_INVAL, "null pointer");
+    HIPCHK(ctx, hipMemcpyAsync(dev, host, bytes, hipMemcpyHostToDevice, ctx->stream));
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    return BNK_OK;
+}
+
+int bnk_copy_to_host(bnk_ctx *ctx, void *host, const void *dev, size_t bytes)
+{
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    if (bytes == 0) return BNK_OK;
+    if (!dev || !host) return fail(ctx, BNK_E_INVAL, "null pointer");
+    HIPCHK(ctx, hipMemcpyAsync(host, dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    return BNK_OK;
+}
+
+int bnk_sync(bnk_ctx *ctx)
+{
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    uint32_t status = 0;
+    int rc = take_status(ctx, &status);
+    if (rc) return rc;
+    if (status & STATUS_PEER_RANGE) return fail(ctx, BNK_E_RANGE, "peer index beyond the key table");
+    if (status & STATUS_FLOWS_FULL) return fail(ctx, BNK_E_NOMEM, "flow table overflow");
+    return BNK_OK;
+}
+
+void *bnk_stream(bnk_ctx *ctx) { return ctx ? (void *)ctx->stream : nullptr; }
+
+int bnk_keys_set(bnk_ctx *ctx, int which, const uint8_t *keys32, uint32_t n_peers)
+{
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    if (which != BNK_KEYS_SEND && which != BNK_KEYS_RECV)
+        return fail(ctx, BNK_E_INVAL, "bad key table selector");
+    if (!keys32 || n_peers == 0) return fail(ctx, BNK_E_INVAL, "empty key table");
+    // in-flight work may still read the old table
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    uint32_t *nk = nullptr;
+    HIPCHK(ctx, hipMalloc((void **)&nk, (size_t)n_peers * 32));
+    hipError_t e = hipMemcpyAsync(nk, keys32, (size_t)n_peers * 32, hipMemcpyHostToDevice, ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) {
+        (void)hipFree(nk);
+        return fail_hip(ctx, "key upload", e);
+    }
+    if (ctx->d_keys[which]) (void)hipFree(ctx->d_keys[which]);
+    ctx->d_keys[which] = nk;
+    ctx->n_keys[which] = n_peers;
+    return BNK_OK;
+}
+
+int bnk_aead_seal_batch(bnk_ctx *ctx, const bnk_batch *in, const bnk_batch *out)
+{
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    return aead_batch(ctx, false, in, out, nullptr);
+}
+
+int bnk_aead_open_batch(bnk_ctx *ctx, const bnk_batch *in, const bnk_batch *out, uint8_t *verdict)
+{
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    return aead_batch(ctx, true, in, out, verdict);
+}
+
+int bnk_probe_valu(bnk_ctx *ctx, int op, uint32_t iters, double *ops_per_sec)
+{
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    if (!ops_per_sec || iters == 0 || op < 0 || op > 6) return fail(ctx, BNK_E_INVAL, "bad probe request");
+    hipDeviceProp_t prop;
+    HIPCHK(ctx, hipGetDeviceProperties(&prop, ctx->device));
+    // 8 workgroups of 4 waves per CU: every SIMD holds 8 waves
+    const uint32_t blocks = (uint32_t)prop.multiProcessorCount * 8u;
+    HIPCHK(ctx, ctx->misc.reserve((size_t)blocks * PROBE_THREADS * 4));
+    HIPCHK(ctx, launch_probe(op, 4, blocks, ctx->misc.as<uint32_t>(), ctx->stream)); // warm-up
+    HIPCHK(ctx, hipEventRecord(ctx->ev0, ctx->stream));
+    HIPCHK(ctx, launch_probe(op, iters, blocks, ctx->misc.as<uint32_t>(), ctx->stream));
+    HIPCHK(ctx, hipEventRecord(ctx->ev1, ctx->stream));
+    HIPCHK(ctx, hipEventSynchronize(ctx->ev1));
+    float ms = 0;
+    HIPCHK(ctx, hipEventElapsedTime(&ms, ctx->ev0, ctx->ev1));
+    const double ops = (double)blocks * PROBE_THREADS * (double)iters * PROBE_CHAINS * PROBE_UNROLL;
+    *ops_per_sec = ops / ((double)ms * 1e-3);
+    return BNK_OK;
+}
+
+} // extern "C"
+
+#include "filter_api.inc"

@@ -1,0 +1,90 @@
+// Context object and host-side helpers shared by the C ABI entry points.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "../../include/bnkhip.h"
+#include "kernels.hpp"
+
+namespace bnk {
+
+// Grow-only device buffer owned by a context.
+struct DevBuf {
+    void *p = nullptr;
+    size_t cap = 0;
+    hipError_t reserve(size_t bytes)
+    {
+        if (bytes <= cap) return hipSuccess;
+        size_t want = cap ? cap : 4096;
+        while (want < bytes) want *= 2;
+        void *np = nullptr;
+        hipError_t e = hipMalloc(&np, want);
+        if (e != hipSuccess) return e;
+        if (p) (void)hipFree(p);
+        p = np;
+        cap = want;
+        return hipSuccess;
+    }
+    void release()
+    {
+        if (p) (void)hipFree(p);
+        p = nullptr;
+        cap = 0;
+    }
+    template <class T> T *as() const { return static_cast<T *>(p); }
+};
+
+// Grow-only pinned host buffer (staging for gathers from [][]byte).
+struct PinBuf {
+    void *p = nullptr;
+    size_t cap = 0;
+    hipError_t reserve(size_t bytes)
+    {
+        if (bytes <= cap) return hipSuccess;
+        size_t want = cap ? cap : 4096;
+        while (want < bytes) want *= 2;
+        void *np = nullptr;
+        hipError_t e = hipHostMalloc(&np, want, hipHostMallocDefault);
+        if (e != hipSuccess) return e;
+        if (p) (void)hipHostFree(p);
+        p = np;
+        cap = want;
+        return hipSuccess;
+    }
+    void release()
+    {
+        if (p) (void)hipHostFree(p);
+        p = nullptr;
+        cap = 0;
+    }
+    template <class T> T *as() const { return static_cast<T *>(p); }
+};
+
+struct FilterState; // filter_host.hpp
+
+} // namespace bnk
+
+struct bnk_ctx {
+    std::mutex mu;
+    int device = -1;
+    hipStream_t stream = nullptr;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    std::string err;
+    bool alive = false;
+
+    uint32_t *d_keys[2] = {nullptr, nullptr};
+    uint32_t n_keys[2] = {0, 0};
+    uint32_t *d_status = nullptr; // one word, see STATUS_*
+
+    // staging for BNK_MEM_HOST batches and scratch for the length sort
+    bnk::DevBuf in_arena, out_arena, off_in, off_out, lens, peer, counters, verdict;
+    bnk::DevBuf order, hist, cursor, misc;
+    bnk::PinBuf pin;
+
+    bnk::FilterState *filter = nullptr;
+};

@@ -1,0 +1,53 @@
+// Launch interfaces between the C ABI (api.hip) and the gfx950 kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace bnk {
+
+// Device-side view of one AEAD launch.  All pointers are device pointers.
+struct AeadArgs {
+    const uint8_t *in;
+    uint8_t *out;
+    const uint32_t *keys;      // n_peers * 8 little-endian words
+    const uint64_t *in_off;    // or nullptr: i * in_stride
+    const uint64_t *out_off;   // or nullptr: i * out_stride
+    const uint32_t *lens;      // or nullptr: len
+    const uint32_t *peer;      // or nullptr: 0
+    const uint64_t *counters;  // or nullptr: counter0 + i
+    const uint32_t *order;     // or nullptr: lane t handles packet t
+    uint8_t *verdict;          // open only
+    uint32_t *status;          // device status word, bit 0 = peer out of range
+    uint64_t counter0;
+    uint32_t n;
+    uint32_t in_stride, out_stride;
+    uint32_t len;
+    uint32_t n_peers;
+};
+
+enum : uint32_t { STATUS_PEER_RANGE = 1u, STATUS_FLOWS_FULL = 2u };
+
+hipError_t launch_aead_seal(const AeadArgs &a, hipStream_t s);
+hipError_t launch_aead_open(const AeadArgs &a, hipStream_t s);
+
+// order[] = packet indices grouped by ChaCha20 block count, longest first, so
+// the lanes of a wave run the same number of rounds.  hist and cursor are
+// device scratch of LEN_BINS words each.
+constexpr uint32_t LEN_BINS = 1032;
+hipError_t launch_length_sort(const uint32_t *lens, uint32_t n, uint32_t tag_bytes,
+                              uint32_t *order, uint32_t *hist, uint32_t *cursor,
+                              hipStream_t s);
+
+// p[0..n) = v on the stream (a kernel, so it is safe under graph capture).
+hipError_t launch_fill_u32(uint32_t *p, uint32_t n, uint32_t v, hipStream_t s);
+
+// VALU throughput probe; out receives one word per thread so nothing is
+// optimised away.
+hipError_t launch_probe(int op, uint32_t iters, uint32_t blocks, uint32_t *out,
+                        hipStream_t s);
+constexpr uint32_t PROBE_THREADS = 256;
+constexpr uint32_t PROBE_CHAINS = 8;   // independent dependency chains per lane
+constexpr uint32_t PROBE_UNROLL = 16;  // instructions per chain per iteration
+
+} // namespace bnk

@@ -1,0 +1,215 @@
+/*
+ * bnkhip.h -- C ABI of libbnkhip.so: the MI355X (gfx950) implementation of
+ * the bnk packet hot path, batched.
+ *
+ *   WireGuard transport seal/open   ChaCha20-Poly1305 (RFC 8439), nonce =
+ *                                   00 00 00 00 || LE64(counter), empty AAD
+ *   internal/filter verdicts        5-tuple ACL + conntrack flow table
+ *   fused relay                     open -> filter -> re-seal
+ *
+ * This is what a cgo shim in the reference would bind.  Each entry point
+ * names the reference interface it stands behind (paths relative to the
+ * reference tree).  Conventions:
+ *   - plain C types only; every buffer is caller-owned and is not retained
+ *     after the call returns (BNK_MEM_HOST) or after the stream reaches the
+ *     call (BNK_MEM_DEVICE);
+ *   - return value 0 on success, a negative BNK_E_* code on failure; nothing
+ *     aborts or throws across the boundary; bnk_last_error() has the text;
+ *   - calls on one context are serialised by an internal mutex, so Go may
+ *     call from many goroutines (the reference serialises its filter the same
+ *     way, internal/filter/filter.go:34,122,190);
+ *   - there is no CPU fallback: without a gfx950 device bnk_init fails.
+ */
+#ifndef BNKHIP_H
+#define BNKHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct bnk_ctx bnk_ctx;
+
+enum {
+    BNK_OK = 0,
+    BNK_E_INVAL = -1, /* null pointer, bad size, layout outside the arena */
+    BNK_E_NODEV = -2, /* no gfx950 device with that ordinal */
+    BNK_E_HIP = -3,   /* HIP runtime failure */
+    BNK_E_NOMEM = -4, /* host or device allocation failed */
+    BNK_E_RANGE = -5, /* peer index beyond the key table */
+    BNK_E_STATE = -6  /* keys not loaded, context shut down */
+};
+
+/* Where the pointers of a bnk_batch live. */
+enum {
+    BNK_MEM_HOST = 0,  /* host memory (pinned rings from bnk_ring_alloc copy
+                          fastest); the call stages, runs and copies back
+                          before it returns */
+    BNK_MEM_DEVICE = 1 /* device memory of the context's GPU; the call only
+                          enqueues work on the context stream (bnk_sync waits) */
+};
+
+/* WireGuard keeps a sending and a receiving key per peer keypair. */
+enum { BNK_KEYS_SEND = 0, BNK_KEYS_RECV = 1 };
+
+/*
+ * A batch of packets in one arena: the flat form of the [][]byte that
+ * tun.Device.Read/Write and conn.Bind.Send/ReceiveFunc carry
+ * (internal/filter/tun_test.go:19-41, internal/magicsock/bind.go:153,296).
+ * Packet i starts at base + (offsets ? offsets[i] : i * stride) and is
+ * (lens ? lens[i] : len) bytes long.
+ */
+typedef struct bnk_batch {
+    void *base;              /* arena */
+    uint64_t bytes;          /* arena size; every packet must lie inside it */
+    uint32_t n;              /* packets */
+    uint32_t mem;            /* BNK_MEM_HOST or BNK_MEM_DEVICE: applies to base
+                                and to every array below */
+    const uint64_t *offsets; /* n byte offsets, or NULL for a uniform stride */
+    uint32_t stride;         /* used when offsets == NULL */
+    uint32_t len;            /* used when lens == NULL */
+    const uint32_t *lens;    /* n lengths, or NULL for a uniform length */
+    const uint32_t *peer;    /* n indices into the key table, or NULL (peer 0) */
+    const uint64_t *counters;/* n 64-bit nonce counters, or NULL for
+                                counter0 + i */
+    uint64_t counter0;
+} bnk_batch;
+
+/* One allowance: the flat form of acl.CompiledRule (internal/acl/acl.go:33-42)
+ * for a single source prefix and a single port range.  A rule with several
+ * prefixes or ranges is the set of all (prefix, range) pairs, which
+ * Match's any-of semantics (acl.go:149-172) make exact; a tcp/udp rule with
+ * no ranges, or any other proto string, matches nothing and has no tuples. */
+typedef struct bnk_rule {
+    uint32_t src_net;    /* host byte order a<<24|b<<16|c<<8|d */
+    uint32_t src_mask;   /* prefix mask; 0 for /0.  Host bits of src_net outside
+                            the mask are ignored, as netip.Prefix.Contains does */
+    uint16_t port_first; /* inclusive; ignored when proto is 1 (icmp) */
+    uint16_t port_last;
+    uint8_t proto;       /* 1 icmp, 6 tcp, 17 udp; anything else never matches */
+    uint8_t pad[3];
+} bnk_rule;
+
+/* ---- lifetime ---------------------------------------------------------- */
+
+/* Opens device `device_ordinal` (must be gfx950) and creates the context's
+ * stream.  Replaces nothing in the reference: it is the library's init. */
+int bnk_init(int device_ordinal, bnk_ctx **out);
+void bnk_shutdown(bnk_ctx *ctx);
+/* Text of the last failure on this context (or of a failed bnk_init when
+ * ctx is NULL).  Valid until the next call on the context. */
+const char *bnk_last_error(bnk_ctx *ctx);
+
+/* Pinned host packet ring for wireguard-go style buffer pools. */
+int bnk_ring_alloc(bnk_ctx *ctx, size_t bytes, void **host_pinned);
+int bnk_ring_free(bnk_ctx *ctx, void *host_pinned);
+/* Device memory for callers that keep batches resident (BNK_MEM_DEVICE). */
+int bnk_dev_alloc(bnk_ctx *ctx, size_t bytes, void **dev);
+int bnk_dev_free(bnk_ctx *ctx, void *dev);
+int bnk_copy_to_device(bnk_ctx *ctx, void *dev, const void *host, size_t bytes);
+int bnk_copy_to_host(bnk_ctx *ctx, void *host, const void *dev, size_t bytes);
+/* Waits for everything enqueued on the context stream. */
+int bnk_sync(bnk_ctx *ctx);
+/* The context's hipStream_t, for callers that time or order work on it. */
+void *bnk_stream(bnk_ctx *ctx);
+
+/* ---- transport AEAD ---------------------------------------------------- */
+
+/* Loads n_peers 32-byte ChaCha20-Poly1305 keys (host memory) into key table
+ * `which`.  Stands where wireguard-go installs a keypair after the Noise
+ * handshake; the reference never sees these keys itself
+ * (internal/dataplane/engine.go:51 hands everything to device.NewDevice). */
+int bnk_keys_set(bnk_ctx *ctx, int which, const uint8_t *keys32,
+                 uint32_t n_peers);
+
+/* Seal: for every packet, ciphertext (len bytes) then the 16-byte tag are
+ * written at the packet's position in `out` (only base, bytes, mem, offsets,
+ * stride of `out` are read).  Keys come from BNK_KEYS_SEND.  in and out may
+ * be the same arena at the same offsets (in place), as wireguard-go's
+ * AEAD.Seal(header, nonce, plaintext, nil) is. */
+int bnk_aead_seal_batch(bnk_ctx *ctx, const bnk_batch *in,
+                        const bnk_batch *out);
+
+/* Open: packet lengths in `in` include the 16-byte tag.  verdict[i] = 1 and
+ * the plaintext (len-16 bytes) is written when the tag verifies; verdict[i] =
+ * 0 and the plaintext region is zero-filled when it does not (what
+ * chacha20poly1305.Open leaves behind); a packet shorter than 16 bytes gets
+ * verdict 0 and nothing is written.  Keys come from BNK_KEYS_RECV.  `verdict`
+ * lives where in->mem says.  wireguard-go drops packets with verdict 0. */
+int bnk_aead_open_batch(bnk_ctx *ctx, const bnk_batch *in,
+                        const bnk_batch *out, uint8_t *verdict);
+
+/* ---- packet filter ----------------------------------------------------- */
+
+/* filter.SetRules (internal/filter/filter.go:46-51): enforcement on, rule
+ * table replaced; n == 0 is deny-all-but-flows (internal/netmap/netmap.go:49-51).
+ * The flow table is kept.  A fresh context is in allow-all mode (filter.New,
+ * filter.go:41-43). */
+int bnk_filter_set_rules(bnk_ctx *ctx, const bnk_rule *rules, uint32_t n);
+/* filter.SetAllowAll (filter.go:54-59): enforcement off, rules dropped,
+ * flows kept. */
+int bnk_filter_set_allow_all(bnk_ctx *ctx);
+/* filter.NoteOutbound over a batch with one `now` (filter.go:160-167,
+ * 189-209), including the len(flows) > 4096 expiry sweep.  now_ns is the
+ * time.Time as Unix nanoseconds.  peer/counters of the batch are ignored. */
+int bnk_filter_note_outbound_batch(bnk_ctx *ctx, const bnk_batch *pkts,
+                                   int64_t now_ns);
+/* filter.CheckInbound over a batch with one `now` (filter.go:121-147,
+ * 171-178): verdict[i] = 1 pass, 0 drop.  `verdict` lives where pkts->mem
+ * says. */
+int bnk_filter_check_inbound_batch(bnk_ctx *ctx, const bnk_batch *pkts,
+                                   int64_t now_ns, uint8_t *verdict);
+/* The [][]byte form the tun.Device wrapper receives (filter.go:160-186):
+ * n host pointers and lengths.  Only the first 64 bytes of a packet can
+ * matter to the filter (IPv4 header of at most 60 bytes plus 4 port bytes),
+ * so only those are staged. */
+int bnk_filter_note_outbound_ptrs(bnk_ctx *ctx, const uint8_t *const *pkts,
+                                  const uint32_t *lens, uint32_t n,
+                                  int64_t now_ns);
+int bnk_filter_check_inbound_ptrs(bnk_ctx *ctx, const uint8_t *const *pkts,
+                                  const uint32_t *lens, uint32_t n,
+                                  int64_t now_ns, uint8_t *verdict);
+/* len(f.flows): entries currently in the flow table (live or expired but not
+ * yet deleted), as the reference's map would hold. */
+int bnk_filter_flow_count(bnk_ctx *ctx, uint32_t *count);
+/* Copies up to cap flow entries to host arrays: key = remote<<32 |
+ * remotePort<<16 | localPort, proto, expiry in Unix ns (the reference's
+ * flowKey and map value, filter.go:26-31,37).  *count receives the number
+ * written.  Order unspecified. */
+int bnk_filter_flow_dump(bnk_ctx *ctx, uint64_t *key, uint8_t *proto,
+                         int64_t *expiry_ns, uint32_t cap, uint32_t *count);
+
+/* ---- fused relay ------------------------------------------------------- */
+
+enum { BNK_RELAY_OK = 0, BNK_RELAY_FORGED = 1, BNK_RELAY_DENIED = 2 };
+
+/* open (BNK_KEYS_RECV, in->peer, in->counters) -> CheckInbound at now_ns ->
+ * seal under BNK_KEYS_SEND[peer_out[i]] with counter ctr_base_out[peer_out[i]]
+ * + (number of earlier packets in the batch with verdict OK and the same
+ * peer_out).  verdict[i] is BNK_RELAY_*; for OK packets the re-sealed packet
+ * (same length as the input) is written to `out` and its counter to
+ * ctr_out[i]; FORGED and DENIED packets leave `out` untouched and get
+ * ctr_out[i] = 0.  The reference has no such function (its server relays
+ * ciphertext unopened, internal/coord/server/server.go:439-453); this is the
+ * composition of the three steps above.  peer_out, ctr_base_out (n_peers_out
+ * entries), verdict and ctr_out live where in->mem says. */
+int bnk_relay_fused_batch(bnk_ctx *ctx, const bnk_batch *in,
+                          const uint32_t *peer_out,
+                          const uint64_t *ctr_base_out, uint32_t n_peers_out,
+                          int64_t now_ns, const bnk_batch *out,
+                          uint8_t *verdict, uint64_t *ctr_out);
+
+/* ---- measurement ------------------------------------------------------- */
+
+/* Runs a dependency-free VALU instruction stream and reports lane-ops per
+ * second: the measured int32 ceiling the AEAD roofline is quoted against.
+ * op: 0 v_add_u32, 1 v_xor_b32, 2 v_alignbit_b32, 3 v_mad_u64_u32,
+ * 4 v_fma_f64, 5 v_mul_lo_u32, 6 v_add_f64. */
+int bnk_probe_valu(bnk_ctx *ctx, int op, uint32_t iters, double *ops_per_sec);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,239 @@
+"""Parity of the HIP seal/open path (through the C ABI) with the CPU oracle:
+bit-exact ciphertexts, tags, verdicts and rejected-plaintext zeroing."""
+import hashlib
+import json
+import os
+
+import numpy as np
+import pytest
+
+from bnk_amd import workloads as W
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    from bnk_amd import lib
+    c = lib.Context(0)
+    yield c
+    c.close()
+
+
+def _oracle_seal(b):
+    from oracle import binding as O
+    out = np.zeros_like(b.plain)
+    O.seal_batch(np.ascontiguousarray(b.keys), b.peer, b.counters, b.plain, b.off, b.lens,
+                 out, b.off, 4)
+    return out
+
+
+def _gpu_seal_host(ctx, b, uniform):
+    from bnk_amd import lib
+    ctx.keys_set(lib.KEYS_SEND, b.keys)
+    ctx.keys_set(lib.KEYS_RECV, b.keys)
+    out = np.zeros_like(b.plain)
+    if uniform:
+        inb = lib.make_batch(b.plain, b.plain.nbytes, b.n, lib.MEM_HOST, stride=b.stride,
+                             length=int(b.lens[0]), counter0=int(b.counters[0]))
+        outb = lib.make_batch(out, out.nbytes, b.n, lib.MEM_HOST, stride=b.stride)
+    else:
+        inb = lib.make_batch(b.plain, b.plain.nbytes, b.n, lib.MEM_HOST, offsets=b.off,
+                             lens=b.lens, peer=b.peer, counters=b.counters)
+        outb = lib.make_batch(out, out.nbytes, b.n, lib.MEM_HOST, offsets=b.off)
+    ctx.seal(inb, outb)
+    return out
+
+
+def _gpu_open_host(ctx, b, sealed, uniform):
+    from bnk_amd import lib
+    out = np.full_like(b.plain, 0xEE)
+    verdict = np.full(b.n, 7, np.uint8)
+    ct_lens = (b.lens + 16).astype(np.uint32)
+    if uniform:
+        inb = lib.make_batch(sealed, sealed.nbytes, b.n, lib.MEM_HOST, stride=b.stride,
+                             length=int(ct_lens[0]), counter0=int(b.counters[0]))
+        outb = lib.make_batch(out, out.nbytes, b.n, lib.MEM_HOST, stride=b.stride)
+    else:
+        inb = lib.make_batch(sealed, sealed.nbytes, b.n, lib.MEM_HOST, offsets=b.off,
+                             lens=ct_lens, peer=b.peer, counters=b.counters)
+        outb = lib.make_batch(out, out.nbytes, b.n, lib.MEM_HOST, offsets=b.off)
+    ctx.open(inb, outb, verdict)
+    return out, verdict
+
+
+def _packets_equal(a, b, off, lens, extra=0):
+    """Compare only the packet bytes (the gaps of `a` keep their fill)."""
+    for i in range(len(lens)):
+        o, L = int(off[i]), int(lens[i]) + extra
+        if not np.array_equal(a[o:o + L], b[o:o + L]):
+            return i
+    return -1
+
+
+def test_cfg1_against_oracle_and_openssl_fixture(ctx):
+    b = W.aead_uniform(1, 128, 1420)
+    got = _gpu_seal_host(ctx, b, uniform=True)
+    want = _oracle_seal(b)
+    assert np.array_equal(got.reshape(128, b.stride)[:, :1436],
+                          want.reshape(128, b.stride)[:, :1436])
+    # bytes of each slot beyond the tag stay as the caller left them
+    assert not got.reshape(128, b.stride)[:, 1436:].any()
+    g = json.load(open(os.path.join(os.path.dirname(__file__), "golden",
+                                    "aead_cfg1_openssl.json")))
+    sealed = got.reshape(128, b.stride)[:, :1436]
+    assert hashlib.sha256(sealed.tobytes()).hexdigest() == g["sha256_all_sealed"]
+    for idx, hx in g["packets"].items():
+        assert sealed[int(idx)].tobytes().hex() == hx
+    back, verdict = _gpu_open_host(ctx, b, got, uniform=True)
+    assert verdict.tolist() == [1] * 128
+    assert np.array_equal(back.reshape(128, b.stride)[:, :1420],
+                          b.plain.reshape(128, b.stride)[:, :1420])
+    assert (back.reshape(128, b.stride)[:, 1420:] == 0xEE).all()
+
+
+EDGE_LENS = [0, 1, 3, 4, 15, 16, 17, 31, 32, 33, 47, 48, 49, 63, 64, 65, 79, 80, 127, 128, 129,
+             255, 256, 575, 576, 1419, 1420, 1421, 1424, 1500, 4096, 9000]
+
+
+def test_edge_lengths_and_high_counters(ctx):
+    lens = np.array(EDGE_LENS * 3, np.uint32)
+    b = W.aead_imix(11, len(lens), n_peers=5, lens=lens)
+    # counters straddling 2^32 and the top of the 64-bit range
+    b.counters[:8] = np.array([0, 1, 0xFFFFFFFF, 1 << 32, (1 << 32) + 1, (1 << 63),
+                               (1 << 64) - 2, (1 << 64) - 1], np.uint64)
+    got = _gpu_seal_host(ctx, b, uniform=False)
+    want = _oracle_seal(b)
+    assert _packets_equal(got, want, b.off, b.lens, 16) == -1
+    assert np.array_equal(got, want)  # gaps untouched too (both started from zeros)
+    back, verdict = _gpu_open_host(ctx, b, got, uniform=False)
+    assert verdict.all()
+    assert _packets_equal(back, b.plain, b.off, b.lens) == -1
+
+
+def test_imix_multi_peer_with_forged_tags(ctx):
+    from oracle import binding as O
+    b = W.aead_imix(3, 6000, n_peers=256)
+    got = _gpu_seal_host(ctx, b, uniform=False)
+    want = _oracle_seal(b)
+    assert np.array_equal(got, want)
+    forged = W.forge_tags(3, got, b.off, b.lens, 0.01)
+    assert forged.sum() == 60
+    back, verdict = _gpu_open_host(ctx, b, got, uniform=False)
+    oback = np.full_like(b.plain, 0xEE)
+    overdict = O.open_batch(np.ascontiguousarray(b.keys), b.peer, b.counters, got, b.off,
+                            (b.lens + 16).astype(np.uint32), oback, b.off, 4)
+    assert np.array_equal(verdict, overdict)
+    assert np.array_equal(verdict == 0, forged)
+    assert np.array_equal(back, oback)  # rejected plaintexts are zero-filled
+    i = int(np.flatnonzero(forged)[0])
+    o, L = int(b.off[i]), int(b.lens[i])
+    assert not back[o:o + L].any()
+
+
+def test_in_place_and_unaligned_slots(ctx):
+    """WireGuard seals in place at offset 16 of its buffers; slots need not be
+    16-byte aligned."""
+    from bnk_amd import lib
+    from oracle import binding as O
+    n, L, stride = 70, 1001, 1051  # odd stride: every alignment class occurs
+    b = W.aead_uniform(12, n, L, stride=stride, counter0=5)
+    ctx.keys_set(lib.KEYS_SEND, b.keys)
+    ctx.keys_set(lib.KEYS_RECV, b.keys)
+    arena = np.concatenate([np.full(13, 0x5A, np.uint8), b.plain])  # odd base offset
+    view = arena[13:]
+    work = arena.copy()
+    wv = work[13:]
+    inb = lib.make_batch(wv, wv.nbytes, n, lib.MEM_HOST, stride=stride, length=L, counter0=5)
+    ctx.seal(inb, inb)
+    want = np.zeros_like(b.plain)
+    O.seal_batch(np.ascontiguousarray(b.keys), b.peer, b.counters, b.plain, b.off, b.lens,
+                 want, b.off, 2)
+    g2 = wv.reshape(n, stride)
+    w2 = want.reshape(n, stride)
+    assert np.array_equal(g2[:, :L + 16], w2[:, :L + 16])
+    assert np.array_equal(g2[:, L + 16:], view.reshape(n, stride)[:, L + 16:])
+    assert (work[:13] == 0x5A).all()
+    verdict = np.zeros(n, np.uint8)
+    opb = lib.make_batch(wv, wv.nbytes, n, lib.MEM_HOST, stride=stride, length=L + 16, counter0=5)
+    ctx.open(opb, opb, verdict)
+    assert verdict.all()
+    assert np.array_equal(wv.reshape(n, stride)[:, :L], view.reshape(n, stride)[:, :L])
+
+
+def test_short_and_error_paths(ctx):
+    from bnk_amd import lib
+    b = W.aead_uniform(13, 4, 32)
+    ctx.keys_set(lib.KEYS_SEND, b.keys)
+    ctx.keys_set(lib.KEYS_RECV, b.keys)
+    # ciphertext shorter than a tag: verdict 0, nothing written
+    buf = np.zeros(64, np.uint8)
+    out = np.full(64, 0xEE, np.uint8)
+    v = np.full(2, 9, np.uint8)
+    inb = lib.make_batch(buf, 64, 2, lib.MEM_HOST, stride=32, length=15)
+    outb = lib.make_batch(out, 64, 2, lib.MEM_HOST, stride=32)
+    ctx.open(inb, outb, v)
+    assert v.tolist() == [0, 0] and (out == 0xEE).all()
+    # empty batch is a no-op
+    ctx.seal(lib.make_batch(buf, 64, 0, lib.MEM_HOST), lib.make_batch(out, 64, 0, lib.MEM_HOST))
+    # packet outside the arena
+    with pytest.raises(lib.BnkError) as ei:
+        ctx.seal(lib.make_batch(buf, 64, 2, lib.MEM_HOST, stride=32, length=32),
+                 lib.make_batch(out, 64, 2, lib.MEM_HOST, stride=32))
+    assert ei.value.code == lib.E_INVAL
+    # peer beyond the key table
+    with pytest.raises(lib.BnkError) as ei:
+        ctx.seal(lib.make_batch(buf, 64, 2, lib.MEM_HOST, stride=32, length=8,
+                                peer=np.array([0, 3], np.uint32)),
+                 lib.make_batch(out, 64, 2, lib.MEM_HOST, stride=32))
+    assert ei.value.code == lib.E_RANGE
+    # keepalive: empty plaintext seals to just a tag, and opens
+    ka = np.zeros(32, np.uint8)
+    ctx.seal(lib.make_batch(ka, 32, 2, lib.MEM_HOST, stride=16, length=0, counter0=9),
+             lib.make_batch(ka, 32, 2, lib.MEM_HOST, stride=16))
+    from oracle import binding as O
+    assert ka[:16].tobytes() == O.aead_seal(b.keys[0].tobytes(), O.wg_nonce(9), b"")
+    v = np.zeros(2, np.uint8)
+    ctx.open(lib.make_batch(ka, 32, 2, lib.MEM_HOST, stride=16, length=16, counter0=9),
+             lib.make_batch(ka, 32, 2, lib.MEM_HOST, stride=16), v)
+    assert v.tolist() == [1, 1]
+
+
+def test_device_resident_large_batch_properties(ctx):
+    """At a size the oracle cannot finish quickly: seal -> open round trip is
+    the identity, every verdict is 1, and a sample of packets is bit-exact
+    against the oracle."""
+    import torch
+    from bnk_amd import lib
+    from oracle import binding as O
+    n, L, stride = 1 << 18, 1420, 1440
+    key = W.rand_bytes(W.stream_seed(2, 0), 32).reshape(1, 32)
+    ctx.keys_set(lib.KEYS_SEND, key)
+    ctx.keys_set(lib.KEYS_RECV, key)
+    g = torch.Generator(device="cuda").manual_seed(2)
+    pt = torch.randint(0, 256, (n, stride), dtype=torch.uint8, device="cuda", generator=g)
+    ct = torch.zeros_like(pt)
+    back = torch.zeros_like(pt)
+    verdict = torch.zeros(n, dtype=torch.uint8, device="cuda")
+    torch.cuda.synchronize()
+    nb = n * stride
+    ctx.seal(lib.make_batch(pt, nb, n, lib.MEM_DEVICE, stride=stride, length=L, counter0=1000),
+             lib.make_batch(ct, nb, n, lib.MEM_DEVICE, stride=stride))
+    ctx.open(lib.make_batch(ct, nb, n, lib.MEM_DEVICE, stride=stride, length=L + 16,
+                            counter0=1000),
+             lib.make_batch(back, nb, n, lib.MEM_DEVICE, stride=stride), verdict)
+    ctx.sync()
+    assert bool(verdict.all())
+    assert torch.equal(back[:, :L], pt[:, :L])
+    assert not bool(back[:, L:].any())
+    for i in (0, 1, 63, 64, 4097, n - 1):
+        want = O.aead_seal(key.tobytes(), O.wg_nonce(1000 + i), pt[i, :L].cpu().numpy().tobytes())
+        assert ct[i, :L + 16].cpu().numpy().tobytes() == want
+    # linearity of the stream cipher: ct(a) ^ ct(b) == a ^ b under the same nonce
+    pt2 = pt.clone(); pt2[:, :L] ^= 0x3C
+    ct2 = torch.zeros_like(pt)
+    ctx.seal(lib.make_batch(pt2, nb, n, lib.MEM_DEVICE, stride=stride, length=L, counter0=1000),
+             lib.make_batch(ct2, nb, n, lib.MEM_DEVICE, stride=stride))
+    ctx.sync()
+    assert bool(((ct[:, :L] ^ ct2[:, :L]) == 0x3C).all())
+    assert not torch.equal(ct[:, L:L + 16], ct2[:, L:L + 16])

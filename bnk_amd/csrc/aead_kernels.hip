@@ -1,4 +1,5 @@
-// Batched WireGuard transport seal/open for gfx950: one lane per packet.
+// Batched WireGuard transport seal/open for gfx950: one lane per packet for
+// the arithmetic, wave-cooperative coalesced memory traffic through LDS.
 //
 // Stands behind wireguard-go's AEAD.Seal / AEAD.Open calls on transport
 // packets (reached in the reference through device.NewDevice,
@@ -11,24 +12,16 @@
 
 namespace bnk {
 
-template <bool AL>
+// Global memory accesses of 16 bytes at any byte alignment (the hardware
+// handles misaligned dwordx4 accesses; aligned ones cost nothing extra).
 BNK_DEV uint4 ld16(const uint8_t *p)
 {
-    if (AL) return *reinterpret_cast<const uint4 *>(p);
     uint4 v;
     __builtin_memcpy(&v, p, 16);
     return v;
 }
 
-template <bool AL>
-BNK_DEV void st16(uint8_t *p, uint4 v)
-{
-    if (AL) {
-        *reinterpret_cast<uint4 *>(p) = v;
-    } else {
-        __builtin_memcpy(p, &v, 16);
-    }
-}
+BNK_DEV void st16(uint8_t *p, uint4 v) { __builtin_memcpy(p, &v, 16); }
 
 // m in 1..15 bytes at p, zero-extended to 16.
 BNK_DEV uint4 ld_partial(const uint8_t *p, uint32_t m)
@@ -63,132 +56,197 @@ BNK_DEV uint4 keep_bytes(uint4 v, uint32_t m)
     return make_uint4(w[0], w[1], w[2], w[3]);
 }
 
-template <bool AL>
 BNK_DEV void zero_fill(uint8_t *dst, uint32_t len)
 {
     uint32_t pos = 0;
-    for (; pos + 16 <= len; pos += 16) st16<AL>(dst + pos, make_uint4(0, 0, 0, 0));
+    for (; pos + 16 <= len; pos += 16) st16(dst + pos, make_uint4(0, 0, 0, 0));
     for (; pos < len; pos++) dst[pos] = 0;
 }
 
-// len is the plaintext length.  Seal reads len bytes at src and writes
-// len + 16 at dst; open reads len + 16 at src and writes len at dst.
-template <bool OPEN, bool AL>
-BNK_DEV void aead_packet(const uint32_t (&k)[8], uint64_t counter,
-                         const uint8_t *src, uint8_t *dst, uint32_t len,
-                         uint8_t *verdict)
+BNK_DEV uint64_t shfl64(uint64_t v, int src_lane)
 {
-    const uint32_t n1 = (uint32_t)counter, n2 = (uint32_t)(counter >> 32);
+    const uint32_t lo = (uint32_t)__shfl((int)(uint32_t)v, src_lane, 64);
+    const uint32_t hi = (uint32_t)__shfl((int)(uint32_t)(v >> 32), src_lane, 64);
+    return (uint64_t)hi << 32 | lo;
+}
+
+// Orders this wave's LDS traffic: the lanes of a wave run in lockstep and the
+// LDS serves one wave's instructions in order, so no hardware wait is needed,
+// only a barrier the compiler will not move memory operations across.
+BNK_DEV void wave_sync()
+{
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
+
+// One wave = 64 packets, one lane per packet for the arithmetic.  Memory is
+// touched cooperatively: in step b the wave moves bytes [64b, 64b+64) of all
+// its 64 packets with four 16-byte accesses per lane, four adjacent lanes
+// covering one packet's 64 contiguous bytes, and a 64 x 80-byte LDS tile
+// (64 data bytes + 16 bytes of padding per row, which keeps the per-lane row
+// reads free of bank conflicts) turns that layout into one row per lane.
+constexpr uint32_t LDS_ROW = 80;
+constexpr uint32_t WAVES_PER_BLOCK = 4;
+
+template <bool OPEN>
+__global__ __launch_bounds__(256) void aead_wave_kernel(AeadArgs a)
+{
+    __shared__ __attribute__((aligned(16))) uint8_t tile_all[WAVES_PER_BLOCK][64 * LDS_ROW];
+    const uint32_t lane = threadIdx.x & 63u;
+    uint8_t *tile = tile_all[threadIdx.x >> 6];
+    const uint32_t t = blockIdx.x * 256u + threadIdx.x;
+
+    // ---- this lane's packet ----
+    bool have = t < a.n;
+    uint32_t i = 0, len = 0;
+    const uint8_t *src = nullptr;
+    uint8_t *dst = nullptr;
+    uint32_t k[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    uint64_t ctr = 0;
+    if (have) {
+        i = a.order ? a.order[t] : t;
+        len = a.lens ? a.lens[i] : a.len;
+        const uint32_t pr = a.peer ? a.peer[i] : 0u;
+        if (pr >= a.n_peers) {
+            atomicOr(a.status, STATUS_PEER_RANGE);
+            if (OPEN) a.verdict[i] = 0;
+            have = false;
+        } else if (OPEN && len < 16u) {
+            a.verdict[i] = 0;
+            have = false;
+        } else {
+            if (OPEN) len -= 16u;
+            src = a.in + (a.in_off ? a.in_off[i] : (uint64_t)i * a.in_stride);
+            dst = a.out + (a.out_off ? a.out_off[i] : (uint64_t)i * a.out_stride);
+            const uint4 *kp = reinterpret_cast<const uint4 *>(a.keys + 8u * pr);
+            const uint4 k0 = kp[0], k1 = kp[1];
+            k[0] = k0.x; k[1] = k0.y; k[2] = k0.z; k[3] = k0.w;
+            k[4] = k1.x; k[5] = k1.y; k[6] = k1.z; k[7] = k1.w;
+            ctr = a.counters ? a.counters[i] : a.counter0 + i;
+        }
+    }
+    if (!have) len = 0;
+    const uint32_t nfull = len >> 6, rem = len & 63u;
+    const uint32_t steps = nfull + (rem ? 1u : 0u);
+
+    // ---- the four (packet, 16-byte column) cells this lane moves per step ----
+    const uint32_t col = lane & 3u;
+    const uint8_t *csrc[4];
+    uint8_t *cdst[4];
+    uint32_t clen[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int owner = 16 * j + (int)(lane >> 2);
+        csrc[j] = reinterpret_cast<const uint8_t *>(shfl64((uint64_t)(uintptr_t)src, owner)) + 16u * col;
+        cdst[j] = reinterpret_cast<uint8_t *>(shfl64((uint64_t)(uintptr_t)dst, owner)) + 16u * col;
+        clen[j] = (uint32_t)__shfl((int)len, owner, 64);
+    }
+
+    const uint32_t n1 = (uint32_t)ctr, n2 = (uint32_t)(ctr >> 32);
     uint32_t x[16];
     chacha_block(k, 0, n1, n2, x);
     Poly26 mac;
     mac.init(x);
 
-    const uint32_t nfull = len >> 6;
-    for (uint32_t b = 0; b < nfull; b++) {
-        chacha_block(k, b + 1, n1, n2, x);
-        const uint8_t *s = src + 64u * b;
-        uint8_t *d = dst + 64u * b;
+    for (uint32_t b = 0; __ballot(b < steps) != 0ull; b++) {
+        const uint32_t pos = 64u * b + 16u * col;
+        // global -> LDS, all 64 lanes, only 16-byte cells that lie fully inside a packet
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            const uint4 v = ld16<AL>(s + 16 * j);
-            const uint4 o = make_uint4(v.x ^ x[4 * j], v.y ^ x[4 * j + 1],
-                                       v.z ^ x[4 * j + 2], v.w ^ x[4 * j + 3]);
-            if (OPEN) mac.block(v.x, v.y, v.z, v.w);
-            else mac.block(o.x, o.y, o.z, o.w);
-            st16<AL>(d + 16 * j, o);
-        }
-    }
-    const uint32_t rem = len & 63u;
-    if (rem) {
-        chacha_block(k, nfull + 1, n1, n2, x);
-        const uint8_t *s = src + 64u * nfull;
-        uint8_t *d = dst + 64u * nfull;
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            if (rem >= 16u * (j + 1)) {
-                const uint4 v = ld16<AL>(s + 16 * j);
-                const uint4 o = make_uint4(v.x ^ x[4 * j], v.y ^ x[4 * j + 1],
-                                           v.z ^ x[4 * j + 2], v.w ^ x[4 * j + 3]);
-                if (OPEN) mac.block(v.x, v.y, v.z, v.w);
-                else mac.block(o.x, o.y, o.z, o.w);
-                st16<AL>(d + 16 * j, o);
-            } else if (rem > 16u * j) {
-                const uint32_t m = rem - 16u * j;
-                const uint4 v = ld_partial(s + 16 * j, m);
-                const uint4 o = keep_bytes(
-                    make_uint4(v.x ^ x[4 * j], v.y ^ x[4 * j + 1],
-                               v.z ^ x[4 * j + 2], v.w ^ x[4 * j + 3]), m);
-                // the MAC sees the ciphertext zero-padded to 16 bytes
-                if (OPEN) mac.block(v.x, v.y, v.z, v.w);
-                else mac.block(o.x, o.y, o.z, o.w);
-                st_partial(d + 16 * j, o, m);
+            if (pos + 16u <= clen[j]) {
+                const uint4 v = ld16(csrc[j] + 64u * b);
+                *reinterpret_cast<uint4 *>(tile + (16u * j + (lane >> 2)) * LDS_ROW + 16u * col) = v;
             }
         }
-    }
-    // LE64(len(aad) = 0) || LE64(len(ciphertext))
-    mac.block(0, 0, len, 0);
-    uint32_t tag[4];
-    mac.finish(tag);
-
-    if (!OPEN) {
-        st16<false>(dst + len, make_uint4(tag[0], tag[1], tag[2], tag[3]));
-    } else {
-        const uint4 t = ld16<false>(src + len);
-        // all 16 bytes are compared, no early exit
-        const uint32_t diff = (t.x ^ tag[0]) | (t.y ^ tag[1]) | (t.z ^ tag[2]) |
-                              (t.w ^ tag[3]);
-        const bool ok = diff == 0;
-        *verdict = ok ? 1 : 0;
-        if (!ok) zero_fill<AL>(dst, len);
-    }
-}
-
-template <bool OPEN>
-__global__ __launch_bounds__(256) void aead_lane_kernel(AeadArgs a)
-{
-    const uint32_t t = blockIdx.x * 256u + threadIdx.x;
-    if (t >= a.n) return;
-    const uint32_t i = a.order ? a.order[t] : t;
-    uint32_t len = a.lens ? a.lens[i] : a.len;
-    const uint64_t ioff = a.in_off ? a.in_off[i] : (uint64_t)i * a.in_stride;
-    const uint64_t ooff = a.out_off ? a.out_off[i] : (uint64_t)i * a.out_stride;
-    const uint32_t pr = a.peer ? a.peer[i] : 0u;
-    if (pr >= a.n_peers) {
-        atomicOr(a.status, STATUS_PEER_RANGE);
-        if (OPEN) a.verdict[i] = 0;
-        return;
-    }
-    if (OPEN) {
-        if (len < 16u) {
-            a.verdict[i] = 0;
-            return;
+        wave_sync();
+        if (b < steps) {
+            chacha_block(k, b + 1, n1, n2, x);
+            uint8_t *row = tile + lane * LDS_ROW;
+            if (b < nfull) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const uint4 v = *reinterpret_cast<const uint4 *>(row + 16 * j);
+                    const uint4 o = make_uint4(v.x ^ x[4 * j], v.y ^ x[4 * j + 1],
+                                               v.z ^ x[4 * j + 2], v.w ^ x[4 * j + 3]);
+                    if (OPEN) mac.block(v.x, v.y, v.z, v.w);
+                    else mac.block(o.x, o.y, o.z, o.w);
+                    *reinterpret_cast<uint4 *>(row + 16 * j) = o;
+                }
+            } else {
+                // last, partial block: whole cells through the tile, the
+                // final 1..15 bytes straight from and to global memory
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    if (rem >= 16u * (j + 1)) {
+                        const uint4 v = *reinterpret_cast<const uint4 *>(row + 16 * j);
+                        const uint4 o = make_uint4(v.x ^ x[4 * j], v.y ^ x[4 * j + 1],
+                                                   v.z ^ x[4 * j + 2], v.w ^ x[4 * j + 3]);
+                        if (OPEN) mac.block(v.x, v.y, v.z, v.w);
+                        else mac.block(o.x, o.y, o.z, o.w);
+                        *reinterpret_cast<uint4 *>(row + 16 * j) = o;
+                    } else if (rem > 16u * j) {
+                        const uint32_t m = rem - 16u * j;
+                        const uint4 v = ld_partial(src + 64u * b + 16 * j, m);
+                        const uint4 o = keep_bytes(
+                            make_uint4(v.x ^ x[4 * j], v.y ^ x[4 * j + 1],
+                                       v.z ^ x[4 * j + 2], v.w ^ x[4 * j + 3]), m);
+                        // the MAC sees the ciphertext zero-padded to 16 bytes
+                        if (OPEN) mac.block(v.x, v.y, v.z, v.w);
+                        else mac.block(o.x, o.y, o.z, o.w);
+                        st_partial(dst + 64u * b + 16 * j, o, m);
+                    }
+                }
+            }
         }
-        len -= 16u;
+        wave_sync();
+        // LDS -> global
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            if (pos + 16u <= clen[j]) {
+                const uint4 v = *reinterpret_cast<const uint4 *>(
+                    tile + (16u * j + (lane >> 2)) * LDS_ROW + 16u * col);
+                st16(cdst[j] + 64u * b, v);
+            }
+        }
+        wave_sync();
     }
-    const uint4 *kp = reinterpret_cast<const uint4 *>(a.keys + 8u * pr);
-    const uint4 k0 = kp[0], k1 = kp[1];
-    const uint32_t k[8] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
-    const uint64_t ctr = a.counters ? a.counters[i] : a.counter0 + i;
-    const uint8_t *src = a.in + ioff;
-    uint8_t *dst = a.out + ooff;
-    uint8_t *vd = OPEN ? a.verdict + i : nullptr;
-    const bool al = (((uintptr_t)src | (uintptr_t)dst) & 15u) == 0;
-    if (al) aead_packet<OPEN, true>(k, ctr, src, dst, len, vd);
-    else aead_packet<OPEN, false>(k, ctr, src, dst, len, vd);
+
+    bool reject = false;
+    if (have) {
+        // LE64(len(aad) = 0) || LE64(len(ciphertext))
+        mac.block(0, 0, len, 0);
+        uint32_t tag[4];
+        mac.finish(tag);
+        if (!OPEN) {
+            st16(dst + len, make_uint4(tag[0], tag[1], tag[2], tag[3]));
+        } else {
+            const uint4 tg = ld16(src + len);
+            // all 16 bytes are compared, no early exit
+            const uint32_t diff = (tg.x ^ tag[0]) | (tg.y ^ tag[1]) | (tg.z ^ tag[2]) |
+                                  (tg.w ^ tag[3]);
+            reject = diff != 0;
+            a.verdict[i] = reject ? 0 : 1;
+        }
+    }
+    if (OPEN && __ballot(reject) != 0ull) {
+        // the plaintext cells were stored by other lanes of this wave: make
+        // those stores land before this lane overwrites them with zeros
+        __threadfence();
+        if (reject) zero_fill(dst, len);
+    }
 }
 
 hipError_t launch_aead_seal(const AeadArgs &a, hipStream_t s)
 {
     if (a.n == 0) return hipSuccess;
-    hipLaunchKernelGGL(aead_lane_kernel<false>, dim3((a.n + 255u) / 256u), dim3(256), 0, s, a);
+    hipLaunchKernelGGL(aead_wave_kernel<false>, dim3((a.n + 255u) / 256u), dim3(256), 0, s, a);
     return hipGetLastError();
 }
 
 hipError_t launch_aead_open(const AeadArgs &a, hipStream_t s)
 {
     if (a.n == 0) return hipSuccess;
-    hipLaunchKernelGGL(aead_lane_kernel<true>, dim3((a.n + 255u) / 256u), dim3(256), 0, s, a);
+    hipLaunchKernelGGL(aead_wave_kernel<true>, dim3((a.n + 255u) / 256u), dim3(256), 0, s, a);
     return hipGetLastError();
 }
 

@@ -478,7 +478,7 @@ int bnk_probe_valu(bnk_ctx *ctx, int op, uint32_t iters, double *ops_per_sec)
 {
     Guard g(ctx);
     if (g.rc) return g.rc;
-    if (!ops_per_sec || iters == 0 || op < 0 || op > 6) return fail(ctx, BNK_E_INVAL, "bad probe request");
+    if (!ops_per_sec || iters == 0 || op < 0 || op >= PROBE_OPS) return fail(ctx, BNK_E_INVAL, "bad probe request");
     hipDeviceProp_t prop;
     HIPCHK(ctx, hipGetDeviceProperties(&prop, ctx->device));
     // 8 workgroups of 4 waves per CU: every SIMD holds 8 waves

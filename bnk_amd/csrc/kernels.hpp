@@ -46,6 +46,7 @@ hipError_t launch_fill_u32(uint32_t *p, uint32_t n, uint32_t v, hipStream_t s);
 // optimised away.
 hipError_t launch_probe(int op, uint32_t iters, uint32_t blocks, uint32_t *out,
                         hipStream_t s);
+constexpr int PROBE_OPS = 24;
 constexpr uint32_t PROBE_THREADS = 256;
 constexpr uint32_t PROBE_CHAINS = 8;   // independent dependency chains per lane
 constexpr uint32_t PROBE_UNROLL = 16;  // instructions per chain per iteration

@@ -35,6 +35,27 @@ __global__ __launch_bounds__(256) void probe_kernel(uint32_t iters, uint32_t *ou
                 if (OP == 4) asm volatile("v_fma_f64 %0, %0, %1, %2" : "+v"(d[c]) : "v"(one), "v"(zero));
                 if (OP == 5) asm volatile("v_mul_lo_u32 %0, %0, %1" : "+v"(a[c]) : "v"(b));
                 if (OP == 6) asm volatile("v_add_f64 %0, %0, %1" : "+v"(d[c]) : "v"(zero));
+                if (OP == 7) asm volatile("v_add_u32_e64 %0, %0, %1" : "+v"(a[c]) : "v"(b));
+                if (OP == 8) asm volatile("v_xad_u32 %0, %0, %1, %2" : "+v"(a[c]) : "v"(b), "v"(m));
+                if (OP == 9) asm volatile("v_add3_u32 %0, %0, %1, %2" : "+v"(a[c]) : "v"(b), "v"(m));
+                if (OP == 10) asm volatile("v_perm_b32 %0, %0, %0, %1" : "+v"(a[c]) : "v"(m));
+                if (OP == 11) asm volatile("v_lshl_or_b32 %0, %0, 7, %1" : "+v"(a[c]) : "v"(b));
+                if (OP == 12)
+                    asm volatile("v_xor_b32_sdwa %0, %0, %1 dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE "
+                                 "src0_sel:WORD_0 src1_sel:WORD_0" : "+v"(a[c]) : "v"(b));
+                if (OP == 13)
+                    asm volatile("v_mov_b32_dpp %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf"
+                                 : "+v"(a[c]));
+                if (OP == 14) asm volatile("v_lshlrev_b32 %0, 7, %0" : "+v"(a[c]));
+                if (OP == 15) asm volatile("v_and_or_b32 %0, %0, %1, %2" : "+v"(a[c]) : "v"(b), "v"(m));
+                if (OP == 16) asm volatile("v_bfe_u32 %0, %0, 3, 22" : "+v"(a[c]));
+                if (OP == 17) asm volatile("v_mad_u32_u24 %0, %0, %1, %2" : "+v"(a[c]) : "v"(b), "v"(m));
+                if (OP == 18) asm volatile("v_pk_add_u16 %0, %0, %1" : "+v"(a[c]) : "v"(b));
+                if (OP == 19) asm volatile("v_alignbit_b32 %0, %0, %1, 7" : "+v"(a[c]) : "v"(b));
+                if (OP == 20) asm volatile("v_mul_u32_u24 %0, %0, %1" : "+v"(a[c]) : "v"(b));
+                if (OP == 21) asm volatile("v_mul_f64 %0, %0, %1" : "+v"(d[c]) : "v"(one));
+                if (OP == 22) asm volatile("v_add_f32 %0, %0, %1" : "+v"(a[c]) : "v"(b));
+                if (OP == 23) asm volatile("v_fma_f32 %0, %0, %1, %2" : "+v"(a[c]) : "v"(b), "v"(m));
             }
         }
     }
@@ -45,19 +66,20 @@ __global__ __launch_bounds__(256) void probe_kernel(uint32_t iters, uint32_t *ou
     out[tid] = acc;
 }
 
+template <int OP>
+static hipError_t probe_dispatch(int op, uint32_t iters, uint32_t blocks, uint32_t *out, hipStream_t s)
+{
+    if (op == OP) {
+        hipLaunchKernelGGL(probe_kernel<OP>, dim3(blocks), dim3(256), 0, s, iters, out);
+        return hipGetLastError();
+    }
+    if constexpr (OP + 1 < PROBE_OPS) return probe_dispatch<OP + 1>(op, iters, blocks, out, s);
+    return hipErrorInvalidValue;
+}
+
 hipError_t launch_probe(int op, uint32_t iters, uint32_t blocks, uint32_t *out, hipStream_t s)
 {
-    switch (op) {
-    case 0: hipLaunchKernelGGL(probe_kernel<0>, dim3(blocks), dim3(256), 0, s, iters, out); break;
-    case 1: hipLaunchKernelGGL(probe_kernel<1>, dim3(blocks), dim3(256), 0, s, iters, out); break;
-    case 2: hipLaunchKernelGGL(probe_kernel<2>, dim3(blocks), dim3(256), 0, s, iters, out); break;
-    case 3: hipLaunchKernelGGL(probe_kernel<3>, dim3(blocks), dim3(256), 0, s, iters, out); break;
-    case 4: hipLaunchKernelGGL(probe_kernel<4>, dim3(blocks), dim3(256), 0, s, iters, out); break;
-    case 5: hipLaunchKernelGGL(probe_kernel<5>, dim3(blocks), dim3(256), 0, s, iters, out); break;
-    case 6: hipLaunchKernelGGL(probe_kernel<6>, dim3(blocks), dim3(256), 0, s, iters, out); break;
-    default: return hipErrorInvalidValue;
-    }
-    return hipGetLastError();
+    return probe_dispatch<0>(op, iters, blocks, out, s);
 }
 
 } // namespace bnk

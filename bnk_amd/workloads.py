@@ -46,6 +46,36 @@ def rand_bytes(seed: int, nbytes: int) -> np.ndarray:
     return words.view(np.uint8)[:nbytes].copy()
 
 
+def rand_bytes_torch(seed: int, nbytes: int, device):
+    """Same bytes as rand_bytes, produced by torch on ``device`` (int64
+    arithmetic wraps like uint64; right shifts are made logical by masking)."""
+    import torch
+    n = (nbytes + 7) // 8
+
+    def lsr(z, s):
+        return (z >> s) & ((1 << (64 - s)) - 1)
+
+    def s64(v):  # Python int -> the int64 with the same 64-bit pattern
+        v &= 0xFFFFFFFFFFFFFFFF
+        return v - (1 << 64) if v >= (1 << 63) else v
+
+    k = torch.arange(1, n + 1, dtype=torch.int64, device=device)
+    z = k * s64(0x9E3779B97F4A7C15) + s64(seed)
+    z = (z ^ lsr(z, 30)) * s64(0xBF58476D1CE4E5B9)
+    z = (z ^ lsr(z, 27)) * s64(0x94D049BB133111EB)
+    z = z ^ lsr(z, 31)
+    return z.view(torch.uint8)[:nbytes]
+
+
+def aead_uniform_torch(cfg: int, n: int, length: int, stride: int, device):
+    """The plaintext arena of aead_uniform(cfg, n, length, stride) as a torch
+    uint8 tensor [n, stride] on ``device``, byte for byte."""
+    import torch
+    plain = torch.zeros((n, stride), dtype=torch.uint8, device=device)
+    plain[:, :length] = rand_bytes_torch(stream_seed(cfg, 1), n * length, device).view(n, length)
+    return plain
+
+
 def rand_u64(seed: int, n: int) -> np.ndarray:
     return splitmix64(seed, n)
 

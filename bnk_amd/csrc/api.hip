@@ -1,91 +1,11 @@
 // C ABI of libbnkhip.so (see include/bnkhip.h): argument checking, staging of
 // host batches through the context's device buffers, kernel launches.
-#include <string.h>
-
-#include <algorithm>
-#include <new>
-
-#include "ctx.hpp"
+#include "api_common.hpp"
 #include "filter_host.hpp"
 
 using namespace bnk;
 
 namespace {
-
-thread_local std::string g_init_err;
-
-int fail(bnk_ctx *ctx, int code, const std::string &what)
-{
-    if (ctx) ctx->err = what;
-    else g_init_err = what;
-    return code;
-}
-
-int fail_hip(bnk_ctx *ctx, const char *what, hipError_t e)
-{
-    return fail(ctx, e == hipErrorOutOfMemory ? BNK_E_NOMEM : BNK_E_HIP,
-                std::string(what) + ": " + hipGetErrorString(e));
-}
-
-#define HIPCHK(ctx, expr)                                         \
-    do {                                                          \
-        hipError_t e_ = (expr);                                   \
-        if (e_ != hipSuccess) return fail_hip((ctx), #expr, e_);  \
-    } while (0)
-
-// Every entry point takes the context lock and makes the context's device
-// current for the calling thread.
-struct Guard {
-    std::unique_lock<std::mutex> lk;
-    int rc = BNK_OK;
-    explicit Guard(bnk_ctx *ctx)
-    {
-        if (!ctx) { rc = fail(nullptr, BNK_E_INVAL, "null context"); return; }
-        lk = std::unique_lock<std::mutex>(ctx->mu);
-        if (!ctx->alive) { rc = fail(ctx, BNK_E_STATE, "context is shut down"); return; }
-        hipError_t e = hipSetDevice(ctx->device);
-        if (e != hipSuccess) rc = fail_hip(ctx, "hipSetDevice", e);
-    }
-};
-
-inline uint64_t pkt_off(const bnk_batch *b, uint32_t i)
-{
-    return b->offsets ? b->offsets[i] : (uint64_t)i * b->stride;
-}
-
-struct Span {
-    uint64_t lo = UINT64_MAX, hi = 0;
-    void add(uint64_t a, uint64_t b) { lo = std::min(lo, a); hi = std::max(hi, b); }
-    uint64_t size() const { return hi > lo ? hi - lo : 0; }
-};
-
-// Checks that packet i of a host batch occupies [off, off + len + delta)
-// inside the arena and accumulates the touched span.  lens come from `src`
-// (the input batch) because an output batch only carries a layout.
-int scan_host_layout(bnk_ctx *ctx, const bnk_batch *lay, const bnk_batch *src, int delta,
-                     Span *span, const char *name)
-{
-    const uint32_t n = src->n;
-    for (uint32_t i = 0; i < n; i++) {
-        const uint64_t off = pkt_off(lay, i);
-        int64_t len = (int64_t)(src->lens ? src->lens[i] : src->len) + delta;
-        if (len < 0) len = 0;
-        if (off > lay->bytes || (uint64_t)len > lay->bytes - off)
-            return fail(ctx, BNK_E_INVAL, std::string(name) + ": packet " + std::to_string(i) +
-                                              " lies outside the arena");
-        span->add(off, off + (uint64_t)len);
-    }
-    return BNK_OK;
-}
-
-int check_batch_common(bnk_ctx *ctx, const bnk_batch *b, const char *name)
-{
-    if (!b) return fail(ctx, BNK_E_INVAL, std::string(name) + ": null batch");
-    if (b->mem != BNK_MEM_HOST && b->mem != BNK_MEM_DEVICE)
-        return fail(ctx, BNK_E_INVAL, std::string(name) + ": bad mem kind");
-    if (b->n && !b->base) return fail(ctx, BNK_E_INVAL, std::string(name) + ": null arena");
-    return BNK_OK;
-}
 
 // Host-resident view of a batch staged on the device.
 struct Staged {
@@ -203,15 +123,6 @@ int maybe_sort(bnk_ctx *ctx, const uint32_t *d_lens, uint32_t n, uint32_t tag_by
     return BNK_OK;
 }
 
-// Reads and clears the device status word; the stream must be idle.
-int take_status(bnk_ctx *ctx, uint32_t *status)
-{
-    HIPCHK(ctx, hipMemcpyAsync(status, ctx->d_status, 4, hipMemcpyDeviceToHost, ctx->stream));
-    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
-    if (*status) HIPCHK(ctx, launch_fill_u32(ctx->d_status, 1, 0, ctx->stream));
-    return BNK_OK;
-}
-
 int aead_batch(bnk_ctx *ctx, bool open, const bnk_batch *in, const bnk_batch *out,
                uint8_t *verdict)
 {
@@ -286,11 +197,30 @@ int aead_batch(bnk_ctx *ctx, bool open, const bnk_batch *in, const bnk_batch *ou
     uint32_t status = 0;
     rc = take_status(ctx, &status);
     if (rc) return rc;
-    if (status & STATUS_PEER_RANGE) return fail(ctx, BNK_E_RANGE, "peer index beyond the key table");
-    return BNK_OK;
+    return status_to_rc(ctx, status);
 }
 
 } // namespace
+
+namespace bnk {
+
+// Reads and clears the device status word; the stream must be idle.
+int take_status(bnk_ctx *ctx, uint32_t *status)
+{
+    HIPCHK(ctx, hipMemcpyAsync(status, ctx->d_status, 4, hipMemcpyDeviceToHost, ctx->stream));
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    if (*status) HIPCHK(ctx, launch_fill_u32(ctx->d_status, 1, 0, ctx->stream));
+    return BNK_OK;
+}
+
+int status_to_rc(bnk_ctx *ctx, uint32_t status)
+{
+    if (status & STATUS_PEER_RANGE) return fail(ctx, BNK_E_RANGE, "peer index beyond the key table");
+    if (status & STATUS_FLOWS_FULL) return fail(ctx, BNK_E_NOMEM, "flow table overflow");
+    return BNK_OK;
+}
+
+} // namespace bnk
 
 extern "C" {
 
@@ -328,7 +258,7 @@ int bnk_init(int device_ordinal, bnk_ctx **out)
     if ((e = hipMalloc((void **)&ctx->d_status, 256)) != hipSuccess) return bail("hipMalloc", e);
     if ((e = launch_fill_u32(ctx->d_status, 64, 0, ctx->stream)) != hipSuccess)
         return bail("status clear", e);
-    ctx->filter = filter_create();
+    ctx->filter = filter_create(ctx->stream, prop.multiProcessorCount);
     if (!ctx->filter) return bail("filter state", hipErrorOutOfMemory);
     if ((e = hipStreamSynchronize(ctx->stream)) != hipSuccess) return bail("hipStreamSynchronize", e);
     ctx->alive = true;
@@ -430,9 +360,7 @@ int bnk_sync(bnk_ctx *ctx)
     uint32_t status = 0;
     int rc = take_status(ctx, &status);
     if (rc) return rc;
-    if (status & STATUS_PEER_RANGE) return fail(ctx, BNK_E_RANGE, "peer index beyond the key table");
-    if (status & STATUS_FLOWS_FULL) return fail(ctx, BNK_E_NOMEM, "flow table overflow");
-    return BNK_OK;
+    return status_to_rc(ctx, status);
 }
 
 void *bnk_stream(bnk_ctx *ctx) { return ctx ? (void *)ctx->stream : nullptr; }
@@ -497,5 +425,3 @@ int bnk_probe_valu(bnk_ctx *ctx, int op, uint32_t iters, double *ops_per_sec)
 }
 
 } // extern "C"
-
-#include "filter_api.inc"

@@ -1,0 +1,377 @@
+// C ABI entry points of the packet filter (see include/bnkhip.h).
+#include "api_common.hpp"
+#include "filter_host.hpp"
+
+using namespace bnk;
+
+namespace bnk {
+
+static hipError_t flow_table_alloc(uint32_t cap, DevBuf &keys, DevBuf &exp, DevBuf &counters,
+                                   FlowTableDev &ft, hipStream_t s)
+{
+    const size_t slots = (size_t)cap * FLOW_REGIONS;
+    hipError_t e;
+    if ((e = keys.reserve(slots * 8)) != hipSuccess) return e;
+    if ((e = exp.reserve(slots * 8)) != hipSuccess) return e;
+    if ((e = counters.reserve(FLOW_COUNTERS * 4)) != hipSuccess) return e;
+    ft.keys = keys.as<uint64_t>();
+    ft.exp = exp.as<int64_t>();
+    ft.counters = counters.as<uint32_t>();
+    ft.cap = cap;
+    if ((e = launch_fill_u64(ft.keys, (uint32_t)slots, 0, s)) != hipSuccess) return e;
+    if ((e = launch_fill_u64(reinterpret_cast<uint64_t *>(ft.exp), (uint32_t)slots,
+                             (uint64_t)FLOW_TOMB, s)) != hipSuccess)
+        return e;
+    return launch_fill_u32(ft.counters, FLOW_COUNTERS, 0, s);
+}
+
+static hipError_t upload_rule_index(FilterState *f, const HostRuleIndex &h, hipStream_t s)
+{
+    hipError_t e;
+    const size_t nb = h.bounds.size();
+    if ((e = f->bounds.reserve(std::max<size_t>(nb, 1) * 4)) != hipSuccess) return e;
+    if ((e = f->starts.reserve((nb + 1) * 4)) != hipSuccess) return e;
+    if ((e = f->ranges.reserve(std::max<size_t>(h.ranges.size(), 1) * 8)) != hipSuccess) return e;
+    if ((e = f->wide.reserve(std::max<size_t>(h.wide.size(), 1) * 16)) != hipSuccess) return e;
+    if ((e = hipMemcpyAsync(f->bounds.p, h.bounds.data(), nb * 4, hipMemcpyHostToDevice, s)) != hipSuccess)
+        return e;
+    if ((e = hipMemcpyAsync(f->starts.p, h.starts.data(), (nb + 1) * 4, hipMemcpyHostToDevice, s)) !=
+        hipSuccess)
+        return e;
+    if (!h.ranges.empty() &&
+        (e = hipMemcpyAsync(f->ranges.p, h.ranges.data(), h.ranges.size() * 8, hipMemcpyHostToDevice,
+                            s)) != hipSuccess)
+        return e;
+    if (!h.wide.empty() &&
+        (e = hipMemcpyAsync(f->wide.p, h.wide.data(), h.wide.size() * 16, hipMemcpyHostToDevice, s)) !=
+            hipSuccess)
+        return e;
+    // the host vectors die with the caller's frame
+    if ((e = hipStreamSynchronize(s)) != hipSuccess) return e;
+    f->ridx.bounds = f->bounds.as<uint32_t>();
+    f->ridx.starts = f->starts.as<uint32_t>();
+    f->ridx.ranges = f->ranges.as<uint2>();
+    f->ridx.wide = f->wide.as<uint4>();
+    f->ridx.n_bounds = (uint32_t)nb;
+    f->ridx.n_wide = (uint32_t)h.wide.size();
+    uint32_t step = 0;
+    if (nb >= 2) {
+        step = 1;
+        while ((size_t)step * 2 <= nb - 1) step *= 2;
+    }
+    f->ridx.top_step = step;
+    return hipSuccess;
+}
+
+FilterState *filter_create(hipStream_t s, int cu_count)
+{
+    FilterState *f = new (std::nothrow) FilterState;
+    if (!f) return nullptr;
+    f->max_blocks = (uint32_t)std::max(cu_count, 1) * 8u;
+    HostRuleIndex h;
+    std::string err;
+    build_rule_index(nullptr, 0, h, err);
+    if (flow_table_alloc(FLOW_CAP_INITIAL, f->keys, f->exp, f->counters, f->flows, s) != hipSuccess ||
+        upload_rule_index(f, h, s) != hipSuccess) {
+        filter_destroy(f);
+        return nullptr;
+    }
+    return f;
+}
+
+void filter_destroy(FilterState *f)
+{
+    if (!f) return;
+    f->release();
+    delete f;
+}
+
+} // namespace bnk
+
+namespace {
+
+// Makes room for n_new more distinct flows: open addressing stays below half
+// full per region, growing (and dropping tombstones) when it would not.
+int flows_reserve(bnk_ctx *ctx, uint32_t n_new)
+{
+    FilterState *f = ctx->filter;
+    const uint64_t half = f->flows.cap / 2;
+    if (f->claimed_upper + n_new <= half) {
+        f->claimed_upper += n_new;
+        return BNK_OK;
+    }
+    uint32_t c[FLOW_COUNTERS];
+    HIPCHK(ctx, hipMemcpyAsync(c, f->flows.counters, sizeof c, hipMemcpyDeviceToHost, ctx->stream));
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    f->claimed_upper = c[FLOW_CLAIMED];
+    if (f->claimed_upper + n_new <= half) {
+        f->claimed_upper += n_new;
+        return BNK_OK;
+    }
+    uint64_t need = 4ull * ((uint64_t)c[FLOW_LIVE] + n_new); // at most a quarter full afterwards
+    uint64_t cap = FLOW_CAP_INITIAL;
+    while (cap < need) cap *= 2;
+    if (cap > FLOW_CAP_MAX) return fail(ctx, BNK_E_NOMEM, "flow table would exceed its maximum size");
+    DevBuf nk, ne, nc;
+    FlowTableDev nt{};
+    hipError_t e = flow_table_alloc((uint32_t)cap, nk, ne, nc, nt, ctx->stream);
+    if (e == hipSuccess)
+        e = launch_flow_rehash(f->flows, nt, ctx->d_status, f->max_blocks, ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (e != hipSuccess) {
+        nk.release(); ne.release(); nc.release();
+        return fail_hip(ctx, "flow table growth", e);
+    }
+    f->keys.release(); f->exp.release(); f->counters.release();
+    f->keys = nk; f->exp = ne; f->counters = nc;
+    f->flows = nt;
+    f->claimed_upper = (uint64_t)c[FLOW_LIVE] + n_new;
+    return BNK_OK;
+}
+
+// The filter reads at most the first 64 bytes of a packet (IPv4 header of up
+// to 60 bytes, then 4 port bytes): host packets are gathered at a 64-byte
+// stride into pinned staging and only that is uploaded.
+constexpr uint32_t HDR_BYTES = 64;
+
+template <class GetPtr, class GetLen>
+int stage_headers(bnk_ctx *ctx, uint32_t n, GetPtr ptr_of, GetLen len_of, FilterArgs *a)
+{
+    const size_t hdr_bytes = (size_t)n * HDR_BYTES, len_bytes = (size_t)n * 4;
+    HIPCHK(ctx, ctx->pin.reserve(hdr_bytes + len_bytes));
+    uint8_t *hp = ctx->pin.as<uint8_t>();
+    uint32_t *hl = reinterpret_cast<uint32_t *>(hp + hdr_bytes);
+    for (uint32_t i = 0; i < n; i++) {
+        const uint32_t len = len_of(i);
+        hl[i] = len;
+        const uint32_t c = len < HDR_BYTES ? len : HDR_BYTES;
+        if (c) memcpy(hp + (size_t)i * HDR_BYTES, ptr_of(i), c);
+    }
+    HIPCHK(ctx, ctx->in_arena.reserve(hdr_bytes));
+    HIPCHK(ctx, ctx->lens.reserve(len_bytes));
+    HIPCHK(ctx, hipMemcpyAsync(ctx->in_arena.p, hp, hdr_bytes, hipMemcpyHostToDevice, ctx->stream));
+    HIPCHK(ctx, hipMemcpyAsync(ctx->lens.p, hl, len_bytes, hipMemcpyHostToDevice, ctx->stream));
+    a->pkts = ctx->in_arena.as<uint8_t>();
+    a->off = nullptr;
+    a->stride = HDR_BYTES;
+    a->lens = ctx->lens.as<uint32_t>();
+    return BNK_OK;
+}
+
+void base_args(bnk_ctx *ctx, uint32_t n, int64_t now_ns, FilterArgs *a)
+{
+    *a = FilterArgs{};
+    a->n = n;
+    a->now = now_ns;
+    a->status = ctx->d_status;
+    a->rules = ctx->filter->ridx;
+    a->flows = ctx->filter->flows;
+}
+
+int check_device_layout(bnk_ctx *ctx, const bnk_batch *b)
+{
+    if (!b->offsets && !b->lens && b->n &&
+        (uint64_t)(b->n - 1) * b->stride + b->len > b->bytes)
+        return fail(ctx, BNK_E_INVAL, "pkts: uniform layout exceeds the arena");
+    return BNK_OK;
+}
+
+int filter_batch(bnk_ctx *ctx, bool check, const bnk_batch *pkts, int64_t now_ns, uint8_t *verdict)
+{
+    int rc = check_batch_common(ctx, pkts, "pkts");
+    if (rc) return rc;
+    const uint32_t n = pkts->n;
+    if (n == 0) return BNK_OK;
+    if (check && !verdict) return fail(ctx, BNK_E_INVAL, "null verdict array");
+    FilterState *f = ctx->filter;
+    if (!f->enforce) {
+        // filter.go:124-126 / :192-194
+        if (!check) return BNK_OK;
+        if (pkts->mem == BNK_MEM_HOST) memset(verdict, 1, n);
+        else HIPCHK(ctx, launch_fill_u8(verdict, n, 1, ctx->stream));
+        return BNK_OK;
+    }
+    if (!check) {
+        rc = flows_reserve(ctx, n);
+        if (rc) return rc;
+    }
+    FilterArgs a;
+    base_args(ctx, n, now_ns, &a);
+    if (pkts->mem == BNK_MEM_DEVICE) {
+        rc = check_device_layout(ctx, pkts);
+        if (rc) return rc;
+        a.pkts = (const uint8_t *)pkts->base;
+        a.off = pkts->offsets;
+        a.lens = pkts->lens;
+        a.stride = pkts->stride;
+        a.len = pkts->len;
+        a.verdict = verdict;
+        HIPCHK(ctx, check ? launch_filter_check(a, f->max_blocks, ctx->stream)
+                          : launch_filter_note(a, f->max_blocks, ctx->stream));
+        return BNK_OK;
+    }
+    Span span;
+    rc = scan_host_layout(ctx, pkts, pkts, 0, &span, "pkts");
+    if (rc) return rc;
+    const uint8_t *base = (const uint8_t *)pkts->base;
+    rc = stage_headers(
+        ctx, n, [&](uint32_t i) { return base + pkt_off(pkts, i); },
+        [&](uint32_t i) { return pkts->lens ? pkts->lens[i] : pkts->len; }, &a);
+    if (rc) return rc;
+    if (check) {
+        HIPCHK(ctx, ctx->verdict.reserve(n));
+        a.verdict = ctx->verdict.as<uint8_t>();
+        HIPCHK(ctx, launch_filter_check(a, f->max_blocks, ctx->stream));
+        HIPCHK(ctx, hipMemcpyAsync(verdict, a.verdict, n, hipMemcpyDeviceToHost, ctx->stream));
+    } else {
+        HIPCHK(ctx, launch_filter_note(a, f->max_blocks, ctx->stream));
+    }
+    uint32_t status = 0;
+    rc = take_status(ctx, &status);
+    if (rc) return rc;
+    return status_to_rc(ctx, status);
+}
+
+int filter_ptrs(bnk_ctx *ctx, bool check, const uint8_t *const *pkts, const uint32_t *lens,
+                uint32_t n, int64_t now_ns, uint8_t *verdict)
+{
+    if (n == 0) return BNK_OK;
+    if (!pkts || !lens) return fail(ctx, BNK_E_INVAL, "null packet list");
+    if (check && !verdict) return fail(ctx, BNK_E_INVAL, "null verdict array");
+    for (uint32_t i = 0; i < n; i++)
+        if (lens[i] && !pkts[i]) return fail(ctx, BNK_E_INVAL, "null packet pointer");
+    FilterState *f = ctx->filter;
+    if (!f->enforce) {
+        if (check) memset(verdict, 1, n);
+        return BNK_OK;
+    }
+    int rc;
+    if (!check) {
+        rc = flows_reserve(ctx, n);
+        if (rc) return rc;
+    }
+    FilterArgs a;
+    base_args(ctx, n, now_ns, &a);
+    rc = stage_headers(
+        ctx, n, [&](uint32_t i) { return pkts[i]; }, [&](uint32_t i) { return lens[i]; }, &a);
+    if (rc) return rc;
+    if (check) {
+        HIPCHK(ctx, ctx->verdict.reserve(n));
+        a.verdict = ctx->verdict.as<uint8_t>();
+        HIPCHK(ctx, launch_filter_check(a, f->max_blocks, ctx->stream));
+        HIPCHK(ctx, hipMemcpyAsync(verdict, a.verdict, n, hipMemcpyDeviceToHost, ctx->stream));
+    } else {
+        HIPCHK(ctx, launch_filter_note(a, f->max_blocks, ctx->stream));
+    }
+    uint32_t status = 0;
+    rc = take_status(ctx, &status);
+    if (rc) return rc;
+    return status_to_rc(ctx, status);
+}
+
+} // namespace
+
+extern "C" {
+
+int bnk_filter_set_rules(bnk_ctx *ctx, const bnk_rule *rules, uint32_t n)
+{
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    if (n && !rules) return fail(ctx, BNK_E_INVAL, "null rule array");
+    HostRuleIndex h;
+    std::string err;
+    if (!build_rule_index(rules, n, h, err)) return fail(ctx, BNK_E_INVAL, err);
+    // work already queued may still read the old tables
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    HIPCHK(ctx, upload_rule_index(ctx->filter, h, ctx->stream));
+    ctx->filter->enforce = true;
+    return BNK_OK;
+}
+
+int bnk_filter_set_allow_all(bnk_ctx *ctx)
+{
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    HostRuleIndex h;
+    std::string err;
+    build_rule_index(nullptr, 0, h, err);
+    HIPCHK(ctx, upload_rule_index(ctx->filter, h, ctx->stream));
+    ctx->filter->enforce = false;
+    return BNK_OK;
+}
+
+int bnk_filter_note_outbound_batch(bnk_ctx *ctx, const bnk_batch *pkts, int64_t now_ns)
+{
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    return filter_batch(ctx, false, pkts, now_ns, nullptr);
+}
+
+int bnk_filter_check_inbound_batch(bnk_ctx *ctx, const bnk_batch *pkts, int64_t now_ns,
+                                   uint8_t *verdict)
+{
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    return filter_batch(ctx, true, pkts, now_ns, verdict);
+}
+
+int bnk_filter_note_outbound_ptrs(bnk_ctx *ctx, const uint8_t *const *pkts, const uint32_t *lens,
+                                  uint32_t n, int64_t now_ns)
+{
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    return filter_ptrs(ctx, false, pkts, lens, n, now_ns, nullptr);
+}
+
+int bnk_filter_check_inbound_ptrs(bnk_ctx *ctx, const uint8_t *const *pkts, const uint32_t *lens,
+                                  uint32_t n, int64_t now_ns, uint8_t *verdict)
+{
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    return filter_ptrs(ctx, true, pkts, lens, n, now_ns, verdict);
+}
+
+int bnk_filter_flow_count(bnk_ctx *ctx, uint32_t *count)
+{
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    if (!count) return fail(ctx, BNK_E_INVAL, "null count");
+    uint32_t c[FLOW_COUNTERS];
+    HIPCHK(ctx, hipMemcpyAsync(c, ctx->filter->flows.counters, sizeof c, hipMemcpyDeviceToHost,
+                               ctx->stream));
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    *count = c[FLOW_LIVE];
+    return BNK_OK;
+}
+
+int bnk_filter_flow_dump(bnk_ctx *ctx, uint64_t *key, uint8_t *proto, int64_t *expiry_ns,
+                         uint32_t cap, uint32_t *count)
+{
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    if (!count || (cap && (!key || !proto || !expiry_ns))) return fail(ctx, BNK_E_INVAL, "null output");
+    const FlowTableDev &ft = ctx->filter->flows;
+    const size_t slots = (size_t)ft.cap * FLOW_REGIONS;
+    std::vector<uint64_t> hk(slots);
+    std::vector<int64_t> he(slots);
+    HIPCHK(ctx, hipMemcpyAsync(hk.data(), ft.keys, slots * 8, hipMemcpyDeviceToHost, ctx->stream));
+    HIPCHK(ctx, hipMemcpyAsync(he.data(), ft.exp, slots * 8, hipMemcpyDeviceToHost, ctx->stream));
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    static const uint8_t class_proto[3] = {1, 6, 17};
+    uint32_t k = 0;
+    for (size_t idx = 0; idx < slots && k < cap; idx++) {
+        if (hk[idx] == 0 || he[idx] == FLOW_TOMB) continue;
+        const uint32_t region = (uint32_t)(idx / ft.cap);
+        const uint64_t w = hk[idx];
+        const uint64_t remote = ((uint64_t)(region & 1u) << 31) | ((w >> 32) & 0x7FFFFFFFu);
+        key[k] = remote << 32 | (w & 0xFFFFFFFFu);
+        proto[k] = class_proto[region >> 1];
+        expiry_ns[k] = he[idx];
+        k++;
+    }
+    *count = k;
+    return BNK_OK;
+}
+
+} // extern "C"

@@ -1,0 +1,52 @@
+// Device-side views of the filter's tables, shared by kernels and host code.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace bnk {
+
+constexpr uint32_t FLOW_REGIONS = 6;     // protocol class (3) x top address bit (2)
+constexpr int64_t FLOW_TOMB = INT64_MIN; // expiry of a deleted (or never used) slot
+enum : uint32_t { FLOW_LIVE = 0, FLOW_CLAIMED = 1, FLOW_SWEEP = 2, FLOW_COUNTERS = 4 };
+
+struct FlowTableDev {
+    uint64_t *keys;     // [FLOW_REGIONS * cap], 0 = empty
+    int64_t *exp;       // [FLOW_REGIONS * cap] expiry in Unix ns, FLOW_TOMB = not in the map
+    uint32_t *counters; // [FLOW_COUNTERS]: entries in the map, slots ever claimed, sweep flag
+    uint32_t cap;       // slots per region, a power of two
+};
+
+struct RuleIndexDev {
+    const uint32_t *bounds; // [n_bounds] ascending starts of the elementary source intervals
+    const uint32_t *starts; // [n_bounds + 1] offsets into ranges
+    const uint2 *ranges;    // sorted disjoint (key_lo, key_hi) per interval
+    const uint4 *wide;      // [n_wide] (net, mask, key_lo, key_hi) scanned by every packet
+    uint32_t n_bounds;
+    uint32_t top_step;      // largest power of two < n_bounds (0 when n_bounds == 1)
+    uint32_t n_wide;
+};
+
+struct FilterArgs {
+    const uint8_t *pkts;
+    const uint64_t *off;  // or nullptr: i * stride
+    const uint32_t *lens; // or nullptr: len
+    const uint8_t *gate;  // or nullptr; gate[i] == 0 skips packet i (verdict 0)
+    uint8_t *verdict;     // check only
+    uint32_t *status;
+    int64_t now;
+    uint32_t n, stride, len;
+    uint32_t trim;        // bytes at the end of each packet that are not payload
+    RuleIndexDev rules;
+    FlowTableDev flows;
+};
+
+hipError_t launch_fill_u64(uint64_t *p, uint32_t n, uint64_t v, hipStream_t s);
+hipError_t launch_fill_u8(uint8_t *p, uint32_t n, uint8_t v, hipStream_t s);
+hipError_t launch_filter_check(const FilterArgs &a, uint32_t max_blocks, hipStream_t s);
+// inserts, then the reference's conditional expiry sweep
+hipError_t launch_filter_note(const FilterArgs &a, uint32_t max_blocks, hipStream_t s);
+hipError_t launch_flow_rehash(const FlowTableDev &from, const FlowTableDev &to, uint32_t *status,
+                              uint32_t max_blocks, hipStream_t s);
+
+} // namespace bnk

@@ -258,3 +258,126 @@ def icmp_echo(src: int, dst: int, reply: bool = False) -> bytes:
     hdr = bytearray(8)
     hdr[0] = 0 if reply else 8
     return ipv4(1, src, dst, bytes(hdr))
+
+
+# --------------------------------------------------------------------------
+# ACL / conntrack workload (configuration 4)
+# --------------------------------------------------------------------------
+
+CGNAT_BASE = 100 << 24 | 64 << 16  # 100.64.0.0/10
+RECORD_STRIDE = 32                 # 20-byte IPv4 header + 8 L4 bytes, padded to 32
+_WELL_KNOWN = (80, 443, 22, 53, 25, 123, 8080, 3389, 5432, 3306, 6379, 8443, 21, 23, 110, 143)
+
+
+def zipf_ports(seed: int, n: int, s: float = 1.1) -> np.ndarray:
+    """Ports drawn from Zipf(s) over ranks 1..65535; rank 1.. map to the
+    well-known ports above, the remaining ranks to a seeded permutation of all
+    other ports."""
+    ranks = np.arange(1, 65536, dtype=np.float64)
+    cdf = np.cumsum(ranks ** (-s))
+    cdf /= cdf[-1]
+    u = (splitmix64(seed, n) >> np.uint64(11)).astype(np.float64) / float(1 << 53)
+    r = np.searchsorted(cdf, u, side="left")
+    rest = np.setdiff1d(np.arange(1, 65536, dtype=np.uint32), np.array(_WELL_KNOWN, np.uint32))
+    rest = rest[permutation(seed ^ 0x5A5A, rest.shape[0])]
+    table = np.concatenate([np.array(_WELL_KNOWN, np.uint32), rest])
+    return table[np.minimum(r, table.shape[0] - 1)].astype(np.uint32)
+
+
+def proto_mix(seed: int, n: int) -> np.ndarray:
+    """TCP:UDP:ICMP = 6:3:1 as IP protocol numbers."""
+    r = rand_below(seed, n, 10)
+    return np.where(r < 6, 6, np.where(r < 9, 17, 1)).astype(np.uint32)
+
+
+def header_records(proto: np.ndarray, src: np.ndarray, dst: np.ndarray, sport: np.ndarray,
+                   dport: np.ndarray) -> np.ndarray:
+    """[n, 32] u8 records: IPv4 header as filter_test.go:13-24 builds it (0x45,
+    total length 28, TTL 64) followed by 8 L4 bytes (ports first for TCP/UDP;
+    echo request type 8 for ICMP)."""
+    n = proto.shape[0]
+    rec = np.zeros((n, RECORD_STRIDE), np.uint8)
+    rec[:, 0] = 0x45
+    rec[:, 3] = 28
+    rec[:, 8] = 64
+    rec[:, 9] = proto
+    for k in range(4):
+        rec[:, 12 + k] = (src >> (24 - 8 * k)) & 0xFF
+        rec[:, 16 + k] = (dst >> (24 - 8 * k)) & 0xFF
+    l4 = proto != 1
+    rec[l4, 20] = (sport[l4] >> 8) & 0xFF
+    rec[l4, 21] = sport[l4] & 0xFF
+    rec[l4, 22] = (dport[l4] >> 8) & 0xFF
+    rec[l4, 23] = dport[l4] & 0xFF
+    rec[~l4, 20] = 8
+    return rec
+
+
+@dataclass
+class AclWorkload:
+    rules_ref: list            # [(srcs, proto_name, ports)] in the reference's shape
+    rule_tuples: np.ndarray    # [n_rules, 5] u32: net, mask, first, last, proto
+    note_batches: list         # [(now_ns, records [m, 32] u8)] ascending in time
+    check: np.ndarray          # [n, 32] u8 records
+    now_ns: int
+    record_len: int = 28
+
+
+def acl_workload(cfg: int = 4, n: int = 1 << 22, n_rules: int = 4096, n_flows: int = 65536,
+                 note_rounds: int = 16, mirror_fraction: float = 0.125) -> AclWorkload:
+    """Configuration 4: ``n`` inbound headers against ``n_rules`` single-prefix
+    single-range rules and a flow table built by ``n_flows`` earlier outbound
+    packets noted at t0 - U[0, 150 s) (so some are expired at check time t0)."""
+    ss = lambda k: stream_seed(cfg, k)  # noqa: E731
+    # rules: prefix length uniform /16../32 under 100.64/10, proto 6:3:1, one
+    # port range (half single ports, else geometric width)
+    bits = 16 + rand_below(ss(10), n_rules, 17)
+    host = rand_below(ss(11), n_rules, 1 << 22)
+    mask = ((0xFFFFFFFF << (32 - bits.astype(np.uint64))) & 0xFFFFFFFF).astype(np.uint32)
+    net = ((CGNAT_BASE | host) & mask).astype(np.uint32)
+    rproto = proto_mix(ss(12), n_rules)
+    first = zipf_ports(ss(13), n_rules)
+    single = rand_below(ss(14), n_rules, 2) == 0
+    u = (splitmix64(ss(15), n_rules) >> np.uint64(11)).astype(np.float64) / float(1 << 53)
+    width = np.where(single, 0, np.floor(np.log(np.maximum(u, 1e-12)) / np.log(0.99)).astype(np.int64))
+    last = np.minimum(first.astype(np.int64) + width, 65535).astype(np.uint32)
+    tuples = np.stack([net, mask, first, last, rproto], axis=1).astype(np.uint32)
+    name = {6: "tcp", 17: "udp", 1: "icmp"}
+    rules_ref = [([(int(net[i]), int(bits[i]))], name[int(rproto[i])],
+                  [] if rproto[i] == 1 else [(int(first[i]), int(last[i]))]) for i in range(n_rules)]
+
+    # earlier outbound traffic from this host
+    self_addr = CGNAT_BASE | 1
+    fproto = proto_mix(ss(20), n_flows)
+    fdst = (CGNAT_BASE | rand_below(ss(21), n_flows, 1 << 22)).astype(np.uint32)
+    fsport = (32768 + rand_below(ss(22), n_flows, 28000)).astype(np.uint32)
+    fdport = zipf_ports(ss(23), n_flows)
+    age_ns = (splitmix64(ss(24), n_flows) % np.uint64(150 * 1_000_000_000)).astype(np.int64)
+    order = np.argsort(-age_ns, kind="stable")  # oldest first
+    rec = header_records(fproto, np.full(n_flows, self_addr, np.uint32), fdst, fsport, fdport)
+    note_batches = []
+    for chunk in np.array_split(order, note_rounds):
+        if chunk.shape[0] == 0:
+            continue
+        # one `now` per batch, as one tun.Read delivers: the batch's newest packet
+        now = T0_NS - int(age_ns[chunk].min())
+        note_batches.append((now, np.ascontiguousarray(rec[chunk])))
+
+    # inbound headers to check at t0
+    cproto = proto_mix(ss(30), n)
+    csrc = (CGNAT_BASE | rand_below(ss(31), n, 1 << 22)).astype(np.uint32)
+    cdst = np.full(n, self_addr, np.uint32)
+    csport = zipf_ports(ss(32), n)
+    cdport = zipf_ports(ss(33), n)
+    # a seeded share of them are replies to recorded flows
+    m = int(mirror_fraction * n)
+    if m and n_flows:
+        which = permutation(ss(34), n)[:m]
+        pick = rand_below(ss(35), m, n_flows)
+        cproto[which] = fproto[pick]
+        csrc[which] = fdst[pick]
+        csport[which] = fdport[pick]
+        cdport[which] = fsport[pick]
+    check = header_records(cproto, csrc, cdst, csport, cdport)
+    return AclWorkload(rules_ref=rules_ref, rule_tuples=tuples, note_batches=note_batches,
+                       check=check, now_ns=T0_NS)

@@ -106,8 +106,11 @@ __global__ __launch_bounds__(256) void aead_wave_kernel(AeadArgs a)
     if (have) {
         i = a.order ? a.order[t] : t;
         len = a.lens ? a.lens[i] : a.len;
+        if (!OPEN) len = len >= a.trim ? len - a.trim : 0u;
         const uint32_t pr = a.peer ? a.peer[i] : 0u;
-        if (pr >= a.n_peers) {
+        if (a.skip && a.skip[i] != 0) {
+            have = false;
+        } else if (pr >= a.n_peers) {
             atomicOr(a.status, STATUS_PEER_RANGE);
             if (OPEN) a.verdict[i] = 0;
             have = false;

@@ -7,122 +7,6 @@ using namespace bnk;
 
 namespace {
 
-// Host-resident view of a batch staged on the device.
-struct Staged {
-    uint8_t *d_in = nullptr, *d_out = nullptr;
-    const uint64_t *d_in_off = nullptr, *d_out_off = nullptr;
-    const uint32_t *d_lens = nullptr, *d_peer = nullptr;
-    const uint64_t *d_counters = nullptr;
-    Span sin, sout;
-    bool in_place = false;
-};
-
-bool same_layout(const bnk_batch *a, const bnk_batch *b)
-{
-    if (a->base != b->base) return false;
-    if (a->offsets || b->offsets) return a->offsets == b->offsets;
-    return a->stride == b->stride;
-}
-
-// Copies the rebased offsets of `lay` into pinned staging at `slot` and
-// queues the upload.
-int upload_offsets(bnk_ctx *ctx, const bnk_batch *lay, uint32_t n, uint64_t lo, DevBuf *dst,
-                   size_t pin_off, const uint64_t **out)
-{
-    if (!lay->offsets) { *out = nullptr; return BNK_OK; }
-    HIPCHK(ctx, dst->reserve((size_t)n * 8));
-    uint64_t *h = reinterpret_cast<uint64_t *>(ctx->pin.as<uint8_t>() + pin_off);
-    for (uint32_t i = 0; i < n; i++) h[i] = lay->offsets[i] - lo;
-    HIPCHK(ctx, hipMemcpyAsync(dst->p, h, (size_t)n * 8, hipMemcpyHostToDevice, ctx->stream));
-    *out = dst->as<uint64_t>();
-    return BNK_OK;
-}
-
-// Stages a host input batch (and the layout of its output batch) on the
-// device.  in_delta/out_delta adjust the per-packet byte counts: seal writes
-// len + 16, open writes len - 16.
-int stage_host(bnk_ctx *ctx, const bnk_batch *in, const bnk_batch *out, int out_delta,
-               uint32_t n_keys, Staged *st)
-{
-    const uint32_t n = in->n;
-    int rc = scan_host_layout(ctx, in, in, 0, &st->sin, "in");
-    if (rc) return rc;
-    rc = scan_host_layout(ctx, out, in, out_delta, &st->sout, "out");
-    if (rc) return rc;
-    if (in->peer)
-        for (uint32_t i = 0; i < n; i++)
-            if (in->peer[i] >= n_keys)
-                return fail(ctx, BNK_E_RANGE, "peer index " + std::to_string(in->peer[i]) +
-                                                  " beyond the key table");
-    // pinned staging for the two rebased offset arrays
-    HIPCHK(ctx, ctx->pin.reserve((size_t)n * 16 + 64));
-
-    st->in_place = same_layout(in, out);
-    if (st->in_place) {
-        Span u = st->sin;
-        u.add(st->sout.lo, st->sout.hi);
-        st->sin = st->sout = u;
-    }
-    HIPCHK(ctx, ctx->in_arena.reserve(st->sin.size() + 16));
-    st->d_in = ctx->in_arena.as<uint8_t>();
-    HIPCHK(ctx, hipMemcpyAsync(st->d_in, (const uint8_t *)in->base + st->sin.lo, st->sin.size(),
-                               hipMemcpyHostToDevice, ctx->stream));
-    if (st->in_place) {
-        st->d_out = st->d_in;
-    } else {
-        HIPCHK(ctx, ctx->out_arena.reserve(st->sout.size() + 16));
-        st->d_out = ctx->out_arena.as<uint8_t>();
-        // bytes between packets of the output arena must survive the round
-        // trip, so the device copy starts from the host's content
-        HIPCHK(ctx, hipMemcpyAsync(st->d_out, (const uint8_t *)out->base + st->sout.lo,
-                                   st->sout.size(), hipMemcpyHostToDevice, ctx->stream));
-    }
-    rc = upload_offsets(ctx, in, n, st->sin.lo, &ctx->off_in, 0, &st->d_in_off);
-    if (rc) return rc;
-    if (st->in_place) {
-        st->d_out_off = st->d_in_off;
-    } else {
-        rc = upload_offsets(ctx, out, n, st->sout.lo, &ctx->off_out, (size_t)n * 8, &st->d_out_off);
-        if (rc) return rc;
-    }
-    if (in->lens) {
-        HIPCHK(ctx, ctx->lens.reserve((size_t)n * 4));
-        HIPCHK(ctx, hipMemcpyAsync(ctx->lens.p, in->lens, (size_t)n * 4, hipMemcpyHostToDevice,
-                                   ctx->stream));
-        st->d_lens = ctx->lens.as<uint32_t>();
-    }
-    if (in->peer) {
-        HIPCHK(ctx, ctx->peer.reserve((size_t)n * 4));
-        HIPCHK(ctx, hipMemcpyAsync(ctx->peer.p, in->peer, (size_t)n * 4, hipMemcpyHostToDevice,
-                                   ctx->stream));
-        st->d_peer = ctx->peer.as<uint32_t>();
-    }
-    if (in->counters) {
-        HIPCHK(ctx, ctx->counters.reserve((size_t)n * 8));
-        HIPCHK(ctx, hipMemcpyAsync(ctx->counters.p, in->counters, (size_t)n * 8,
-                                   hipMemcpyHostToDevice, ctx->stream));
-        st->d_counters = ctx->counters.as<uint64_t>();
-    }
-    return BNK_OK;
-}
-
-// Lanes of a wave should run the same number of ChaCha20 blocks: when lengths
-// vary, hand packets to lanes in length order.
-int maybe_sort(bnk_ctx *ctx, const uint32_t *d_lens, uint32_t n, uint32_t tag_bytes,
-               const uint32_t **order)
-{
-    *order = nullptr;
-    if (!d_lens || n <= 64) return BNK_OK;
-    HIPCHK(ctx, ctx->order.reserve((size_t)n * 4));
-    HIPCHK(ctx, ctx->hist.reserve(LEN_BINS * 4));
-    HIPCHK(ctx, ctx->cursor.reserve(LEN_BINS * 4));
-    HIPCHK(ctx, launch_length_sort(d_lens, n, tag_bytes, ctx->order.as<uint32_t>(),
-                                   ctx->hist.as<uint32_t>(), ctx->cursor.as<uint32_t>(),
-                                   ctx->stream));
-    *order = ctx->order.as<uint32_t>();
-    return BNK_OK;
-}
-
 int aead_batch(bnk_ctx *ctx, bool open, const bnk_batch *in, const bnk_batch *out,
                uint8_t *verdict)
 {
@@ -277,7 +161,9 @@ void bnk_shutdown(bnk_ctx *ctx)
         if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
         for (DevBuf *b : {&ctx->in_arena, &ctx->out_arena, &ctx->off_in, &ctx->off_out, &ctx->lens,
                           &ctx->peer, &ctx->counters, &ctx->verdict, &ctx->order, &ctx->hist,
-                          &ctx->cursor, &ctx->misc})
+                          &ctx->cursor, &ctx->misc, &ctx->r_plain, &ctx->r_auth, &ctx->r_pass,
+                          &ctx->r_keys, &ctx->r_idx, &ctx->r_skeys, &ctx->r_sidx, &ctx->r_tmp,
+                          &ctx->r_peer_out, &ctx->r_ctr_base, &ctx->r_ctr_out, &ctx->r_verdict})
             b->release();
         ctx->pin.release();
         for (int w = 0; w < 2; w++)

@@ -85,6 +85,9 @@ struct bnk_ctx {
     bnk::DevBuf in_arena, out_arena, off_in, off_out, lens, peer, counters, verdict;
     bnk::DevBuf order, hist, cursor, misc;
     bnk::PinBuf pin;
+    // fused relay: plaintext scratch, per-packet flags, sort buffers, staged arrays
+    bnk::DevBuf r_plain, r_auth, r_pass, r_keys, r_idx, r_skeys, r_sidx, r_tmp;
+    bnk::DevBuf r_peer_out, r_ctr_base, r_ctr_out, r_verdict;
 
     bnk::FilterState *filter = nullptr;
 };

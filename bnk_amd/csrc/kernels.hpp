@@ -18,12 +18,14 @@ struct AeadArgs {
     const uint64_t *counters;  // or nullptr: counter0 + i
     const uint32_t *order;     // or nullptr: lane t handles packet t
     uint8_t *verdict;          // open only
+    const uint8_t *skip;       // or nullptr; skip[i] != 0 leaves packet i alone
     uint32_t *status;          // device status word, bit 0 = peer out of range
     uint64_t counter0;
     uint32_t n;
     uint32_t in_stride, out_stride;
     uint32_t len;
     uint32_t n_peers;
+    uint32_t trim;             // seal only: lens[i] - trim is the plaintext length
 };
 
 enum : uint32_t { STATUS_PEER_RANGE = 1u, STATUS_FLOWS_FULL = 2u };
@@ -41,6 +43,16 @@ hipError_t launch_length_sort(const uint32_t *lens, uint32_t n, uint32_t tag_byt
 
 // p[0..n) = v on the stream (a kernel, so it is safe under graph capture).
 hipError_t launch_fill_u32(uint32_t *p, uint32_t n, uint32_t v, hipStream_t s);
+
+// Fused relay bookkeeping (relay_kernels.hip).  After open (auth[i]) and the
+// filter (pass[i]): verdicts, then per-peer batch-order counters for the
+// survivors.  sort_tmp holds sort_tmp_bytes of scratch (relay_sort_tmp_bytes).
+size_t relay_sort_tmp_bytes(uint32_t n);
+hipError_t launch_relay_assign(const uint8_t *auth, const uint8_t *pass, const uint32_t *peer_out,
+                               const uint64_t *ctr_base_out, uint32_t n_peers_out, uint32_t n,
+                               uint32_t *keys, uint32_t *idx, uint32_t *skeys, uint32_t *sidx,
+                               void *sort_tmp, size_t sort_tmp_bytes, uint8_t *verdict,
+                               uint64_t *ctr_out, uint32_t *status, hipStream_t s);
 
 // VALU throughput probe; out receives one word per thread so nothing is
 // optimised away.

@@ -1,0 +1,170 @@
+// C ABI entry point of the fused relay step (see include/bnkhip.h):
+// open -> filter -> re-seal, composed from the AEAD and filter kernels plus
+// the counter assignment of relay_kernels.hip.
+#include "api_common.hpp"
+#include "filter_host.hpp"
+
+using namespace bnk;
+
+extern "C" int bnk_relay_fused_batch(bnk_ctx *ctx, const bnk_batch *in, const uint32_t *peer_out,
+                                     const uint64_t *ctr_base_out, uint32_t n_peers_out,
+                                     int64_t now_ns, const bnk_batch *out, uint8_t *verdict,
+                                     uint64_t *ctr_out)
+{
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    int rc = check_batch_common(ctx, in, "in");
+    if (rc) return rc;
+    rc = check_batch_common(ctx, out, "out");
+    if (rc) return rc;
+    if (in->mem != out->mem) return fail(ctx, BNK_E_INVAL, "in and out must use the same mem kind");
+    const uint32_t n = in->n;
+    if (n == 0) return BNK_OK;
+    if (!peer_out || !ctr_base_out || !verdict || !ctr_out || n_peers_out == 0)
+        return fail(ctx, BNK_E_INVAL, "null relay array");
+    if (!ctx->d_keys[BNK_KEYS_RECV] || !ctx->d_keys[BNK_KEYS_SEND])
+        return fail(ctx, BNK_E_STATE, "relay needs both key tables loaded");
+    if (n_peers_out > ctx->n_keys[BNK_KEYS_SEND])
+        return fail(ctx, BNK_E_RANGE, "n_peers_out exceeds the send key table");
+    const bool host = in->mem == BNK_MEM_HOST;
+
+    // ---- where everything lives on the device ----
+    AeadArgs op{};
+    op.keys = ctx->d_keys[BNK_KEYS_RECV];
+    op.n_peers = ctx->n_keys[BNK_KEYS_RECV];
+    op.status = ctx->d_status;
+    op.counter0 = in->counter0;
+    op.n = n;
+    op.in_stride = in->stride;
+    op.len = in->len;
+    uint8_t *d_out = nullptr;
+    const uint64_t *d_out_off = nullptr;
+    const uint32_t *d_peer_out = nullptr;
+    const uint64_t *d_ctr_base = nullptr;
+    uint8_t *d_verdict = nullptr;
+    uint64_t *d_ctr_out = nullptr;
+    uint64_t plain_bytes = 0;
+    Staged st;
+    if (host) {
+        // the re-sealed packet has the input's length: out_delta 0
+        rc = stage_host(ctx, in, out, 0, ctx->n_keys[BNK_KEYS_RECV], &st);
+        if (rc) return rc;
+        for (uint32_t i = 0; i < n; i++)
+            if (peer_out[i] >= n_peers_out)
+                return fail(ctx, BNK_E_RANGE, "peer_out index beyond n_peers_out");
+        op.in = st.d_in;
+        op.in_off = st.d_in_off;
+        op.lens = st.d_lens;
+        op.peer = st.d_peer;
+        op.counters = st.d_counters;
+        d_out = st.d_out;
+        d_out_off = st.d_out_off;
+        plain_bytes = st.sin.size();
+        HIPCHK(ctx, ctx->r_peer_out.reserve((size_t)n * 4));
+        HIPCHK(ctx, ctx->r_ctr_base.reserve((size_t)n_peers_out * 8));
+        HIPCHK(ctx, ctx->r_ctr_out.reserve((size_t)n * 8));
+        HIPCHK(ctx, ctx->r_verdict.reserve(n));
+        HIPCHK(ctx, hipMemcpyAsync(ctx->r_peer_out.p, peer_out, (size_t)n * 4, hipMemcpyHostToDevice,
+                                   ctx->stream));
+        HIPCHK(ctx, hipMemcpyAsync(ctx->r_ctr_base.p, ctr_base_out, (size_t)n_peers_out * 8,
+                                   hipMemcpyHostToDevice, ctx->stream));
+        d_peer_out = ctx->r_peer_out.as<uint32_t>();
+        d_ctr_base = ctx->r_ctr_base.as<uint64_t>();
+        d_verdict = ctx->r_verdict.as<uint8_t>();
+        d_ctr_out = ctx->r_ctr_out.as<uint64_t>();
+    } else {
+        if (!in->offsets && !in->lens && (uint64_t)(n - 1) * in->stride + in->len > in->bytes)
+            return fail(ctx, BNK_E_INVAL, "in: uniform layout exceeds the arena");
+        if (!out->offsets && !in->lens && (uint64_t)(n - 1) * out->stride + in->len > out->bytes)
+            return fail(ctx, BNK_E_INVAL, "out: uniform layout exceeds the arena");
+        op.in = (const uint8_t *)in->base;
+        op.in_off = in->offsets;
+        op.lens = in->lens;
+        op.peer = in->peer;
+        op.counters = in->counters;
+        d_out = (uint8_t *)out->base;
+        d_out_off = out->offsets;
+        plain_bytes = in->bytes;
+        d_peer_out = peer_out;
+        d_ctr_base = ctr_base_out;
+        d_verdict = verdict;
+        d_ctr_out = ctr_out;
+    }
+    HIPCHK(ctx, ctx->r_plain.reserve(plain_bytes + 16));
+    HIPCHK(ctx, ctx->r_auth.reserve(n));
+    HIPCHK(ctx, ctx->r_pass.reserve(n));
+    for (DevBuf *b : {&ctx->r_keys, &ctx->r_idx, &ctx->r_skeys, &ctx->r_sidx})
+        HIPCHK(ctx, b->reserve((size_t)n * 4));
+    const size_t tmp_bytes = relay_sort_tmp_bytes(n);
+    HIPCHK(ctx, ctx->r_tmp.reserve(tmp_bytes + 16));
+
+    // ---- 1. open into the plaintext scratch (same offsets as the input) ----
+    op.out = ctx->r_plain.as<uint8_t>();
+    op.out_off = op.in_off;
+    op.out_stride = in->stride;
+    op.verdict = ctx->r_auth.as<uint8_t>();
+    rc = maybe_sort(ctx, op.lens, n, 16, &op.order);
+    if (rc) return rc;
+    HIPCHK(ctx, launch_aead_open(op, ctx->stream));
+
+    // ---- 2. CheckInbound on the authentic plaintexts ----
+    FilterState *f = ctx->filter;
+    uint8_t *d_pass = ctx->r_pass.as<uint8_t>();
+    if (!f->enforce) {
+        HIPCHK(ctx, launch_fill_u8(d_pass, n, 1, ctx->stream)); // filter.go:124-126
+    } else {
+        FilterArgs fa{};
+        fa.pkts = op.out;
+        fa.off = op.in_off;
+        fa.lens = op.lens;
+        fa.stride = in->stride;
+        fa.len = in->len;
+        fa.trim = 16; // lens count the tag
+        fa.gate = op.verdict;
+        fa.verdict = d_pass;
+        fa.status = ctx->d_status;
+        fa.now = now_ns;
+        fa.n = n;
+        fa.rules = f->ridx;
+        fa.flows = f->flows;
+        HIPCHK(ctx, launch_filter_check(fa, f->max_blocks, ctx->stream));
+    }
+
+    // ---- 3. verdicts and outbound counters ----
+    HIPCHK(ctx, launch_relay_assign(op.verdict, d_pass, d_peer_out, d_ctr_base, n_peers_out, n,
+                                    ctx->r_keys.as<uint32_t>(), ctx->r_idx.as<uint32_t>(),
+                                    ctx->r_skeys.as<uint32_t>(), ctx->r_sidx.as<uint32_t>(),
+                                    ctx->r_tmp.p, tmp_bytes, d_verdict, d_ctr_out, ctx->d_status,
+                                    ctx->stream));
+
+    // ---- 4. re-seal the survivors under the outbound keys ----
+    AeadArgs se{};
+    se.keys = ctx->d_keys[BNK_KEYS_SEND];
+    se.n_peers = n_peers_out;
+    se.status = ctx->d_status;
+    se.n = n;
+    se.in = op.out;
+    se.in_off = op.in_off;
+    se.in_stride = in->stride;
+    se.out = d_out;
+    se.out_off = d_out_off;
+    se.out_stride = out->stride;
+    se.lens = op.lens;
+    se.len = in->len;
+    se.trim = 16;
+    se.peer = d_peer_out;
+    se.counters = d_ctr_out;
+    se.skip = d_verdict; // BNK_RELAY_OK is 0
+    se.order = op.order;
+    HIPCHK(ctx, launch_aead_seal(se, ctx->stream));
+    if (!host) return BNK_OK;
+
+    HIPCHK(ctx, hipMemcpyAsync((uint8_t *)out->base + st.sout.lo, d_out, st.sout.size(),
+                               hipMemcpyDeviceToHost, ctx->stream));
+    HIPCHK(ctx, hipMemcpyAsync(verdict, d_verdict, n, hipMemcpyDeviceToHost, ctx->stream));
+    HIPCHK(ctx, hipMemcpyAsync(ctr_out, d_ctr_out, (size_t)n * 8, hipMemcpyDeviceToHost, ctx->stream));
+    uint32_t status = 0;
+    rc = take_status(ctx, &status);
+    if (rc) return rc;
+    return status_to_rc(ctx, status);
+}

@@ -1,0 +1,85 @@
+// Bookkeeping of the fused relay step open -> filter -> re-seal: verdicts and
+// the outbound nonce counters.  A packet that survives takes the next counter
+// of its outbound peer in batch order; dropped packets consume none (as in
+// wireguard-go, where the nonce is assigned when a packet is queued for
+// sending).  That is a segmented exclusive count over the survivors keyed by
+// peer: a stable radix sort of (peer, index) pairs puts each peer's survivors
+// together in batch order, and a survivor's rank is its distance from the
+// first element of its segment.
+#include <string.h>
+
+#include <rocprim/rocprim.hpp>
+
+#include "../../include/bnkhip.h"
+#include "kernels.hpp"
+
+namespace bnk {
+
+constexpr uint32_t NO_PEER = 0xFFFFFFFFu;
+
+__global__ __launch_bounds__(256) void relay_verdict_kernel(
+    const uint8_t *auth, const uint8_t *pass, const uint32_t *peer_out, uint32_t n_peers_out,
+    uint32_t n, uint32_t *keys, uint32_t *idx, uint8_t *verdict, uint64_t *ctr_out, uint32_t *status)
+{
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i >= n) return;
+    uint8_t v = !auth[i] ? BNK_RELAY_FORGED : !pass[i] ? BNK_RELAY_DENIED : BNK_RELAY_OK;
+    uint32_t key = NO_PEER;
+    if (v == BNK_RELAY_OK) {
+        key = peer_out[i];
+        if (key >= n_peers_out) {
+            atomicOr(status, STATUS_PEER_RANGE);
+            v = BNK_RELAY_DENIED;
+            key = NO_PEER;
+        }
+    }
+    verdict[i] = v;
+    keys[i] = key;
+    idx[i] = i;
+    ctr_out[i] = 0;
+}
+
+__global__ __launch_bounds__(256) void relay_rank_kernel(const uint32_t *skeys, const uint32_t *sidx,
+                                                         const uint64_t *ctr_base_out, uint32_t n,
+                                                         uint64_t *ctr_out)
+{
+    const uint32_t p = blockIdx.x * 256u + threadIdx.x;
+    if (p >= n) return;
+    const uint32_t key = skeys[p];
+    if (key == NO_PEER) return;
+    // first position holding this key
+    uint32_t lo = 0, hi = p;
+    while (lo < hi) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (skeys[mid] < key) lo = mid + 1;
+        else hi = mid;
+    }
+    ctr_out[sidx[p]] = ctr_base_out[key] + (uint64_t)(p - lo);
+}
+
+size_t relay_sort_tmp_bytes(uint32_t n)
+{
+    size_t bytes = 0;
+    (void)rocprim::radix_sort_pairs(nullptr, bytes, (const uint32_t *)nullptr, (uint32_t *)nullptr,
+                                    (const uint32_t *)nullptr, (uint32_t *)nullptr, (size_t)n);
+    return bytes;
+}
+
+hipError_t launch_relay_assign(const uint8_t *auth, const uint8_t *pass, const uint32_t *peer_out,
+                               const uint64_t *ctr_base_out, uint32_t n_peers_out, uint32_t n,
+                               uint32_t *keys, uint32_t *idx, uint32_t *skeys, uint32_t *sidx,
+                               void *sort_tmp, size_t sort_tmp_bytes, uint8_t *verdict,
+                               uint64_t *ctr_out, uint32_t *status, hipStream_t s)
+{
+    if (n == 0) return hipSuccess;
+    const dim3 grid((n + 255u) / 256u);
+    hipLaunchKernelGGL(relay_verdict_kernel, grid, dim3(256), 0, s, auth, pass, peer_out, n_peers_out,
+                       n, keys, idx, verdict, ctr_out, status);
+    hipError_t e = rocprim::radix_sort_pairs(sort_tmp, sort_tmp_bytes, keys, skeys, idx, sidx, (size_t)n,
+                                             0, 32, s);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(relay_rank_kernel, grid, dim3(256), 0, s, skeys, sidx, ctr_base_out, n, ctr_out);
+    return hipGetLastError();
+}
+
+} // namespace bnk

@@ -29,11 +29,18 @@ _M2 = np.uint64(0x94D049BB133111EB)
 def splitmix64(seed: int, n: int, start: int = 0) -> np.ndarray:
     """Outputs start+1 .. start+n of SplitMix64 seeded with ``seed``."""
     with np.errstate(over="ignore"):
-        k = np.arange(start + 1, start + n + 1, dtype=np.uint64)
-        z = np.uint64(seed & 0xFFFFFFFFFFFFFFFF) + k * _GOLDEN
-        z = (z ^ (z >> np.uint64(30))) * _M1
-        z = (z ^ (z >> np.uint64(27))) * _M2
-        return z ^ (z >> np.uint64(31))
+        z = np.arange(start + 1, start + n + 1, dtype=np.uint64)
+        z *= _GOLDEN
+        z += np.uint64(seed & 0xFFFFFFFFFFFFFFFF)
+        t = z >> np.uint64(30)
+        z ^= t
+        z *= _M1
+        np.right_shift(z, np.uint64(27), out=t)
+        z ^= t
+        z *= _M2
+        np.right_shift(z, np.uint64(31), out=t)
+        z ^= t
+        return z
 
 
 def stream_seed(cfg: int, stream: int) -> int:
@@ -43,7 +50,7 @@ def stream_seed(cfg: int, stream: int) -> int:
 
 def rand_bytes(seed: int, nbytes: int) -> np.ndarray:
     words = splitmix64(seed, (nbytes + 7) // 8)
-    return words.view(np.uint8)[:nbytes].copy()
+    return words.view(np.uint8)[:nbytes]
 
 
 def rand_bytes_torch(seed: int, nbytes: int, device):
@@ -122,7 +129,7 @@ class AeadBatch:
 
     @property
     def arena_bytes(self) -> int:
-        return int(self.plain.shape[0])
+        return int(self.plain.shape[0]) if self.plain is not None else int(self.meta["total"])
 
 
 def aead_uniform(cfg: int, n: int, length: int = 1420, stride: int | None = None,
@@ -167,7 +174,7 @@ def per_peer_sequence(peer: np.ndarray, n_peers: int) -> np.ndarray:
     return seq
 
 
-def aead_imix(cfg: int, n: int, n_peers: int = 256, payload: np.ndarray | None = None,
+def aead_imix(cfg: int, n: int, n_peers: int = 256, payload: bool = True,
               lens: np.ndarray | None = None) -> AeadBatch:
     """Configuration 3 (and the AEAD half of 5): IMIX sizes, ``n_peers`` keys,
     per-peer counter = random base below 2^48 plus the per-peer sequence
@@ -183,20 +190,34 @@ def aead_imix(cfg: int, n: int, n_peers: int = 256, payload: np.ndarray | None =
     off = np.zeros(n, np.uint64)
     np.cumsum(slot[:-1], out=off[1:])
     total = int(off[-1] + slot[-1]) if n else 0
-    plain = np.zeros(total, np.uint8)
-    if payload is None:
+    plain = None
+    if payload:
         # random fill of the whole arena, then clear the tag/pad gaps so the
         # arena content is a function of the packets only
-        plain[:] = rand_bytes(stream_seed(cfg, 1), total)
-        mark = np.zeros(total + 1, np.int32)
-        np.add.at(mark, off.astype(np.int64), 1)
-        np.add.at(mark, (off + lens.astype(np.uint64)).astype(np.int64), -1)
-        inside = np.cumsum(mark)[:total] > 0
-        plain[~inside] = 0
-    else:
-        plain[:] = payload
+        plain = rand_bytes(stream_seed(cfg, 1), total)
+        gap = (slot - lens.astype(np.uint64)).astype(np.int64)
+        end = (off + lens.astype(np.uint64)).astype(np.int64)
+        for k in range(int(gap.max()) if n else 0):
+            sel = gap > k
+            plain[end[sel] + k] = 0
     return AeadBatch(keys=keys, peer=peer, counters=counters, lens=lens, off=off,
-                     plain=plain, stride=0, meta={"cfg": cfg, "n_peers": n_peers})
+                     plain=plain, stride=0,
+                     meta={"cfg": cfg, "n_peers": n_peers, "total": total})
+
+
+def imix_plain_torch(b: AeadBatch, device):
+    """The arena aead_imix(..., payload=True) would hold, built by torch on
+    ``device`` (for sizes where the numpy path takes too long)."""
+    import torch
+    total = b.meta["total"]
+    plain = rand_bytes_torch(stream_seed(b.meta["cfg"], 1), total, device).clone()
+    slot = ((b.lens.astype(np.uint64) + np.uint64(TAG + 15)) // np.uint64(16)) * np.uint64(16)
+    gap = (slot - b.lens.astype(np.uint64)).astype(np.int64)
+    end = (b.off + b.lens.astype(np.uint64)).astype(np.int64)
+    for k in range(int(gap.max()) if b.n else 0):
+        sel = gap > k
+        plain[torch.from_numpy(end[sel] + k).to(device)] = 0
+    return plain
 
 
 def forge_tags(cfg: int, sealed: np.ndarray, off: np.ndarray, lens: np.ndarray,
@@ -381,3 +402,88 @@ def acl_workload(cfg: int = 4, n: int = 1 << 22, n_rules: int = 4096, n_flows: i
     check = header_records(cproto, csrc, cdst, csport, cdport)
     return AclWorkload(rules_ref=rules_ref, rule_tuples=tuples, note_batches=note_batches,
                        check=check, now_ns=T0_NS)
+
+
+# --------------------------------------------------------------------------
+# Fused relay workload (configuration 5)
+# --------------------------------------------------------------------------
+
+@dataclass
+class RelayWorkload:
+    batch: AeadBatch           # inbound plaintexts (before sealing), keys = inbound keys
+    keys_out: np.ndarray       # [n_peers, 32]
+    peer_out: np.ndarray       # [n] u32
+    ctr_base_out: np.ndarray   # [n_peers] u64
+    rules_ref: list
+    note_batch: tuple          # (now_ns, records) noted before the relay step
+    denied: np.ndarray         # [n] bool: constructed to fail the filter
+    flow_allowed: np.ndarray   # [n] bool: pass only through the flow table
+    forged_fraction: float
+    now_ns: int
+
+
+def relay_workload(cfg: int = 5, n: int = 1 << 22, n_peers: int = 4096, n_rules: int = 4096,
+                   forged_fraction: float = 0.005, denied_fraction: float = 0.05,
+                   flow_fraction: float = 0.01, payload: bool = True) -> RelayWorkload:
+    """Configuration 5: IMIX packets whose plaintext starts with an IPv4 + L4
+    header.  denied_fraction of them come from 10.0.0.0/8, which no rule
+    covers; flow_fraction come from 10.0.0.0/8 too but answer a noted outbound
+    flow; every other packet is built to match one seeded rule."""
+    ss = lambda k: stream_seed(cfg, k)  # noqa: E731
+    acl = acl_workload(cfg, n=1, n_rules=n_rules, n_flows=0)
+    t = acl.rule_tuples
+    b = aead_imix(cfg, n, n_peers=n_peers, payload=payload)
+    pick = rand_below(ss(40), n, n_rules)
+    net, mask, first, last, rproto = (t[pick, k] for k in range(5))
+    r1 = splitmix64(ss(41), n)
+    src = (net | ((r1 & np.uint64(0xFFFFFFFF)).astype(np.uint32) & ~mask)).astype(np.uint32)
+    span = (last - first + 1).astype(np.uint64)
+    dport = (first + ((r1 >> np.uint64(32)) % span).astype(np.uint32)).astype(np.uint32)
+    sport = (1024 + rand_below(ss(42), n, 60000)).astype(np.uint32)
+    proto = rproto.copy()
+    order = permutation(ss(43), n)
+    n_denied = int(denied_fraction * n)
+    n_flow = int(flow_fraction * n)
+    denied = np.zeros(n, bool)
+    flow_allowed = np.zeros(n, bool)
+    denied[order[:n_denied]] = True
+    flow_allowed[order[n_denied:n_denied + n_flow]] = True
+    outside = denied | flow_allowed
+    ten = (10 << 24 | rand_below(ss(44), n, 1 << 24)).astype(np.uint32)
+    src[outside] = ten[outside]
+    # flow-admitted packets must not be ICMP duplicates of each other's keys;
+    # give them tcp/udp and distinct port pairs
+    proto[flow_allowed] = np.where(rand_below(ss(45), n, 2)[flow_allowed] == 0, 6, 17)
+    self_addr = CGNAT_BASE | 1
+    rec = header_records(proto, src, np.full(n, self_addr, np.uint32), sport, dport)
+    # total length field = plaintext length (not looked at by the filter)
+    rec[:, 2] = (b.lens >> 8) & 0xFF
+    rec[:, 3] = b.lens & 0xFF
+    if payload:
+        off64 = b.off.astype(np.int64)
+        for k in range(28):
+            b.plain[off64 + k] = rec[:, k]
+    # the outbound packets this host sent earlier, which the flow_allowed ones answer
+    fa = np.flatnonzero(flow_allowed)
+    note_rec = header_records(proto[fa], np.full(fa.shape[0], self_addr, np.uint32), src[fa],
+                              dport[fa], sport[fa])
+    keys_out = rand_bytes(ss(46), 32 * n_peers).reshape(n_peers, 32)
+    peer_out = rand_below(ss(47), n, n_peers)
+    ctr_base_out = rand_u64(ss(48), n_peers) >> np.uint64(16)
+    b.meta["headers"] = rec
+    return RelayWorkload(batch=b, keys_out=keys_out, peer_out=peer_out, ctr_base_out=ctr_base_out,
+                         rules_ref=acl.rules_ref, note_batch=(T0_NS - 1_000_000_000, note_rec),
+                         denied=denied, flow_allowed=flow_allowed,
+                         forged_fraction=forged_fraction, now_ns=T0_NS)
+
+
+def relay_plain_torch(w: RelayWorkload, device):
+    """Plaintext arena of a relay_workload(..., payload=False), built on
+    ``device``: the IMIX payload with each packet's 28 header bytes written in."""
+    import torch
+    plain = imix_plain_torch(w.batch, device)
+    rec = torch.from_numpy(np.ascontiguousarray(w.batch.meta["headers"][:, :28])).to(device)
+    off = torch.from_numpy(w.batch.off.astype(np.int64)).to(device)
+    for k in range(28):
+        plain[off + k] = rec[:, k]
+    return plain

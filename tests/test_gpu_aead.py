@@ -232,6 +232,7 @@ def test_device_resident_large_batch_properties(ctx):
     # linearity of the stream cipher: ct(a) ^ ct(b) == a ^ b under the same nonce
     pt2 = pt.clone(); pt2[:, :L] ^= 0x3C
     ct2 = torch.zeros_like(pt)
+    torch.cuda.synchronize()  # torch's fills run on its own stream
     ctx.seal(lib.make_batch(pt2, nb, n, lib.MEM_DEVICE, stride=stride, length=L, counter0=1000),
              lib.make_batch(ct2, nb, n, lib.MEM_DEVICE, stride=stride))
     ctx.sync()

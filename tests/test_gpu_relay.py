@@ -1,0 +1,155 @@
+"""Fused relay open -> filter -> re-seal on the GPU against the CPU
+definition (oracle/relay.c): identical verdicts, outbound counters and output
+ciphertexts."""
+import numpy as np
+import pytest
+
+from bnk_amd import workloads as W
+
+pytestmark = pytest.mark.gpu
+
+
+def _note(ctx, ora, w):
+    from bnk_amd import lib
+    now, rec = w.note_batch
+    m = rec.shape[0]
+    buf = np.ascontiguousarray(rec).reshape(-1)
+    if ora is not None:
+        ora.note_outbound_batch(buf, np.arange(m, dtype=np.uint64) * 32, np.full(m, 28, np.uint32), now)
+    ctx.filter_note_outbound(lib.make_batch(buf, buf.nbytes, m, lib.MEM_HOST, stride=32, length=28), now)
+
+
+def test_relay_matches_oracle_host_path():
+    from bnk_amd import lib
+    from oracle import binding as O
+    w = W.relay_workload(n=12000, n_peers=64, n_rules=512)
+    b = w.batch
+    keys_in = np.ascontiguousarray(b.keys)
+    keys_out = np.ascontiguousarray(w.keys_out)
+    sealed = np.zeros_like(b.plain)
+    O.seal_batch(keys_in, b.peer, b.counters, b.plain, b.off, b.lens, sealed, b.off, 4)
+    forged = W.forge_tags(5, sealed, b.off, b.lens, w.forged_fraction)
+    # a truncated packet is FORGED too
+    ct_lens = (b.lens + 16).astype(np.uint32)
+    ct_lens[7] = 9
+    ora = O.Filter()
+    ora.set_rules(w.rules_ref)
+    ctx = lib.Context(0)
+    ctx.filter_set_rules(w.rules_ref)
+    ctx.keys_set(lib.KEYS_RECV, keys_in)
+    ctx.keys_set(lib.KEYS_SEND, keys_out)
+    _note(ctx, ora, w)
+    want_out = np.full_like(b.plain, 0x77)
+    want_v, want_c = ora.relay_fused_batch(keys_in, b.peer, b.counters, keys_out, w.peer_out,
+                                           w.ctr_base_out, sealed, b.off, ct_lens, want_out, b.off,
+                                           w.now_ns)
+    got_out = np.full_like(b.plain, 0x77)
+    got_v = np.full(b.n, 9, np.uint8)
+    got_c = np.full(b.n, 123, np.uint64)
+    ctx.relay_fused(
+        lib.make_batch(sealed, sealed.nbytes, b.n, lib.MEM_HOST, offsets=b.off, lens=ct_lens,
+                       peer=b.peer, counters=b.counters),
+        w.peer_out, w.ctr_base_out, len(w.ctr_base_out), w.now_ns,
+        lib.make_batch(got_out, got_out.nbytes, b.n, lib.MEM_HOST, offsets=b.off), got_v, got_c)
+    assert np.array_equal(got_v, want_v)
+    assert np.array_equal(got_c, want_c)
+    assert np.array_equal(got_out, want_out)  # dropped packets' slots keep their 0x77 fill
+    expect = np.where(forged, 1, np.where(w.denied, 2, 0))
+    expect[7] = 1
+    assert np.array_equal(got_v, expect)
+    assert ctx.filter_flows() == ora.flows()
+    # in allow-all mode nothing is DENIED
+    ctx.filter_set_allow_all()
+    ctx.relay_fused(
+        lib.make_batch(sealed, sealed.nbytes, b.n, lib.MEM_HOST, offsets=b.off, lens=ct_lens,
+                       peer=b.peer, counters=b.counters),
+        w.peer_out, w.ctr_base_out, len(w.ctr_base_out), w.now_ns,
+        lib.make_batch(got_out, got_out.nbytes, b.n, lib.MEM_HOST, offsets=b.off), got_v, got_c)
+    assert np.array_equal(got_v == 1, expect == 1) and not (got_v == 2).any()
+    ctx.close()
+
+
+def test_relay_full_size_device_resident_properties():
+    """Configuration 5 at full size (2^22 IMIX packets, 4096 peers, 4096
+    rules): verdicts equal the construction, counters equal base + per-peer
+    rank among survivors in batch order, every re-sealed packet opens under the
+    outbound key to the original plaintext, and a sample is bit-exact against
+    the oracle."""
+    import torch
+    from bnk_amd import lib
+    from oracle import binding as O
+    n = 1 << 22
+    w = W.relay_workload(n=n, payload=False)
+    b = w.batch
+    dev = torch.device("cuda:0")
+    keys_in = np.ascontiguousarray(b.keys)
+    keys_out = np.ascontiguousarray(w.keys_out)
+    plain = W.relay_plain_torch(w, dev)
+    total = plain.numel()
+    d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)  # noqa: E731
+    d_off, d_peer, d_ctr = d(b.off.astype(np.int64)), d(b.peer.astype(np.int32)), d(b.counters.astype(np.int64))
+    d_lens, d_ctlens = d(b.lens.astype(np.int32)), d((b.lens + 16).astype(np.int32))
+    d_peer_out, d_base = d(w.peer_out.astype(np.int32)), d(w.ctr_base_out.astype(np.int64))
+    sealed = torch.zeros(total, dtype=torch.uint8, device=dev)
+    out = torch.full((total,), 0x77, dtype=torch.uint8, device=dev)
+    verdict = torch.zeros(n, dtype=torch.uint8, device=dev)
+    ctr_out = torch.zeros(n, dtype=torch.int64, device=dev)
+    torch.cuda.synchronize()
+    ctx = lib.Context(0)
+    ctx.filter_set_rules(w.rules_ref)
+    _note(ctx, None, w)
+    # inbound traffic: sealed under the inbound keys, then 0.5 % of tags forged
+    ctx.keys_set(lib.KEYS_SEND, keys_in)
+    ctx.seal(lib.make_batch(plain, total, n, lib.MEM_DEVICE, offsets=d_off, lens=d_lens, peer=d_peer,
+                            counters=d_ctr),
+             lib.make_batch(sealed, total, n, lib.MEM_DEVICE, offsets=d_off))
+    ctx.sync()
+    k = int(w.forged_fraction * n)
+    which = W.permutation(W.stream_seed(5, 5), n)[:k].astype(np.int64)
+    bit = W.rand_below(W.stream_seed(5, 6), k, 128)
+    pos = b.off[which].astype(np.int64) + b.lens[which].astype(np.int64) + (bit >> 3).astype(np.int64)
+    sealed[d(pos)] ^= d((1 << (bit & 7)).astype(np.uint8))
+    forged = np.zeros(n, bool)
+    forged[which] = True
+    torch.cuda.synchronize()
+    ctx.keys_set(lib.KEYS_RECV, keys_in)
+    ctx.keys_set(lib.KEYS_SEND, keys_out)
+    ctx.relay_fused(lib.make_batch(sealed, total, n, lib.MEM_DEVICE, offsets=d_off, lens=d_ctlens,
+                                   peer=d_peer, counters=d_ctr),
+                    d_peer_out, d_base, len(w.ctr_base_out), w.now_ns,
+                    lib.make_batch(out, total, n, lib.MEM_DEVICE, offsets=d_off), verdict, ctr_out)
+    ctx.sync()
+    v = verdict.cpu().numpy()
+    c = ctr_out.cpu().numpy().astype(np.uint64)
+    expect = np.where(forged, 1, np.where(w.denied, 2, 0))
+    assert np.array_equal(v, expect)
+    assert abs((v == 2).mean() - 0.05) < 0.002 and (v == 1).sum() == k
+    # counters: base + rank among the same peer's survivors, batch order
+    ok = v == 0
+    surv = np.flatnonzero(ok)
+    want_c = np.zeros(n, np.uint64)
+    want_c[surv] = w.ctr_base_out[w.peer_out[surv]] + W.per_peer_sequence(w.peer_out[surv],
+                                                                        len(w.ctr_base_out))
+    assert np.array_equal(c, want_c)
+    # every survivor opens under the outbound key/counter to the original plaintext
+    ctx.keys_set(lib.KEYS_RECV, keys_out)
+    back = torch.zeros(total, dtype=torch.uint8, device=dev)
+    v2 = torch.zeros(n, dtype=torch.uint8, device=dev)
+    torch.cuda.synchronize()  # torch's fills run on its own stream
+    ctx.open(lib.make_batch(out, total, n, lib.MEM_DEVICE, offsets=d_off, lens=d_ctlens,
+                            peer=d_peer_out, counters=ctr_out),
+             lib.make_batch(back, total, n, lib.MEM_DEVICE, offsets=d_off), v2)
+    ctx.sync()
+    assert np.array_equal(v2.cpu().numpy().astype(bool), ok)
+    # compare plaintext bytes of survivors; dropped slots of `out` kept the fill
+    o_host, p_host, b_host = out.cpu().numpy(), plain.cpu().numpy(), back.cpu().numpy()
+    for i in np.concatenate([surv[:300], surv[-300:]]):
+        o, L = int(b.off[i]), int(b.lens[i])
+        assert np.array_equal(b_host[o:o + L], p_host[o:o + L])
+        want = O.aead_seal(keys_out[w.peer_out[i]].tobytes(), O.wg_nonce(int(c[i])),
+                           p_host[o:o + L].tobytes())
+        assert o_host[o:o + L + 16].tobytes() == want
+    for i in np.flatnonzero(~ok)[:300]:
+        o, L = int(b.off[i]), int(b.lens[i])
+        assert (o_host[o:o + L + 16] == 0x77).all()
+    ctx.close()

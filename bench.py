@@ -45,12 +45,257 @@ def ops_aead(length: int) -> int:
     return ops_chacha(length) + ops_poly(length)
 
 
+def _events(torch, stream, k):
+    return [[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(k)]
+
+
+def bench_filter(args) -> dict:
+    """Configuration 4: 2^22 IPv4 headers (32-byte records) against 4096 rules
+    and a flow table built from 65,536 noted outbound packets; one step = one
+    CheckInbound batch."""
+    import numpy as np
+    import torch
+    from bnk_amd import lib, workloads as W
+    n = 1 << 22
+    w = W.acl_workload(n=n)
+    ctx = lib.Context(0)
+    ctx.filter_set_rules(w.rules_ref)
+    for now, rec in w.note_batches:
+        buf = np.ascontiguousarray(rec).reshape(-1)
+        ctx.filter_note_outbound(
+            lib.make_batch(buf, buf.nbytes, rec.shape[0], lib.MEM_HOST, stride=32, length=28), now)
+    dev = torch.device("cuda:0")
+    d_rec = torch.from_numpy(w.check).to(dev)
+    d_v = torch.zeros(n, dtype=torch.uint8, device=dev)
+    torch.cuda.synchronize()
+    batch = lib.make_batch(d_rec, n * 32, n, lib.MEM_DEVICE, stride=32, length=28)
+    for _ in range(args.warmup):
+        ctx.filter_check_inbound(batch, w.now_ns, d_v)
+    ctx.sync()
+    stream = torch.cuda.ExternalStream(ctx.stream, device=dev)
+    ev = _events(torch, stream, args.steps)
+    t0 = time.perf_counter()
+    for s in range(args.steps):
+        ev[s][0].record(stream)
+        ctx.filter_check_inbound(batch, w.now_ns, d_v)
+        ev[s][1].record(stream)
+    ctx.sync()
+    t1 = time.perf_counter()
+    ms = (t1 - t0) * 1e3 / args.steps
+    kern_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / args.steps
+    v = d_v.cpu().numpy()
+    allowed = float(v.mean())
+    # algorithmic bytes: 20-byte header + 4 port bytes in, 1 verdict byte out, and one 16-byte
+    # flow slot for every packet no rule admits (the reference probes its map for those)
+    alg_bytes = n * 25 + int((1.0 - allowed) * n) * 16
+    gbs = alg_bytes / (kern_ms * 1e-3) / 1e9
+    out = {
+        "metric": "acl_filter_mpkt_per_s", "value": round(n / (ms * 1e-3) / 1e6, 1),
+        "unit": "Mpkt/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "u32", "data": "synthetic",
+        "config": {"workload": "cfg4: CheckInbound of %d IPv4 headers, 4096 rules, flow table from "
+                               "65536 noted packets, device resident" % n,
+                   "packets": n, "rules": 4096, "allowed_fraction": round(allowed, 4)},
+        "roofline": {"bound": "hbm", "kernel": "filter_check_kernel", "achieved": round(gbs, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+                     "traffic": None, "bytes_per_launch": alg_bytes,
+                     "avg_launch_ms": round(kern_ms, 4)},
+    }
+    if not args.no_cpu_baseline:
+        from oracle import binding as O
+        ora = O.Filter()
+        ora.set_rules(w.rules_ref)
+        for now, rec in w.note_batches:
+            m = rec.shape[0]
+            ora.note_outbound_batch(np.ascontiguousarray(rec).reshape(-1),
+                                    np.arange(m, dtype=np.uint64) * 32, np.full(m, 28, np.uint32), now)
+        sample = args.cpu_sample or 1 << 16
+        buf = np.ascontiguousarray(w.check[:sample]).reshape(-1)
+        tp = time.perf_counter()
+        ov = ora.check_inbound_batch(buf, np.arange(sample, dtype=np.uint64) * 32,
+                                     np.full(sample, 28, np.uint32), w.now_ns)
+        dt = time.perf_counter() - tp
+        out["cpu_baseline"] = {
+            "value": round(sample / dt / 1e6, 4), "unit": "Mpkt/s", "cores": 1, "kind": "port",
+            "sample": "CheckInbound of the first %d headers of the same workload, C restatement "
+                      "of filter.go/acl.go (linear rule scan under one lock, as the reference), "
+                      "1 thread" % sample,
+            "gpu_output_matches": bool(np.array_equal(ov, v[:sample])),
+        }
+    ctx.close()
+    return out
+
+
+def _imix_device(torch, np, W, b, dev):
+    d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)  # noqa: E731
+    return (d(b.off.astype(np.int64)), d(b.peer.astype(np.int32)), d(b.counters.astype(np.int64)),
+            d(b.lens.astype(np.int32)), d((b.lens + 16).astype(np.int32)))
+
+
+def bench_imix(args) -> dict:
+    """Configuration 3: 2^20 IMIX packets (60/576/1420 B, 7:4:1), 256 peers;
+    seal, then open with 1 % of the tags forged."""
+    import numpy as np
+    import torch
+    from bnk_amd import lib, workloads as W
+    n = 1 << 20
+    b = W.aead_imix(3, n, n_peers=256, payload=False)
+    dev = torch.device("cuda:0")
+    total = b.meta["total"]
+    plain = W.imix_plain_torch(b, dev)
+    d_off, d_peer, d_ctr, d_lens, d_ctl = _imix_device(torch, np, W, b, dev)
+    sealed = torch.zeros(total, dtype=torch.uint8, device=dev)
+    forged_copy = torch.zeros(total, dtype=torch.uint8, device=dev)
+    back = torch.zeros(total, dtype=torch.uint8, device=dev)
+    v = torch.zeros(n, dtype=torch.uint8, device=dev)
+    torch.cuda.synchronize()
+    ctx = lib.Context(0)
+    ctx.keys_set(lib.KEYS_SEND, b.keys)
+    ctx.keys_set(lib.KEYS_RECV, b.keys)
+    sb = lib.make_batch(plain, total, n, lib.MEM_DEVICE, offsets=d_off, lens=d_lens, peer=d_peer,
+                        counters=d_ctr)
+    so = lib.make_batch(sealed, total, n, lib.MEM_DEVICE, offsets=d_off)
+    ctx.seal(sb, so)
+    ctx.sync()
+    forged_copy.copy_(sealed)
+    k = int(0.01 * n)
+    which = W.permutation(W.stream_seed(3, 5), n)[:k].astype(np.int64)
+    bit = W.rand_below(W.stream_seed(3, 6), k, 128)
+    pos = b.off[which].astype(np.int64) + b.lens[which].astype(np.int64) + (bit >> 3).astype(np.int64)
+    forged_copy[torch.from_numpy(pos).to(dev)] ^= torch.from_numpy((1 << (bit & 7)).astype(np.uint8)).to(dev)
+    torch.cuda.synchronize()
+    ob = lib.make_batch(forged_copy, total, n, lib.MEM_DEVICE, offsets=d_off, lens=d_ctl, peer=d_peer,
+                        counters=d_ctr)
+    oo = lib.make_batch(back, total, n, lib.MEM_DEVICE, offsets=d_off)
+    for _ in range(args.warmup):
+        ctx.seal(sb, so)
+        ctx.open(ob, oo, v)
+    ctx.sync()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        ctx.seal(sb, so)
+        ctx.open(ob, oo, v)
+    ctx.sync()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    vv = v.cpu().numpy()
+    forged = np.zeros(n, bool)
+    forged[which] = True
+    assert np.array_equal(vv == 0, forged), "forged tags and rejects differ"
+    payload = int(b.lens.sum())
+    ops = sum(int((b.lens == L_).sum()) * ops_aead(L_) for L_ in (60, 576, 1420))
+    ctx.close()
+    return {
+        "metric": "aead_seal_open_gbit_per_s_imix", "value": round(payload * 8 / (ms * 1e-3) / 1e9, 1),
+        "unit": "Gbit/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u32", "data": "synthetic",
+        "config": {"workload": "cfg3: seal+open of %d IMIX packets (60/576/1420 B 7:4:1), 256 peers, "
+                               "1%% forged tags on open, device resident" % n, "packets": n},
+        "mpkt_per_s_pair": round(n / (ms * 1e-3) / 1e6, 1),
+        "rejected": int((vv == 0).sum()),
+        "roofline_valu": {"achieved": round(2 * ops / (ms * 1e-3) / 1e12, 2), "peak": VALU_PEAK_TOPS,
+                          "unit": "Top/s (int32 op-equivalents)",
+                          "frac": round(2 * ops / (ms * 1e-3) / 1e12 / VALU_PEAK_TOPS, 4)},
+    }
+
+
+def bench_relay(args) -> dict:
+    """Configuration 5: open -> filter -> re-seal of 2^22 IMIX packets across
+    4096 peers, 0.5 % forged tags, 5 % denied by the ACL."""
+    import numpy as np
+    import torch
+    from bnk_amd import lib, workloads as W
+    n = 1 << 22
+    w = W.relay_workload(n=n, payload=False)
+    b = w.batch
+    dev = torch.device("cuda:0")
+    total = b.meta["total"]
+    plain = W.relay_plain_torch(w, dev)
+    d_off, d_peer, d_ctr, d_lens, d_ctl = _imix_device(torch, np, W, b, dev)
+    d_peer_out = torch.from_numpy(w.peer_out.astype(np.int32)).to(dev)
+    d_base = torch.from_numpy(w.ctr_base_out.astype(np.int64)).to(dev)
+    sealed = torch.zeros(total, dtype=torch.uint8, device=dev)
+    out = torch.zeros(total, dtype=torch.uint8, device=dev)
+    verdict = torch.zeros(n, dtype=torch.uint8, device=dev)
+    ctr_out = torch.zeros(n, dtype=torch.int64, device=dev)
+    torch.cuda.synchronize()
+    ctx = lib.Context(0)
+    ctx.filter_set_rules(w.rules_ref)
+    now, rec = w.note_batch
+    buf = np.ascontiguousarray(rec).reshape(-1)
+    ctx.filter_note_outbound(lib.make_batch(buf, buf.nbytes, rec.shape[0], lib.MEM_HOST, stride=32,
+                                            length=28), now)
+    ctx.keys_set(lib.KEYS_SEND, b.keys)
+    ctx.seal(lib.make_batch(plain, total, n, lib.MEM_DEVICE, offsets=d_off, lens=d_lens, peer=d_peer,
+                            counters=d_ctr),
+             lib.make_batch(sealed, total, n, lib.MEM_DEVICE, offsets=d_off))
+    ctx.sync()
+    k = int(w.forged_fraction * n)
+    which = W.permutation(W.stream_seed(5, 5), n)[:k].astype(np.int64)
+    bit = W.rand_below(W.stream_seed(5, 6), k, 128)
+    pos = b.off[which].astype(np.int64) + b.lens[which].astype(np.int64) + (bit >> 3).astype(np.int64)
+    sealed[torch.from_numpy(pos).to(dev)] ^= torch.from_numpy((1 << (bit & 7)).astype(np.uint8)).to(dev)
+    torch.cuda.synchronize()
+    ctx.keys_set(lib.KEYS_RECV, b.keys)
+    ctx.keys_set(lib.KEYS_SEND, w.keys_out)
+    ib = lib.make_batch(sealed, total, n, lib.MEM_DEVICE, offsets=d_off, lens=d_ctl, peer=d_peer,
+                        counters=d_ctr)
+    ob = lib.make_batch(out, total, n, lib.MEM_DEVICE, offsets=d_off)
+
+    def step():
+        ctx.relay_fused(ib, d_peer_out, d_base, len(w.ctr_base_out), w.now_ns, ob, verdict, ctr_out)
+
+    for _ in range(args.warmup):
+        step()
+    ctx.sync()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    ctx.sync()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    v = verdict.cpu().numpy()
+    forged = np.zeros(n, bool)
+    forged[which] = True
+    assert np.array_equal(v, np.where(forged, 1, np.where(w.denied, 2, 0))), "verdicts differ"
+    payload = int(b.lens.sum())
+    ctx.close()
+    return {
+        "metric": "relay_open_filter_reseal_mpkt_per_s", "value": round(n / (ms * 1e-3) / 1e6, 1),
+        "unit": "Mpkt/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u32", "data": "synthetic",
+        "config": {"workload": "cfg5: open->filter->re-seal of %d IMIX packets, 4096 peers, 4096 rules, "
+                               "0.5%% forged, 5%% denied, device resident" % n, "packets": n},
+        "gbit_per_s_plaintext": round(payload * 8 / (ms * 1e-3) / 1e9, 1),
+        "verdicts": {"ok": int((v == 0).sum()), "forged": int((v == 1).sum()),
+                     "denied": int((v == 2).sum())},
+    }
+
+
+def bench_copy(args) -> dict:
+    """Plain device-to-device copy of 1 GiB: the measured HBM ceiling and the
+    known-size launch the FETCH_SIZE / WRITE_SIZE counters are scaled by."""
+    from bnk_amd import lib
+    ctx = lib.Context(0)
+    nbytes = 1 << 30
+    rate = ctx.probe_copy(nbytes, max(args.steps, 1))
+    ctx.close()
+    return {"metric": "hbm_copy_gb_per_s", "value": round(rate / 1e9, 1), "unit": "GB/s",
+            "n_gpus": 1, "steps": args.steps, "warmup": 1, "higher_is_better": True,
+            "config": {"workload": "copy_kernel: %d bytes read + %d bytes written per launch"
+                                   % (nbytes, nbytes)}}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--packets", type=int, default=1 << 20)
+    ap.add_argument("--workload", default="aead", choices=["aead", "filter", "imix", "relay", "copy"],
+                    help="aead (default, the headline line, with the ACL filter rate as an extra); "
+                         "filter / imix / relay / copy print one line for that workload alone")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample", type=int, default=0,
                     help="packets in the CPU baseline sample (0 = sized for ~10 s)")
@@ -67,6 +312,11 @@ def main() -> int:
     if not torch.cuda.is_available():
         print("no GPU visible: bench.py needs an MI355X", file=sys.stderr)
         return 2
+    if args.workload != "aead":
+        out = {"filter": bench_filter, "imix": bench_imix, "relay": bench_relay,
+               "copy": bench_copy}[args.workload](args)
+        print(json.dumps(out))
+        return 0
     n = args.packets
     ctx = lib.Context(0)
     key = W.rand_bytes(W.stream_seed(2, 0), 32).reshape(1, 32)
@@ -202,6 +452,11 @@ def main() -> int:
                       "cannot be built offline (no Go toolchain)" % (sample, threads),
             "gpu_output_matches": same,
         }
+    ctx.close()
+    acl = bench_filter(args)
+    out["extra"] = {"acl_filter": {k: acl[k] for k in ("metric", "value", "unit", "ms_per_step",
+                                                       "config", "roofline", "cpu_baseline")
+                                   if k in acl}}
     print(json.dumps(out))
     return 0
 

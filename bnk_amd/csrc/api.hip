@@ -310,4 +310,38 @@ int bnk_probe_valu(bnk_ctx *ctx, int op, uint32_t iters, double *ops_per_sec)
     return BNK_OK;
 }
 
+int bnk_probe_copy(bnk_ctx *ctx, size_t bytes, uint32_t iters, double *bytes_per_sec)
+{
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    if (!bytes_per_sec || iters == 0 || bytes < 4096 || (bytes & 15))
+        return fail(ctx, BNK_E_INVAL, "bad copy probe request");
+    hipDeviceProp_t prop;
+    HIPCHK(ctx, hipGetDeviceProperties(&prop, ctx->device));
+    const uint32_t blocks = (uint32_t)prop.multiProcessorCount * 16u;
+    void *src = nullptr, *dst = nullptr;
+    HIPCHK(ctx, hipMalloc(&src, bytes));
+    hipError_t e = hipMalloc(&dst, bytes);
+    if (e != hipSuccess) {
+        (void)hipFree(src);
+        return fail_hip(ctx, "hipMalloc", e);
+    }
+    float ms = 0;
+    e = launch_fill_u32((uint32_t *)src, (uint32_t)std::min<size_t>(bytes / 4, 1u << 30), 0x5a5a5a5au,
+                        ctx->stream);
+    if (e == hipSuccess) e = launch_copy(src, dst, bytes, blocks, ctx->stream); // warm-up
+    if (e == hipSuccess) e = hipEventRecord(ctx->ev0, ctx->stream);
+    for (uint32_t i = 0; i < iters && e == hipSuccess; i++)
+        e = launch_copy(src, dst, bytes, blocks, ctx->stream);
+    if (e == hipSuccess) e = hipEventRecord(ctx->ev1, ctx->stream);
+    if (e == hipSuccess) e = hipEventSynchronize(ctx->ev1);
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, ctx->ev0, ctx->ev1);
+    (void)hipFree(src);
+    (void)hipFree(dst);
+    if (e != hipSuccess) return fail_hip(ctx, "copy probe", e);
+    // bytes read plus bytes written
+    *bytes_per_sec = 2.0 * (double)bytes * iters / ((double)ms * 1e-3);
+    return BNK_OK;
+}
+
 } // extern "C"

@@ -58,6 +58,7 @@ hipError_t launch_relay_assign(const uint8_t *auth, const uint8_t *pass, const u
 // optimised away.
 hipError_t launch_probe(int op, uint32_t iters, uint32_t blocks, uint32_t *out,
                         hipStream_t s);
+hipError_t launch_copy(const void *src, void *dst, size_t bytes, uint32_t blocks, hipStream_t s);
 constexpr int PROBE_OPS = 24;
 constexpr uint32_t PROBE_THREADS = 256;
 constexpr uint32_t PROBE_CHAINS = 8;   // independent dependency chains per lane

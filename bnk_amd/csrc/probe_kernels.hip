@@ -66,6 +66,21 @@ __global__ __launch_bounds__(256) void probe_kernel(uint32_t iters, uint32_t *ou
     out[tid] = acc;
 }
 
+// Plain streaming copy: the measured HBM ceiling, and the known-size kernel
+// the FETCH_SIZE / WRITE_SIZE counters are scaled against.
+__global__ __launch_bounds__(256) void copy_kernel(const uint4 *src, uint4 *dst, size_t n16)
+{
+    const size_t stride = (size_t)gridDim.x * 256u;
+    for (size_t i = (size_t)blockIdx.x * 256u + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
+}
+
+hipError_t launch_copy(const void *src, void *dst, size_t bytes, uint32_t blocks, hipStream_t s)
+{
+    hipLaunchKernelGGL(copy_kernel, dim3(blocks), dim3(256), 0, s, (const uint4 *)src, (uint4 *)dst,
+                       bytes / 16);
+    return hipGetLastError();
+}
+
 template <int OP>
 static hipError_t probe_dispatch(int op, uint32_t iters, uint32_t blocks, uint32_t *out, hipStream_t s)
 {

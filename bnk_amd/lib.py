@@ -294,6 +294,13 @@ class Context:
         return float(r.value)
 
 
+    def probe_copy(self, nbytes: int, iters: int) -> float:
+        r = C.c_double()
+        self._chk(self._lib.bnk_probe_copy(self._h, C.c_size_t(nbytes), C.c_uint32(iters),
+                                           C.byref(r)))
+        return float(r.value)
+
+
 class HostFilter:
     """The reference's filter.Filter method set (internal/filter/filter.go:41-59,
     121, 189) over a Context, one packet per call."""

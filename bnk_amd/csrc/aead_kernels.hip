@@ -12,16 +12,43 @@
 
 namespace bnk {
 
-// Global memory accesses of 16 bytes at any byte alignment (the hardware
-// handles misaligned dwordx4 accesses; aligned ones cost nothing extra).
+// Packet pointers travel between lanes as integers, which would leave the
+// compiler with flat accesses (and flat accesses also tick the LDS counter,
+// stalling LDS waits behind loads still in flight): name the global address
+// space explicitly.
+#define BNK_GLOBAL __attribute__((address_space(1)))
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef u32x4 __attribute__((aligned(1))) u32x4_unaligned;
+
+// 16 bytes of global memory at any byte alignment (the hardware handles
+// misaligned dwordx4 accesses; aligned ones cost nothing extra).
 BNK_DEV uint4 ld16(const uint8_t *p)
 {
-    uint4 v;
-    __builtin_memcpy(&v, p, 16);
-    return v;
+    const u32x4 v = *reinterpret_cast<const BNK_GLOBAL u32x4_unaligned *>((uintptr_t)p);
+    return make_uint4(v.x, v.y, v.z, v.w);
 }
 
-BNK_DEV void st16(uint8_t *p, uint4 v) { __builtin_memcpy(p, &v, 16); }
+BNK_DEV void st16(uint8_t *p, uint4 v)
+{
+    const u32x4 t = {v.x, v.y, v.z, v.w};
+    *reinterpret_cast<BNK_GLOBAL u32x4_unaligned *>((uintptr_t)p) = t;
+}
+
+// The same for addresses known to be 16-byte aligned.
+BNK_DEV uint4 ld16a(const uint8_t *p)
+{
+    const u32x4 v = *reinterpret_cast<const BNK_GLOBAL u32x4 *>((uintptr_t)p);
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+
+BNK_DEV void st16a(uint8_t *p, uint4 v)
+{
+    const u32x4 t = {v.x, v.y, v.z, v.w};
+    *reinterpret_cast<BNK_GLOBAL u32x4 *>((uintptr_t)p) = t;
+}
+
+BNK_DEV uint8_t ld8(const uint8_t *p) { return *reinterpret_cast<const BNK_GLOBAL uint8_t *>((uintptr_t)p); }
+BNK_DEV void st8(uint8_t *p, uint8_t v) { *reinterpret_cast<BNK_GLOBAL uint8_t *>((uintptr_t)p) = v; }
 
 // m in 1..15 bytes at p, zero-extended to 16.
 BNK_DEV uint4 ld_partial(const uint8_t *p, uint32_t m)
@@ -29,7 +56,7 @@ BNK_DEV uint4 ld_partial(const uint8_t *p, uint32_t m)
     uint32_t w[4] = {0, 0, 0, 0};
 #pragma unroll
     for (int i = 0; i < 15; i++)
-        if ((uint32_t)i < m) w[i >> 2] |= (uint32_t)p[i] << (8 * (i & 3));
+        if ((uint32_t)i < m) w[i >> 2] |= (uint32_t)ld8(p + i) << (8 * (i & 3));
     return make_uint4(w[0], w[1], w[2], w[3]);
 }
 
@@ -38,7 +65,7 @@ BNK_DEV void st_partial(uint8_t *p, uint4 v, uint32_t m)
     const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
     for (int i = 0; i < 15; i++)
-        if ((uint32_t)i < m) p[i] = (uint8_t)(w[i >> 2] >> (8 * (i & 3)));
+        if ((uint32_t)i < m) st8(p + i, (uint8_t)(w[i >> 2] >> (8 * (i & 3))));
 }
 
 // Keeps the low m (0..16) bytes of a 16-byte little-endian value.
@@ -60,7 +87,7 @@ BNK_DEV void zero_fill(uint8_t *dst, uint32_t len)
 {
     uint32_t pos = 0;
     for (; pos + 16 <= len; pos += 16) st16(dst + pos, make_uint4(0, 0, 0, 0));
-    for (; pos < len; pos++) dst[pos] = 0;
+    for (; pos < len; pos++) st8(dst + pos, 0);
 }
 
 BNK_DEV uint64_t shfl64(uint64_t v, int src_lane)
@@ -80,18 +107,229 @@ BNK_DEV void wave_sync()
 }
 
 // One wave = 64 packets, one lane per packet for the arithmetic.  Memory is
-// touched cooperatively: in step b the wave moves bytes [64b, 64b+64) of all
-// its 64 packets with four 16-byte accesses per lane, four adjacent lanes
-// covering one packet's 64 contiguous bytes, and a 64 x 80-byte LDS tile
-// (64 data bytes + 16 bytes of padding per row, which keeps the per-lane row
-// reads free of bank conflicts) turns that layout into one row per lane.
-constexpr uint32_t LDS_ROW = 80;
+// touched cooperatively through a per-wave LDS tile, in one of two ways.
+//
+// Line path (every packet of the wave 16-byte aligned, source and destination
+// at the same offset within a 128-byte line): the wave moves whole aligned
+// 128-byte lines, eight adjacent lanes per line, so every HBM/L2 access is a
+// full line touched exactly once.  A packet rarely starts on a line boundary,
+// so each LDS row is a ring of two lines: step s consumes packet bytes
+// [128s, 128s+128), which live in lines s and s+1 of the packet; line s+1 is
+// fetched just before step s, line s is complete and written back just after.
+// Only the 16-byte cells that belong to the packet are ever read or written,
+// so neighbours sharing a line are never disturbed.
+//
+// Generic path (anything else): 64 bytes per packet per step, four adjacent
+// lanes per packet, any byte alignment.
+constexpr uint32_t LDS_ROW = 80;    // generic: 64 data bytes + 16 pad
+constexpr uint32_t RING_ROW = 272;  // line path: 2 x 128-byte lines + 16 pad
 constexpr uint32_t WAVES_PER_BLOCK = 4;
 
 template <bool OPEN>
-__global__ __launch_bounds__(256) void aead_wave_kernel(AeadArgs a)
+BNK_DEV void crypt_cell(Poly26 &mac, const uint32_t (&x)[16], int j, uint8_t *cell)
 {
-    __shared__ __attribute__((aligned(16))) uint8_t tile_all[WAVES_PER_BLOCK][64 * LDS_ROW];
+    const uint4 v = *reinterpret_cast<const uint4 *>(cell);
+    const uint4 o = make_uint4(v.x ^ x[4 * j], v.y ^ x[4 * j + 1], v.z ^ x[4 * j + 2],
+                               v.w ^ x[4 * j + 3]);
+    if (OPEN) mac.block(v.x, v.y, v.z, v.w);
+    else mac.block(o.x, o.y, o.z, o.w);
+    *reinterpret_cast<uint4 *>(cell) = o;
+}
+
+// The final 1..15 bytes of a packet go straight from and to global memory.
+template <bool OPEN>
+BNK_DEV void crypt_tail(Poly26 &mac, const uint32_t (&x)[16], int j, const uint8_t *s, uint8_t *d,
+                        uint32_t m)
+{
+    const uint4 v = ld_partial(s, m);
+    const uint4 o = keep_bytes(make_uint4(v.x ^ x[4 * j], v.y ^ x[4 * j + 1], v.z ^ x[4 * j + 2],
+                                          v.w ^ x[4 * j + 3]), m);
+    // the MAC sees the ciphertext zero-padded to 16 bytes
+    if (OPEN) mac.block(v.x, v.y, v.z, v.w);
+    else mac.block(o.x, o.y, o.z, o.w);
+    st_partial(d, o, m);
+}
+
+template <bool OPEN>
+BNK_DEV void body_generic(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_t *dst,
+                          uint32_t len, const uint32_t (&k)[8], uint32_t n1, uint32_t n2,
+                          Poly26 &mac, uint32_t (&x)[16])
+{
+    const uint32_t nfull = len >> 6, rem = len & 63u;
+    const uint32_t steps = nfull + (rem ? 1u : 0u);
+    // the four (packet, 16-byte column) cells this lane moves per step
+    const uint32_t col = lane & 3u;
+    const uint8_t *csrc[4];
+    uint8_t *cdst[4];
+    uint32_t clen[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int owner = 16 * j + (int)(lane >> 2);
+        csrc[j] = reinterpret_cast<const uint8_t *>(shfl64((uint64_t)(uintptr_t)src, owner)) + 16u * col;
+        cdst[j] = reinterpret_cast<uint8_t *>(shfl64((uint64_t)(uintptr_t)dst, owner)) + 16u * col;
+        clen[j] = (uint32_t)__shfl((int)len, owner, 64);
+    }
+    for (uint32_t b = 0; __ballot(b < steps) != 0ull; b++) {
+        const uint32_t pos = 64u * b + 16u * col;
+        // global -> LDS, all 64 lanes, only 16-byte cells that lie fully inside a packet
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            if (pos + 16u <= clen[j]) {
+                const uint4 v = ld16(csrc[j] + 64u * b);
+                *reinterpret_cast<uint4 *>(tile + (16u * j + (lane >> 2)) * LDS_ROW + 16u * col) = v;
+            }
+        }
+        wave_sync();
+        if (b < steps) {
+            chacha_block(k, b + 1, n1, n2, x);
+            uint8_t *row = tile + lane * LDS_ROW;
+            if (b < nfull) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) crypt_cell<OPEN>(mac, x, j, row + 16 * j);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    if (rem >= 16u * (j + 1)) crypt_cell<OPEN>(mac, x, j, row + 16 * j);
+                    else if (rem > 16u * j)
+                        crypt_tail<OPEN>(mac, x, j, src + 64u * b + 16 * j, dst + 64u * b + 16 * j,
+                                         rem - 16u * j);
+                }
+            }
+        }
+        wave_sync();
+        // LDS -> global
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            if (pos + 16u <= clen[j]) {
+                const uint4 v = *reinterpret_cast<const uint4 *>(
+                    tile + (16u * j + (lane >> 2)) * LDS_ROW + 16u * col);
+                st16(cdst[j] + 64u * b, v);
+            }
+        }
+        wave_sync();
+    }
+}
+
+template <bool OPEN>
+BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_t *dst, uint32_t len,
+                        const uint32_t (&k)[8], uint32_t n1, uint32_t n2, Poly26 &mac,
+                        uint32_t (&x)[16])
+{
+    // Cells are 16 bytes; a packet's cell kc sits at stream position c0 + kc,
+    // where the stream starts at the 128-byte line holding the packet's first
+    // byte.  Stream position K lives in line K / 8 and in ring cell K % 16.
+    const uint32_t skew = (uint32_t)(uintptr_t)src & 127u;
+    const uint32_t c0 = skew >> 4;
+    const uint32_t ncell = len >> 4; // whole cells; a shorter tail is handled by its owner
+    const uint32_t steps = (len + 127u) >> 7;
+    const uint32_t sub = lane & 7u;
+    // the eight (packet, cell-of-line) positions this lane moves per line
+    const uint8_t *csrc[8];
+    uint8_t *cdst[8];
+    uint32_t cfirst[8], cend[8];
+#pragma unroll
+    for (int q = 0; q < 8; q++) {
+        const int owner = 8 * q + (int)(lane >> 3);
+        csrc[q] = reinterpret_cast<const uint8_t *>(shfl64((uint64_t)(uintptr_t)(src - skew), owner)) + 16u * sub;
+        cdst[q] = reinterpret_cast<uint8_t *>(shfl64((uint64_t)(uintptr_t)(dst - skew), owner)) + 16u * sub;
+        cfirst[q] = (uint32_t)__shfl((int)c0, owner, 64);
+        cend[q] = cfirst[q] + (uint32_t)__shfl((int)ncell, owner, 64);
+    }
+    uint32_t maxsteps = steps;
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        const uint32_t o = (uint32_t)__shfl_xor((int)maxsteps, off, 64);
+        maxsteps = o > maxsteps ? o : maxsteps;
+    }
+    maxsteps = __builtin_amdgcn_readfirstlane(maxsteps);
+
+    // Lines are fetched one iteration ahead into registers (issue), so the
+    // loads fly while the wave computes, and only then moved into the ring
+    // (commit), which overwrites the half whose line was written back last.
+    uint4 pre0 = make_uint4(0, 0, 0, 0), pre1 = pre0, pre2 = pre0, pre3 = pre0, pre4 = pre0,
+          pre5 = pre0, pre6 = pre0, pre7 = pre0;
+#define BNK_ISSUE(q, m)                                                                     \
+    if (8u * (m) + sub >= cfirst[q] && 8u * (m) + sub < cend[q])                            \
+        pre##q = ld16a(csrc[q] + 128u * (m))
+#define BNK_COMMIT(q, m)                                                                    \
+    if (8u * (m) + sub >= cfirst[q] && 8u * (m) + sub < cend[q])                            \
+        *reinterpret_cast<uint4 *>(tile + (8u * q + (lane >> 3)) * RING_ROW +               \
+                                   (((8u * (m) + sub) & 15u) << 4)) = pre##q
+#define BNK_ISSUE_LINE(m)                                                                   \
+    do {                                                                                    \
+        BNK_ISSUE(0, m); BNK_ISSUE(1, m); BNK_ISSUE(2, m); BNK_ISSUE(3, m);                 \
+        BNK_ISSUE(4, m); BNK_ISSUE(5, m); BNK_ISSUE(6, m); BNK_ISSUE(7, m);                 \
+    } while (0)
+#define BNK_COMMIT_LINE(m)                                                                  \
+    do {                                                                                    \
+        BNK_COMMIT(0, m); BNK_COMMIT(1, m); BNK_COMMIT(2, m); BNK_COMMIT(3, m);             \
+        BNK_COMMIT(4, m); BNK_COMMIT(5, m); BNK_COMMIT(6, m); BNK_COMMIT(7, m);             \
+    } while (0)
+    auto store_line = [&](uint32_t m) __attribute__((always_inline)) {
+        const uint32_t K = 8u * m + sub;
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+            if (K >= cfirst[q] && K < cend[q]) {
+                const uint4 v = *reinterpret_cast<const uint4 *>(
+                    tile + (8u * q + (lane >> 3)) * RING_ROW + ((K & 15u) << 4));
+                st16a(cdst[q] + 128u * m, v);
+            }
+        }
+    };
+
+    uint8_t *row = tile + lane * RING_ROW;
+    BNK_ISSUE_LINE(0u);
+    BNK_COMMIT_LINE(0u);
+    BNK_ISSUE_LINE(1u);
+    // iteration s: line s+1 enters the ring, line s+2 starts flying, packet
+    // bytes [128s, 128s+128) are processed, line s is written back; the extra
+    // last iteration only writes back the final line
+    for (uint32_t s = 0; s <= maxsteps; s++) {
+        BNK_COMMIT_LINE(s + 1);
+        if (s + 2 <= maxsteps) BNK_ISSUE_LINE(s + 2);
+        wave_sync();
+        if (s < steps) {
+            if (8u * s + 8u <= ncell) {
+                // all eight cells of this step are whole cells of the packet
+#pragma unroll 1
+                for (uint32_t h = 0; h < 2; h++) {
+                    chacha_block(k, 2u * s + h + 1, n1, n2, x);
+                    const uint32_t r0 = c0 + 8u * s + 4u * h;
+#pragma unroll
+                    for (int j = 0; j < 4; j++) crypt_cell<OPEN>(mac, x, j, row + (((r0 + j) & 15u) << 4));
+                }
+            } else {
+#pragma unroll 1
+                for (uint32_t h = 0; h < 2; h++) {
+                    const uint32_t b = 2u * s + h;
+                    if (64u * b < len) {
+                        chacha_block(k, b + 1, n1, n2, x);
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            const uint32_t kc = 4u * b + j;
+                            if (kc < ncell) crypt_cell<OPEN>(mac, x, j, row + (((c0 + kc) & 15u) << 4));
+                            else if (kc == ncell && (len & 15u))
+                                crypt_tail<OPEN>(mac, x, j, src + 16u * kc, dst + 16u * kc, len & 15u);
+                        }
+                    }
+                }
+            }
+        }
+        wave_sync();
+        store_line(s);
+        wave_sync();
+    }
+#undef BNK_ISSUE
+#undef BNK_COMMIT
+#undef BNK_ISSUE_LINE
+#undef BNK_COMMIT_LINE
+}
+
+template <bool OPEN>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void aead_wave_kernel(AeadArgs a)
+{
+    __shared__ __attribute__((aligned(16))) uint8_t tile_all[WAVES_PER_BLOCK][64 * RING_ROW];
+    static_assert(RING_ROW >= LDS_ROW, "the generic path reuses the tile");
     const uint32_t lane = threadIdx.x & 63u;
     uint8_t *tile = tile_all[threadIdx.x >> 6];
     const uint32_t t = blockIdx.x * 256u + threadIdx.x;
@@ -128,21 +366,10 @@ __global__ __launch_bounds__(256) void aead_wave_kernel(AeadArgs a)
             ctr = a.counters ? a.counters[i] : a.counter0 + i;
         }
     }
-    if (!have) len = 0;
-    const uint32_t nfull = len >> 6, rem = len & 63u;
-    const uint32_t steps = nfull + (rem ? 1u : 0u);
-
-    // ---- the four (packet, 16-byte column) cells this lane moves per step ----
-    const uint32_t col = lane & 3u;
-    const uint8_t *csrc[4];
-    uint8_t *cdst[4];
-    uint32_t clen[4];
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-        const int owner = 16 * j + (int)(lane >> 2);
-        csrc[j] = reinterpret_cast<const uint8_t *>(shfl64((uint64_t)(uintptr_t)src, owner)) + 16u * col;
-        cdst[j] = reinterpret_cast<uint8_t *>(shfl64((uint64_t)(uintptr_t)dst, owner)) + 16u * col;
-        clen[j] = (uint32_t)__shfl((int)len, owner, 64);
+    if (!have) {
+        len = 0;
+        src = nullptr;
+        dst = nullptr;
     }
 
     const uint32_t n1 = (uint32_t)ctr, n2 = (uint32_t)(ctr >> 32);
@@ -151,68 +378,10 @@ __global__ __launch_bounds__(256) void aead_wave_kernel(AeadArgs a)
     Poly26 mac;
     mac.init(x);
 
-    for (uint32_t b = 0; __ballot(b < steps) != 0ull; b++) {
-        const uint32_t pos = 64u * b + 16u * col;
-        // global -> LDS, all 64 lanes, only 16-byte cells that lie fully inside a packet
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            if (pos + 16u <= clen[j]) {
-                const uint4 v = ld16(csrc[j] + 64u * b);
-                *reinterpret_cast<uint4 *>(tile + (16u * j + (lane >> 2)) * LDS_ROW + 16u * col) = v;
-            }
-        }
-        wave_sync();
-        if (b < steps) {
-            chacha_block(k, b + 1, n1, n2, x);
-            uint8_t *row = tile + lane * LDS_ROW;
-            if (b < nfull) {
-#pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    const uint4 v = *reinterpret_cast<const uint4 *>(row + 16 * j);
-                    const uint4 o = make_uint4(v.x ^ x[4 * j], v.y ^ x[4 * j + 1],
-                                               v.z ^ x[4 * j + 2], v.w ^ x[4 * j + 3]);
-                    if (OPEN) mac.block(v.x, v.y, v.z, v.w);
-                    else mac.block(o.x, o.y, o.z, o.w);
-                    *reinterpret_cast<uint4 *>(row + 16 * j) = o;
-                }
-            } else {
-                // last, partial block: whole cells through the tile, the
-                // final 1..15 bytes straight from and to global memory
-#pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    if (rem >= 16u * (j + 1)) {
-                        const uint4 v = *reinterpret_cast<const uint4 *>(row + 16 * j);
-                        const uint4 o = make_uint4(v.x ^ x[4 * j], v.y ^ x[4 * j + 1],
-                                                   v.z ^ x[4 * j + 2], v.w ^ x[4 * j + 3]);
-                        if (OPEN) mac.block(v.x, v.y, v.z, v.w);
-                        else mac.block(o.x, o.y, o.z, o.w);
-                        *reinterpret_cast<uint4 *>(row + 16 * j) = o;
-                    } else if (rem > 16u * j) {
-                        const uint32_t m = rem - 16u * j;
-                        const uint4 v = ld_partial(src + 64u * b + 16 * j, m);
-                        const uint4 o = keep_bytes(
-                            make_uint4(v.x ^ x[4 * j], v.y ^ x[4 * j + 1],
-                                       v.z ^ x[4 * j + 2], v.w ^ x[4 * j + 3]), m);
-                        // the MAC sees the ciphertext zero-padded to 16 bytes
-                        if (OPEN) mac.block(v.x, v.y, v.z, v.w);
-                        else mac.block(o.x, o.y, o.z, o.w);
-                        st_partial(dst + 64u * b + 16 * j, o, m);
-                    }
-                }
-            }
-        }
-        wave_sync();
-        // LDS -> global
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            if (pos + 16u <= clen[j]) {
-                const uint4 v = *reinterpret_cast<const uint4 *>(
-                    tile + (16u * j + (lane >> 2)) * LDS_ROW + 16u * col);
-                st16(cdst[j] + 64u * b, v);
-            }
-        }
-        wave_sync();
-    }
+    const bool lane_lines = (((uintptr_t)src | (uintptr_t)dst) & 15u) == 0 &&
+                            (((uintptr_t)src ^ (uintptr_t)dst) & 127u) == 0;
+    if (__ballot(!lane_lines) == 0ull) body_lines<OPEN>(tile, lane, src, dst, len, k, n1, n2, mac, x);
+    else body_generic<OPEN>(tile, lane, src, dst, len, k, n1, n2, mac, x);
 
     bool reject = false;
     if (have) {

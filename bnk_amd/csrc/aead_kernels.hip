@@ -83,13 +83,6 @@ BNK_DEV uint4 keep_bytes(uint4 v, uint32_t m)
     return make_uint4(w[0], w[1], w[2], w[3]);
 }
 
-BNK_DEV void zero_fill(uint8_t *dst, uint32_t len)
-{
-    uint32_t pos = 0;
-    for (; pos + 16 <= len; pos += 16) st16(dst + pos, make_uint4(0, 0, 0, 0));
-    for (; pos < len; pos++) st8(dst + pos, 0);
-}
-
 BNK_DEV uint64_t shfl64(uint64_t v, int src_lane)
 {
     const uint32_t lo = (uint32_t)__shfl((int)(uint32_t)v, src_lane, 64);
@@ -400,11 +393,25 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             a.verdict[i] = reject ? 0 : 1;
         }
     }
-    if (OPEN && __ballot(reject) != 0ull) {
-        // the plaintext cells were stored by other lanes of this wave: make
-        // those stores land before this lane overwrites them with zeros
-        __threadfence();
-        if (reject) zero_fill(dst, len);
+    if (OPEN) {
+        unsigned long long rej = __ballot(reject);
+        if (rej != 0ull) {
+            // the plaintext cells were stored by other lanes of this wave: wait
+            // until those stores have been acknowledged (a workgroup-scope
+            // release is just that wait; a wider fence would write back the
+            // whole L2), then the wave clears each rejected packet together
+            // (chacha20poly1305.Open leaves zeros behind)
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+            while (rej != 0ull) {
+                const int r = __ffsll((long long)rej) - 1;
+                rej &= rej - 1ull;
+                uint8_t *d = reinterpret_cast<uint8_t *>(shfl64((uint64_t)(uintptr_t)dst, r));
+                const uint32_t L = (uint32_t)__shfl((int)len, r, 64);
+                for (uint32_t pos = 16u * lane; pos + 16u <= L; pos += 1024u)
+                    st16(d + pos, make_uint4(0, 0, 0, 0));
+                if (lane < (L & 15u)) st8(d + (L & ~15u) + lane, 0);
+            }
+        }
     }
 }
 

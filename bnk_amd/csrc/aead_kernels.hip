@@ -119,7 +119,7 @@ constexpr uint32_t RING_ROW = 272;  // line path: 2 x 128-byte lines + 16 pad
 constexpr uint32_t WAVES_PER_BLOCK = 4;
 
 template <bool OPEN>
-BNK_DEV void crypt_cell(Poly26 &mac, const uint32_t (&x)[16], int j, uint8_t *cell)
+BNK_DEV void crypt_cell(Poly32 &mac, const uint32_t (&x)[16], int j, uint8_t *cell)
 {
     const uint4 v = *reinterpret_cast<const uint4 *>(cell);
     const uint4 o = make_uint4(v.x ^ x[4 * j], v.y ^ x[4 * j + 1], v.z ^ x[4 * j + 2],
@@ -131,7 +131,7 @@ BNK_DEV void crypt_cell(Poly26 &mac, const uint32_t (&x)[16], int j, uint8_t *ce
 
 // The final 1..15 bytes of a packet go straight from and to global memory.
 template <bool OPEN>
-BNK_DEV void crypt_tail(Poly26 &mac, const uint32_t (&x)[16], int j, const uint8_t *s, uint8_t *d,
+BNK_DEV void crypt_tail(Poly32 &mac, const uint32_t (&x)[16], int j, const uint8_t *s, uint8_t *d,
                         uint32_t m)
 {
     const uint4 v = ld_partial(s, m);
@@ -146,7 +146,7 @@ BNK_DEV void crypt_tail(Poly26 &mac, const uint32_t (&x)[16], int j, const uint8
 template <bool OPEN>
 BNK_DEV void body_generic(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_t *dst,
                           uint32_t len, const uint32_t (&k)[8], uint32_t n1, uint32_t n2,
-                          Poly26 &mac, uint32_t (&x)[16])
+                          Poly32 &mac, uint32_t (&x)[16])
 {
     const uint32_t nfull = len >> 6, rem = len & 63u;
     const uint32_t steps = nfull + (rem ? 1u : 0u);
@@ -205,7 +205,7 @@ BNK_DEV void body_generic(uint8_t *tile, uint32_t lane, const uint8_t *src, uint
 
 template <bool OPEN>
 BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_t *dst, uint32_t len,
-                        const uint32_t (&k)[8], uint32_t n1, uint32_t n2, Poly26 &mac,
+                        const uint32_t (&k)[8], uint32_t n1, uint32_t n2, Poly32 &mac,
                         uint32_t (&x)[16])
 {
     // Cells are 16 bytes; a packet's cell kc sits at stream position c0 + kc,
@@ -368,7 +368,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const uint32_t n1 = (uint32_t)ctr, n2 = (uint32_t)(ctr >> 32);
     uint32_t x[16];
     chacha_block(k, 0, n1, n2, x);
-    Poly26 mac;
+    Poly32 mac;
     mac.init(x);
 
     const bool lane_lines = (((uintptr_t)src | (uintptr_t)dst) & 15u) == 0 &&

@@ -3,17 +3,28 @@
 // One lane owns one packet end to end: the 16-word ChaCha20 state and the
 // Poly1305 accumulator stay in VGPRs for the packet's whole life, there is no
 // cross-lane traffic and no LDS.  32-bit add/xor/rotate (v_alignbit_b32) for
-// ChaCha20; Poly1305 in radix 2^26 with v_mad_u64_u32 partial products.
+// ChaCha20; Poly1305 with v_mad_u64_u32 partial products (radix 2^32 in the
+// kernels; the radix 2^26 layout is kept as an independent cross-check).
 #pragma once
 
-#include <hip/hip_runtime.h>
 #include <stdint.h>
+
+// The arithmetic in this header is plain 32/64-bit integer C++, so the same
+// source also compiles for the host: tests/cpp/lane_test.cpp runs it on the
+// CPU against the RFC 8439 vectors (including Poly1305 carry edge cases that
+// random packets never reach).  The library itself only ever uses it on the GPU.
+#if defined(__HIPCC__)
+#include <hip/hip_runtime.h>
+#define BNK_DEV __device__ __forceinline__
+#else
+#define BNK_DEV inline
+#endif
 
 namespace bnk {
 
-#define BNK_DEV __device__ __forceinline__
-
-BNK_DEV uint32_t rotl32(uint32_t v, int c) { return __builtin_rotateleft32(v, c); }
+BNK_DEV uint32_t rotl32(uint32_t v, int c) { return v << c | v >> (32 - c); }
+// low 32 bits of (hi:lo) >> s, 0 < s < 32 (one v_alignbit_b32 on the GPU)
+BNK_DEV uint32_t funnel(uint32_t hi, uint32_t lo, int s) { return lo >> s | hi << (32 - s); }
 
 #define BNK_QR(a, b, c, d)                          \
     a += b; d ^= a; d = rotl32(d, 16);              \
@@ -73,9 +84,9 @@ struct Poly26 {
     BNK_DEV void block(uint32_t w0, uint32_t w1, uint32_t w2, uint32_t w3)
     {
         const uint32_t a0 = h0 + (w0 & 0x3ffffffu);
-        const uint32_t a1 = h1 + (__builtin_amdgcn_alignbit(w1, w0, 26) & 0x3ffffffu);
-        const uint32_t a2 = h2 + (__builtin_amdgcn_alignbit(w2, w1, 20) & 0x3ffffffu);
-        const uint32_t a3 = h3 + (__builtin_amdgcn_alignbit(w3, w2, 14) & 0x3ffffffu);
+        const uint32_t a1 = h1 + (funnel(w1, w0, 26) & 0x3ffffffu);
+        const uint32_t a2 = h2 + (funnel(w2, w1, 20) & 0x3ffffffu);
+        const uint32_t a3 = h3 + (funnel(w3, w2, 14) & 0x3ffffffu);
         const uint32_t a4 = h4 + ((w3 >> 8) | (1u << 24));
 
         uint64_t d0 = (uint64_t)a0 * r0 + (uint64_t)a1 * s4 + (uint64_t)a2 * s3 +
@@ -132,6 +143,82 @@ struct Poly26 {
         f = (uint64_t)w1 + pad1 + (f >> 32); tag[1] = (uint32_t)f;
         f = (uint64_t)w2 + pad2 + (f >> 32); tag[2] = (uint32_t)f;
         f = (uint64_t)w3 + pad3 + (f >> 32); tag[3] = (uint32_t)f;
+    }
+};
+
+// Poly1305 in radix 2^32: the accumulator is four 32-bit words plus a small
+// fifth, r is its four clamped words.  The clamp clears the low two bits of
+// r1..r3, so a product that lands at 2^128 or above folds back exactly with
+// s_j = r_j + r_j/4 = 5*r_j/4 (2^130 = 5 mod p).  Message words are used as
+// they are: no limb extraction, 20 multiplies per block.
+struct Poly32 {
+    uint32_t r0, r1, r2, r3;
+    uint32_t s1, s2, s3;
+    uint32_t h0, h1, h2, h3, h4;
+    uint32_t pad0, pad1, pad2, pad3;
+
+    // otk = first 8 words of ChaCha20 block 0
+    BNK_DEV void init(const uint32_t (&x)[16])
+    {
+        r0 = x[0] & 0x0fffffffu; r1 = x[1] & 0x0ffffffcu;
+        r2 = x[2] & 0x0ffffffcu; r3 = x[3] & 0x0ffffffcu;
+        s1 = r1 + (r1 >> 2); s2 = r2 + (r2 >> 2); s3 = r3 + (r3 >> 2);
+        h0 = h1 = h2 = h3 = h4 = 0;
+        pad0 = x[4]; pad1 = x[5]; pad2 = x[6]; pad3 = x[7];
+    }
+
+    // One full 16-byte block (little-endian words w0..w3) with bit 128 set.
+    BNK_DEV void block(uint32_t w0, uint32_t w1, uint32_t w2, uint32_t w3)
+    {
+        uint64_t t;
+        t = (uint64_t)h0 + w0;             const uint32_t a0 = (uint32_t)t;
+        t = (uint64_t)h1 + w1 + (t >> 32); const uint32_t a1 = (uint32_t)t;
+        t = (uint64_t)h2 + w2 + (t >> 32); const uint32_t a2 = (uint32_t)t;
+        t = (uint64_t)h3 + w3 + (t >> 32); const uint32_t a3 = (uint32_t)t;
+        const uint32_t a4 = h4 + (uint32_t)(t >> 32) + 1u; // at most 9
+
+        // a_i < 2^32, r_j < 2^28, s_j < 1.25 * 2^28: four terms stay below 2^63
+        uint64_t d0 = (uint64_t)a0 * r0 + (uint64_t)a1 * s3 + (uint64_t)a2 * s2 + (uint64_t)a3 * s1;
+        uint64_t d1 = (uint64_t)a0 * r1 + (uint64_t)a1 * r0 + (uint64_t)a2 * s3 + (uint64_t)a3 * s2 +
+                      (uint64_t)(a4 * s1);
+        uint64_t d2 = (uint64_t)a0 * r2 + (uint64_t)a1 * r1 + (uint64_t)a2 * r0 + (uint64_t)a3 * s3 +
+                      (uint64_t)(a4 * s2);
+        uint64_t d3 = (uint64_t)a0 * r3 + (uint64_t)a1 * r2 + (uint64_t)a2 * r1 + (uint64_t)a3 * r0 +
+                      (uint64_t)(a4 * s3);
+        uint32_t e4 = a4 * r0; // stays at 2^128; below 2^32 because a4 <= 9
+
+        d1 += d0 >> 32;
+        d2 += d1 >> 32;
+        d3 += d2 >> 32;
+        e4 += (uint32_t)(d3 >> 32);
+        // everything at and above 2^130 comes back times 5
+        const uint32_t c = (e4 >> 2) * 5u;
+        t = (uint64_t)(uint32_t)d0 + c;             h0 = (uint32_t)t;
+        t = (uint64_t)(uint32_t)d1 + (t >> 32);     h1 = (uint32_t)t;
+        t = (uint64_t)(uint32_t)d2 + (t >> 32);     h2 = (uint32_t)t;
+        t = (uint64_t)(uint32_t)d3 + (t >> 32);     h3 = (uint32_t)t;
+        h4 = (e4 & 3u) + (uint32_t)(t >> 32);
+    }
+
+    // tag = ((h mod 2^130-5) + s) mod 2^128 as four little-endian words
+    BNK_DEV void finish(uint32_t (&tag)[4])
+    {
+        // h < 2^130 + small: h >= p  <=>  h + 5 >= 2^130
+        uint64_t t;
+        t = (uint64_t)h0 + 5u;         const uint32_t g0 = (uint32_t)t;
+        t = (uint64_t)h1 + (t >> 32);  const uint32_t g1 = (uint32_t)t;
+        t = (uint64_t)h2 + (t >> 32);  const uint32_t g2 = (uint32_t)t;
+        t = (uint64_t)h3 + (t >> 32);  const uint32_t g3 = (uint32_t)t;
+        const uint32_t g4 = h4 + (uint32_t)(t >> 32);
+        const uint32_t take_g = 0u - (uint32_t)((g4 >> 2) != 0); // all ones when h + 5 >= 2^130
+        const uint32_t f0 = (h0 & ~take_g) | (g0 & take_g);
+        const uint32_t f1 = (h1 & ~take_g) | (g1 & take_g);
+        const uint32_t f2 = (h2 & ~take_g) | (g2 & take_g);
+        const uint32_t f3 = (h3 & ~take_g) | (g3 & take_g);
+        t = (uint64_t)f0 + pad0;             tag[0] = (uint32_t)t;
+        t = (uint64_t)f1 + pad1 + (t >> 32); tag[1] = (uint32_t)t;
+        t = (uint64_t)f2 + pad2 + (t >> 32); tag[2] = (uint32_t)t;
+        t = (uint64_t)f3 + pad3 + (t >> 32); tag[3] = (uint32_t)t;
     }
 };
 

@@ -6,22 +6,17 @@ using namespace bnk;
 
 namespace bnk {
 
-static hipError_t flow_table_alloc(uint32_t cap, DevBuf &keys, DevBuf &exp, DevBuf &counters,
-                                   FlowTableDev &ft, hipStream_t s)
+static hipError_t flow_table_alloc(uint32_t cap, DevBuf &slots, DevBuf &counters, FlowTableDev &ft,
+                                   hipStream_t s)
 {
-    const size_t slots = (size_t)cap * FLOW_REGIONS;
+    const size_t n = (size_t)cap * FLOW_REGIONS;
     hipError_t e;
-    if ((e = keys.reserve(slots * 8)) != hipSuccess) return e;
-    if ((e = exp.reserve(slots * 8)) != hipSuccess) return e;
+    if ((e = slots.reserve(n * sizeof(FlowSlotMem))) != hipSuccess) return e;
     if ((e = counters.reserve(FLOW_COUNTERS * 4)) != hipSuccess) return e;
-    ft.keys = keys.as<uint64_t>();
-    ft.exp = exp.as<int64_t>();
+    ft.slots = slots.as<FlowSlotMem>();
     ft.counters = counters.as<uint32_t>();
     ft.cap = cap;
-    if ((e = launch_fill_u64(ft.keys, (uint32_t)slots, 0, s)) != hipSuccess) return e;
-    if ((e = launch_fill_u64(reinterpret_cast<uint64_t *>(ft.exp), (uint32_t)slots,
-                             (uint64_t)FLOW_TOMB, s)) != hipSuccess)
-        return e;
+    if ((e = launch_flow_clear(ft.slots, (uint32_t)n, s)) != hipSuccess) return e;
     return launch_fill_u32(ft.counters, FLOW_COUNTERS, 0, s);
 }
 
@@ -30,12 +25,12 @@ static hipError_t upload_rule_index(FilterState *f, const HostRuleIndex &h, hipS
     hipError_t e;
     const size_t nb = h.bounds.size();
     if ((e = f->bounds.reserve(std::max<size_t>(nb, 1) * 4)) != hipSuccess) return e;
-    if ((e = f->starts.reserve((nb + 1) * 4)) != hipSuccess) return e;
+    if ((e = f->meta.reserve((nb + 1) * 4)) != hipSuccess) return e;
     if ((e = f->ranges.reserve(std::max<size_t>(h.ranges.size(), 1) * 8)) != hipSuccess) return e;
     if ((e = f->wide.reserve(std::max<size_t>(h.wide.size(), 1) * 16)) != hipSuccess) return e;
     if ((e = hipMemcpyAsync(f->bounds.p, h.bounds.data(), nb * 4, hipMemcpyHostToDevice, s)) != hipSuccess)
         return e;
-    if ((e = hipMemcpyAsync(f->starts.p, h.starts.data(), (nb + 1) * 4, hipMemcpyHostToDevice, s)) !=
+    if ((e = hipMemcpyAsync(f->meta.p, h.meta.data(), (nb + 1) * 4, hipMemcpyHostToDevice, s)) !=
         hipSuccess)
         return e;
     if (!h.ranges.empty() &&
@@ -49,7 +44,7 @@ static hipError_t upload_rule_index(FilterState *f, const HostRuleIndex &h, hipS
     // the host vectors die with the caller's frame
     if ((e = hipStreamSynchronize(s)) != hipSuccess) return e;
     f->ridx.bounds = f->bounds.as<uint32_t>();
-    f->ridx.starts = f->starts.as<uint32_t>();
+    f->ridx.meta = f->meta.as<uint32_t>();
     f->ridx.ranges = f->ranges.as<uint2>();
     f->ridx.wide = f->wide.as<uint4>();
     f->ridx.n_bounds = (uint32_t)nb;
@@ -71,7 +66,7 @@ FilterState *filter_create(hipStream_t s, int cu_count)
     HostRuleIndex h;
     std::string err;
     build_rule_index(nullptr, 0, h, err);
-    if (flow_table_alloc(FLOW_CAP_INITIAL, f->keys, f->exp, f->counters, f->flows, s) != hipSuccess ||
+    if (flow_table_alloc(FLOW_CAP_INITIAL, f->slots, f->counters, f->flows, s) != hipSuccess ||
         upload_rule_index(f, h, s) != hipSuccess) {
         filter_destroy(f);
         return nullptr;
@@ -112,18 +107,18 @@ int flows_reserve(bnk_ctx *ctx, uint32_t n_new)
     uint64_t cap = FLOW_CAP_INITIAL;
     while (cap < need) cap *= 2;
     if (cap > FLOW_CAP_MAX) return fail(ctx, BNK_E_NOMEM, "flow table would exceed its maximum size");
-    DevBuf nk, ne, nc;
+    DevBuf ns, nc;
     FlowTableDev nt{};
-    hipError_t e = flow_table_alloc((uint32_t)cap, nk, ne, nc, nt, ctx->stream);
+    hipError_t e = flow_table_alloc((uint32_t)cap, ns, nc, nt, ctx->stream);
     if (e == hipSuccess)
         e = launch_flow_rehash(f->flows, nt, ctx->d_status, f->max_blocks, ctx->stream);
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
     if (e != hipSuccess) {
-        nk.release(); ne.release(); nc.release();
+        ns.release(); nc.release();
         return fail_hip(ctx, "flow table growth", e);
     }
-    f->keys.release(); f->exp.release(); f->counters.release();
-    f->keys = nk; f->exp = ne; f->counters = nc;
+    f->slots.release(); f->counters.release();
+    f->slots = ns; f->counters = nc;
     f->flows = nt;
     f->claimed_upper = (uint64_t)c[FLOW_LIVE] + n_new;
     return BNK_OK;
@@ -353,21 +348,20 @@ int bnk_filter_flow_dump(bnk_ctx *ctx, uint64_t *key, uint8_t *proto, int64_t *e
     if (!count || (cap && (!key || !proto || !expiry_ns))) return fail(ctx, BNK_E_INVAL, "null output");
     const FlowTableDev &ft = ctx->filter->flows;
     const size_t slots = (size_t)ft.cap * FLOW_REGIONS;
-    std::vector<uint64_t> hk(slots);
-    std::vector<int64_t> he(slots);
-    HIPCHK(ctx, hipMemcpyAsync(hk.data(), ft.keys, slots * 8, hipMemcpyDeviceToHost, ctx->stream));
-    HIPCHK(ctx, hipMemcpyAsync(he.data(), ft.exp, slots * 8, hipMemcpyDeviceToHost, ctx->stream));
+    std::vector<FlowSlotMem> hs(slots);
+    HIPCHK(ctx, hipMemcpyAsync(hs.data(), ft.slots, slots * sizeof(FlowSlotMem), hipMemcpyDeviceToHost,
+                               ctx->stream));
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
     static const uint8_t class_proto[3] = {1, 6, 17};
     uint32_t k = 0;
     for (size_t idx = 0; idx < slots && k < cap; idx++) {
-        if (hk[idx] == 0 || he[idx] == FLOW_TOMB) continue;
+        if (hs[idx].key == 0 || hs[idx].exp == FLOW_TOMB) continue;
         const uint32_t region = (uint32_t)(idx / ft.cap);
-        const uint64_t w = hk[idx];
+        const uint64_t w = hs[idx].key;
         const uint64_t remote = ((uint64_t)(region & 1u) << 31) | ((w >> 32) & 0x7FFFFFFFu);
         key[k] = remote << 32 | (w & 0xFFFFFFFFu);
         proto[k] = class_proto[region >> 1];
-        expiry_ns[k] = he[idx];
+        expiry_ns[k] = hs[idx].exp;
         k++;
     }
     *count = k;

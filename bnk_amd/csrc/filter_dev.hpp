@@ -10,17 +10,24 @@ constexpr uint32_t FLOW_REGIONS = 6;     // protocol class (3) x top address bit
 constexpr int64_t FLOW_TOMB = INT64_MIN; // expiry of a deleted (or never used) slot
 enum : uint32_t { FLOW_LIVE = 0, FLOW_CLAIMED = 1, FLOW_SWEEP = 2, FLOW_COUNTERS = 4 };
 
+// One 16-byte slot, so a probe is a single memory transaction.
+struct FlowSlotMem {
+    uint64_t key; // 0 = empty
+    int64_t exp;  // expiry in Unix ns, FLOW_TOMB = not in the map
+};
+
 struct FlowTableDev {
-    uint64_t *keys;     // [FLOW_REGIONS * cap], 0 = empty
-    int64_t *exp;       // [FLOW_REGIONS * cap] expiry in Unix ns, FLOW_TOMB = not in the map
+    FlowSlotMem *slots; // [FLOW_REGIONS * cap]
     uint32_t *counters; // [FLOW_COUNTERS]: entries in the map, slots ever claimed, sweep flag
     uint32_t cap;       // slots per region, a power of two
 };
 
 struct RuleIndexDev {
     const uint32_t *bounds; // [n_bounds] ascending starts of the elementary source intervals
-    const uint32_t *starts; // [n_bounds + 1] offsets into ranges
-    const uint2 *ranges;    // sorted disjoint (key_lo, key_hi) per interval
+    const uint32_t *meta;   // [n_bounds + 1] (first 64-byte block of the interval's list) << 8 |
+                            // min(entries, 255); the last element only carries the block count
+    const uint2 *ranges;    // per interval: sorted disjoint (key_lo, key_hi), padded to a multiple
+                            // of 8 entries (one 64-byte block) with never-matching (~0, 0)
     const uint4 *wide;      // [n_wide] (net, mask, key_lo, key_hi) scanned by every packet
     uint32_t n_bounds;
     uint32_t top_step;      // largest power of two < n_bounds (0 when n_bounds == 1)
@@ -42,6 +49,7 @@ struct FilterArgs {
 };
 
 hipError_t launch_fill_u64(uint64_t *p, uint32_t n, uint64_t v, hipStream_t s);
+hipError_t launch_flow_clear(FlowSlotMem *p, uint32_t n, hipStream_t s);
 hipError_t launch_fill_u8(uint8_t *p, uint32_t n, uint8_t v, hipStream_t s);
 hipError_t launch_filter_check(const FilterArgs &a, uint32_t max_blocks, hipStream_t s);
 // inserts, then the reference's conditional expiry sweep

@@ -12,14 +12,14 @@
 namespace bnk {
 
 struct HostRuleIndex {
-    std::vector<uint32_t> bounds, starts;
+    std::vector<uint32_t> bounds, meta;
     std::vector<uint2> ranges;
     std::vector<uint4> wide;
 };
 
 // Upper limit on expanded (interval, key range) entries; rules that would push
 // the total beyond it are kept in the wide list instead.
-constexpr size_t RULE_EXPANSION_BUDGET = size_t(1) << 22;
+constexpr size_t RULE_EXPANSION_BUDGET = size_t(1) << 22; // keeps block numbers within 24 bits
 
 // Compiles bnk_rule tuples (each one prefix x one port range of an
 // acl.CompiledRule, internal/acl/acl.go:33-42) into the interval index the
@@ -106,36 +106,40 @@ inline bool build_rule_index(const bnk_rule *rules, uint32_t n, HostRuleIndex &o
     for (const Tuple &t : ts)
         if (!t.wide)
             for (uint32_t j = t.a; j < t.b; j++) raw[fill[j]++] = make_uint2(t.klo, t.khi);
-    // per interval: sort by key_lo, merge overlapping or adjacent key ranges
-    out.starts.assign(nb + 1, 0);
+    // per interval: sort by key_lo, merge overlapping or adjacent key ranges,
+    // pad the list to whole 64-byte blocks
+    out.meta.assign(nb + 1, 0);
     out.ranges.clear();
     for (uint32_t j = 0; j < nb; j++) {
-        out.starts[j] = (uint32_t)out.ranges.size();
-        auto first = raw.begin() + raw_start[j], last = raw.begin() + raw_start[j + 1];
-        std::sort(first, last, [](const uint2 &x, const uint2 &y) { return x.x < y.x; });
-        for (auto it = first; it != last; ++it) {
-            if (out.ranges.size() > out.starts[j] && it->x <= out.ranges.back().y + 1u) {
+        const size_t first = out.ranges.size();
+        auto lo = raw.begin() + raw_start[j], hi = raw.begin() + raw_start[j + 1];
+        std::sort(lo, hi, [](const uint2 &x, const uint2 &y) { return x.x < y.x; });
+        for (auto it = lo; it != hi; ++it) {
+            if (out.ranges.size() > first && it->x <= out.ranges.back().y + 1u) {
                 if (it->y > out.ranges.back().y) out.ranges.back().y = it->y;
             } else {
                 out.ranges.push_back(*it);
             }
         }
+        const size_t cnt = out.ranges.size() - first;
+        while (out.ranges.size() % 8) out.ranges.push_back(make_uint2(0xFFFFFFFFu, 0u));
+        out.meta[j] = (uint32_t)(first / 8) << 8 | (uint32_t)std::min<size_t>(cnt, 255);
     }
-    out.starts[nb] = (uint32_t)out.ranges.size();
+    out.meta[nb] = (uint32_t)(out.ranges.size() / 8) << 8;
     return true;
 }
 
 struct FilterState {
     bool enforce = false; // filter.New: allow-all until a policy arrives (filter.go:41-43)
-    DevBuf bounds, starts, ranges, wide;
+    DevBuf bounds, meta, ranges, wide;
     RuleIndexDev ridx{};
-    DevBuf keys, exp, counters;
+    DevBuf slots, counters;
     FlowTableDev flows{};
     uint64_t claimed_upper = 0; // host bound on slots ever claimed in the current table
     uint32_t max_blocks = 2048;
     void release()
     {
-        for (DevBuf *b : {&bounds, &starts, &ranges, &wide, &keys, &exp, &counters}) b->release();
+        for (DevBuf *b : {&bounds, &meta, &ranges, &wide, &slots, &counters}) b->release();
     }
 };
 

@@ -11,13 +11,15 @@
 // 2 udp; icmp packets carry key 0 and icmp rules cover the whole class).  The
 // host cuts the 32-bit source space at every interval end into elementary
 // intervals and stores, per elementary interval, the sorted disjoint union of
-// the key intervals of all rules covering it.  A packet does one binary search
-// over the cut points (staged in LDS) and one over its interval's key list.
+// the key intervals of all rules covering it, in 64-byte blocks.  A packet does
+// one binary search over the cut points (staged in LDS together with each
+// interval's block number and length) and then reads its interval's list: one
+// memory transaction when the list fits a block, a binary search otherwise.
 // "Any rule matches" is all the reference asks (filter.go:131-135), so this is
 // exact.  Rules too wide to expand go to a short list every packet scans.
 //
-// Flow table.  Open addressing in HBM, one 64-bit key word and one 64-bit
-// expiry per slot.  The reference's flowKey (remote addr, remote port, local
+// Flow table.  Open addressing in HBM, one 16-byte slot (64-bit key word,
+// 64-bit expiry) so a probe is one memory transaction.  The reference's flowKey (remote addr, remote port, local
 // port, proto) is 66 bits with the protocol class; the class and the top
 // address bit select one of six equal regions and the other 63 bits plus a
 // marker bit form the key word, so 0 can mean "empty" and a slot is claimed
@@ -120,18 +122,38 @@ BNK_DEV uint32_t interval_of(Ptr bounds, uint32_t n, uint32_t top_step, uint32_t
     return pos;
 }
 
-BNK_DEV bool rules_match(const RuleIndexDev &ri, uint32_t interval, uint32_t src, uint32_t key)
+BNK_DEV bool in_range(uint2 r, uint32_t key) { return key >= r.x && key <= r.y; }
+
+// meta_j / meta_next: the interval's and the following interval's meta words.
+BNK_DEV bool rules_match(const RuleIndexDev &ri, uint32_t meta_j, uint32_t meta_next, uint32_t src,
+                         uint32_t key)
 {
-    uint32_t lo = ri.starts[interval], hi = ri.starts[interval + 1];
-    // last range with klo <= key
-    while (lo < hi) {
-        const uint32_t mid = (lo + hi) >> 1;
-        const uint2 r = ri.ranges[mid];
-        if (r.x <= key) {
-            if (key <= r.y) return true;
-            lo = mid + 1;
-        } else {
-            hi = mid;
+    const uint32_t cnt = meta_j & 255u;
+    const uint2 *list = ri.ranges + (size_t)(meta_j >> 8) * 8u;
+    if (cnt != 0u && cnt <= 8u) {
+        // the whole list is one 64-byte block: two entries per 16-byte load
+        const uint4 *blk = reinterpret_cast<const uint4 *>(list);
+        bool hit = false;
+#pragma unroll
+        for (uint32_t q = 0; q < 4; q++) {
+            if (2u * q < cnt) {
+                const uint4 v = blk[q];
+                hit = hit || in_range(make_uint2(v.x, v.y), key) || in_range(make_uint2(v.z, v.w), key);
+            }
+        }
+        if (hit) return true;
+    } else if (cnt > 8u) {
+        // last range with key_lo <= key (padding entries sort to the end)
+        uint32_t lo = 0, hi = ((meta_next >> 8) - (meta_j >> 8)) * 8u;
+        while (lo < hi) {
+            const uint32_t mid = (lo + hi) >> 1;
+            const uint2 r = list[mid];
+            if (r.x <= key) {
+                if (key <= r.y) return true;
+                lo = mid + 1;
+            } else {
+                hi = mid;
+            }
         }
     }
     for (uint32_t w = 0; w < ri.n_wide; w++) {
@@ -141,21 +163,24 @@ BNK_DEV bool rules_match(const RuleIndexDev &ri, uint32_t interval, uint32_t src
     return false;
 }
 
-constexpr uint32_t LDS_BOUNDS_MAX = 12288; // 48 KiB of cut points
+constexpr uint32_t LDS_BOUNDS_MAX = 12288; // 96 KiB: cut points and meta words
+constexpr uint32_t FILTER_THREADS = 1024; // one copy of the index serves 16 waves
 
 // filter.go:121-147 for a batch; enforcement is on (the host short-circuits
 // allow-all mode).
-__global__ __launch_bounds__(256) void filter_check_kernel(FilterArgs a)
+__global__ __launch_bounds__(FILTER_THREADS) void filter_check_kernel(FilterArgs a)
 {
-    extern __shared__ uint32_t lb[]; // n_bounds words when they fit, else unused
+    extern __shared__ uint32_t lds[]; // bounds then meta (n_bounds + 1) when they fit, else unused
     const RuleIndexDev ri = a.rules;
     const bool in_lds = ri.n_bounds <= LDS_BOUNDS_MAX;
+    uint32_t *lb = lds, *lm = lds + ri.n_bounds;
     if (in_lds) {
-        for (uint32_t q = threadIdx.x; q < ri.n_bounds; q += 256u) lb[q] = ri.bounds[q];
+        for (uint32_t q = threadIdx.x; q < ri.n_bounds; q += FILTER_THREADS) lb[q] = ri.bounds[q];
+        for (uint32_t q = threadIdx.x; q <= ri.n_bounds; q += FILTER_THREADS) lm[q] = ri.meta[q];
         __syncthreads();
     }
-    const uint32_t stride = gridDim.x * 256u;
-    for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < a.n; i += stride) {
+    const uint32_t stride = gridDim.x * FILTER_THREADS;
+    for (uint32_t i = blockIdx.x * FILTER_THREADS + threadIdx.x; i < a.n; i += stride) {
         if (a.gate && a.gate[i] == 0) {
             a.verdict[i] = 0;
             continue;
@@ -166,20 +191,31 @@ __global__ __launch_bounds__(256) void filter_check_kernel(FilterArgs a)
         uint8_t pass = 0;
         if (parse_packet(p, len - (len >= a.trim ? a.trim : len), h)) {
             const uint32_t key = proto_class(h.proto) << 16 | h.dport;
-            const uint32_t iv = in_lds ? interval_of(lb, ri.n_bounds, ri.top_step, h.src)
-                                       : interval_of(ri.bounds, ri.n_bounds, ri.top_step, h.src);
-            if (rules_match(ri, iv, h.src, key)) {
+            uint32_t mj, mn;
+            if (in_lds) {
+                const uint32_t iv = interval_of(lb, ri.n_bounds, ri.top_step, h.src);
+                mj = lm[iv];
+                mn = lm[iv + 1];
+            } else {
+                const uint32_t iv = interval_of(ri.bounds, ri.n_bounds, ri.top_step, h.src);
+                mj = ri.meta[iv];
+                mn = ri.meta[iv + 1];
+            }
+            if (rules_match(ri, mj, mn, h.src, key)) {
                 pass = 1;
             } else {
                 // return traffic: remote = src, remotePort = srcPort, localPort = dstPort
                 const FlowSlot s = flow_slot(a.flows, h.src, h.sport, h.dport, h.proto);
                 for (uint32_t probe = 0; probe < a.flows.cap; probe++) {
-                    const uint32_t idx = s.base + ((s.start + probe) & (a.flows.cap - 1u));
-                    const uint64_t kw = __atomic_load_n(&a.flows.keys[idx], __ATOMIC_RELAXED);
-                    if (kw == 0) break; // miss
-                    if (kw != s.word) continue;
-                    unsigned long long *ep = reinterpret_cast<unsigned long long *>(&a.flows.exp[idx]);
-                    const int64_t e = (int64_t)__atomic_load_n(ep, __ATOMIC_RELAXED);
+                    FlowSlotMem *slot = a.flows.slots + s.base + ((s.start + probe) & (a.flows.cap - 1u));
+                    // Keys only change in NoteOutbound batches, never during this
+                    // kernel.  An expiry that another lane is refreshing may be seen
+                    // old or new: both are values this batch's single `now` allows.
+                    const ulonglong2 cur = *reinterpret_cast<const ulonglong2 *>(slot);
+                    if (cur.x == 0) break; // miss
+                    if (cur.x != s.word) continue;
+                    unsigned long long *ep = reinterpret_cast<unsigned long long *>(&slot->exp);
+                    const int64_t e = (int64_t)cur.y;
                     if (e == FLOW_TOMB) break; // deleted earlier
                     if (a.now < e) {
                         // keep-alive on traffic (filter.go:141)
@@ -215,12 +251,12 @@ __global__ __launch_bounds__(256) void filter_note_kernel(FilterArgs a)
         const unsigned long long expiry = (unsigned long long)(a.now + flow_ttl_ns(h.proto));
         bool placed = false;
         for (uint32_t probe = 0; probe < a.flows.cap; probe++) {
-            const uint32_t idx = s.base + ((s.start + probe) & (a.flows.cap - 1u));
-            unsigned long long *kp = reinterpret_cast<unsigned long long *>(&a.flows.keys[idx]);
+            FlowSlotMem *slot = a.flows.slots + s.base + ((s.start + probe) & (a.flows.cap - 1u));
+            unsigned long long *kp = reinterpret_cast<unsigned long long *>(&slot->key);
             const unsigned long long old = atomicCAS(kp, 0ULL, (unsigned long long)s.word);
             if (old == 0ULL) atomicAdd(&a.flows.counters[FLOW_CLAIMED], 1u);
             if (old == 0ULL || old == s.word) {
-                unsigned long long *ep = reinterpret_cast<unsigned long long *>(&a.flows.exp[idx]);
+                unsigned long long *ep = reinterpret_cast<unsigned long long *>(&slot->exp);
                 // every lane of this batch writes the same expiry for this key;
                 // the one that replaces a tombstone (fresh slots start as
                 // tombstones) brings the entry into the map
@@ -249,10 +285,10 @@ __global__ __launch_bounds__(256) void flow_sweep_kernel(FlowTableDev ft, int64_
     const uint32_t total = ft.cap * FLOW_REGIONS;
     const uint32_t stride = gridDim.x * 256u;
     for (uint32_t idx = blockIdx.x * 256u + threadIdx.x; idx < total; idx += stride) {
-        if (ft.keys[idx] == 0) continue;
-        const int64_t e = ft.exp[idx];
+        if (ft.slots[idx].key == 0) continue;
+        const int64_t e = ft.slots[idx].exp;
         if (e != FLOW_TOMB && now > e) {
-            ft.exp[idx] = FLOW_TOMB;
+            ft.slots[idx].exp = FLOW_TOMB;
             atomicSub(&ft.counters[FLOW_LIVE], 1u);
         }
     }
@@ -265,17 +301,17 @@ __global__ __launch_bounds__(256) void flow_rehash_kernel(FlowTableDev from, Flo
     const uint32_t total = from.cap * FLOW_REGIONS;
     const uint32_t stride = gridDim.x * 256u;
     for (uint32_t idx = blockIdx.x * 256u + threadIdx.x; idx < total; idx += stride) {
-        const uint64_t word = from.keys[idx];
-        const int64_t e = from.exp[idx];
+        const uint64_t word = from.slots[idx].key;
+        const int64_t e = from.slots[idx].exp;
         if (word == 0 || e == FLOW_TOMB) continue;
         const uint32_t region = idx / from.cap;
         const uint32_t start = (uint32_t)mix64(word ^ ((uint64_t)region << 59)) & (to.cap - 1u);
         bool placed = false;
         for (uint32_t probe = 0; probe < to.cap; probe++) {
             const uint32_t t = region * to.cap + ((start + probe) & (to.cap - 1u));
-            unsigned long long *kp = reinterpret_cast<unsigned long long *>(&to.keys[t]);
+            unsigned long long *kp = reinterpret_cast<unsigned long long *>(&to.slots[t].key);
             if (atomicCAS(kp, 0ULL, (unsigned long long)word) == 0ULL) {
-                to.exp[t] = e;
+                to.slots[t].exp = e;
                 atomicAdd(&to.counters[FLOW_CLAIMED], 1u);
                 atomicAdd(&to.counters[FLOW_LIVE], 1u);
                 placed = true;
@@ -290,6 +326,15 @@ __global__ __launch_bounds__(256) void fill_u64_kernel(uint64_t *p, uint32_t n, 
 {
     const uint32_t stride = gridDim.x * 256u;
     for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < n; i += stride) p[i] = v;
+}
+
+__global__ __launch_bounds__(256) void flow_clear_kernel(FlowSlotMem *p, uint32_t n)
+{
+    const uint32_t stride = gridDim.x * 256u;
+    for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < n; i += stride) {
+        p[i].key = 0;
+        p[i].exp = FLOW_TOMB;
+    }
 }
 
 __global__ __launch_bounds__(256) void fill_u8_kernel(uint8_t *p, uint32_t n, uint8_t v)
@@ -311,6 +356,13 @@ hipError_t launch_fill_u64(uint64_t *p, uint32_t n, uint64_t v, hipStream_t s)
     return hipGetLastError();
 }
 
+hipError_t launch_flow_clear(FlowSlotMem *p, uint32_t n, hipStream_t s)
+{
+    if (n == 0) return hipSuccess;
+    hipLaunchKernelGGL(flow_clear_kernel, dim3(grid_for(n, 4096)), dim3(256), 0, s, p, n);
+    return hipGetLastError();
+}
+
 hipError_t launch_fill_u8(uint8_t *p, uint32_t n, uint8_t v, hipStream_t s)
 {
     if (n == 0) return hipSuccess;
@@ -321,8 +373,20 @@ hipError_t launch_fill_u8(uint8_t *p, uint32_t n, uint8_t v, hipStream_t s)
 hipError_t launch_filter_check(const FilterArgs &a, uint32_t max_blocks, hipStream_t s)
 {
     if (a.n == 0) return hipSuccess;
-    const uint32_t lds = a.rules.n_bounds <= LDS_BOUNDS_MAX ? a.rules.n_bounds * 4u : 0u;
-    hipLaunchKernelGGL(filter_check_kernel, dim3(grid_for(a.n, max_blocks)), dim3(256), lds, s, a);
+    const uint32_t lds = a.rules.n_bounds <= LDS_BOUNDS_MAX ? (2u * a.rules.n_bounds + 1u) * 4u : 0u;
+    if (lds > 48u * 1024u) {
+        // more dynamic LDS than the default limit: opt in (gfx950 has 160 KiB per CU)
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(filter_check_kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)((2u * LDS_BOUNDS_MAX + 1u) * 4u));
+        if (e != hipSuccess) return e;
+    }
+    // one index copy per workgroup: as many workgroups per CU as their LDS allows, two at most
+    const uint32_t per_cu = lds > 80u * 1024u ? 1u : 2u;
+    uint32_t blocks = (a.n + FILTER_THREADS - 1u) / FILTER_THREADS;
+    const uint32_t cap = (max_blocks / 8u) * per_cu; // max_blocks is 8 per CU
+    if (blocks > cap) blocks = cap;
+    hipLaunchKernelGGL(filter_check_kernel, dim3(blocks), dim3(FILTER_THREADS), lds, s, a);
     return hipGetLastError();
 }
 

@@ -6,17 +6,23 @@ using namespace bnk;
 
 namespace bnk {
 
-static hipError_t flow_table_alloc(uint32_t cap, DevBuf &slots, DevBuf &counters, FlowTableDev &ft,
-                                   hipStream_t s)
+static hipError_t flow_table_alloc(uint32_t cap, DevBuf &slots, DevBuf &counters, DevBuf &present,
+                                   FlowTableDev &ft, hipStream_t s)
 {
     const size_t n = (size_t)cap * FLOW_REGIONS;
+    // the table is kept under half full, so 8 * cap bits see at most one key per 16 bits
+    const uint32_t bits = cap * 8u;
     hipError_t e;
     if ((e = slots.reserve(n * sizeof(FlowSlotMem))) != hipSuccess) return e;
     if ((e = counters.reserve(FLOW_COUNTERS * 4)) != hipSuccess) return e;
+    if ((e = present.reserve(bits / 8)) != hipSuccess) return e;
     ft.slots = slots.as<FlowSlotMem>();
     ft.counters = counters.as<uint32_t>();
+    ft.present = present.as<uint32_t>();
     ft.cap = cap;
+    ft.present_mask = bits - 1u;
     if ((e = launch_flow_clear(ft.slots, (uint32_t)n, s)) != hipSuccess) return e;
+    if ((e = launch_fill_u32(ft.present, bits / 32, 0, s)) != hipSuccess) return e;
     return launch_fill_u32(ft.counters, FLOW_COUNTERS, 0, s);
 }
 
@@ -66,7 +72,7 @@ FilterState *filter_create(hipStream_t s, int cu_count)
     HostRuleIndex h;
     std::string err;
     build_rule_index(nullptr, 0, h, err);
-    if (flow_table_alloc(FLOW_CAP_INITIAL, f->slots, f->counters, f->flows, s) != hipSuccess ||
+    if (flow_table_alloc(FLOW_CAP_INITIAL, f->slots, f->counters, f->present, f->flows, s) != hipSuccess ||
         upload_rule_index(f, h, s) != hipSuccess) {
         filter_destroy(f);
         return nullptr;
@@ -107,18 +113,18 @@ int flows_reserve(bnk_ctx *ctx, uint32_t n_new)
     uint64_t cap = FLOW_CAP_INITIAL;
     while (cap < need) cap *= 2;
     if (cap > FLOW_CAP_MAX) return fail(ctx, BNK_E_NOMEM, "flow table would exceed its maximum size");
-    DevBuf ns, nc;
+    DevBuf ns, nc, np;
     FlowTableDev nt{};
-    hipError_t e = flow_table_alloc((uint32_t)cap, ns, nc, nt, ctx->stream);
+    hipError_t e = flow_table_alloc((uint32_t)cap, ns, nc, np, nt, ctx->stream);
     if (e == hipSuccess)
         e = launch_flow_rehash(f->flows, nt, ctx->d_status, f->max_blocks, ctx->stream);
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
     if (e != hipSuccess) {
-        ns.release(); nc.release();
+        ns.release(); nc.release(); np.release();
         return fail_hip(ctx, "flow table growth", e);
     }
-    f->slots.release(); f->counters.release();
-    f->slots = ns; f->counters = nc;
+    f->slots.release(); f->counters.release(); f->present.release();
+    f->slots = ns; f->counters = nc; f->present = np;
     f->flows = nt;
     f->claimed_upper = (uint64_t)c[FLOW_LIVE] + n_new;
     return BNK_OK;

@@ -19,7 +19,10 @@ struct FlowSlotMem {
 struct FlowTableDev {
     FlowSlotMem *slots; // [FLOW_REGIONS * cap]
     uint32_t *counters; // [FLOW_COUNTERS]: entries in the map, slots ever claimed, sweep flag
+    uint32_t *present;  // [present_bits / 32] one hashed bit per key ever stored in this table:
+                        // small enough to stay in L2, it answers most misses without a probe
     uint32_t cap;       // slots per region, a power of two
+    uint32_t present_mask; // present_bits - 1 (a power of two)
 };
 
 struct RuleIndexDev {

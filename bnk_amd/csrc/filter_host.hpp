@@ -133,13 +133,13 @@ struct FilterState {
     bool enforce = false; // filter.New: allow-all until a policy arrives (filter.go:41-43)
     DevBuf bounds, meta, ranges, wide;
     RuleIndexDev ridx{};
-    DevBuf slots, counters;
+    DevBuf slots, counters, present;
     FlowTableDev flows{};
     uint64_t claimed_upper = 0; // host bound on slots ever claimed in the current table
     uint32_t max_blocks = 2048;
     void release()
     {
-        for (DevBuf *b : {&bounds, &meta, &ranges, &wide, &slots, &counters}) b->release();
+        for (DevBuf *b : {&bounds, &meta, &ranges, &wide, &slots, &counters, &present}) b->release();
     }
 };
 

@@ -95,6 +95,7 @@ struct FlowSlot {
     uint64_t word;   // stored key word (never 0)
     uint32_t base;   // first slot of the region
     uint32_t start;  // probe start within the region
+    uint32_t bit;    // this key's bit in the presence bitmap
 };
 
 BNK_DEV FlowSlot flow_slot(const FlowTableDev &ft, uint32_t remote, uint32_t rport, uint32_t lport,
@@ -104,7 +105,9 @@ BNK_DEV FlowSlot flow_slot(const FlowTableDev &ft, uint32_t remote, uint32_t rpo
     const uint32_t region = proto_class(proto) * 2u + (remote >> 31);
     s.word = (1ULL << 63) | ((uint64_t)(remote & 0x7FFFFFFFu) << 32) | ((uint64_t)rport << 16) | lport;
     s.base = region * ft.cap;
-    s.start = (uint32_t)mix64(s.word ^ ((uint64_t)region << 59)) & (ft.cap - 1u);
+    const uint64_t hsh = mix64(s.word ^ ((uint64_t)region << 59));
+    s.start = (uint32_t)hsh & (ft.cap - 1u);
+    s.bit = (uint32_t)(hsh >> 32) & ft.present_mask;
     return s;
 }
 
@@ -206,7 +209,9 @@ __global__ __launch_bounds__(FILTER_THREADS) void filter_check_kernel(FilterArgs
             } else {
                 // return traffic: remote = src, remotePort = srcPort, localPort = dstPort
                 const FlowSlot s = flow_slot(a.flows, h.src, h.sport, h.dport, h.proto);
-                for (uint32_t probe = 0; probe < a.flows.cap; probe++) {
+                // a clear bit means the key was never stored: no probe needed
+                const bool maybe = (a.flows.present[s.bit >> 5] >> (s.bit & 31u)) & 1u;
+                for (uint32_t probe = 0; maybe && probe < a.flows.cap; probe++) {
                     FlowSlotMem *slot = a.flows.slots + s.base + ((s.start + probe) & (a.flows.cap - 1u));
                     // Keys only change in NoteOutbound batches, never during this
                     // kernel.  An expiry that another lane is refreshing may be seen
@@ -254,7 +259,10 @@ __global__ __launch_bounds__(256) void filter_note_kernel(FilterArgs a)
             FlowSlotMem *slot = a.flows.slots + s.base + ((s.start + probe) & (a.flows.cap - 1u));
             unsigned long long *kp = reinterpret_cast<unsigned long long *>(&slot->key);
             const unsigned long long old = atomicCAS(kp, 0ULL, (unsigned long long)s.word);
-            if (old == 0ULL) atomicAdd(&a.flows.counters[FLOW_CLAIMED], 1u);
+            if (old == 0ULL) {
+                atomicAdd(&a.flows.counters[FLOW_CLAIMED], 1u);
+                atomicOr(&a.flows.present[s.bit >> 5], 1u << (s.bit & 31u));
+            }
             if (old == 0ULL || old == s.word) {
                 unsigned long long *ep = reinterpret_cast<unsigned long long *>(&slot->exp);
                 // every lane of this batch writes the same expiry for this key;
@@ -305,13 +313,16 @@ __global__ __launch_bounds__(256) void flow_rehash_kernel(FlowTableDev from, Flo
         const int64_t e = from.slots[idx].exp;
         if (word == 0 || e == FLOW_TOMB) continue;
         const uint32_t region = idx / from.cap;
-        const uint32_t start = (uint32_t)mix64(word ^ ((uint64_t)region << 59)) & (to.cap - 1u);
+        const uint64_t hsh = mix64(word ^ ((uint64_t)region << 59));
+        const uint32_t start = (uint32_t)hsh & (to.cap - 1u);
+        const uint32_t bit = (uint32_t)(hsh >> 32) & to.present_mask;
         bool placed = false;
         for (uint32_t probe = 0; probe < to.cap; probe++) {
             const uint32_t t = region * to.cap + ((start + probe) & (to.cap - 1u));
             unsigned long long *kp = reinterpret_cast<unsigned long long *>(&to.slots[t].key);
             if (atomicCAS(kp, 0ULL, (unsigned long long)word) == 0ULL) {
                 to.slots[t].exp = e;
+                atomicOr(&to.present[bit >> 5], 1u << (bit & 31u));
                 atomicAdd(&to.counters[FLOW_CLAIMED], 1u);
                 atomicAdd(&to.counters[FLOW_LIVE], 1u);
                 placed = true;

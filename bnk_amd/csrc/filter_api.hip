@@ -1,6 +1,7 @@
 // C ABI entry points of the packet filter (see include/bnkhip.h).
 #include "api_common.hpp"
 #include "filter_host.hpp"
+#include "netmap_json.hpp"
 
 using namespace bnk;
 
@@ -287,6 +288,42 @@ int bnk_filter_set_rules(bnk_ctx *ctx, const bnk_rule *rules, uint32_t n)
     HIPCHK(ctx, upload_rule_index(ctx->filter, h, ctx->stream));
     ctx->filter->enforce = true;
     return BNK_OK;
+}
+
+int bnk_rules_from_netmap_json(const char *json, size_t len, bnk_rule *out, uint32_t cap,
+                               uint32_t *n_tuples, int *filter_enabled, char *err, size_t err_cap)
+{
+    if (err && err_cap) err[0] = '\0';
+    if (!json || !n_tuples || !filter_enabled || (cap && !out)) return BNK_E_INVAL;
+    NetmapFilter nf;
+    std::string msg;
+    if (!NetmapJson(json, len).parse(nf, msg)) {
+        if (err && err_cap) {
+            strncpy(err, msg.c_str(), err_cap - 1);
+            err[err_cap - 1] = '\0';
+        }
+        return BNK_E_INVAL;
+    }
+    *n_tuples = (uint32_t)nf.tuples.size();
+    *filter_enabled = nf.filter_enabled ? 1 : 0;
+    const size_t k = std::min<size_t>(cap, nf.tuples.size());
+    if (k) memcpy(out, nf.tuples.data(), k * sizeof(bnk_rule));
+    return BNK_OK;
+}
+
+int bnk_filter_apply_netmap_json(bnk_ctx *ctx, const char *json, size_t len)
+{
+    if (!ctx) return fail(nullptr, BNK_E_INVAL, "null context");
+    if (!json) return fail(ctx, BNK_E_INVAL, "null document");
+    NetmapFilter nf;
+    std::string msg;
+    {
+        std::lock_guard<std::mutex> lk(ctx->mu);
+        if (!NetmapJson(json, len).parse(nf, msg)) return fail(ctx, BNK_E_INVAL, msg);
+    }
+    // engine.go:279-283
+    if (nf.filter_enabled) return bnk_filter_set_rules(ctx, nf.tuples.data(), (uint32_t)nf.tuples.size());
+    return bnk_filter_set_allow_all(ctx);
 }
 
 int bnk_filter_set_allow_all(bnk_ctx *ctx)

@@ -125,6 +125,29 @@ def flatten_rules(rules) -> np.ndarray:
     return arr, len(out)
 
 
+def rules_from_netmap_json(doc: str | bytes):
+    """(filter_enabled, [(src_net, src_mask, first, last, proto)]) from a netmap
+    JSON document; raises BnkError(E_INVAL) on a document Go would reject.
+    Needs no GPU."""
+    lib = load()
+    raw = doc.encode() if isinstance(doc, str) else bytes(doc)
+    n = C.c_uint32()
+    en = C.c_int()
+    err = C.create_string_buffer(256)
+    cap = 64
+    while True:
+        arr = (Rule * cap)()
+        rc = lib.bnk_rules_from_netmap_json(raw, C.c_size_t(len(raw)), arr, C.c_uint32(cap),
+                                            C.byref(n), C.byref(en), err, C.c_size_t(256))
+        if rc != 0:
+            raise BnkError(rc, err.value.decode())
+        if n.value <= cap:
+            break
+        cap = n.value
+    return bool(en.value), [(arr[i].src_net, arr[i].src_mask, arr[i].port_first,
+                             arr[i].port_last, arr[i].proto) for i in range(n.value)]
+
+
 class Context:
     """One bnk_ctx: a GPU, a stream, key tables, a filter."""
 
@@ -224,6 +247,10 @@ class Context:
 
     def filter_set_rule_tuples(self, arr, n: int) -> None:
         self._chk(self._lib.bnk_filter_set_rules(self._h, arr, C.c_uint32(n)))
+
+    def filter_apply_netmap_json(self, doc: str | bytes) -> None:
+        raw = doc.encode() if isinstance(doc, str) else bytes(doc)
+        self._chk(self._lib.bnk_filter_apply_netmap_json(self._h, raw, C.c_size_t(len(raw))))
 
     def filter_set_allow_all(self) -> None:
         self._chk(self._lib.bnk_filter_set_allow_all(self._h))

@@ -151,6 +151,22 @@ int bnk_filter_set_rules(bnk_ctx *ctx, const bnk_rule *rules, uint32_t n);
 /* filter.SetAllowAll (filter.go:54-59): enforcement off, rules dropped,
  * flows kept. */
 int bnk_filter_set_allow_all(bnk_ctx *ctx);
+/* The filter half of Engine.ApplyNetmap (internal/dataplane/engine.go:279-283)
+ * fed with the wire format the control server pushes: a netmap JSON document
+ * whose "filter_enabled" / "filter" fields carry []acl.CompiledRule
+ * (internal/netmap/netmap.go:44-53, internal/acl/acl.go:33-42); a bare JSON array
+ * of rules is accepted too and means filter_enabled.  filter_enabled true ->
+ * SetRules(filter), false -> SetAllowAll().  A document Go's decoder would
+ * reject (malformed JSON, bad prefix text, port outside 0..65535) returns
+ * BNK_E_INVAL and leaves the filter as it was. */
+int bnk_filter_apply_netmap_json(bnk_ctx *ctx, const char *json, size_t len);
+/* The same parse without a context (no GPU needed): writes up to cap tuples,
+ * the total number of tuples to *n_tuples (call again with a larger array when
+ * it exceeds cap), filter_enabled as 0/1, and on failure a message to err. */
+int bnk_rules_from_netmap_json(const char *json, size_t len, bnk_rule *out, uint32_t cap,
+                               uint32_t *n_tuples, int *filter_enabled, char *err,
+                               size_t err_cap);
+
 /* filter.NoteOutbound over a batch with one `now` (filter.go:160-167,
  * 189-209), including the len(flows) > 4096 expiry sweep.  now_ns is the
  * time.Time as Unix nanoseconds.  peer/counters of the batch are ignored. */

@@ -244,3 +244,27 @@ def test_cfg4_full_size_device_resident_properties():
     assert ctxs[0].filter_flows() == ctxs[1].filter_flows()
     for c in ctxs:
         c.close()
+
+
+def test_apply_netmap_json_end_to_end():
+    """Engine.ApplyNetmap's filter half fed with the control server's wire
+    format: the reference's integration test allows one port and blocks another
+    (internal/dataplane/acl_integration_test.go:20-80)."""
+    import json
+    from bnk_amd import lib
+    ctx = lib.Context(0)
+    a, b = W.ip("100.64.0.1"), W.ip("100.64.0.2")
+    doc = {"self_id": 2, "self_ip": "100.64.0.2/32", "peers": [], "filter_enabled": True,
+           "filter": [{"srcs": ["100.64.0.1/32"], "proto": "tcp", "ports": [{"first": 7777, "last": 7777}]}]}
+    ctx.filter_apply_netmap_json(json.dumps(doc))
+    got = ctx.filter_check_inbound_ptrs([W.tcp(a, b, 40000, 7777), W.tcp(a, b, 40000, 8888),
+                                         W.udp(a, b, 40000, 7777)], FC.T0)
+    assert got.tolist() == [1, 0, 0]
+    # a malformed push leaves the filter as it was
+    with pytest.raises(lib.BnkError):
+        ctx.filter_apply_netmap_json('{"filter_enabled":true,"filter":[{"srcs":["bogus"]}]}')
+    assert ctx.filter_check_inbound_ptrs([W.tcp(a, b, 1, 7777)], FC.T0).tolist() == [1]
+    # policy removed: allow-all again
+    ctx.filter_apply_netmap_json(json.dumps({"self_id": 2, "peers": []}))
+    assert ctx.filter_check_inbound_ptrs([W.tcp(a, b, 1, 8888)], FC.T0).tolist() == [1]
+    ctx.close()

@@ -350,8 +350,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             have = false;
         } else {
             if (OPEN) len -= 16u;
-            src = a.in + (a.in_off ? a.in_off[i] : (uint64_t)i * a.in_stride);
-            dst = a.out + (a.out_off ? a.out_off[i] : (uint64_t)i * a.out_stride);
+            src = a.in + (a.in_off ? a.in_off[i] : (uint64_t)i * a.in_stride) + a.in_skip;
+            dst = a.out + (a.out_off ? a.out_off[i] : (uint64_t)i * a.out_stride) + a.out_skip;
             const uint4 *kp = reinterpret_cast<const uint4 *>(a.keys + 8u * pr);
             const uint4 k0 = kp[0], k1 = kp[1];
             k[0] = k0.x; k[1] = k0.y; k[2] = k0.z; k[3] = k0.w;

@@ -163,7 +163,10 @@ void bnk_shutdown(bnk_ctx *ctx)
                           &ctx->peer, &ctx->counters, &ctx->verdict, &ctx->order, &ctx->hist,
                           &ctx->cursor, &ctx->misc, &ctx->r_plain, &ctx->r_auth, &ctx->r_pass,
                           &ctx->r_keys, &ctx->r_idx, &ctx->r_skeys, &ctx->r_sidx, &ctx->r_tmp,
-                          &ctx->r_peer_out, &ctx->r_ctr_base, &ctx->r_ctr_out, &ctx->r_verdict})
+                          &ctx->r_peer_out, &ctx->r_ctr_base, &ctx->r_ctr_out, &ctx->r_verdict,
+                          &ctx->wg_index, &ctx->wg_remote, &ctx->wg_allowed, &ctx->wg_send_ctr,
+                          &ctx->wg_peer, &ctx->wg_counter, &ctx->wg_ctlen, &ctx->wg_result,
+                          &ctx->wg_outlen, &ctx->wg_padded, &ctx->wg_wirelen, &ctx->wg_skip})
             b->release();
         ctx->pin.release();
         for (int w = 0; w < 2; w++)

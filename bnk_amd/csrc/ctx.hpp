@@ -89,5 +89,10 @@ struct bnk_ctx {
     bnk::DevBuf r_plain, r_auth, r_pass, r_keys, r_idx, r_skeys, r_sidx, r_tmp;
     bnk::DevBuf r_peer_out, r_ctr_base, r_ctr_out, r_verdict;
 
+    // WireGuard framing: peer tables and per-packet scratch
+    bnk::DevBuf wg_index, wg_remote, wg_allowed, wg_send_ctr;
+    uint32_t n_wg_peers = 0;
+    bnk::DevBuf wg_peer, wg_counter, wg_ctlen, wg_result, wg_outlen, wg_padded, wg_wirelen, wg_skip;
+
     bnk::FilterState *filter = nullptr;
 };

@@ -26,6 +26,7 @@ struct AeadArgs {
     uint32_t len;
     uint32_t n_peers;
     uint32_t trim;             // seal only: lens[i] - trim is the plaintext length
+    uint32_t in_skip, out_skip; // bytes between a packet's offset and its AEAD data
 };
 
 enum : uint32_t { STATUS_PEER_RANGE = 1u, STATUS_FLOWS_FULL = 2u };
@@ -53,6 +54,14 @@ hipError_t launch_relay_assign(const uint8_t *auth, const uint8_t *pass, const u
                                uint32_t *keys, uint32_t *idx, uint32_t *skeys, uint32_t *sidx,
                                void *sort_tmp, size_t sort_tmp_bytes, uint8_t *verdict,
                                uint64_t *ctr_out, uint32_t *status, hipStream_t s);
+
+// Batch-order counters per peer: ctr_out[i] = ctr_base[keys[i]] + (number of
+// earlier i' with the same key), for keys[i] != 0xFFFFFFFF.  keys/idx are
+// inputs (idx[i] = i), skeys/sidx and sort_tmp scratch.  With advance set,
+// ctr_base[key] moves past the counters handed out.
+hipError_t launch_peer_rank(uint32_t *keys, uint32_t *idx, uint32_t *skeys, uint32_t *sidx,
+                            void *sort_tmp, size_t sort_tmp_bytes, uint64_t *ctr_base, uint32_t n,
+                            uint64_t *ctr_out, bool advance, hipStream_t s);
 
 // VALU throughput probe; out receives one word per thread so nothing is
 // optimised away.

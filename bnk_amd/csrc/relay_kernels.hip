@@ -57,6 +57,19 @@ __global__ __launch_bounds__(256) void relay_rank_kernel(const uint32_t *skeys, 
     ctr_out[sidx[p]] = ctr_base_out[key] + (uint64_t)(p - lo);
 }
 
+// The last element of each peer's segment holds the largest counter handed out.
+__global__ __launch_bounds__(256) void peer_advance_kernel(const uint32_t *skeys, const uint32_t *sidx,
+                                                           const uint64_t *ctr_out, uint32_t n,
+                                                           uint64_t *ctr_base)
+{
+    const uint32_t p = blockIdx.x * 256u + threadIdx.x;
+    if (p >= n) return;
+    const uint32_t key = skeys[p];
+    if (key == NO_PEER) return;
+    if (p + 1u < n && skeys[p + 1u] == key) return;
+    ctr_base[key] = ctr_out[sidx[p]] + 1u;
+}
+
 size_t relay_sort_tmp_bytes(uint32_t n)
 {
     size_t bytes = 0;
@@ -75,10 +88,22 @@ hipError_t launch_relay_assign(const uint8_t *auth, const uint8_t *pass, const u
     const dim3 grid((n + 255u) / 256u);
     hipLaunchKernelGGL(relay_verdict_kernel, grid, dim3(256), 0, s, auth, pass, peer_out, n_peers_out,
                        n, keys, idx, verdict, ctr_out, status);
+    return launch_peer_rank(keys, idx, skeys, sidx, sort_tmp, sort_tmp_bytes,
+                            const_cast<uint64_t *>(ctr_base_out), n, ctr_out, false, s);
+}
+
+hipError_t launch_peer_rank(uint32_t *keys, uint32_t *idx, uint32_t *skeys, uint32_t *sidx,
+                            void *sort_tmp, size_t sort_tmp_bytes, uint64_t *ctr_base, uint32_t n,
+                            uint64_t *ctr_out, bool advance, hipStream_t s)
+{
+    if (n == 0) return hipSuccess;
+    const dim3 grid((n + 255u) / 256u);
     hipError_t e = rocprim::radix_sort_pairs(sort_tmp, sort_tmp_bytes, keys, skeys, idx, sidx, (size_t)n,
                                              0, 32, s);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(relay_rank_kernel, grid, dim3(256), 0, s, skeys, sidx, ctr_base_out, n, ctr_out);
+    hipLaunchKernelGGL(relay_rank_kernel, grid, dim3(256), 0, s, skeys, sidx, ctr_base, n, ctr_out);
+    if (advance)
+        hipLaunchKernelGGL(peer_advance_kernel, grid, dim3(256), 0, s, skeys, sidx, ctr_out, n, ctr_base);
     return hipGetLastError();
 }
 

@@ -1,0 +1,300 @@
+// C ABI entry points of the WireGuard transport framing (see
+// include/bnkhip.h): peer table, encapsulation, decapsulation.
+#include <vector>
+
+#include "api_common.hpp"
+#include "wg_dev.hpp"
+
+using namespace bnk;
+
+namespace {
+
+uint32_t wg_padding_host(uint32_t len, uint32_t mtu)
+{
+    uint32_t last = len;
+    if (mtu == 0) return ((last + 15u) & ~15u) - last;
+    if (last > mtu) last %= mtu;
+    uint32_t padded = (last + 15u) & ~15u;
+    if (padded > mtu) padded = mtu;
+    return padded - last;
+}
+
+WgPeersDev peers_view(bnk_ctx *ctx)
+{
+    WgPeersDev pe{};
+    pe.index_sorted = ctx->wg_index.as<uint2>();
+    pe.remote_index = ctx->wg_remote.as<uint32_t>();
+    pe.allowed = ctx->wg_allowed.as<uint2>();
+    pe.send_ctr = ctx->wg_send_ctr.as<uint64_t>();
+    pe.n = ctx->n_wg_peers;
+    return pe;
+}
+
+int upload(bnk_ctx *ctx, DevBuf *dst, const void *src, size_t bytes)
+{
+    HIPCHK(ctx, dst->reserve(bytes));
+    HIPCHK(ctx, hipMemcpyAsync(dst->p, src, bytes, hipMemcpyHostToDevice, ctx->stream));
+    return BNK_OK;
+}
+
+} // namespace
+
+extern "C" int bnk_wg_peers_set(bnk_ctx *ctx, const bnk_wg_peer *peers, uint32_t n)
+{
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    if (!peers || n == 0) return fail(ctx, BNK_E_INVAL, "empty peer table");
+    std::vector<uint2> index(n), allowed(n);
+    std::vector<uint32_t> remote(n);
+    for (uint32_t i = 0; i < n; i++) {
+        const uint32_t inv = ~peers[i].allowed_mask;
+        if ((inv & (inv + 1u)) != 0u)
+            return fail(ctx, BNK_E_INVAL, "peer " + std::to_string(i) + ": allowed_mask is not a prefix mask");
+        index[i] = make_uint2(peers[i].local_index, i);
+        remote[i] = peers[i].remote_index;
+        allowed[i] = make_uint2(peers[i].allowed_net, peers[i].allowed_mask);
+    }
+    std::sort(index.begin(), index.end(), [](const uint2 &a, const uint2 &b) { return a.x < b.x; });
+    for (uint32_t i = 1; i < n; i++)
+        if (index[i].x == index[i - 1].x)
+            return fail(ctx, BNK_E_INVAL, "local_index " + std::to_string(index[i].x) + " is used by two peers");
+    // in-flight batches may still read the old tables
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    std::vector<uint64_t> zeros(n, 0);
+    int rc = upload(ctx, &ctx->wg_index, index.data(), (size_t)n * 8);
+    if (!rc) rc = upload(ctx, &ctx->wg_remote, remote.data(), (size_t)n * 4);
+    if (!rc) rc = upload(ctx, &ctx->wg_allowed, allowed.data(), (size_t)n * 8);
+    if (!rc) rc = upload(ctx, &ctx->wg_send_ctr, zeros.data(), (size_t)n * 8);
+    if (rc) return rc;
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream)); // the vectors above go away
+    ctx->n_wg_peers = n;
+    return BNK_OK;
+}
+
+extern "C" int bnk_wg_send_counters(bnk_ctx *ctx, uint64_t *out, uint32_t n)
+{
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    if (!out) return fail(ctx, BNK_E_INVAL, "null out pointer");
+    if (n > ctx->n_wg_peers) return fail(ctx, BNK_E_RANGE, "more counters asked for than peers");
+    if (n == 0) return BNK_OK;
+    HIPCHK(ctx, hipMemcpyAsync(out, ctx->wg_send_ctr.p, (size_t)n * 8, hipMemcpyDeviceToHost, ctx->stream));
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    return BNK_OK;
+}
+
+extern "C" int bnk_wg_encap_batch(bnk_ctx *ctx, const bnk_batch *slots, uint32_t mtu, uint32_t *wire_len)
+{
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    int rc = check_batch_common(ctx, slots, "slots");
+    if (rc) return rc;
+    const uint32_t n = slots->n;
+    if (n == 0) return BNK_OK;
+    if (!wire_len) return fail(ctx, BNK_E_INVAL, "null wire_len array");
+    if (ctx->n_wg_peers == 0) return fail(ctx, BNK_E_STATE, "no peer table loaded");
+    if (!ctx->d_keys[BNK_KEYS_SEND] || ctx->n_keys[BNK_KEYS_SEND] < ctx->n_wg_peers)
+        return fail(ctx, BNK_E_STATE, "send key table is smaller than the peer table");
+    const bool host = slots->mem == BNK_MEM_HOST;
+
+    WgBatch b{};
+    b.n = n;
+    b.stride = slots->stride;
+    b.len = slots->len;
+    const uint32_t *d_peer = nullptr;
+    uint32_t *d_wire_len = nullptr;
+    Span span;
+    if (host) {
+        for (uint32_t i = 0; i < n; i++) {
+            const uint64_t off = pkt_off(slots, i);
+            const uint32_t len = slots->lens ? slots->lens[i] : slots->len;
+            const uint64_t need = 16ull + len + wg_padding_host(len, mtu) + 16ull;
+            if (off > slots->bytes || need > slots->bytes - off)
+                return fail(ctx, BNK_E_INVAL, "slots: packet " + std::to_string(i) + " lies outside the arena");
+            if (slots->peer && slots->peer[i] >= ctx->n_wg_peers)
+                return fail(ctx, BNK_E_RANGE, "peer index " + std::to_string(slots->peer[i]) +
+                                                  " beyond the peer table");
+            span.add(off, off + need);
+        }
+        HIPCHK(ctx, ctx->pin.reserve((size_t)n * 16 + 64));
+        HIPCHK(ctx, ctx->in_arena.reserve(span.size() + 16));
+        HIPCHK(ctx, hipMemcpyAsync(ctx->in_arena.p, (const uint8_t *)slots->base + span.lo, span.size(),
+                                   hipMemcpyHostToDevice, ctx->stream));
+        b.base = ctx->in_arena.as<uint8_t>();
+        rc = upload_offsets(ctx, slots, n, span.lo, &ctx->off_in, 0, &b.off);
+        if (rc) return rc;
+        if (slots->lens) {
+            rc = upload(ctx, &ctx->lens, slots->lens, (size_t)n * 4);
+            if (rc) return rc;
+            b.lens = ctx->lens.as<uint32_t>();
+        }
+        if (slots->peer) {
+            rc = upload(ctx, &ctx->peer, slots->peer, (size_t)n * 4);
+            if (rc) return rc;
+            d_peer = ctx->peer.as<uint32_t>();
+        }
+        HIPCHK(ctx, ctx->wg_wirelen.reserve((size_t)n * 4));
+        d_wire_len = ctx->wg_wirelen.as<uint32_t>();
+    } else {
+        if (!slots->offsets && !slots->lens &&
+            (uint64_t)(n - 1) * slots->stride + 16ull + slots->len + wg_padding_host(slots->len, mtu) + 16ull >
+                slots->bytes)
+            return fail(ctx, BNK_E_INVAL, "slots: uniform layout exceeds the arena");
+        b.base = (const uint8_t *)slots->base;
+        b.off = slots->offsets;
+        b.lens = slots->lens;
+        d_peer = slots->peer;
+        d_wire_len = wire_len;
+    }
+
+    for (DevBuf *buf : {&ctx->r_keys, &ctx->r_idx, &ctx->r_skeys, &ctx->r_sidx, &ctx->wg_padded})
+        HIPCHK(ctx, buf->reserve((size_t)n * 4));
+    HIPCHK(ctx, ctx->r_ctr_out.reserve((size_t)n * 8));
+    HIPCHK(ctx, ctx->wg_skip.reserve(n));
+    const size_t tmp_bytes = relay_sort_tmp_bytes(n);
+    HIPCHK(ctx, ctx->r_tmp.reserve(tmp_bytes + 16));
+    const WgPeersDev pe = peers_view(ctx);
+    uint64_t *d_ctr = ctx->r_ctr_out.as<uint64_t>();
+    uint32_t *d_padded = ctx->wg_padded.as<uint32_t>();
+    uint8_t *d_skip = ctx->wg_skip.as<uint8_t>();
+
+    // counters in batch order per peer, advancing the peers' send counters
+    HIPCHK(ctx, launch_wg_keys(d_peer, pe.n, n, ctx->r_keys.as<uint32_t>(), ctx->r_idx.as<uint32_t>(),
+                               ctx->d_status, ctx->stream));
+    HIPCHK(ctx, launch_peer_rank(ctx->r_keys.as<uint32_t>(), ctx->r_idx.as<uint32_t>(),
+                                 ctx->r_skeys.as<uint32_t>(), ctx->r_sidx.as<uint32_t>(), ctx->r_tmp.p,
+                                 tmp_bytes, pe.send_ctr, n, d_ctr, true, ctx->stream));
+    HIPCHK(ctx, launch_wg_encap_prep(b, pe, d_peer, d_ctr, mtu, d_padded, d_wire_len, d_skip, ctx->stream));
+
+    AeadArgs se{};
+    se.keys = ctx->d_keys[BNK_KEYS_SEND];
+    se.n_peers = pe.n;
+    se.status = ctx->d_status;
+    se.n = n;
+    se.in = b.base;
+    se.out = const_cast<uint8_t *>(b.base);
+    se.in_off = se.out_off = b.off;
+    se.in_stride = se.out_stride = slots->stride;
+    se.in_skip = se.out_skip = 16;
+    se.lens = d_padded;
+    se.peer = d_peer;
+    se.counters = d_ctr;
+    se.skip = d_skip;
+    rc = maybe_sort(ctx, se.lens, n, 0, &se.order);
+    if (rc) return rc;
+    HIPCHK(ctx, launch_aead_seal(se, ctx->stream));
+    if (!host) return BNK_OK;
+
+    HIPCHK(ctx, hipMemcpyAsync((uint8_t *)slots->base + span.lo, ctx->in_arena.p, span.size(),
+                               hipMemcpyDeviceToHost, ctx->stream));
+    HIPCHK(ctx, hipMemcpyAsync(wire_len, d_wire_len, (size_t)n * 4, hipMemcpyDeviceToHost, ctx->stream));
+    uint32_t status = 0;
+    rc = take_status(ctx, &status);
+    if (rc) return rc;
+    return status_to_rc(ctx, status);
+}
+
+extern "C" int bnk_wg_decap_batch(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *out,
+                                  uint8_t *result, uint32_t *out_len, uint32_t *peer, uint64_t *counter)
+{
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    int rc = check_batch_common(ctx, wire, "wire");
+    if (rc) return rc;
+    rc = check_batch_common(ctx, out, "out");
+    if (rc) return rc;
+    if (wire->mem != out->mem) return fail(ctx, BNK_E_INVAL, "wire and out must use the same mem kind");
+    const uint32_t n = wire->n;
+    if (n == 0) return BNK_OK;
+    if (!result || !out_len || !peer || !counter) return fail(ctx, BNK_E_INVAL, "null result array");
+    if (ctx->n_wg_peers == 0) return fail(ctx, BNK_E_STATE, "no peer table loaded");
+    if (!ctx->d_keys[BNK_KEYS_RECV] || ctx->n_keys[BNK_KEYS_RECV] < ctx->n_wg_peers)
+        return fail(ctx, BNK_E_STATE, "receive key table is smaller than the peer table");
+    const bool host = wire->mem == BNK_MEM_HOST;
+
+    WgBatch wb{}, ob{};
+    wb.n = ob.n = n;
+    wb.stride = wire->stride;
+    wb.len = wire->len;
+    ob.stride = out->stride;
+    uint8_t *d_result = nullptr;
+    uint32_t *d_out_len = nullptr, *d_peer = nullptr;
+    uint64_t *d_counter = nullptr;
+    Staged st;
+    if (host) {
+        bnk_batch w2 = *wire;
+        w2.peer = nullptr;
+        w2.counters = nullptr;
+        rc = stage_host(ctx, &w2, out, -32, 0, &st);
+        if (rc) return rc;
+        wb.base = st.d_in;
+        wb.off = st.d_in_off;
+        wb.lens = st.d_lens;
+        ob.base = st.d_out;
+        ob.off = st.d_out_off;
+        HIPCHK(ctx, ctx->wg_result.reserve(n));
+        HIPCHK(ctx, ctx->wg_outlen.reserve((size_t)n * 4));
+        HIPCHK(ctx, ctx->wg_peer.reserve((size_t)n * 4));
+        HIPCHK(ctx, ctx->wg_counter.reserve((size_t)n * 8));
+        d_result = ctx->wg_result.as<uint8_t>();
+        d_out_len = ctx->wg_outlen.as<uint32_t>();
+        d_peer = ctx->wg_peer.as<uint32_t>();
+        d_counter = ctx->wg_counter.as<uint64_t>();
+    } else {
+        if (!wire->offsets && !wire->lens && (uint64_t)(n - 1) * wire->stride + wire->len > wire->bytes)
+            return fail(ctx, BNK_E_INVAL, "wire: uniform layout exceeds the arena");
+        if (!out->offsets && !wire->lens &&
+            (uint64_t)(n - 1) * out->stride + (wire->len >= 32u ? wire->len - 32u : 0u) > out->bytes)
+            return fail(ctx, BNK_E_INVAL, "out: uniform layout exceeds the arena");
+        wb.base = (const uint8_t *)wire->base;
+        wb.off = wire->offsets;
+        wb.lens = wire->lens;
+        ob.base = (const uint8_t *)out->base;
+        ob.off = out->offsets;
+        d_result = result;
+        d_out_len = out_len;
+        d_peer = peer;
+        d_counter = counter;
+    }
+    HIPCHK(ctx, ctx->wg_ctlen.reserve((size_t)n * 4));
+    HIPCHK(ctx, ctx->r_auth.reserve(n));
+    uint32_t *d_ctlen = ctx->wg_ctlen.as<uint32_t>();
+    uint8_t *d_auth = ctx->r_auth.as<uint8_t>();
+    const WgPeersDev pe = peers_view(ctx);
+
+    HIPCHK(ctx, launch_wg_parse(wb, pe, d_peer, d_counter, d_ctlen, d_result, ctx->stream));
+
+    AeadArgs op{};
+    op.keys = ctx->d_keys[BNK_KEYS_RECV];
+    op.n_peers = pe.n;
+    op.status = ctx->d_status;
+    op.n = n;
+    op.in = wb.base;
+    op.in_off = wb.off;
+    op.in_stride = wire->stride;
+    op.in_skip = 16;
+    op.out = const_cast<uint8_t *>(ob.base);
+    op.out_off = ob.off;
+    op.out_stride = out->stride;
+    op.lens = d_ctlen;
+    op.peer = d_peer;
+    op.counters = d_counter;
+    op.verdict = d_auth;
+    op.skip = d_result; // BNK_WG_OK is 0: header failures are not opened
+    rc = maybe_sort(ctx, op.lens, n, 16, &op.order);
+    if (rc) return rc;
+    HIPCHK(ctx, launch_aead_open(op, ctx->stream));
+    HIPCHK(ctx, launch_wg_finish(ob, 0, pe, d_peer, d_ctlen, d_auth, d_result, d_out_len, ctx->stream));
+    if (!host) return BNK_OK;
+
+    HIPCHK(ctx, hipMemcpyAsync((uint8_t *)out->base + st.sout.lo, st.d_out, st.sout.size(),
+                               hipMemcpyDeviceToHost, ctx->stream));
+    HIPCHK(ctx, hipMemcpyAsync(result, d_result, n, hipMemcpyDeviceToHost, ctx->stream));
+    HIPCHK(ctx, hipMemcpyAsync(out_len, d_out_len, (size_t)n * 4, hipMemcpyDeviceToHost, ctx->stream));
+    HIPCHK(ctx, hipMemcpyAsync(peer, d_peer, (size_t)n * 4, hipMemcpyDeviceToHost, ctx->stream));
+    HIPCHK(ctx, hipMemcpyAsync(counter, d_counter, (size_t)n * 8, hipMemcpyDeviceToHost, ctx->stream));
+    uint32_t status = 0;
+    rc = take_status(ctx, &status);
+    if (rc) return rc;
+    return status_to_rc(ctx, status);
+}

@@ -1,0 +1,190 @@
+// WireGuard transport framing around the AEAD kernels: header parse and
+// build, receiver-index lookup, zero padding, IPv4 length trim, allowed-IP
+// check.  Follows the WireGuard protocol paper (section 5.4.6) and
+// wireguard-go's documented behaviour; wireguard-go itself is not part of the
+// reference tree (the reference only instantiates it,
+// internal/dataplane/engine.go:51, and gives every peer one /32 allowed IP,
+// engine.go:292-299).
+#include "../../include/bnkhip.h"
+#include "wg_dev.hpp"
+
+namespace bnk {
+
+#define BNK_DEV __device__ __forceinline__
+
+BNK_DEV uint32_t wg_ld32(const uint8_t *p)
+{
+    uint32_t v;
+    __builtin_memcpy(&v, p, 4);
+    return v;
+}
+
+BNK_DEV void wg_st32(uint8_t *p, uint32_t v) { __builtin_memcpy(p, &v, 4); }
+
+BNK_DEV uint32_t wg_padding(uint32_t len, uint32_t mtu)
+{
+    uint32_t last = len;
+    if (mtu == 0) return ((last + 15u) & ~15u) - last;
+    if (last > mtu) last %= mtu;
+    uint32_t padded = (last + 15u) & ~15u;
+    if (padded > mtu) padded = mtu;
+    return padded - last;
+}
+
+// Header checks and receiver-index lookup of received datagrams.
+__global__ __launch_bounds__(256) void wg_parse_kernel(WgBatch b, WgPeersDev pe, uint32_t *peer,
+                                                       uint64_t *counter, uint32_t *ct_len,
+                                                       uint8_t *result)
+{
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i >= b.n) return;
+    const uint8_t *w = b.base + (b.off ? b.off[i] : (uint64_t)i * b.stride);
+    const uint32_t len = b.lens ? b.lens[i] : b.len;
+    peer[i] = 0xFFFFFFFFu;
+    counter[i] = 0;
+    ct_len[i] = 0;
+    if (len < 32u || wg_ld32(w) != 4u) {
+        result[i] = BNK_WG_BAD_HEADER;
+        return;
+    }
+    const uint32_t idx = wg_ld32(w + 4);
+    uint32_t lo = 0, hi = pe.n;
+    while (lo < hi) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (pe.index_sorted[mid].x < idx) lo = mid + 1;
+        else hi = mid;
+    }
+    if (lo >= pe.n || pe.index_sorted[lo].x != idx) {
+        result[i] = BNK_WG_UNKNOWN_INDEX;
+        return;
+    }
+    peer[i] = pe.index_sorted[lo].y;
+    counter[i] = (uint64_t)wg_ld32(w + 8) | (uint64_t)wg_ld32(w + 12) << 32;
+    ct_len[i] = len - 16u;
+    result[i] = BNK_WG_OK; // so far
+}
+
+// After the open: keepalive, IP version, length trim, allowed source.
+__global__ __launch_bounds__(256) void wg_finish_kernel(WgBatch out, uint32_t out_skip, WgPeersDev pe,
+                                                        const uint32_t *peer, const uint32_t *ct_len,
+                                                        const uint8_t *auth, uint8_t *result,
+                                                        uint32_t *out_len)
+{
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i >= out.n) return;
+    out_len[i] = 0;
+    if (result[i] != BNK_WG_OK) return;
+    if (!auth[i]) {
+        result[i] = BNK_WG_AUTH_FAIL;
+        return;
+    }
+    const uint32_t plen = ct_len[i] - 16u;
+    if (plen == 0u) {
+        result[i] = BNK_WG_KEEPALIVE;
+        return;
+    }
+    const uint8_t *p = out.base + (out.off ? out.off[i] : (uint64_t)i * out.stride) + out_skip;
+    const uint32_t version = p[0] >> 4;
+    if (version == 4u) {
+        if (plen < 20u) { result[i] = BNK_WG_BAD_IP; return; }
+        const uint32_t total = (uint32_t)p[2] << 8 | p[3];
+        if (total > plen || total < 20u) { result[i] = BNK_WG_BAD_IP; return; }
+        const uint32_t src = __builtin_bswap32(wg_ld32(p + 12));
+        const uint2 al = pe.allowed[peer[i]];
+        if ((src & al.y) != (al.x & al.y)) { result[i] = BNK_WG_NOT_ALLOWED; return; }
+        out_len[i] = total;
+        return;
+    }
+    if (version == 6u) {
+        if (plen < 40u) { result[i] = BNK_WG_BAD_IP; return; }
+        const uint32_t total = ((uint32_t)p[4] << 8 | p[5]) + 40u;
+        result[i] = total > plen ? BNK_WG_BAD_IP : BNK_WG_NOT_ALLOWED; // peers own IPv4 addresses only
+        return;
+    }
+    result[i] = BNK_WG_BAD_IP;
+}
+
+// Sort keys for the per-peer counter assignment of an outgoing batch.
+__global__ __launch_bounds__(256) void wg_keys_kernel(const uint32_t *peer, uint32_t n_peers, uint32_t n,
+                                                      uint32_t *keys, uint32_t *idx, uint32_t *status)
+{
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i >= n) return;
+    uint32_t k = peer ? peer[i] : 0u;
+    if (k >= n_peers) {
+        atomicOr(status, 1u); // STATUS_PEER_RANGE
+        k = 0xFFFFFFFFu;
+    }
+    keys[i] = k;
+    idx[i] = i;
+}
+
+// Writes the transport header into the slot's headroom, zero-pads the
+// plaintext, and reports the padded and wire lengths.
+__global__ __launch_bounds__(256) void wg_encap_prep_kernel(WgBatch b, WgPeersDev pe, const uint32_t *peer,
+                                                            const uint64_t *counter, uint32_t mtu,
+                                                            uint32_t *padded_len, uint32_t *wire_len,
+                                                            uint8_t *skip)
+{
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i >= b.n) return;
+    const uint32_t pr = peer ? peer[i] : 0u;
+    const uint32_t len = b.lens ? b.lens[i] : b.len;
+    if (pr >= pe.n) {
+        skip[i] = 1;
+        padded_len[i] = 0;
+        wire_len[i] = 0;
+        return;
+    }
+    uint8_t *w = const_cast<uint8_t *>(b.base) + (b.off ? b.off[i] : (uint64_t)i * b.stride);
+    const uint32_t pad = wg_padding(len, mtu);
+    const uint64_t c = counter[i];
+    wg_st32(w, 4u);
+    wg_st32(w + 4, pe.remote_index[pr]);
+    wg_st32(w + 8, (uint32_t)c);
+    wg_st32(w + 12, (uint32_t)(c >> 32));
+    for (uint32_t k = 0; k < pad; k++) w[16u + len + k] = 0;
+    skip[i] = 0;
+    padded_len[i] = len + pad;
+    wire_len[i] = 16u + len + pad + 16u;
+}
+
+static dim3 grid_of(uint32_t n) { return dim3((n + 255u) / 256u); }
+
+hipError_t launch_wg_parse(const WgBatch &b, const WgPeersDev &pe, uint32_t *peer, uint64_t *counter,
+                           uint32_t *ct_len, uint8_t *result, hipStream_t s)
+{
+    if (b.n == 0) return hipSuccess;
+    hipLaunchKernelGGL(wg_parse_kernel, grid_of(b.n), dim3(256), 0, s, b, pe, peer, counter, ct_len, result);
+    return hipGetLastError();
+}
+
+hipError_t launch_wg_finish(const WgBatch &out, uint32_t out_skip, const WgPeersDev &pe,
+                            const uint32_t *peer, const uint32_t *ct_len, const uint8_t *auth,
+                            uint8_t *result, uint32_t *out_len, hipStream_t s)
+{
+    if (out.n == 0) return hipSuccess;
+    hipLaunchKernelGGL(wg_finish_kernel, grid_of(out.n), dim3(256), 0, s, out, out_skip, pe, peer, ct_len,
+                       auth, result, out_len);
+    return hipGetLastError();
+}
+
+hipError_t launch_wg_keys(const uint32_t *peer, uint32_t n_peers, uint32_t n, uint32_t *keys,
+                          uint32_t *idx, uint32_t *status, hipStream_t s)
+{
+    if (n == 0) return hipSuccess;
+    hipLaunchKernelGGL(wg_keys_kernel, grid_of(n), dim3(256), 0, s, peer, n_peers, n, keys, idx, status);
+    return hipGetLastError();
+}
+
+hipError_t launch_wg_encap_prep(const WgBatch &b, const WgPeersDev &pe, const uint32_t *peer,
+                                const uint64_t *counter, uint32_t mtu, uint32_t *padded_len,
+                                uint32_t *wire_len, uint8_t *skip, hipStream_t s)
+{
+    if (b.n == 0) return hipSuccess;
+    hipLaunchKernelGGL(wg_encap_prep_kernel, grid_of(b.n), dim3(256), 0, s, b, pe, peer, counter, mtu,
+                       padded_len, wire_len, skip);
+    return hipGetLastError();
+}
+
+} // namespace bnk

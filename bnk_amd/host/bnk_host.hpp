@@ -255,4 +255,53 @@ inline std::unique_ptr<tun::Device> WrapTUN(tun::Device *inner, Filter *f)
     return std::unique_ptr<tun::Device>(new FilteredTUN(inner, f));
 }
 
+// Anti-replay window for received transport counters (RFC 6479), with the
+// geometry wireguard-go's replay.Filter uses: a ring of 128 64-bit blocks,
+// so a counter is still acceptable while it trails the newest one by at most
+// (128 - 1) * 64 = 8128.  The reference gets this from
+// golang.zx2c4.com/wireguard/replay through device.NewDevice
+// (internal/dataplane/engine.go:51).  One filter per peer keypair; feed it
+// the (peer, counter) pairs bnk_wg_decap_batch reports for authentic packets,
+// in arrival order.
+class ReplayFilter {
+public:
+    static constexpr uint64_t kBlocks = 128;
+    static constexpr uint64_t kWindow = (kBlocks - 1) * 64;
+    // wireguard-go's RejectAfterMessages: 2^64 - 2^13 - 1
+    static constexpr uint64_t kRejectAfterMessages = ~uint64_t(0) - (uint64_t(1) << 13);
+
+    ReplayFilter() { Reset(); }
+    void Reset()
+    {
+        newest_ = 0;
+        for (uint64_t &w : seen_) w = 0;
+    }
+    // true = first sighting inside the window (accept and remember);
+    // false = duplicate, too old, or at/after `limit`.
+    bool ValidateCounter(uint64_t counter, uint64_t limit = kRejectAfterMessages)
+    {
+        if (counter >= limit) return false;
+        const uint64_t blk = counter / 64;
+        if (counter > newest_) {
+            // blocks between the old head and the new one start empty
+            const uint64_t head = newest_ / 64;
+            uint64_t fresh = blk - head;
+            if (fresh > kBlocks) fresh = kBlocks;
+            for (uint64_t k = 1; k <= fresh; k++) seen_[(head + k) % kBlocks] = 0;
+            newest_ = counter;
+        } else if (newest_ - counter > kWindow) {
+            return false;
+        }
+        uint64_t &word = seen_[blk % kBlocks];
+        const uint64_t bit = uint64_t(1) << (counter % 64);
+        const bool fresh = (word & bit) == 0;
+        word |= bit;
+        return fresh;
+    }
+
+private:
+    uint64_t newest_;
+    uint64_t seen_[kBlocks];
+};
+
 } // namespace bnk_host

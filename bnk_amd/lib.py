@@ -38,6 +38,10 @@ class Batch(C.Structure):
                 ("counters", C.c_void_p), ("counter0", C.c_uint64)]
 
 
+WG_OK, WG_KEEPALIVE, WG_BAD_HEADER, WG_UNKNOWN_INDEX, WG_AUTH_FAIL, WG_BAD_IP, \
+    WG_NOT_ALLOWED = range(7)
+
+
 class Rule(C.Structure):
     """struct bnk_rule"""
     _fields_ = [("src_net", C.c_uint32), ("src_mask", C.c_uint32),
@@ -312,6 +316,28 @@ class Context:
             self._h, C.byref(inb), C.c_void_p(_ptr(peer_out)), C.c_void_p(_ptr(ctr_base_out)),
             C.c_uint32(n_peers_out), C.c_int64(now_ns), C.byref(outb),
             C.c_void_p(_ptr(verdict)), C.c_void_p(_ptr(ctr_out))))
+
+    # ---- WireGuard transport framing ----
+    def wg_peers_set(self, peers) -> None:
+        """peers: [(local_index, remote_index, allowed_net, allowed_mask)]"""
+        arr = np.ascontiguousarray(np.array(peers, dtype=np.uint32).reshape(-1, 4))
+        self._chk(self._lib.bnk_wg_peers_set(self._h, C.c_void_p(arr.ctypes.data),
+                                             C.c_uint32(arr.shape[0])))
+
+    def wg_send_counters(self, n: int) -> np.ndarray:
+        out = np.zeros(max(n, 1), np.uint64)
+        self._chk(self._lib.bnk_wg_send_counters(self._h, C.c_void_p(out.ctypes.data),
+                                                 C.c_uint32(n)))
+        return out[:n]
+
+    def wg_encap(self, slots: Batch, mtu: int, wire_len) -> None:
+        self._chk(self._lib.bnk_wg_encap_batch(self._h, C.byref(slots), C.c_uint32(mtu),
+                                               C.c_void_p(_ptr(wire_len))))
+
+    def wg_decap(self, wire: Batch, outb: Batch, result, out_len, peer, counter) -> None:
+        self._chk(self._lib.bnk_wg_decap_batch(
+            self._h, C.byref(wire), C.byref(outb), C.c_void_p(_ptr(result)),
+            C.c_void_p(_ptr(out_len)), C.c_void_p(_ptr(peer)), C.c_void_p(_ptr(counter))))
 
     # ---- measurement ----
     def probe_valu(self, op: str | int, iters: int = 2000) -> float:

@@ -197,6 +197,63 @@ int bnk_filter_flow_count(bnk_ctx *ctx, uint32_t *count);
 int bnk_filter_flow_dump(bnk_ctx *ctx, uint64_t *key, uint8_t *proto,
                          int64_t *expiry_ns, uint32_t cap, uint32_t *count);
 
+/* ---- WireGuard transport framing ----------------------------------------
+ *
+ * The datagram around the AEAD: type (LE32 = 4) || receiver index (LE32) ||
+ * counter (LE64) || ChaCha20-Poly1305(plaintext zero-padded to 16 bytes).
+ * The reference delegates this to golang.zx2c4.com/wireguard's device
+ * package, which it only instantiates (internal/dataplane/engine.go:51) and
+ * configures with one /32 allowed IP per peer (engine.go:292-299); that
+ * package is not in the reference tree, so these entry points follow the
+ * WireGuard protocol paper (section 5.4.6) and wireguard-go's documented
+ * behaviour (device/send.go, device/receive.go).  The anti-replay window
+ * (RFC 6479) is order dependent and stays on the host, fed with the peer and
+ * counter this call reports. */
+
+enum {
+    BNK_WG_OK = 0,            /* data packet, delivered */
+    BNK_WG_KEEPALIVE = 1,     /* authentic, empty plaintext */
+    BNK_WG_BAD_HEADER = 2,    /* shorter than 32 bytes or type != 4 */
+    BNK_WG_UNKNOWN_INDEX = 3, /* no peer owns the receiver index */
+    BNK_WG_AUTH_FAIL = 4,     /* tag mismatch */
+    BNK_WG_BAD_IP = 5,        /* not IPv4/IPv6 or length fields beyond the plaintext */
+    BNK_WG_NOT_ALLOWED = 6    /* inner source outside the peer's allowed IP */
+};
+
+typedef struct bnk_wg_peer {
+    uint32_t local_index;  /* receiver index we handed out; unique per peer */
+    uint32_t remote_index; /* receiver index the peer expects */
+    uint32_t allowed_net;  /* IPv4 prefix, host order (engine.go:292-299: a /32) */
+    uint32_t allowed_mask;
+} bnk_wg_peer;
+
+/* Installs the peer table; peer i uses row i of both key tables.  Resets
+ * every peer's send counter to 0 (a fresh keypair starts there). */
+int bnk_wg_peers_set(bnk_ctx *ctx, const bnk_wg_peer *peers, uint32_t n);
+/* Copies the next send counter of peers [0, n) to a host array. */
+int bnk_wg_send_counters(bnk_ctx *ctx, uint64_t *out, uint32_t n);
+/* Outgoing: slot i starts at slots' offset i with 16 bytes of headroom,
+ * lens[i] bytes of plaintext after it, and room for the padding and the
+ * tag.  Pads the plaintext with zeros to a multiple of 16 (never beyond
+ * mtu; mtu 0 = no cap), gives each packet its peer's next counter in batch
+ * order, writes the header into the headroom and seals in place.
+ * wire_len[i] = 16 + lens[i] + padding + 16, the datagram to send from the
+ * slot's start.  slots->counters and counter0 are ignored.  wire_len lives
+ * where slots->mem says. */
+int bnk_wg_encap_batch(bnk_ctx *ctx, const bnk_batch *slots, uint32_t mtu,
+                       uint32_t *wire_len);
+/* Incoming: wire->lens[i] bytes at wire's offset i are one datagram.
+ * result[i] is BNK_WG_*; for BNK_WG_OK the inner packet, trimmed to its IP
+ * total length, is out_len[i] bytes at out's offset i.  For every result but
+ * BAD_HEADER/UNKNOWN_INDEX peer[i] and counter[i] name the sender and the
+ * nonce counter (feed them to the replay window when result is OK or
+ * KEEPALIVE); otherwise peer[i] = 0xFFFFFFFF.  A failed open leaves zeros in
+ * `out`, like the AEAD entry points.  wire->peer/counters are ignored.
+ * result, out_len, peer and counter live where wire->mem says. */
+int bnk_wg_decap_batch(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *out,
+                       uint8_t *result, uint32_t *out_len, uint32_t *peer,
+                       uint64_t *counter);
+
 /* ---- fused relay ------------------------------------------------------- */
 
 enum { BNK_RELAY_OK = 0, BNK_RELAY_FORGED = 1, BNK_RELAY_DENIED = 2 };

@@ -270,3 +270,62 @@ class Filter:
             C.c_int64(now_ns), _p(verdict, _u8p), _p(ctr_out, _u64p),
             C.c_uint32(n))
         return verdict, ctr_out
+
+
+# ---- WireGuard transport framing (parity unpinned: see bnk_oracle.h) -----
+
+WG_OK, WG_KEEPALIVE, WG_BAD_HEADER, WG_UNKNOWN_INDEX, WG_AUTH_FAIL, WG_BAD_IP, \
+    WG_NOT_ALLOWED = range(7)
+
+_lib.bnko_wg_padding.restype = C.c_uint32
+_lib.bnko_wg_encap.restype = C.c_uint32
+_lib.bnko_wg_decap.restype = C.c_int
+_lib.bnko_replay_validate.restype = C.c_int
+
+
+def wg_padding(length: int, mtu: int) -> int:
+    return int(_lib.bnko_wg_padding(C.c_uint32(length), C.c_uint32(mtu)))
+
+
+def wg_encap(plain: bytes, mtu: int, key: bytes, remote_index: int, counter: int) -> bytes:
+    """One transport datagram for `plain`."""
+    slot = np.zeros(16 + len(plain) + 16 + 16, np.uint8)
+    slot[16:16 + len(plain)] = np.frombuffer(plain, np.uint8)
+    n = _lib.bnko_wg_encap(_p(slot, _u8p), C.c_uint32(len(plain)), C.c_uint32(mtu),
+                           _p(_b(key), _u8p), C.c_uint32(remote_index), C.c_uint64(counter))
+    return slot[:n].tobytes()
+
+
+def _mk_wg_peers(peers) -> np.ndarray:
+    """[(local_index, remote_index, allowed_net, allowed_mask)] -> u32[n, 4]"""
+    return np.ascontiguousarray(np.array(peers, dtype=np.uint32).reshape(-1, 4))
+
+
+def wg_decap(wire: bytes, peers, keys_recv: np.ndarray):
+    """-> (result, plaintext bytes, peer, counter)"""
+    pe = _mk_wg_peers(peers)
+    src = _b(wire) if len(wire) else np.zeros(1, np.uint8)
+    out = np.zeros(max(len(wire), 1), np.uint8)
+    out_len = C.c_uint32()
+    peer = C.c_uint32()
+    counter = C.c_uint64()
+    rc = _lib.bnko_wg_decap(_p(src, _u8p), C.c_uint32(len(wire)), C.c_void_p(pe.ctypes.data),
+                            _p(np.ascontiguousarray(keys_recv).reshape(-1), _u8p),
+                            C.c_uint32(pe.shape[0]), _p(out, _u8p), C.byref(out_len),
+                            C.byref(peer), C.byref(counter))
+    return int(rc), out[:out_len.value].tobytes(), int(peer.value), int(counter.value)
+
+
+class ReplayFilter:
+    """RFC 6479 window (bnko_replay)."""
+
+    def __init__(self):
+        self._s = np.zeros(129, np.uint64)
+        _lib.bnko_replay_reset(C.c_void_p(self._s.ctypes.data))
+
+    def reset(self) -> None:
+        _lib.bnko_replay_reset(C.c_void_p(self._s.ctypes.data))
+
+    def validate(self, counter: int, limit: int = (1 << 64) - (1 << 13) - 1) -> bool:
+        return bool(_lib.bnko_replay_validate(C.c_void_p(self._s.ctypes.data),
+                                              C.c_uint64(counter), C.c_uint64(limit)))

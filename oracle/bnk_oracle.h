@@ -185,6 +185,60 @@ void bnko_relay_fused_batch(bnko_filter *f, const uint8_t *keys_in,
                             const uint64_t *out_off, int64_t now_ns,
                             uint8_t *verdict, uint64_t *ctr_out, uint32_t n);
 
+/* ---------------- WireGuard transport framing (wireguard-go, not vendored) ----------------
+ *
+ * PARITY UNPINNED: the reference reaches this code only through
+ * device.NewDevice (internal/dataplane/engine.go:51) and wireguard-go's source
+ * is not in the reference tree.  What follows restates the WireGuard protocol
+ * paper (section 5.4.6: type 4, receiver index, 64-bit counter, zero padding of
+ * the plaintext to a multiple of 16) and wireguard-go's documented behaviour
+ * (padding capped at the MTU, IPv4 total-length trim, source must be an
+ * allowed IP of the sending peer, RFC 6479 replay window of 8128 counters).
+ * In-repo corroboration: offset 16 (internal/filter/tun_test.go:50), type byte 4
+ * (internal/magicsock/bind_bench_test.go:29), one /32 allowed IP per peer
+ * (internal/dataplane/engine.go:292-299). */
+
+enum {
+    BNKO_WG_OK = 0,            /* deliver out_len bytes of plaintext */
+    BNKO_WG_KEEPALIVE = 1,     /* authentic, empty */
+    BNKO_WG_BAD_HEADER = 2,    /* shorter than 32 bytes or type != 4 */
+    BNKO_WG_UNKNOWN_INDEX = 3, /* receiver index names no keypair */
+    BNKO_WG_AUTH_FAIL = 4,
+    BNKO_WG_BAD_IP = 5,        /* not IPv4/IPv6, or its length field is inconsistent */
+    BNKO_WG_NOT_ALLOWED = 6    /* source address is not the peer's allowed IP */
+};
+
+typedef struct {
+    uint32_t local_index;  /* index this side handed out; arrives in the header */
+    uint32_t remote_index; /* index the peer handed out; goes into the header */
+    uint32_t allowed_net, allowed_mask; /* the peer's allowed IPv4 prefix */
+} bnko_wg_peer;
+
+/* Bytes of zero padding wireguard-go appends before sealing. */
+uint32_t bnko_wg_padding(uint32_t packet_len, uint32_t mtu);
+
+/* slot: 16 bytes of headroom, then `len` plaintext bytes, then room for the
+ * padding and the tag.  Writes the header, pads, seals in place with `counter`
+ * under key; returns the wire length (16 + padded + 16). */
+uint32_t bnko_wg_encap(uint8_t *slot, uint32_t len, uint32_t mtu, const uint8_t key[32],
+                       uint32_t remote_index, uint64_t counter);
+
+/* wire: a received datagram.  peers/keys_recv: n_peers entries.  On OK writes
+ * the trimmed plaintext to out (may be wire + 16) and its length to *out_len;
+ * *peer and *counter are set whenever the index resolves. */
+int bnko_wg_decap(const uint8_t *wire, uint32_t wire_len, const bnko_wg_peer *peers,
+                  const uint8_t *keys_recv, uint32_t n_peers, uint8_t *out, uint32_t *out_len,
+                  uint32_t *peer, uint64_t *counter);
+
+/* RFC 6479 sliding window as wireguard-go's replay.Filter keeps it. */
+typedef struct {
+    uint64_t last;
+    uint64_t ring[128];
+} bnko_replay;
+void bnko_replay_reset(bnko_replay *f);
+/* 1 = fresh (accept), 0 = replayed, too old, or counter >= limit */
+int bnko_replay_validate(bnko_replay *f, uint64_t counter, uint64_t limit);
+
 #ifdef __cplusplus
 }
 #endif

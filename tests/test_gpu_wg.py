@@ -1,0 +1,354 @@
+"""WireGuard transport framing on the GPU (bnk_wg_encap_batch /
+bnk_wg_decap_batch) against the oracle's per-packet definition: identical
+datagrams, results, lengths, peers, counters and plaintext bytes.  The oracle's
+framing itself is spec-derived (wireguard-go is not in the reference tree), so
+this is parity with the restated protocol, not with a reference artefact."""
+import struct
+
+import numpy as np
+import pytest
+
+from bnk_amd import workloads as W
+
+pytestmark = pytest.mark.gpu
+
+N_PEERS = 37
+MTU = 1420
+
+
+def _peers(rng):
+    local = rng.permutation(1 << 20)[:N_PEERS].astype(np.uint32) * 4099 + 17
+    remote = rng.integers(0, 1 << 32, N_PEERS, dtype=np.uint64).astype(np.uint32)
+    net = (0x64400000 + np.arange(N_PEERS, dtype=np.uint32) * 256 + 1).astype(np.uint32)
+    mask = np.full(N_PEERS, 0xFFFFFFFF, np.uint32)
+    mask[::5] = 0xFFFFFF00  # a few peers own a /24
+    return [(int(a), int(b), int(c), int(d)) for a, b, c, d in zip(local, remote, net, mask)]
+
+
+def _inner(rng, peers, p, length):
+    """An IPv4 packet of `length` bytes from peer p's allowed address."""
+    if length < 20:
+        return bytes(length)  # too short for IPv4; version nibble 0
+    pkt = bytearray(rng.integers(0, 256, length, dtype=np.uint8).tobytes())
+    pkt[0] = 0x45
+    pkt[2:4] = struct.pack(">H", length)
+    pkt[12:16] = struct.pack(">I", peers[p][2])
+    return bytes(pkt)
+
+
+def _layout(rng, sizes, misalign=False):
+    """Slot offsets: 16-aligned with random gaps, or arbitrary."""
+    gaps = rng.integers(0, 5, len(sizes)) * 16
+    off = np.zeros(len(sizes), np.uint64)
+    pos = 0
+    for i, s in enumerate(sizes):
+        pos += int(gaps[i])
+        if misalign:
+            pos += int(rng.integers(0, 16))
+        else:
+            pos = (pos + 15) & ~15
+        off[i] = pos
+        pos += int(s)
+    return off, pos + 64
+
+
+def _ctx(peers, keys_send=None, keys_recv=None):
+    from bnk_amd import lib
+    ctx = lib.Context(0)
+    if keys_send is not None:
+        ctx.keys_set(lib.KEYS_SEND, keys_send)
+    if keys_recv is not None:
+        ctx.keys_set(lib.KEYS_RECV, keys_recv)
+    ctx.wg_peers_set(peers)
+    return ctx
+
+
+@pytest.mark.parametrize("mem", ["host", "device"])
+@pytest.mark.parametrize("misalign", [False, True])
+def test_encap_matches_oracle(mem, misalign):
+    import torch
+    from bnk_amd import lib
+    from oracle import binding as O
+    rng = np.random.default_rng(11 + misalign)
+    peers = _peers(rng)
+    keys = rng.integers(0, 256, (N_PEERS, 32), dtype=np.uint8)
+    n = 3000
+    lens = rng.choice([0, 1, 15, 16, 17, 20, 40, 63, 64, 65, 127, 128, 129, 576, 1399, 1408, 1419, 1420],
+                      n).astype(np.uint32)
+    lens[:200] = rng.integers(0, MTU + 1, 200)
+    peer = rng.integers(0, N_PEERS, n).astype(np.uint32)
+    room = 16 + lens.astype(np.int64) + 15 + 16
+    off, total = _layout(rng, room, misalign)
+    arena = np.full(total, 0xEE, np.uint8)
+    plains = []
+    for i in range(n):
+        pt = _inner(rng, peers, int(peer[i]), int(lens[i]))
+        plains.append(pt)
+        arena[int(off[i]) + 16:int(off[i]) + 16 + len(pt)] = np.frombuffer(pt, np.uint8)
+    ctx = _ctx(peers, keys_send=keys)
+    next_ctr = np.zeros(N_PEERS, np.uint64)
+    for round_ in range(2):  # the second batch continues the peers' counters
+        want = arena.copy()
+        want_len = np.zeros(n, np.uint32)
+        for i in range(n):
+            p = int(peer[i])
+            w = O.wg_encap(plains[i], MTU, keys[p].tobytes(), peers[p][1], int(next_ctr[p]))
+            next_ctr[p] += 1
+            want[int(off[i]):int(off[i]) + len(w)] = np.frombuffer(w, np.uint8)
+            want_len[i] = len(w)
+        if mem == "host":
+            got = arena.copy()
+            got_len = np.zeros(n, np.uint32)
+            ctx.wg_encap(lib.make_batch(got, got.nbytes, n, lib.MEM_HOST, offsets=off, lens=lens, peer=peer),
+                         MTU, got_len)
+        else:
+            dev = torch.device("cuda:0")
+            d_arena = torch.from_numpy(arena).to(dev)
+            d_off = torch.from_numpy(off.astype(np.int64)).to(dev)
+            d_lens = torch.from_numpy(lens.astype(np.int32)).to(dev)
+            d_peer = torch.from_numpy(peer.astype(np.int32)).to(dev)
+            d_wl = torch.zeros(n, dtype=torch.int32, device=dev)
+            torch.cuda.synchronize()
+            ctx.wg_encap(lib.make_batch(d_arena, d_arena.numel(), n, lib.MEM_DEVICE, offsets=d_off,
+                                        lens=d_lens, peer=d_peer), MTU, d_wl)
+            ctx.sync()
+            got = d_arena.cpu().numpy()
+            got_len = d_wl.cpu().numpy().astype(np.uint32)
+        assert np.array_equal(got_len, want_len)
+        bad = np.flatnonzero(got != want)
+        assert bad.size == 0, f"first differing byte at {bad[:5]}"  # gaps keep their 0xEE fill
+        assert np.array_equal(ctx.wg_send_counters(N_PEERS), next_ctr)
+    ctx.close()
+
+
+def _decap_cases(rng, peers, keys, n):
+    """Datagrams as the remote peers would send them, most of them damaged in
+    one of the ways the receive path must tell apart."""
+    from oracle import binding as O
+    wires, kinds = [], []
+    for i in range(n):
+        p = int(rng.integers(0, N_PEERS))
+        kind = int(rng.integers(0, 14))
+        length = int(rng.choice([20, 21, 28, 40, 64, 100, 576, 1300, 1420]))
+        pt = bytearray(_inner(rng, peers, p, length))
+        if kind == 1:
+            pt = bytearray()                           # keepalive
+        elif kind == 2:
+            pt[2:4] = struct.pack(">H", max(20, length - int(rng.integers(0, 9))))  # trailing bytes
+        elif kind == 3:
+            pt[0] = int(rng.choice([0x05, 0x55, 0x75, 0xF5]))
+        elif kind == 4:
+            pt[2:4] = struct.pack(">H", length + 16)
+        elif kind == 5:
+            pt[2:4] = struct.pack(">H", int(rng.integers(0, 20)))
+        elif kind == 6:
+            pt[12:16] = struct.pack(">I", peers[p][2] ^ 0x00010000)  # outside the allowed prefix
+        elif kind == 7:
+            pt = bytearray(max(length, 40))
+            pt[0] = 0x60
+            pt[4:6] = struct.pack(">H", len(pt) - 40 + int(rng.integers(0, 2)) * 8)
+        elif kind == 8:
+            pt = pt[:int(rng.integers(1, 20))]
+            pt[0] = 0x45
+        ctr = int(rng.integers(0, 1 << 62))
+        w = bytearray(O.wg_encap(bytes(pt), MTU, keys[p].tobytes(), peers[p][0], ctr))
+        if kind == 9:
+            w[int(rng.integers(8, len(w)))] ^= 1 << int(rng.integers(0, 8))   # counter, body or tag
+        elif kind == 10:
+            w[0:4] = struct.pack("<I", int(rng.choice([0, 1, 2, 3, 5, 0x0400, 0x04000000])))
+        elif kind == 11:
+            w = w[:int(rng.integers(0, 32))]
+        elif kind == 12:
+            w[4:8] = struct.pack("<I", peers[p][0] ^ 0x40000000)
+        elif kind == 13:
+            w[4:8] = struct.pack("<I", peers[(p + 1) % N_PEERS][0])           # someone else's index
+        wires.append(bytes(w))
+        kinds.append(kind)
+    return wires, np.array(kinds)
+
+
+@pytest.mark.parametrize("mem", ["host", "device"])
+@pytest.mark.parametrize("aligned", [True, False])
+def test_decap_matches_oracle(mem, aligned):
+    import torch
+    from bnk_amd import lib
+    from oracle import binding as O
+    rng = np.random.default_rng(23 + aligned)
+    peers = _peers(rng)
+    keys = rng.integers(0, 256, (N_PEERS, 32), dtype=np.uint8)
+    n = 4000
+    wires, kinds = _decap_cases(rng, peers, keys, n)
+    lens = np.array([len(w) for w in wires], np.uint32)
+    off, total = _layout(rng, lens, misalign=not aligned)
+    arena = np.full(total, 0xEE, np.uint8)
+    for i, w in enumerate(wires):
+        arena[int(off[i]):int(off[i]) + len(w)] = np.frombuffer(w, np.uint8)
+    # plaintext slot i sits 16 bytes into a copy of the wire layout, so that
+    # ciphertext and plaintext share their position within a 128-byte line
+    out_off = off + np.uint64(16)
+    want_out = np.full(total + 16, 0x77, np.uint8)
+    want = np.zeros((n, 4), np.uint64)
+    for i, w in enumerate(wires):
+        rc, pt, p, c = O.wg_decap(w, peers, keys)
+        want[i] = (rc, len(pt), p, c)
+        plen = max(len(w) - 32, 0)
+        if rc not in (O.WG_BAD_HEADER, O.WG_UNKNOWN_INDEX):
+            # an opened packet leaves its whole plaintext (padding included), a
+            # failed open leaves zeros
+            if rc == O.WG_AUTH_FAIL:
+                body = bytes(plen)
+            else:
+                ok, body = O.aead_open(keys[p].tobytes(), O.wg_nonce(c), w[16:])
+                assert ok
+            want_out[int(out_off[i]):int(out_off[i]) + plen] = np.frombuffer(body, np.uint8)
+    assert len(set(want[:, 0].tolist())) == 7  # every result class occurs
+    ctx = _ctx(peers, keys_recv=keys)
+    if mem == "host":
+        got_out = np.full(total + 16, 0x77, np.uint8)
+        res = np.full(n, 99, np.uint8)
+        olen = np.full(n, 99, np.uint32)
+        gp = np.full(n, 99, np.uint32)
+        gc = np.full(n, 99, np.uint64)
+        ctx.wg_decap(lib.make_batch(arena, arena.nbytes, n, lib.MEM_HOST, offsets=off, lens=lens),
+                     lib.make_batch(got_out, got_out.nbytes, n, lib.MEM_HOST, offsets=out_off),
+                     res, olen, gp, gc)
+    else:
+        dev = torch.device("cuda:0")
+        d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)  # noqa: E731
+        d_arena, d_off, d_lens = d(arena), d(off.astype(np.int64)), d(lens.astype(np.int32))
+        d_ooff = d(out_off.astype(np.int64))
+        d_out = torch.full((total + 16,), 0x77, dtype=torch.uint8, device=dev)
+        d_res = torch.full((n,), 99, dtype=torch.uint8, device=dev)
+        d_olen = torch.zeros(n, dtype=torch.int32, device=dev)
+        d_gp = torch.zeros(n, dtype=torch.int32, device=dev)
+        d_gc = torch.zeros(n, dtype=torch.int64, device=dev)
+        torch.cuda.synchronize()
+        ctx.wg_decap(lib.make_batch(d_arena, d_arena.numel(), n, lib.MEM_DEVICE, offsets=d_off, lens=d_lens),
+                     lib.make_batch(d_out, d_out.numel(), n, lib.MEM_DEVICE, offsets=d_ooff),
+                     d_res, d_olen, d_gp, d_gc)
+        ctx.sync()
+        got_out = d_out.cpu().numpy()
+        res = d_res.cpu().numpy()
+        olen = d_olen.cpu().numpy().astype(np.uint32)
+        gp = d_gp.cpu().numpy().astype(np.uint32)
+        gc = d_gc.cpu().numpy().astype(np.uint64)
+    assert np.array_equal(res, want[:, 0].astype(np.uint8))
+    assert np.array_equal(olen, want[:, 1].astype(np.uint32))
+    assert np.array_equal(gp, want[:, 2].astype(np.uint32))
+    assert np.array_equal(gc, want[:, 3])
+    bad = np.flatnonzero(got_out != want_out)
+    assert bad.size == 0, f"first differing byte at {bad[:5]}"
+    ctx.close()
+
+
+def test_encap_then_decap_round_trip_full_size():
+    """2^20 MTU-sized slots, device resident: every datagram decapsulates to
+    its plaintext under the mirrored peer table, counters are each peer's
+    0..k-1 in batch order, and a sample is bit-exact against the oracle."""
+    import torch
+    from bnk_amd import lib
+    from oracle import binding as O
+    dev = torch.device("cuda:0")
+    n, n_peers, plen = 1 << 20, 1024, 1400
+    stride = 1536  # slot: 16 headroom + 1400 + 8 pad + 16 tag = 1440
+    rng = np.random.default_rng(5)
+    keys = rng.integers(0, 256, (n_peers, 32), dtype=np.uint8)
+    idx_a = (np.arange(n_peers, dtype=np.uint32) * 7919 + 3).astype(np.uint32)
+    idx_b = (np.arange(n_peers, dtype=np.uint32) * 104729 + 11).astype(np.uint32)
+    addr = (0x64400000 + np.arange(n_peers, dtype=np.uint32)).astype(np.uint32)
+    full = np.full(n_peers, 0xFFFFFFFF, np.uint32)
+    # side A sends with remote index idx_b; side B receives with local index idx_b
+    side_a = np.stack([idx_a, idx_b, addr, full], 1)
+    side_b = np.stack([idx_b, idx_a, addr, full], 1)
+    peer = rng.integers(0, n_peers, n).astype(np.uint32)
+    arena = W.rand_bytes_torch(W.stream_seed(2, 77), n * stride, dev).view(n, stride)
+    d_peer = torch.from_numpy(peer.astype(np.int32)).to(dev)
+    # valid IPv4 header fields where decap looks: version/IHL, total length, source
+    arena[:, 16] = 0x45
+    arena[:, 18] = plen >> 8
+    arena[:, 19] = plen & 0xFF
+    src = torch.from_numpy(addr.astype(np.int64)).to(dev)[d_peer.long()]
+    for k in range(4):
+        arena[:, 16 + 12 + k] = ((src >> (24 - 8 * k)) & 0xFF).to(torch.uint8)
+    plain = arena[:, 16:16 + plen].clone()
+    d_wl = torch.zeros(n, dtype=torch.int32, device=dev)
+    torch.cuda.synchronize()
+    tx = lib.Context(0)
+    tx.keys_set(lib.KEYS_SEND, keys)
+    tx.wg_peers_set(side_a)
+    tx.wg_encap(lib.make_batch(arena, arena.numel(), n, lib.MEM_DEVICE, stride=stride, length=plen,
+                               peer=d_peer), MTU, d_wl)
+    tx.sync()
+    assert bool((d_wl == 1440).all())
+    sent = np.bincount(peer, minlength=n_peers).astype(np.uint64)
+    assert np.array_equal(tx.wg_send_counters(n_peers), sent)
+    # sample against the oracle
+    sample = rng.choice(n, 64, replace=False)
+    rank = np.zeros(n, np.uint64)
+    seen = np.zeros(n_peers, np.uint64)
+    for i in range(n):
+        rank[i] = seen[peer[i]]
+        seen[peer[i]] += 1
+    h_plain = plain[torch.from_numpy(sample).to(dev)].cpu().numpy()
+    h_wire = arena[torch.from_numpy(sample).to(dev)].cpu().numpy()
+    for j, i in enumerate(sample):
+        p = int(peer[i])
+        w = O.wg_encap(h_plain[j].tobytes(), MTU, keys[p].tobytes(), int(idx_b[p]), int(rank[i]))
+        assert h_wire[j, :1440].tobytes() == w
+    # receive side
+    rx = lib.Context(0)
+    rx.keys_set(lib.KEYS_RECV, keys)
+    rx.wg_peers_set(side_b)
+    out = torch.zeros(n, stride, dtype=torch.uint8, device=dev)
+    d_res = torch.full((n,), 99, dtype=torch.uint8, device=dev)
+    d_olen = torch.zeros(n, dtype=torch.int32, device=dev)
+    d_gp = torch.zeros(n, dtype=torch.int32, device=dev)
+    d_gc = torch.zeros(n, dtype=torch.int64, device=dev)
+    torch.cuda.synchronize()
+    # plaintext lands 16 bytes into its slot, in line with the ciphertext
+    rx.wg_decap(lib.make_batch(arena, arena.numel(), n, lib.MEM_DEVICE, stride=stride, length=1440),
+                lib.make_batch(out.view(-1)[16:], out.numel() - 16, n, lib.MEM_DEVICE, stride=stride),
+                d_res, d_olen, d_gp, d_gc)
+    rx.sync()
+    assert bool((d_res == 0).all())
+    assert bool((d_olen == plen).all())
+    assert bool((d_gp == d_peer).all())
+    assert np.array_equal(d_gc.cpu().numpy().astype(np.uint64), rank)
+    assert torch.equal(out[:, 16:16 + plen], plain)
+    tx.close()
+    rx.close()
+
+
+def test_wg_argument_errors():
+    from bnk_amd import lib
+    ctx = lib.Context(0)
+    arena = np.zeros(4096, np.uint8)
+    wl_ = np.zeros(4, np.uint32)
+    b = lib.make_batch(arena, arena.nbytes, 4, lib.MEM_HOST, stride=256, length=100)
+    with pytest.raises(lib.BnkError) as ei:
+        ctx.wg_encap(b, MTU, wl_)
+    assert ei.value.code == lib.E_STATE  # no peer table
+    with pytest.raises(lib.BnkError) as ei:
+        ctx.wg_peers_set([(1, 2, 3, 0xFFFFFFFF), (1, 5, 6, 0xFFFFFFFF)])
+    assert ei.value.code == lib.E_INVAL  # duplicate local index
+    with pytest.raises(lib.BnkError) as ei:
+        ctx.wg_peers_set([(1, 2, 3, 0xFF00FF00)])
+    assert ei.value.code == lib.E_INVAL
+    ctx.wg_peers_set([(1, 2, 3, 0xFFFFFFFF), (4, 5, 6, 0xFFFFFFFF)])
+    with pytest.raises(lib.BnkError) as ei:
+        ctx.wg_encap(b, MTU, wl_)
+    assert ei.value.code == lib.E_STATE  # no send keys
+    ctx.keys_set(lib.KEYS_SEND, np.zeros((2, 32), np.uint8))
+    peer = np.array([0, 1, 2, 0], np.uint32)
+    with pytest.raises(lib.BnkError) as ei:
+        ctx.wg_encap(lib.make_batch(arena, arena.nbytes, 4, lib.MEM_HOST, stride=256, length=100,
+                                    peer=peer), MTU, wl_)
+    assert ei.value.code == lib.E_RANGE
+    with pytest.raises(lib.BnkError) as ei:
+        ctx.wg_encap(lib.make_batch(arena, 900, 4, lib.MEM_HOST, stride=256, length=100), MTU, wl_)
+    assert ei.value.code == lib.E_INVAL  # last slot has no room for pad + tag
+    assert np.array_equal(ctx.wg_send_counters(2), [0, 0])  # refused calls hand out no counters
+    ctx.wg_encap(b, MTU, wl_)
+    assert np.array_equal(wl_, [16 + 112 + 16] * 4)
+    assert np.array_equal(ctx.wg_send_counters(2), [4, 0])
+    ctx.close()

@@ -273,6 +273,90 @@ def bench_relay(args) -> dict:
     }
 
 
+def bench_wg(args) -> dict:
+    """Transport framing around the AEAD: encapsulate (header, padding, per-peer
+    counters, seal in place) and decapsulate (header checks, index lookup, open,
+    IPv4 trim, allowed-IP check) 2^20 MTU-sized packets across 1024 peers."""
+    import numpy as np
+    import torch
+    from bnk_amd import lib, workloads as W
+    dev = torch.device("cuda:0")
+    n, n_peers, plen, mtu, stride = 1 << 20, 1024, 1420, 1420, 1456
+    wire_len = 16 + plen + 16
+    keys = W.rand_bytes(W.stream_seed(2, 40), n_peers * 32).reshape(n_peers, 32)
+    idx_a = (np.arange(n_peers, dtype=np.uint32) * 7919 + 3).astype(np.uint32)
+    idx_b = (np.arange(n_peers, dtype=np.uint32) * 104729 + 11).astype(np.uint32)
+    addr = (0x64400000 + np.arange(n_peers, dtype=np.uint32)).astype(np.uint32)
+    full = np.full(n_peers, 0xFFFFFFFF, np.uint32)
+    peer = W.rand_below(W.stream_seed(2, 41), n, n_peers).astype(np.uint32)
+    d_peer = torch.from_numpy(peer.astype(np.int32)).to(dev)
+
+    def slots():
+        a = W.rand_bytes_torch(W.stream_seed(2, 42), n * stride, dev).view(n, stride)
+        a[:, 16] = 0x45
+        a[:, 18] = plen >> 8
+        a[:, 19] = plen & 0xFF
+        src = torch.from_numpy(addr.astype(np.int64)).to(dev)[d_peer.long()]
+        for k in range(4):
+            a[:, 28 + k] = ((src >> (24 - 8 * k)) & 0xFF).to(torch.uint8)
+        return a
+
+    wire = slots()       # encapsulated once; the receive side reads it every step
+    scratch = slots()    # encapsulated in place again every step
+    out = torch.zeros(n * stride + 16, dtype=torch.uint8, device=dev)
+    d_wl = torch.zeros(n, dtype=torch.int32, device=dev)
+    d_res = torch.zeros(n, dtype=torch.uint8, device=dev)
+    d_olen = torch.zeros(n, dtype=torch.int32, device=dev)
+    d_gp = torch.zeros(n, dtype=torch.int32, device=dev)
+    d_gc = torch.zeros(n, dtype=torch.int64, device=dev)
+    torch.cuda.synchronize()
+    tx, rx = lib.Context(0), lib.Context(0)
+    tx.keys_set(lib.KEYS_SEND, keys)
+    tx.wg_peers_set(np.stack([idx_a, idx_b, addr, full], 1))
+    rx.keys_set(lib.KEYS_RECV, keys)
+    rx.wg_peers_set(np.stack([idx_b, idx_a, addr, full], 1))
+    nbytes = n * stride
+    tx.wg_encap(lib.make_batch(wire, nbytes, n, lib.MEM_DEVICE, stride=stride, length=plen, peer=d_peer),
+                mtu, d_wl)
+    tx.sync()
+    assert bool((d_wl == wire_len).all())
+    b_enc = lib.make_batch(scratch, nbytes, n, lib.MEM_DEVICE, stride=stride, length=plen, peer=d_peer)
+    b_wire = lib.make_batch(wire, nbytes, n, lib.MEM_DEVICE, stride=stride, length=wire_len)
+    b_out = lib.make_batch(out[16:], nbytes, n, lib.MEM_DEVICE, stride=stride)
+
+    def step():
+        tx.wg_encap(b_enc, mtu, d_wl)
+        rx.wg_decap(b_wire, b_out, d_res, d_olen, d_gp, d_gc)
+
+    for _ in range(args.warmup):
+        step()
+    tx.sync()
+    rx.sync()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    tx.sync()
+    rx.sync()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    assert bool((d_res == 0).all()) and bool((d_olen == plen).all()) and bool((d_gp == d_peer).all())
+    ops = n * ops_aead(plen)
+    tx.close()
+    rx.close()
+    return {
+        "metric": "wg_encap_decap_gbit_per_s", "value": round(n * plen * 8 / (ms * 1e-3) / 1e9, 1),
+        "unit": "Gbit/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u32", "data": "synthetic",
+        "config": {"workload": "transport framing: encapsulate in place + decapsulate %d packets x %d B "
+                               "(wire %d B, slot stride %d), %d peers, device resident"
+                               % (n, plen, wire_len, stride, n_peers), "packets": n},
+        "mpkt_per_s_pair": round(n / (ms * 1e-3) / 1e6, 1),
+        "roofline_valu": {"achieved": round(2 * ops / (ms * 1e-3) / 1e12, 2), "peak": VALU_PEAK_TOPS,
+                          "unit": "Top/s (int32 op-equivalents)",
+                          "frac": round(2 * ops / (ms * 1e-3) / 1e12 / VALU_PEAK_TOPS, 4)},
+    }
+
+
 def bench_copy(args) -> dict:
     """Plain device-to-device copy of 1 GiB: the measured HBM ceiling and the
     known-size launch the FETCH_SIZE / WRITE_SIZE counters are scaled by."""
@@ -293,9 +377,9 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--packets", type=int, default=1 << 20)
-    ap.add_argument("--workload", default="aead", choices=["aead", "filter", "imix", "relay", "copy"],
+    ap.add_argument("--workload", default="aead", choices=["aead", "filter", "imix", "relay", "wg", "copy"],
                     help="aead (default, the headline line, with the ACL filter rate as an extra); "
-                         "filter / imix / relay / copy print one line for that workload alone")
+                         "filter / imix / relay / wg / copy print one line for that workload alone")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample", type=int, default=0,
                     help="packets in the CPU baseline sample (0 = sized for ~10 s)")
@@ -314,7 +398,7 @@ def main() -> int:
         return 2
     if args.workload != "aead":
         out = {"filter": bench_filter, "imix": bench_imix, "relay": bench_relay,
-               "copy": bench_copy}[args.workload](args)
+               "wg": bench_wg, "copy": bench_copy}[args.workload](args)
         print(json.dumps(out))
         return 0
     n = args.packets

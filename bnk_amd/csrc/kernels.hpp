@@ -48,7 +48,7 @@ hipError_t launch_fill_u32(uint32_t *p, uint32_t n, uint32_t v, hipStream_t s);
 // Fused relay bookkeeping (relay_kernels.hip).  After open (auth[i]) and the
 // filter (pass[i]): verdicts, then per-peer batch-order counters for the
 // survivors.  sort_tmp holds sort_tmp_bytes of scratch (relay_sort_tmp_bytes).
-size_t relay_sort_tmp_bytes(uint32_t n);
+size_t relay_sort_tmp_bytes(uint32_t n, uint32_t n_keys);
 hipError_t launch_relay_assign(const uint8_t *auth, const uint8_t *pass, const uint32_t *peer_out,
                                const uint64_t *ctr_base_out, uint32_t n_peers_out, uint32_t n,
                                uint32_t *keys, uint32_t *idx, uint32_t *skeys, uint32_t *sidx,
@@ -56,12 +56,13 @@ hipError_t launch_relay_assign(const uint8_t *auth, const uint8_t *pass, const u
                                uint64_t *ctr_out, uint32_t *status, hipStream_t s);
 
 // Batch-order counters per peer: ctr_out[i] = ctr_base[keys[i]] + (number of
-// earlier i' with the same key), for keys[i] != 0xFFFFFFFF.  keys/idx are
+// earlier i' with the same key), for keys[i] < n_keys; other keys must be
+// 0xFFFFFFFF.  keys/idx are
 // inputs (idx[i] = i), skeys/sidx and sort_tmp scratch.  With advance set,
 // ctr_base[key] moves past the counters handed out.
 hipError_t launch_peer_rank(uint32_t *keys, uint32_t *idx, uint32_t *skeys, uint32_t *sidx,
-                            void *sort_tmp, size_t sort_tmp_bytes, uint64_t *ctr_base, uint32_t n,
-                            uint64_t *ctr_out, bool advance, hipStream_t s);
+                            void *sort_tmp, size_t sort_tmp_bytes, uint64_t *ctr_base, uint32_t n_keys,
+                            uint32_t n, uint64_t *ctr_out, bool advance, hipStream_t s);
 
 // VALU throughput probe; out receives one word per thread so nothing is
 // optimised away.

@@ -95,7 +95,7 @@ extern "C" int bnk_relay_fused_batch(bnk_ctx *ctx, const bnk_batch *in, const ui
     HIPCHK(ctx, ctx->r_pass.reserve(n));
     for (DevBuf *b : {&ctx->r_keys, &ctx->r_idx, &ctx->r_skeys, &ctx->r_sidx})
         HIPCHK(ctx, b->reserve((size_t)n * 4));
-    const size_t tmp_bytes = relay_sort_tmp_bytes(n);
+    const size_t tmp_bytes = relay_sort_tmp_bytes(n, n_peers_out);
     HIPCHK(ctx, ctx->r_tmp.reserve(tmp_bytes + 16));
 
     // ---- 1. open into the plaintext scratch (same offsets as the input) ----

@@ -70,11 +70,21 @@ __global__ __launch_bounds__(256) void peer_advance_kernel(const uint32_t *skeys
     ctr_base[key] = ctr_out[sidx[p]] + 1u;
 }
 
-size_t relay_sort_tmp_bytes(uint32_t n)
+// Peer keys are below n_keys and the "no peer" key is all ones, so the low
+// bit_width(n_keys) bits order them the same way the full word does.
+static unsigned key_bits(uint32_t n_keys)
+{
+    unsigned bits = 1;
+    while (bits < 32 && (n_keys >> bits) != 0) bits++;
+    return bits;
+}
+
+size_t relay_sort_tmp_bytes(uint32_t n, uint32_t n_keys)
 {
     size_t bytes = 0;
     (void)rocprim::radix_sort_pairs(nullptr, bytes, (const uint32_t *)nullptr, (uint32_t *)nullptr,
-                                    (const uint32_t *)nullptr, (uint32_t *)nullptr, (size_t)n);
+                                    (const uint32_t *)nullptr, (uint32_t *)nullptr, (size_t)n, 0,
+                                    key_bits(n_keys));
     return bytes;
 }
 
@@ -89,17 +99,17 @@ hipError_t launch_relay_assign(const uint8_t *auth, const uint8_t *pass, const u
     hipLaunchKernelGGL(relay_verdict_kernel, grid, dim3(256), 0, s, auth, pass, peer_out, n_peers_out,
                        n, keys, idx, verdict, ctr_out, status);
     return launch_peer_rank(keys, idx, skeys, sidx, sort_tmp, sort_tmp_bytes,
-                            const_cast<uint64_t *>(ctr_base_out), n, ctr_out, false, s);
+                            const_cast<uint64_t *>(ctr_base_out), n_peers_out, n, ctr_out, false, s);
 }
 
 hipError_t launch_peer_rank(uint32_t *keys, uint32_t *idx, uint32_t *skeys, uint32_t *sidx,
-                            void *sort_tmp, size_t sort_tmp_bytes, uint64_t *ctr_base, uint32_t n,
-                            uint64_t *ctr_out, bool advance, hipStream_t s)
+                            void *sort_tmp, size_t sort_tmp_bytes, uint64_t *ctr_base, uint32_t n_keys,
+                            uint32_t n, uint64_t *ctr_out, bool advance, hipStream_t s)
 {
     if (n == 0) return hipSuccess;
     const dim3 grid((n + 255u) / 256u);
     hipError_t e = rocprim::radix_sort_pairs(sort_tmp, sort_tmp_bytes, keys, skeys, idx, sidx, (size_t)n,
-                                             0, 32, s);
+                                             0, key_bits(n_keys), s);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(relay_rank_kernel, grid, dim3(256), 0, s, skeys, sidx, ctr_base, n, ctr_out);
     if (advance)

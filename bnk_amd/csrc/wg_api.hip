@@ -151,7 +151,7 @@ extern "C" int bnk_wg_encap_batch(bnk_ctx *ctx, const bnk_batch *slots, uint32_t
         HIPCHK(ctx, buf->reserve((size_t)n * 4));
     HIPCHK(ctx, ctx->r_ctr_out.reserve((size_t)n * 8));
     HIPCHK(ctx, ctx->wg_skip.reserve(n));
-    const size_t tmp_bytes = relay_sort_tmp_bytes(n);
+    const size_t tmp_bytes = relay_sort_tmp_bytes(n, ctx->n_wg_peers);
     HIPCHK(ctx, ctx->r_tmp.reserve(tmp_bytes + 16));
     const WgPeersDev pe = peers_view(ctx);
     uint64_t *d_ctr = ctx->r_ctr_out.as<uint64_t>();
@@ -163,7 +163,7 @@ extern "C" int bnk_wg_encap_batch(bnk_ctx *ctx, const bnk_batch *slots, uint32_t
                                ctx->d_status, ctx->stream));
     HIPCHK(ctx, launch_peer_rank(ctx->r_keys.as<uint32_t>(), ctx->r_idx.as<uint32_t>(),
                                  ctx->r_skeys.as<uint32_t>(), ctx->r_sidx.as<uint32_t>(), ctx->r_tmp.p,
-                                 tmp_bytes, pe.send_ctr, n, d_ctr, true, ctx->stream));
+                                 tmp_bytes, pe.send_ctr, pe.n, n, d_ctr, true, ctx->stream));
     HIPCHK(ctx, launch_wg_encap_prep(b, pe, d_peer, d_ctr, mtu, d_padded, d_wire_len, d_skip, ctx->stream));
 
     AeadArgs se{};
@@ -180,8 +180,10 @@ extern "C" int bnk_wg_encap_batch(bnk_ctx *ctx, const bnk_batch *slots, uint32_t
     se.peer = d_peer;
     se.counters = d_ctr;
     se.skip = d_skip;
-    rc = maybe_sort(ctx, se.lens, n, 0, &se.order);
-    if (rc) return rc;
+    if (slots->lens) { // equal plaintext lengths pad to equal lengths
+        rc = maybe_sort(ctx, se.lens, n, 0, &se.order);
+        if (rc) return rc;
+    }
     HIPCHK(ctx, launch_aead_seal(se, ctx->stream));
     if (!host) return BNK_OK;
 
@@ -281,8 +283,10 @@ extern "C" int bnk_wg_decap_batch(bnk_ctx *ctx, const bnk_batch *wire, const bnk
     op.counters = d_counter;
     op.verdict = d_auth;
     op.skip = d_result; // BNK_WG_OK is 0: header failures are not opened
-    rc = maybe_sort(ctx, op.lens, n, 16, &op.order);
-    if (rc) return rc;
+    if (wire->lens) {
+        rc = maybe_sort(ctx, op.lens, n, 16, &op.order);
+        if (rc) return rc;
+    }
     HIPCHK(ctx, launch_aead_open(op, ctx->stream));
     HIPCHK(ctx, launch_wg_finish(ob, 0, pe, d_peer, d_ctlen, d_auth, d_result, d_out_len, ctx->stream));
     if (!host) return BNK_OK;

@@ -326,7 +326,11 @@ def bench_wg(args) -> dict:
 
     def step():
         tx.wg_encap(b_enc, mtu, d_wl)
+        if args.serial:
+            tx.sync()
         rx.wg_decap(b_wire, b_out, d_res, d_olen, d_gp, d_gc)
+        if args.serial:
+            rx.sync()
 
     for _ in range(args.warmup):
         step()
@@ -380,6 +384,9 @@ def main() -> int:
     ap.add_argument("--workload", default="aead", choices=["aead", "filter", "imix", "relay", "wg", "copy"],
                     help="aead (default, the headline line, with the ACL filter rate as an extra); "
                          "filter / imix / relay / wg / copy print one line for that workload alone")
+    ap.add_argument("--serial", action="store_true",
+                    help="wg: wait for the send side before starting the receive side, so a kernel "
+                         "trace shows undisturbed durations (the two sides use separate streams)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample", type=int, default=0,
                     help="packets in the CPU baseline sample (0 = sized for ~10 s)")

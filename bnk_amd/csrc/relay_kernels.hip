@@ -79,10 +79,15 @@ static unsigned key_bits(uint32_t n_keys)
     return bits;
 }
 
+// A few key bits sort faster in one or two Onesweep passes than in the merge
+// sort rocPRIM picks by default for up to 2^20 items.
+using SortConfig = rocprim::radix_sort_config<rocprim::default_config, rocprim::default_config,
+                                              rocprim::default_config, 32768>;
+
 size_t relay_sort_tmp_bytes(uint32_t n, uint32_t n_keys)
 {
     size_t bytes = 0;
-    (void)rocprim::radix_sort_pairs(nullptr, bytes, (const uint32_t *)nullptr, (uint32_t *)nullptr,
+    (void)rocprim::radix_sort_pairs<SortConfig>(nullptr, bytes, (const uint32_t *)nullptr, (uint32_t *)nullptr,
                                     (const uint32_t *)nullptr, (uint32_t *)nullptr, (size_t)n, 0,
                                     key_bits(n_keys));
     return bytes;
@@ -108,7 +113,7 @@ hipError_t launch_peer_rank(uint32_t *keys, uint32_t *idx, uint32_t *skeys, uint
 {
     if (n == 0) return hipSuccess;
     const dim3 grid((n + 255u) / 256u);
-    hipError_t e = rocprim::radix_sort_pairs(sort_tmp, sort_tmp_bytes, keys, skeys, idx, sidx, (size_t)n,
+    hipError_t e = rocprim::radix_sort_pairs<SortConfig>(sort_tmp, sort_tmp_bytes, keys, skeys, idx, sidx, (size_t)n,
                                              0, key_bits(n_keys), s);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(relay_rank_kernel, grid, dim3(256), 0, s, skeys, sidx, ctr_base, n, ctr_out);

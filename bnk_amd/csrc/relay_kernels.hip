@@ -8,6 +8,8 @@
 // first element of its segment.
 #include <string.h>
 
+#include <algorithm>
+
 #include <rocprim/rocprim.hpp>
 
 #include "../../include/bnkhip.h"
@@ -39,7 +41,19 @@ __global__ __launch_bounds__(256) void relay_verdict_kernel(
     ctr_out[i] = 0;
 }
 
+// Where each peer's run starts in the sorted sequence.
+__global__ __launch_bounds__(256) void peer_heads_kernel(const uint32_t *skeys, uint32_t n,
+                                                         uint32_t *seg_start)
+{
+    const uint32_t p = blockIdx.x * 256u + threadIdx.x;
+    if (p >= n) return;
+    const uint32_t key = skeys[p];
+    if (key == NO_PEER) return;
+    if (p == 0u || skeys[p - 1u] != key) seg_start[key] = p;
+}
+
 __global__ __launch_bounds__(256) void relay_rank_kernel(const uint32_t *skeys, const uint32_t *sidx,
+                                                         const uint32_t *seg_start,
                                                          const uint64_t *ctr_base_out, uint32_t n,
                                                          uint64_t *ctr_out)
 {
@@ -47,14 +61,7 @@ __global__ __launch_bounds__(256) void relay_rank_kernel(const uint32_t *skeys, 
     if (p >= n) return;
     const uint32_t key = skeys[p];
     if (key == NO_PEER) return;
-    // first position holding this key
-    uint32_t lo = 0, hi = p;
-    while (lo < hi) {
-        const uint32_t mid = (lo + hi) >> 1;
-        if (skeys[mid] < key) lo = mid + 1;
-        else hi = mid;
-    }
-    ctr_out[sidx[p]] = ctr_base_out[key] + (uint64_t)(p - lo);
+    ctr_out[sidx[p]] = ctr_base_out[key] + (uint64_t)(p - seg_start[key]);
 }
 
 // The last element of each peer's segment holds the largest counter handed out.
@@ -90,7 +97,8 @@ size_t relay_sort_tmp_bytes(uint32_t n, uint32_t n_keys)
     (void)rocprim::radix_sort_pairs<SortConfig>(nullptr, bytes, (const uint32_t *)nullptr, (uint32_t *)nullptr,
                                     (const uint32_t *)nullptr, (uint32_t *)nullptr, (size_t)n, 0,
                                     key_bits(n_keys));
-    return bytes;
+    // once the sort is done the same scratch holds one run start per key
+    return std::max(bytes, (size_t)n_keys * 4);
 }
 
 hipError_t launch_relay_assign(const uint8_t *auth, const uint8_t *pass, const uint32_t *peer_out,
@@ -116,7 +124,9 @@ hipError_t launch_peer_rank(uint32_t *keys, uint32_t *idx, uint32_t *skeys, uint
     hipError_t e = rocprim::radix_sort_pairs<SortConfig>(sort_tmp, sort_tmp_bytes, keys, skeys, idx, sidx, (size_t)n,
                                              0, key_bits(n_keys), s);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(relay_rank_kernel, grid, dim3(256), 0, s, skeys, sidx, ctr_base, n, ctr_out);
+    uint32_t *seg_start = static_cast<uint32_t *>(sort_tmp);
+    hipLaunchKernelGGL(peer_heads_kernel, grid, dim3(256), 0, s, skeys, n, seg_start);
+    hipLaunchKernelGGL(relay_rank_kernel, grid, dim3(256), 0, s, skeys, sidx, seg_start, ctr_base, n, ctr_out);
     if (advance)
         hipLaunchKernelGGL(peer_advance_kernel, grid, dim3(256), 0, s, skeys, sidx, ctr_out, n, ctr_base);
     return hipGetLastError();

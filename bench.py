@@ -361,6 +361,52 @@ def bench_wg(args) -> dict:
     }
 
 
+def bench_host(args) -> dict:
+    """Configuration 2 handed over as BNK_MEM_HOST batches in a pinned ring:
+    every call uploads the arena, runs the kernel and downloads the result, so
+    the rate is bound by the host link, not by the kernel."""
+    import numpy as np
+    from bnk_amd import lib, workloads as W
+    n = min(args.packets, 1 << 18)
+    ctx = lib.Context(0)
+    key = W.rand_bytes(W.stream_seed(2, 0), 32).reshape(1, 32)
+    ctx.keys_set(lib.KEYS_SEND, key)
+    ctx.keys_set(lib.KEYS_RECV, key)
+    nbytes = n * STRIDE
+    plain, sealed, opened = (ctx.ring_alloc(nbytes) for _ in range(3))
+    plain.reshape(n, STRIDE)[:, :L] = W.rand_bytes(W.stream_seed(2, 1), n * L).reshape(n, L)
+    verdict = np.zeros(n, np.uint8)
+    b_plain = lib.make_batch(plain, nbytes, n, lib.MEM_HOST, stride=STRIDE, length=L)
+    b_sealed_out = lib.make_batch(sealed, nbytes, n, lib.MEM_HOST, stride=STRIDE)
+    b_sealed_in = lib.make_batch(sealed, nbytes, n, lib.MEM_HOST, stride=STRIDE, length=L + 16)
+    b_opened = lib.make_batch(opened, nbytes, n, lib.MEM_HOST, stride=STRIDE)
+
+    def step():
+        ctx.seal(b_plain, b_sealed_out)
+        ctx.open(b_sealed_in, b_opened, verdict)
+
+    for _ in range(args.warmup):
+        step()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    assert verdict.all() and np.array_equal(opened.reshape(n, STRIDE)[:, :L], plain.reshape(n, STRIDE)[:, :L])
+    for r in (plain, sealed, opened):
+        ctx.ring_free(r)
+    ctx.close()
+    moved = 2 * (n * STRIDE + n * STRIDE)  # per step: arena up and arena down, twice
+    return {
+        "metric": "aead_seal_open_gbit_per_s_1420B_host_memory", "value": round(n * L * 8 / (ms * 1e-3) / 1e9, 1),
+        "unit": "Gbit/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u32", "data": "synthetic",
+        "config": {"workload": "cfg2 through BNK_MEM_HOST: seal+open of %d packets x %d B from pinned host "
+                               "rings, upload and download inside every call" % (n, L), "packets": n},
+        "host_link_gb_per_s": round(moved / (ms * 1e-3) / 1e9, 1),
+    }
+
+
 def bench_copy(args) -> dict:
     """Plain device-to-device copy of 1 GiB: the measured HBM ceiling and the
     known-size launch the FETCH_SIZE / WRITE_SIZE counters are scaled by."""
@@ -381,9 +427,9 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--packets", type=int, default=1 << 20)
-    ap.add_argument("--workload", default="aead", choices=["aead", "filter", "imix", "relay", "wg", "copy"],
+    ap.add_argument("--workload", default="aead", choices=["aead", "filter", "imix", "relay", "wg", "host", "copy"],
                     help="aead (default, the headline line, with the ACL filter rate as an extra); "
-                         "filter / imix / relay / wg / copy print one line for that workload alone")
+                         "filter / imix / relay / wg / host / copy print one line for that workload alone")
     ap.add_argument("--serial", action="store_true",
                     help="wg: wait for the send side before starting the receive side, so a kernel "
                          "trace shows undisturbed durations (the two sides use separate streams)")
@@ -405,7 +451,7 @@ def main() -> int:
         return 2
     if args.workload != "aead":
         out = {"filter": bench_filter, "imix": bench_imix, "relay": bench_relay,
-               "wg": bench_wg, "copy": bench_copy}[args.workload](args)
+               "wg": bench_wg, "host": bench_host, "copy": bench_copy}[args.workload](args)
         print(json.dumps(out))
         return 0
     n = args.packets

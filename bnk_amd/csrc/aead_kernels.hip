@@ -236,39 +236,45 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
     }
     maxsteps = __builtin_amdgcn_readfirstlane(maxsteps);
 
+    // Lines m_lo <= m < m_hi lie wholly inside every packet of the wave: those
+    // move without per-cell bounds checks.
+    uint32_t maxc0 = c0, minend = c0 + ncell;
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        const uint32_t a = (uint32_t)__shfl_xor((int)maxc0, off, 64);
+        const uint32_t b = (uint32_t)__shfl_xor((int)minend, off, 64);
+        maxc0 = a > maxc0 ? a : maxc0;
+        minend = b < minend ? b : minend;
+    }
+    const uint32_t m_lo = __builtin_amdgcn_readfirstlane(maxc0) ? 1u : 0u;
+    const uint32_t m_hi = __builtin_amdgcn_readfirstlane(minend) >> 3;
+
     // Lines are fetched one iteration ahead into registers (issue), so the
     // loads fly while the wave computes, and only then moved into the ring
     // (commit), which overwrites the half whose line was written back last.
     uint4 pre0 = make_uint4(0, 0, 0, 0), pre1 = pre0, pre2 = pre0, pre3 = pre0, pre4 = pre0,
           pre5 = pre0, pre6 = pre0, pre7 = pre0;
-#define BNK_ISSUE(q, m)                                                                     \
-    if (8u * (m) + sub >= cfirst[q] && 8u * (m) + sub < cend[q])                            \
-        pre##q = ld16a(csrc[q] + 128u * (m))
-#define BNK_COMMIT(q, m)                                                                    \
-    if (8u * (m) + sub >= cfirst[q] && 8u * (m) + sub < cend[q])                            \
-        *reinterpret_cast<uint4 *>(tile + (8u * q + (lane >> 3)) * RING_ROW +               \
-                                   (((8u * (m) + sub) & 15u) << 4)) = pre##q
-#define BNK_ISSUE_LINE(m)                                                                   \
+    uint8_t *mycell = tile + (lane >> 3) * RING_ROW;
+#define BNK_INSIDE(q, m) (8u * (m) + sub >= cfirst[q] && 8u * (m) + sub < cend[q])
+#define BNK_SLOT(q, m) reinterpret_cast<uint4 *>(mycell + 8u * q * RING_ROW + (((8u * (m) + sub) & 15u) << 4))
+#define BNK_ISSUE(q, m) if (BNK_INSIDE(q, m)) pre##q = ld16a(csrc[q] + 128u * (m))
+#define BNK_ISSUE_ALL(q, m) pre##q = ld16a(csrc[q] + 128u * (m))
+#define BNK_COMMIT(q, m) if (BNK_INSIDE(q, m)) *BNK_SLOT(q, m) = pre##q
+#define BNK_COMMIT_ALL(q, m) *BNK_SLOT(q, m) = pre##q
+#define BNK_STORE(q, m) if (BNK_INSIDE(q, m)) st16a(cdst[q] + 128u * (m), *BNK_SLOT(q, m))
+#define BNK_STORE_ALL(q, m) st16a(cdst[q] + 128u * (m), *BNK_SLOT(q, m))
+#define BNK_EIGHT(OP, m)                                                                    \
     do {                                                                                    \
-        BNK_ISSUE(0, m); BNK_ISSUE(1, m); BNK_ISSUE(2, m); BNK_ISSUE(3, m);                 \
-        BNK_ISSUE(4, m); BNK_ISSUE(5, m); BNK_ISSUE(6, m); BNK_ISSUE(7, m);                 \
+        OP(0, m); OP(1, m); OP(2, m); OP(3, m); OP(4, m); OP(5, m); OP(6, m); OP(7, m);     \
     } while (0)
-#define BNK_COMMIT_LINE(m)                                                                  \
+#define BNK_LINE(OP, m)                                                                     \
     do {                                                                                    \
-        BNK_COMMIT(0, m); BNK_COMMIT(1, m); BNK_COMMIT(2, m); BNK_COMMIT(3, m);             \
-        BNK_COMMIT(4, m); BNK_COMMIT(5, m); BNK_COMMIT(6, m); BNK_COMMIT(7, m);             \
+        if ((m) >= m_lo && (m) < m_hi) BNK_EIGHT(OP##_ALL, m);                              \
+        else BNK_EIGHT(OP, m);                                                              \
     } while (0)
-    auto store_line = [&](uint32_t m) __attribute__((always_inline)) {
-        const uint32_t K = 8u * m + sub;
-#pragma unroll
-        for (int q = 0; q < 8; q++) {
-            if (K >= cfirst[q] && K < cend[q]) {
-                const uint4 v = *reinterpret_cast<const uint4 *>(
-                    tile + (8u * q + (lane >> 3)) * RING_ROW + ((K & 15u) << 4));
-                st16a(cdst[q] + 128u * m, v);
-            }
-        }
-    };
+#define BNK_ISSUE_LINE(m) BNK_LINE(BNK_ISSUE, m)
+#define BNK_COMMIT_LINE(m) BNK_LINE(BNK_COMMIT, m)
+    auto store_line = [&](uint32_t m) __attribute__((always_inline)) { BNK_LINE(BNK_STORE, m); };
 
     uint8_t *row = tile + lane * RING_ROW;
     BNK_ISSUE_LINE(0u);
@@ -312,8 +318,16 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
         store_line(s);
         wave_sync();
     }
+#undef BNK_INSIDE
+#undef BNK_SLOT
 #undef BNK_ISSUE
+#undef BNK_ISSUE_ALL
 #undef BNK_COMMIT
+#undef BNK_COMMIT_ALL
+#undef BNK_STORE
+#undef BNK_STORE_ALL
+#undef BNK_EIGHT
+#undef BNK_LINE
 #undef BNK_ISSUE_LINE
 #undef BNK_COMMIT_LINE
 }

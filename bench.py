@@ -99,7 +99,9 @@ def bench_filter(args) -> dict:
                    "packets": n, "rules": 4096, "allowed_fraction": round(allowed, 4)},
         "roofline": {"bound": "hbm", "kernel": "filter_check_kernel", "achieved": round(gbs, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
-                     "traffic": None, "bytes_per_launch": alg_bytes,
+                     # FETCH_SIZE x2 + WRITE_SIZE under rocprofv3 --pmc for this launch
+                     # (profiles/filter_check_kernel_cfg4.md); not re-measured by this run
+                     "traffic": 232.8e6 if n == 1 << 22 else None, "bytes_per_launch": alg_bytes,
                      "avg_launch_ms": round(kern_ms, 4)},
     }
     if not args.no_cpu_baseline:
@@ -544,7 +546,9 @@ def main() -> int:
             "bound": "hbm", "kernel": "aead_wave_kernel",
             "achieved": round(achieved_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": round(achieved_gbs / HBM_PEAK_GBS, 4),
-            "traffic": None,
+            # FETCH_SIZE x2 + WRITE_SIZE under rocprofv3 --pmc, mean of the seal and the open
+            # launch (profiles/aead_wave_kernel_cfg2.md); not re-measured by this run
+            "traffic": 3.214e9 if n == 1 << 20 else None,
             "bytes_per_launch": alg_bytes, "avg_launch_ms": round(kern_ms, 4),
         },
         "roofline_valu": {

@@ -18,3 +18,14 @@ def test_cpp_host_mirror_suite():
     print(r.stdout, r.stderr)
     assert r.returncode == 0, r.stdout + r.stderr
     assert "PASS all host-mirror tests" in r.stdout
+
+
+def test_cpp_tunnel_over_loopback():
+    """encapsulate -> sendmmsg from the pinned ring -> recvmmsg into a pinned
+    ring -> decapsulate -> replay window (tests/cpp/tunnel_test.cpp)."""
+    exe = os.path.join(HERE, "cpp", "tunnel_test")
+    assert os.path.exists(exe), "build it first: make -C tests/cpp (or __graft_entry__.build())"
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    print(r.stdout, r.stderr)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "PASS tunnel over loopback" in r.stdout

@@ -25,6 +25,7 @@
 #include <vector>
 
 #include "../../include/bnkhip.h"
+#include "bnk_coalesce.hpp"
 
 namespace bnk_host {
 
@@ -104,9 +105,17 @@ inline int64_t UnixNano(std::chrono::system_clock::time_point t)
     return std::chrono::duration_cast<std::chrono::nanoseconds>(t.time_since_epoch()).count();
 }
 
+// What the TUN wrapper needs from a filter: one verdict per packet of a batch,
+// and the outbound packets of a batch recorded.
+struct PacketFilter {
+    virtual ~PacketFilter() = default;
+    virtual std::vector<uint8_t> CheckInboundBatch(const std::vector<ByteSlice> &pkts, int64_t now_ns) = 0;
+    virtual void NoteOutboundBatch(const std::vector<ByteSlice> &pkts, int64_t now_ns) = 0;
+};
+
 // filter.Filter.  One GPU context per filter; calls are serialised inside the
 // library as the reference serialises them with its mutex (filter.go:34).
-class Filter {
+class Filter : public PacketFilter {
 public:
     // filter.New: allow-all until a policy arrives.
     explicit Filter(int device = 0)
@@ -141,7 +150,7 @@ public:
         check(bnk_filter_note_outbound_ptrs(ctx_, &p, &len, 1, now_ns));
     }
     // One verdict per packet with one `now`, as filteredTUN.Write needs.
-    std::vector<uint8_t> CheckInboundBatch(const std::vector<ByteSlice> &pkts, int64_t now_ns)
+    std::vector<uint8_t> CheckInboundBatch(const std::vector<ByteSlice> &pkts, int64_t now_ns) override
     {
         std::vector<const uint8_t *> ptrs(pkts.size());
         std::vector<uint32_t> lens(pkts.size());
@@ -154,7 +163,7 @@ public:
                                             now_ns, v.data()));
         return v;
     }
-    void NoteOutboundBatch(const std::vector<ByteSlice> &pkts, int64_t now_ns)
+    void NoteOutboundBatch(const std::vector<ByteSlice> &pkts, int64_t now_ns) override
     {
         std::vector<const uint8_t *> ptrs(pkts.size());
         std::vector<uint32_t> lens(pkts.size());
@@ -181,6 +190,83 @@ private:
     bnk_ctx *ctx_ = nullptr;
 };
 
+// A Filter behind a BatchCoalescer: calls from many threads (one per peer in
+// wireguard-go) that arrive within max_wait of each other become one GPU
+// batch.  The `now_ns` arguments are ignored: a merged batch takes the clock
+// when it is flushed.
+class CoalescedFilter : public PacketFilter {
+public:
+    CoalescedFilter(Filter *f, size_t max_packets = 8192,
+                    std::chrono::microseconds max_wait = std::chrono::microseconds(200))
+        : f_(f), co_([this](const uint8_t *const *ptrs, const uint32_t *lens, const uint8_t *note,
+                            uint32_t n, int64_t now, uint8_t *verdict) { Run(ptrs, lens, note, n, now, verdict); },
+                     max_packets, max_wait)
+    {
+    }
+    bool CheckInbound(ByteSlice pkt)
+    {
+        const uint8_t *p = pkt.data;
+        const uint32_t len = (uint32_t)pkt.len;
+        uint8_t v = 0;
+        co_.Submit(&p, &len, 1, false, &v);
+        return v != 0;
+    }
+    void NoteOutbound(ByteSlice pkt)
+    {
+        const uint8_t *p = pkt.data;
+        const uint32_t len = (uint32_t)pkt.len;
+        co_.Submit(&p, &len, 1, true, nullptr);
+    }
+    std::vector<uint8_t> CheckInboundBatch(const std::vector<ByteSlice> &pkts, int64_t) override
+    {
+        std::vector<const uint8_t *> ptrs(pkts.size());
+        std::vector<uint32_t> lens(pkts.size());
+        for (size_t i = 0; i < pkts.size(); i++) {
+            ptrs[i] = pkts[i].data;
+            lens[i] = (uint32_t)pkts[i].len;
+        }
+        std::vector<uint8_t> v(pkts.size());
+        co_.Submit(ptrs.data(), lens.data(), (uint32_t)pkts.size(), false, v.data());
+        return v;
+    }
+    void NoteOutboundBatch(const std::vector<ByteSlice> &pkts, int64_t) override
+    {
+        std::vector<const uint8_t *> ptrs(pkts.size());
+        std::vector<uint32_t> lens(pkts.size());
+        for (size_t i = 0; i < pkts.size(); i++) {
+            ptrs[i] = pkts[i].data;
+            lens[i] = (uint32_t)pkts[i].len;
+        }
+        co_.Submit(ptrs.data(), lens.data(), (uint32_t)pkts.size(), true, nullptr);
+    }
+    CoalesceStats Stats() { return co_.Stats(); }
+
+private:
+    // notes first, then checks, each as one call
+    void Run(const uint8_t *const *ptrs, const uint32_t *lens, const uint8_t *note, uint32_t n,
+             int64_t now, uint8_t *verdict)
+    {
+        std::vector<const uint8_t *> p[2];
+        std::vector<uint32_t> l[2], where;
+        for (uint32_t i = 0; i < n; i++) {
+            p[note[i] ? 1 : 0].push_back(ptrs[i]);
+            l[note[i] ? 1 : 0].push_back(lens[i]);
+            if (!note[i]) where.push_back(i);
+        }
+        bnk_ctx *ctx = f_->ctx();
+        if (!p[1].empty() &&
+            bnk_filter_note_outbound_ptrs(ctx, p[1].data(), l[1].data(), (uint32_t)p[1].size(), now))
+            throw std::runtime_error(std::string("libbnkhip: ") + bnk_last_error(ctx));
+        if (p[0].empty()) return;
+        std::vector<uint8_t> v(p[0].size());
+        if (bnk_filter_check_inbound_ptrs(ctx, p[0].data(), l[0].data(), (uint32_t)p[0].size(), now, v.data()))
+            throw std::runtime_error(std::string("libbnkhip: ") + bnk_last_error(ctx));
+        for (size_t k = 0; k < where.size(); k++) verdict[where[k]] = v[k];
+    }
+    Filter *f_;
+    BatchCoalescer co_;
+};
+
 namespace tun {
 
 enum Event { EventUp = 1, EventDown = 2, EventMTUUpdate = 4 };
@@ -204,7 +290,7 @@ struct Device {
 // filteredTUN (filter.go:155-186).
 class FilteredTUN : public tun::Device {
 public:
-    FilteredTUN(tun::Device *inner, Filter *f) : inner_(inner), f_(f) {}
+    FilteredTUN(tun::Device *inner, PacketFilter *f) : inner_(inner), f_(f) {}
 
     // filter.go:160-167
     std::pair<int, Error> Read(std::vector<ByteSlice> &bufs, std::vector<int> &sizes, int offset) override
@@ -246,11 +332,11 @@ public:
 
 private:
     tun::Device *inner_;
-    Filter *f_;
+    PacketFilter *f_;
 };
 
 // filter.WrapTUN (filter.go:151-153)
-inline std::unique_ptr<tun::Device> WrapTUN(tun::Device *inner, Filter *f)
+inline std::unique_ptr<tun::Device> WrapTUN(tun::Device *inner, PacketFilter *f)
 {
     return std::unique_ptr<tun::Device>(new FilteredTUN(inner, f));
 }

@@ -4,6 +4,9 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <atomic>
+#include <thread>
+
 #include "../../bnk_amd/host/bnk_host.hpp"
 
 using namespace bnk_host;
@@ -226,6 +229,53 @@ static void TestWrapTUNReadRecordsOutboundFlows()
            "other Device methods pass through");
 }
 
+// Per-peer writers in parallel, as wireguard-go calls filteredTUN.Write: each
+// thread's own packets get their own verdicts, the same as a direct filter
+// gives, while the GPU sees merged batches.
+static void TestCoalescedWritesFromManyThreads()
+{
+    Filter f; sshOnly(f);
+    note(f, udp(self, peer, 40000, 9999), UnixNano(std::chrono::system_clock::now()));
+    CoalescedFilter cf(&f, 4096, std::chrono::microseconds(500));
+    constexpr int T = 16, ROUNDS = 25;
+    std::atomic<int> wrong{0}, delivered{0};
+    std::vector<std::thread> th;
+    for (int t = 0; t < T; t++)
+        th.emplace_back([&, t] {
+            fakeTUN inner;
+            auto wrapped = WrapTUN(&inner, &cf);
+            for (int r = 0; r < ROUNDS; r++) {
+                // ssh (rule), a reply to the noted flow, and two packets nothing admits
+                std::vector<Bytes> pk{pad(tcp(peer, self, (uint16_t)(1000 + t), 22, true), 16),
+                                      pad(tcp(peer, self, (uint16_t)(1000 + t), 23, true), 16),
+                                      pad(udp(peer, self, 9999, 40000), 16),
+                                      pad(udp(peer, self, 9999, (uint16_t)(40001 + r)), 16)};
+                std::vector<ByteSlice> bufs;
+                for (Bytes &b : pk) bufs.push_back(ByteSlice(b));
+                const size_t before = inner.written.size();
+                auto res = wrapped->Write(bufs, 16);
+                if (res.first != 4 || !res.second.empty()) wrong++;
+                if (inner.written.size() != before + 2) wrong++;
+                else {
+                    if (inner.written[before][9] != 6 || inner.written[before + 1][9] != 17) wrong++;
+                    delivered += 2;
+                }
+            }
+        });
+    for (auto &x : th) x.join();
+    EXPECT(wrong == 0, "coalesced verdicts differ from the direct filter's");
+    EXPECT(delivered == T * ROUNDS * 2, "two of four packets pass in every write");
+    const CoalesceStats st = cf.Stats();
+    EXPECT(st.calls == (uint64_t)T * ROUNDS && st.batches < st.calls, "writes were merged into fewer launches");
+    printf("coalescer: %llu writes -> %llu batches, largest %llu packets\n", (unsigned long long)st.calls,
+           (unsigned long long)st.batches, (unsigned long long)st.largest_batch);
+    // outbound notes go through the same window and are seen by later checks
+    Bytes query = udp(self, peer, 41000, 53);
+    cf.NoteOutbound(ByteSlice(query));
+    Bytes reply = udp(peer, self, 53, 41000);
+    EXPECT(cf.CheckInbound(ByteSlice(reply)), "reply to a coalesced note must pass");
+}
+
 int main()
 {
     try {
@@ -240,6 +290,7 @@ int main()
         TestSetAllowAllDisablesEnforcement();
         TestWrapTUNDropsDeniedInboundWrites();
         TestWrapTUNReadRecordsOutboundFlows();
+        TestCoalescedWritesFromManyThreads();
     } catch (const std::exception &e) {
         printf("FAIL exception: %s\n", e.what());
         return 2;

@@ -12,3 +12,13 @@ def test_ring_bind_over_loopback():
     r = subprocess.run([os.path.join(HERE, "cpp", "bind_test")], capture_output=True, text=True,
                        timeout=120)
     assert r.returncode == 0, r.stdout + r.stderr
+
+
+def test_batch_coalescer_with_a_stand_in_executor():
+    """bnk_amd/host/bnk_coalesce.hpp: callers get their own verdicts, windows
+    fill and flush, a lone caller waits at most the window, failures reach
+    every caller (tests/cpp/coalesce_test.cpp)."""
+    subprocess.run(["make", "-s", "-C", os.path.join(HERE, "cpp"), "coalesce_test"], check=True)
+    r = subprocess.run([os.path.join(HERE, "cpp", "coalesce_test")], capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode == 0, r.stdout + r.stderr

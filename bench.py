@@ -593,6 +593,26 @@ def main() -> int:
                       "cannot be built offline (no Go toolchain)" % (sample, threads),
             "gpu_output_matches": same,
         }
+        if O.ossl_available():
+            # the same sample through OpenSSL's assembly implementation, the nearest
+            # stand-in on this box for the assembly the Go reference runs
+            so = np.zeros_like(hb.plain)
+            sv = np.zeros_like(hb.plain)
+            res = {}
+            for nt in (1, threads):
+                tp = time.perf_counter()
+                okc = O.ossl_seal_open_batch(keys, hb.peer, hb.counters, hb.plain, hb.off, hb.lens,
+                                             so, sv, nt)
+                res[nt] = time.perf_counter() - tp
+                assert okc == sample
+            out["cpu_baseline_openssl"] = {
+                "value": round(sample * L * 8 / res[threads] / 1e9, 3), "unit": "Gbit/s",
+                "cores": threads, "one_thread": round(sample * L * 8 / res[1] / 1e9, 3),
+                "kind": "library",
+                "sample": "the same %d packets, EVP_chacha20_poly1305 seal+open, %d pthreads"
+                          % (sample, threads),
+                "matches_oracle": bool(np.array_equal(so, ho)),
+            }
     ctx.close()
     acl = bench_filter(args)
     out["extra"] = {"acl_filter": {k: acl[k] for k in ("metric", "value", "unit", "ms_per_step",

@@ -329,3 +329,19 @@ class ReplayFilter:
     def validate(self, counter: int, limit: int = (1 << 64) - (1 << 13) - 1) -> bool:
         return bool(_lib.bnko_replay_validate(C.c_void_p(self._s.ctypes.data),
                                               C.c_uint64(counter), C.c_uint64(limit)))
+
+
+# ---- OpenSSL as a second CPU baseline ------------------------------------
+
+def ossl_available() -> bool:
+    return bool(_lib.bnko_ossl_available())
+
+
+def ossl_seal_open_batch(keys, peer, counters, inbuf, off, lens, sealed, opened, nthreads: int) -> int:
+    """EVP_chacha20_poly1305 seal then open of every packet; returns how many
+    round trips verified."""
+    _lib.bnko_ossl_seal_open_batch.restype = C.c_uint32
+    return int(_lib.bnko_ossl_seal_open_batch(
+        _p(keys, _u8p), _p(peer, _u32p), _p(counters, _u64p), _p(inbuf, _u8p), _p(off, _u64p),
+        _p(lens, _u32p), _p(sealed, _u8p), _p(opened, _u8p), C.c_uint32(len(lens)),
+        C.c_int(nthreads)))

@@ -239,6 +239,16 @@ void bnko_replay_reset(bnko_replay *f);
 /* 1 = fresh (accept), 0 = replayed, too old, or counter >= limit */
 int bnko_replay_validate(bnko_replay *f, uint64_t counter, uint64_t limit);
 
+/* ---- OpenSSL as a second CPU baseline (openssl_batch.c) ------------------ */
+
+/* 1 when libcrypto could be loaded at run time. */
+int bnko_ossl_available(void);
+/* EVP_chacha20_poly1305 seal into `sealed` then open into `opened`, split over
+ * nthreads; returns the number of packets whose round trip verified. */
+uint32_t bnko_ossl_seal_open_batch(const uint8_t *keys, const uint32_t *peer, const uint64_t *counters,
+                                   const uint8_t *in, const uint64_t *off, const uint32_t *len,
+                                   uint8_t *sealed, uint8_t *opened, uint32_t n, int nthreads);
+
 #ifdef __cplusplus
 }
 #endif

@@ -222,3 +222,22 @@ def test_cfg1_golden_fixture():
     assert hashlib.sha256(sealed.tobytes()).hexdigest() == g["sha256_all_sealed"]
     for idx, hx in g["packets"].items():
         assert sealed[int(idx)].tobytes().hex() == hx
+
+
+def test_openssl_batch_baseline_agrees_with_the_oracle():
+    """The second CPU baseline bench.py reports (oracle/openssl_batch.c) seals
+    to the same bytes as the restatement and opens back to the plaintext."""
+    from bnk_amd import workloads as W
+    if not O.ossl_available():
+        pytest.skip("libcrypto not on this machine")
+    b = W.aead_imix(3, 3000, n_peers=16)
+    keys = np.ascontiguousarray(b.keys)
+    want = np.zeros_like(b.plain)
+    O.seal_batch(keys, b.peer, b.counters, b.plain, b.off, b.lens, want, b.off, 4)
+    sealed = np.zeros_like(b.plain)
+    opened = np.zeros_like(b.plain)
+    assert O.ossl_seal_open_batch(keys, b.peer, b.counters, b.plain, b.off, b.lens, sealed, opened, 3) == b.n
+    assert np.array_equal(sealed, want)
+    for i in (0, 1, b.n - 1):
+        o, l = int(b.off[i]), int(b.lens[i])
+        assert np.array_equal(opened[o:o + l], b.plain[o:o + l])

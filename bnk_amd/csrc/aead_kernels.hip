@@ -349,7 +349,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     uint32_t k[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     uint64_t ctr = 0;
     if (have) {
-        i = a.order ? a.order[t] : t;
+        i = a.first + (a.order ? a.order[t] : t);
         len = a.lens ? a.lens[i] : a.len;
         if (!OPEN) len = len >= a.trim ? len - a.trim : 0u;
         const uint32_t pr = a.peer ? a.peer[i] : 0u;

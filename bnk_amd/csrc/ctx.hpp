@@ -74,6 +74,9 @@ struct bnk_ctx {
     int device = -1;
     hipStream_t stream = nullptr;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    // chunked host batches: upload and download streams, one event pair per chunk
+    hipStream_t s_up = nullptr, s_down = nullptr;
+    std::vector<hipEvent_t> ev_up, ev_done;
     std::string err;
     bool alive = false;
 

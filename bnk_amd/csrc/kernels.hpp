@@ -27,6 +27,7 @@ struct AeadArgs {
     uint32_t n_peers;
     uint32_t trim;             // seal only: lens[i] - trim is the plaintext length
     uint32_t in_skip, out_skip; // bytes between a packet's offset and its AEAD data
+    uint32_t first;            // the launch covers packets first .. first+n-1; order[] is relative to first
 };
 
 enum : uint32_t { STATUS_PEER_RANGE = 1u, STATUS_FLOWS_FULL = 2u };

@@ -111,6 +111,31 @@ def test_edge_lengths_and_high_counters(ctx):
     assert _packets_equal(back, b.plain, b.off, b.lens) == -1
 
 
+@pytest.mark.parametrize("n", [64, 128, 100])
+def test_unsorted_mixed_lengths_within_a_wave(ctx, n):
+    """Up to 64 packets are not grouped by length, so one wave holds long and
+    short packets at once: the lines inside every packet of the wave take the
+    unchecked route, the others the bounds-checked one, and a partly filled
+    wave takes the checked one throughout.  Every alignment class of a
+    128-byte line occurs as the first byte of some packet."""
+    rng = np.random.default_rng(n)
+    lens = rng.integers(130, 1500, n).astype(np.uint32)
+    lens[::7] = rng.choice([128, 129, 255, 256, 257, 1408, 1420, 1499], len(lens[::7]))
+    b = W.aead_imix(13, n, n_peers=3, lens=lens)
+    assert len({int(o) & 127 for o in b.off}) >= 6
+    got = _gpu_seal_host(ctx, b, uniform=False)
+    want = _oracle_seal(b)
+    assert np.array_equal(got, want)
+    W.forge_tags(13, got, b.off, b.lens, 0.1)
+    back, verdict = _gpu_open_host(ctx, b, got, uniform=False)
+    from oracle import binding as O
+    oback = np.full_like(b.plain, 0xEE)
+    overdict = O.open_batch(np.ascontiguousarray(b.keys), b.peer, b.counters, got, b.off,
+                            (b.lens + 16).astype(np.uint32), oback, b.off, 2)
+    assert np.array_equal(verdict, overdict) and 0 < int((verdict == 0).sum()) < n
+    assert np.array_equal(back, oback)
+
+
 def test_imix_multi_peer_with_forged_tags(ctx):
     from oracle import binding as O
     b = W.aead_imix(3, 6000, n_peers=256)
@@ -129,6 +154,65 @@ def test_imix_multi_peer_with_forged_tags(ctx):
     i = int(np.flatnonzero(forged)[0])
     o, L = int(b.off[i]), int(b.lens[i])
     assert not back[o:o + L].any()
+
+
+@pytest.mark.parametrize("layout", ["offsets", "reversed", "in_place", "uniform"])
+def test_large_host_batches_take_the_chunked_route(ctx, layout):
+    """Host batches of several chunks' worth are uploaded, computed and
+    downloaded chunk by chunk with the three overlapped; a layout whose packets
+    do not ascend through the arena takes the single-shot route.  Either way:
+    oracle-exact bytes, verdicts, zero-filled rejects and untouched gaps."""
+    from bnk_amd import lib
+    from oracle import binding as O
+    if layout == "uniform":
+        n, L, stride = 20000, 1420, 1472
+        b = W.aead_uniform(14, n, L, stride=stride, counter0=1 << 33)
+    else:
+        n = 40000
+        b = W.aead_imix(14, n, n_peers=64)
+    assert b.plain.nbytes > 3 * (4 << 20)
+    off = b.off
+    peer, counters, lens = b.peer, b.counters, b.lens
+    if layout == "reversed":
+        perm = np.arange(n)[::-1].copy()
+        off, peer, counters, lens = off[perm].copy(), peer[perm].copy(), counters[perm].copy(), lens[perm].copy()
+    keys = np.ascontiguousarray(b.keys)
+    ctx.keys_set(lib.KEYS_SEND, keys)
+    ctx.keys_set(lib.KEYS_RECV, keys)
+    want = np.full_like(b.plain, 0x5A)
+    O.seal_batch(keys, peer, counters, b.plain, off, lens, want, off, 4)
+    ct_lens = (lens + 16).astype(np.uint32)
+
+    def batch(buf, ln, with_meta=True):
+        if layout == "uniform":
+            return lib.make_batch(buf, buf.nbytes, n, lib.MEM_HOST, stride=b.stride,
+                                  length=int(ln[0]) if with_meta else 0, counter0=1 << 33)
+        return lib.make_batch(buf, buf.nbytes, n, lib.MEM_HOST, offsets=off,
+                              lens=ln if with_meta else None, peer=peer if with_meta else None,
+                              counters=counters if with_meta else None)
+
+    if layout == "in_place":
+        got = b.plain.copy()
+        ctx.seal(batch(got, lens), batch(got, lens, False))
+        # only the packets and their tags changed
+        assert _packets_equal(got, want, off, lens, 16) == -1
+        mask = np.ones(got.size, bool)
+        for o, l in zip(off.astype(np.int64), lens.astype(np.int64)):
+            mask[o:o + l + 16] = False
+        assert np.array_equal(got[mask], b.plain[mask])
+    else:
+        got = np.full_like(b.plain, 0x5A)
+        ctx.seal(batch(b.plain, lens), batch(got, lens, False))
+        assert np.array_equal(got, want)  # the 0x5A between packets survived
+    forged = W.forge_tags(14, got, off, lens, 0.02)
+    back = np.full_like(b.plain, 0xEE)
+    verdict = np.full(n, 7, np.uint8)
+    ctx.open(batch(got, ct_lens), batch(back, lens, False), verdict)
+    oback = np.full_like(b.plain, 0xEE)
+    overdict = O.open_batch(keys, peer, counters, got, off, ct_lens, oback, off, 4)
+    assert np.array_equal(verdict, overdict)
+    assert np.array_equal(verdict == 0, forged) and forged.sum() == int(0.02 * n)
+    assert np.array_equal(back, oback)
 
 
 def test_in_place_and_unaligned_slots(ctx):

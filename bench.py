@@ -16,6 +16,7 @@ from __future__ import annotations
 import argparse
 import json
 import os
+import shutil
 import sys
 import time
 
@@ -592,6 +593,10 @@ def main() -> int:
                       "restatement of RFC 8439 (oracle/aead.c), %d pthreads; the Go reference "
                       "cannot be built offline (no Go toolchain)" % (sample, threads),
             "gpu_output_matches": same,
+            # the reference's own Go path (x/crypto via wireguard-go) would be timed here with
+            # GOMAXPROCS stated; it needs a Go toolchain and the module cache on this box
+            "go_toolchain_on_box": shutil.which("go") is not None,
+            "host_cpus": os.cpu_count(),
         }
         if O.ossl_available():
             # the same sample through OpenSSL's assembly implementation, the nearest

@@ -148,6 +148,8 @@ BNK_DEV void body_generic(uint8_t *tile, uint32_t lane, const uint8_t *src, uint
                           uint32_t len, const uint32_t (&k)[8], uint32_t n1, uint32_t n2,
                           Poly32 &mac, uint32_t (&x)[16])
 {
+    chacha_block(k, 0, n1, n2, x);
+    mac.init(x);
     const uint32_t nfull = len >> 6, rem = len & 63u;
     const uint32_t steps = nfull + (rem ? 1u : 0u);
     // the four (packet, 16-byte column) cells this lane moves per step
@@ -278,6 +280,9 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
 
     uint8_t *row = tile + lane * RING_ROW;
     BNK_ISSUE_LINE(0u);
+    // keystream block 0 (the Poly1305 key) is computed while the first line flies
+    chacha_block(k, 0, n1, n2, x);
+    mac.init(x);
     BNK_COMMIT_LINE(0u);
     BNK_ISSUE_LINE(1u);
     // iteration s: line s+1 enters the ring, line s+2 starts flying, packet
@@ -381,9 +386,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
     const uint32_t n1 = (uint32_t)ctr, n2 = (uint32_t)(ctr >> 32);
     uint32_t x[16];
-    chacha_block(k, 0, n1, n2, x);
-    Poly32 mac;
-    mac.init(x);
+    Poly32 mac; // keyed from keystream block 0 inside the body, once its first loads are out
 
     const bool lane_lines = (((uintptr_t)src | (uintptr_t)dst) & 15u) == 0 &&
                             (((uintptr_t)src ^ (uintptr_t)dst) & 127u) == 0;
@@ -455,6 +458,36 @@ BNK_DEV uint32_t len_bin(uint32_t len, uint32_t tag_bytes)
     return nb >= LEN_BINS - 1 ? 0u : (LEN_BINS - 1 - nb);
 }
 
+// Adds one to bins[b] for every participating lane and returns what the
+// lane's own atomicAdd would have returned, with one LDS atomic per distinct
+// bin of the wave instead of one per lane: traffic is a handful of sizes, so
+// most lanes of a wave hit the same bin and would serialise on it.  After
+// eight rounds the remaining lanes (a wave with many distinct sizes) go one
+// by one.
+BNK_DEV uint32_t wave_bin_add(uint32_t *bins, uint32_t b, bool active)
+{
+    const uint32_t lane = threadIdx.x & 63u;
+    uint32_t result = 0;
+    bool todo = active;
+    for (int round = 0; round < 8; round++) {
+        const unsigned long long left = __ballot(todo);
+        if (left == 0ull) return result;
+        const int leader = __ffsll((long long)left) - 1;
+        const uint32_t lb = (uint32_t)__shfl((int)b, leader, 64);
+        const bool mine = todo && b == lb;
+        const unsigned long long same = __ballot(mine);
+        uint32_t old = 0;
+        if ((int)lane == leader) old = atomicAdd(&bins[lb], (uint32_t)__popcll(same));
+        old = (uint32_t)__shfl((int)old, leader, 64);
+        if (mine) {
+            result = old + (uint32_t)__popcll(same & ((1ull << lane) - 1ull));
+            todo = false;
+        }
+    }
+    if (todo) result = atomicAdd(&bins[b], 1u);
+    return result;
+}
+
 __global__ __launch_bounds__(256) void len_hist_kernel(const uint32_t *lens, uint32_t n,
                                                        uint32_t tag_bytes, uint32_t *hist)
 {
@@ -462,8 +495,12 @@ __global__ __launch_bounds__(256) void len_hist_kernel(const uint32_t *lens, uin
     for (uint32_t b = threadIdx.x; b < LEN_BINS; b += 256) lh[b] = 0;
     __syncthreads();
     const uint32_t stride = gridDim.x * 256u;
-    for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < n; i += stride)
-        atomicAdd(&lh[len_bin(lens[i], tag_bytes)], 1u);
+    // whole waves stay in the loop together (the helper uses wave-wide votes)
+    for (uint32_t i0 = blockIdx.x * 256u; i0 < n; i0 += stride) {
+        const uint32_t i = i0 + threadIdx.x;
+        const bool in = i < n;
+        (void)wave_bin_add(lh, in ? len_bin(lens[i], tag_bytes) : 0u, in);
+    }
     __syncthreads();
     for (uint32_t b = threadIdx.x; b < LEN_BINS; b += 256)
         if (lh[b]) atomicAdd(&hist[b], lh[b]);
@@ -512,8 +549,11 @@ __global__ __launch_bounds__(256) void len_scatter_kernel(const uint32_t *lens, 
     __syncthreads();
     const uint32_t stride = gridDim.x * 256u;
     // every block walks its strided share twice: count, reserve, place
-    for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < n; i += stride)
-        atomicAdd(&cnt[len_bin(lens[i], tag_bytes)], 1u);
+    for (uint32_t i0 = blockIdx.x * 256u; i0 < n; i0 += stride) {
+        const uint32_t i = i0 + threadIdx.x;
+        const bool in = i < n;
+        (void)wave_bin_add(cnt, in ? len_bin(lens[i], tag_bytes) : 0u, in);
+    }
     __syncthreads();
     for (uint32_t b = threadIdx.x; b < LEN_BINS; b += 256) {
         const uint32_t c = cnt[b];
@@ -521,9 +561,12 @@ __global__ __launch_bounds__(256) void len_scatter_kernel(const uint32_t *lens, 
         cnt[b] = 0;
     }
     __syncthreads();
-    for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < n; i += stride) {
-        const uint32_t b = len_bin(lens[i], tag_bytes);
-        order[base[b] + atomicAdd(&cnt[b], 1u)] = i;
+    for (uint32_t i0 = blockIdx.x * 256u; i0 < n; i0 += stride) {
+        const uint32_t i = i0 + threadIdx.x;
+        const bool in = i < n;
+        const uint32_t b = in ? len_bin(lens[i], tag_bytes) : 0u;
+        const uint32_t at = wave_bin_add(cnt, b, in);
+        if (in) order[base[b] + at] = i;
     }
 }
 

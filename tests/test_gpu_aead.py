@@ -156,6 +156,26 @@ def test_imix_multi_peer_with_forged_tags(ctx):
     assert not back[o:o + L].any()
 
 
+def test_maximum_packet_sizes(ctx):
+    """Jumbo frames and the largest length a 16-bit IP total-length field can
+    name (65,535), next to minimum-size packets: more ChaCha20 blocks than the
+    length grouping has bins, in both memory paths' batch sizes."""
+    lens = np.array([65535, 65519, 65520, 9000, 8999, 9001, 4096, 60, 0, 1] * 7, np.uint32)
+    b = W.aead_imix(15, len(lens), n_peers=4, lens=lens)
+    got = _gpu_seal_host(ctx, b, uniform=False)
+    want = _oracle_seal(b)
+    assert np.array_equal(got, want)
+    forged = W.forge_tags(15, got, b.off, b.lens, 0.1)
+    back, verdict = _gpu_open_host(ctx, b, got, uniform=False)
+    assert np.array_equal(verdict == 0, forged)
+    for i in range(b.n):
+        o, L = int(b.off[i]), int(b.lens[i])
+        if forged[i]:
+            assert not back[o:o + L].any()
+        else:
+            assert np.array_equal(back[o:o + L], b.plain[o:o + L])
+
+
 @pytest.mark.parametrize("layout", ["offsets", "reversed", "in_place", "uniform"])
 def test_large_host_batches_take_the_chunked_route(ctx, layout):
     """Host batches of several chunks' worth are uploaded, computed and

@@ -33,7 +33,7 @@ static hipError_t upload_rule_index(FilterState *f, const HostRuleIndex &h, hipS
     const size_t nb = h.bounds.size();
     if ((e = f->bounds.reserve(std::max<size_t>(nb, 1) * 4)) != hipSuccess) return e;
     if ((e = f->meta.reserve((nb + 1) * 4)) != hipSuccess) return e;
-    if ((e = f->ranges.reserve(std::max<size_t>(h.ranges.size(), 1) * 8)) != hipSuccess) return e;
+    if ((e = f->ranges.reserve(std::max<size_t>(h.ranges.size(), 1) * 4)) != hipSuccess) return e;
     if ((e = f->wide.reserve(std::max<size_t>(h.wide.size(), 1) * 16)) != hipSuccess) return e;
     if ((e = hipMemcpyAsync(f->bounds.p, h.bounds.data(), nb * 4, hipMemcpyHostToDevice, s)) != hipSuccess)
         return e;
@@ -41,7 +41,7 @@ static hipError_t upload_rule_index(FilterState *f, const HostRuleIndex &h, hipS
         hipSuccess)
         return e;
     if (!h.ranges.empty() &&
-        (e = hipMemcpyAsync(f->ranges.p, h.ranges.data(), h.ranges.size() * 8, hipMemcpyHostToDevice,
+        (e = hipMemcpyAsync(f->ranges.p, h.ranges.data(), h.ranges.size() * 4, hipMemcpyHostToDevice,
                             s)) != hipSuccess)
         return e;
     if (!h.wide.empty() &&
@@ -52,7 +52,7 @@ static hipError_t upload_rule_index(FilterState *f, const HostRuleIndex &h, hipS
     if ((e = hipStreamSynchronize(s)) != hipSuccess) return e;
     f->ridx.bounds = f->bounds.as<uint32_t>();
     f->ridx.meta = f->meta.as<uint32_t>();
-    f->ridx.ranges = f->ranges.as<uint2>();
+    f->ridx.ranges = f->ranges.as<uint32_t>();
     f->ridx.wide = f->wide.as<uint4>();
     f->ridx.n_bounds = (uint32_t)nb;
     f->ridx.n_wide = (uint32_t)h.wide.size();

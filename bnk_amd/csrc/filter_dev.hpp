@@ -25,12 +25,19 @@ struct FlowTableDev {
     uint32_t present_mask; // present_bits - 1 (a power of two)
 };
 
+// A key is class << 16 | port with class < 3, so key_lo 0x3FFFF never occurs.
+constexpr uint32_t RANGE_PAD = 0x3FFFFu << 14;
+constexpr uint32_t RANGE_MAX_SPAN = (1u << 14) - 1u; // largest key_hi - key_lo one entry holds
+constexpr uint32_t RANGE_BLOCK = 16;                 // entries per 64-byte block
+
 struct RuleIndexDev {
     const uint32_t *bounds; // [n_bounds] ascending starts of the elementary source intervals
     const uint32_t *meta;   // [n_bounds + 1] (first 64-byte block of the interval's list) << 8 |
                             // min(entries, 255); the last element only carries the block count
-    const uint2 *ranges;    // per interval: sorted disjoint (key_lo, key_hi), padded to a multiple
-                            // of 8 entries (one 64-byte block) with never-matching (~0, 0)
+    const uint32_t *ranges; // per interval: sorted disjoint key ranges, one word each
+                            // (key_lo << 14 | key_hi - key_lo; wider ranges are cut into
+                            // pieces), padded to a multiple of 16 entries (one 64-byte block)
+                            // with RANGE_PAD, which contains no key
     const uint4 *wide;      // [n_wide] (net, mask, key_lo, key_hi) scanned by every packet
     uint32_t n_bounds;
     uint32_t top_step;      // largest power of two < n_bounds (0 when n_bounds == 1)

@@ -13,7 +13,7 @@ namespace bnk {
 
 struct HostRuleIndex {
     std::vector<uint32_t> bounds, meta;
-    std::vector<uint2> ranges;
+    std::vector<uint32_t> ranges;
     std::vector<uint4> wide;
 };
 
@@ -107,25 +107,33 @@ inline bool build_rule_index(const bnk_rule *rules, uint32_t n, HostRuleIndex &o
         if (!t.wide)
             for (uint32_t j = t.a; j < t.b; j++) raw[fill[j]++] = make_uint2(t.klo, t.khi);
     // per interval: sort by key_lo, merge overlapping or adjacent key ranges,
-    // pad the list to whole 64-byte blocks
+    // cut what is left into one-word pieces, pad the list to whole 64-byte blocks
     out.meta.assign(nb + 1, 0);
     out.ranges.clear();
+    std::vector<uint2> merged;
     for (uint32_t j = 0; j < nb; j++) {
         const size_t first = out.ranges.size();
         auto lo = raw.begin() + raw_start[j], hi = raw.begin() + raw_start[j + 1];
         std::sort(lo, hi, [](const uint2 &x, const uint2 &y) { return x.x < y.x; });
+        merged.clear();
         for (auto it = lo; it != hi; ++it) {
-            if (out.ranges.size() > first && it->x <= out.ranges.back().y + 1u) {
-                if (it->y > out.ranges.back().y) out.ranges.back().y = it->y;
+            if (!merged.empty() && it->x <= merged.back().y + 1u) {
+                if (it->y > merged.back().y) merged.back().y = it->y;
             } else {
-                out.ranges.push_back(*it);
+                merged.push_back(*it);
             }
         }
+        for (const uint2 &r : merged)
+            for (uint32_t at = r.x;; at += RANGE_MAX_SPAN + 1u) {
+                const uint32_t span = std::min(r.y - at, RANGE_MAX_SPAN);
+                out.ranges.push_back(at << 14 | span);
+                if (at + span == r.y) break;
+            }
         const size_t cnt = out.ranges.size() - first;
-        while (out.ranges.size() % 8) out.ranges.push_back(make_uint2(0xFFFFFFFFu, 0u));
-        out.meta[j] = (uint32_t)(first / 8) << 8 | (uint32_t)std::min<size_t>(cnt, 255);
+        while (out.ranges.size() % RANGE_BLOCK) out.ranges.push_back(RANGE_PAD);
+        out.meta[j] = (uint32_t)(first / RANGE_BLOCK) << 8 | (uint32_t)std::min<size_t>(cnt, 255);
     }
-    out.meta[nb] = (uint32_t)(out.ranges.size() / 8) << 8;
+    out.meta[nb] = (uint32_t)(out.ranges.size() / RANGE_BLOCK) << 8;
     return true;
 }
 

@@ -45,21 +45,39 @@ struct Parsed {
     uint32_t proto;
 };
 
-// filter.go:71-106
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef u32x4 __attribute__((aligned(1))) u32x4_unaligned;
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef u32x2 __attribute__((aligned(1))) u32x2_unaligned;
+
+// filter.go:71-106.  Bytes 0-15 come in one load and bytes 16-23 (destination
+// and, without IP options, the ports) in a second when the packet has them:
+// every load instruction here reads 64 different lines, so their number is
+// what the kernel pays for.
 BNK_DEV bool parse_packet(const uint8_t *p, uint32_t len, Parsed &o)
 {
     if (len < 20u) return false;
-    const uint32_t w0 = ld32u(p);
+    const u32x4 a = *reinterpret_cast<const u32x4_unaligned *>(p);
+    const uint32_t w0 = a.x;
     if (((w0 >> 4) & 0xFu) != 4u) return false;
     const uint32_t ihl = (w0 & 0xFu) * 4u;
     if (ihl < 20u || len < ihl) return false;
-    o.proto = (ld32u(p + 8) >> 8) & 0xFFu;
-    o.src = __builtin_bswap32(ld32u(p + 12));
-    o.dst = __builtin_bswap32(ld32u(p + 16));
+    o.proto = (a.z >> 8) & 0xFFu;
+    o.src = __builtin_bswap32(a.w);
+    uint32_t dst_w, l4_w = 0;
+    const bool wide = len >= 24u;
+    if (wide) {
+        const u32x2 b = *reinterpret_cast<const u32x2_unaligned *>(p + 16);
+        dst_w = b.x;
+        l4_w = b.y;
+    } else {
+        dst_w = ld32u(p + 16);
+    }
+    o.dst = __builtin_bswap32(dst_w);
     const uint32_t body = len - ihl;
     if (o.proto == 6u || o.proto == 17u) {
         if (body < 4u) return false;
-        const uint32_t w = __builtin_bswap32(ld32u(p + ihl));
+        const uint32_t w = __builtin_bswap32(wide && ihl == 20u ? l4_w : ld32u(p + ihl));
         o.sport = w >> 16;
         o.dport = w & 0xFFFFu;
         return true;
@@ -125,39 +143,45 @@ BNK_DEV uint32_t interval_of(Ptr bounds, uint32_t n, uint32_t top_step, uint32_t
     return pos;
 }
 
-BNK_DEV bool in_range(uint2 r, uint32_t key) { return key >= r.x && key <= r.y; }
+// One word holds a range: key_lo << 14 | key_hi - key_lo.
+BNK_DEV bool in_range(uint32_t e, uint32_t key) { return key - (e >> 14) <= (e & RANGE_MAX_SPAN); }
+
+BNK_DEV bool quad_hit(uint4 v, uint32_t key)
+{
+    return in_range(v.x, key) || in_range(v.y, key) || in_range(v.z, key) || in_range(v.w, key);
+}
 
 // meta_j / meta_next: the interval's and the following interval's meta words.
+// The kernel is bound by the number of scattered load instructions a wave
+// issues (every lane reads a different line), and a wave waits for its slowest
+// lane: a list of up to 16 ranges is one 64-byte block read with as many
+// 16-byte loads as it has quads of entries, all issued together; longer lists
+// first find their block by its first key.
 BNK_DEV bool rules_match(const RuleIndexDev &ri, uint32_t meta_j, uint32_t meta_next, uint32_t src,
                          uint32_t key)
 {
-    const uint32_t cnt = meta_j & 255u;
-    const uint2 *list = ri.ranges + (size_t)(meta_j >> 8) * 8u;
-    if (cnt != 0u && cnt <= 8u) {
-        // the whole list is one 64-byte block: two entries per 16-byte load
-        const uint4 *blk = reinterpret_cast<const uint4 *>(list);
-        bool hit = false;
-#pragma unroll
-        for (uint32_t q = 0; q < 4; q++) {
-            if (2u * q < cnt) {
-                const uint4 v = blk[q];
-                hit = hit || in_range(make_uint2(v.x, v.y), key) || in_range(make_uint2(v.z, v.w), key);
-            }
-        }
-        if (hit) return true;
-    } else if (cnt > 8u) {
-        // last range with key_lo <= key (padding entries sort to the end)
-        uint32_t lo = 0, hi = ((meta_next >> 8) - (meta_j >> 8)) * 8u;
-        while (lo < hi) {
+    const uint32_t nblk = (meta_next >> 8) - (meta_j >> 8);
+    const uint4 *blk = reinterpret_cast<const uint4 *>(ri.ranges + (size_t)(meta_j >> 8) * RANGE_BLOCK);
+    if (nblk == 1u) {
+        const uint32_t cnt = meta_j & 255u;
+        const uint4 pad = make_uint4(RANGE_PAD, RANGE_PAD, RANGE_PAD, RANGE_PAD);
+        const uint4 v0 = blk[0];
+        const uint4 v1 = cnt > 4u ? blk[1] : pad;
+        const uint4 v2 = cnt > 8u ? blk[2] : pad;
+        const uint4 v3 = cnt > 12u ? blk[3] : pad;
+        if (quad_hit(v0, key) || quad_hit(v1, key) || quad_hit(v2, key) || quad_hit(v3, key)) return true;
+    } else if (nblk > 1u) {
+        // last block whose first key_lo <= key; the ranges are sorted and
+        // disjoint, so only that block can hold the key
+        uint32_t lo = 0, hi = nblk;
+        while (hi - lo > 1u) {
             const uint32_t mid = (lo + hi) >> 1;
-            const uint2 r = list[mid];
-            if (r.x <= key) {
-                if (key <= r.y) return true;
-                lo = mid + 1;
-            } else {
-                hi = mid;
-            }
+            if ((blk[4u * mid].x >> 14) <= key) lo = mid;
+            else hi = mid;
         }
+        const uint4 *b = blk + 4u * lo;
+        const uint4 v0 = b[0], v1 = b[1], v2 = b[2], v3 = b[3];
+        if (quad_hit(v0, key) || quad_hit(v1, key) || quad_hit(v2, key) || quad_hit(v3, key)) return true;
     }
     for (uint32_t w = 0; w < ri.n_wide; w++) {
         const uint4 r = ri.wide[w];
@@ -171,7 +195,7 @@ constexpr uint32_t FILTER_THREADS = 1024; // one copy of the index serves 16 wav
 
 // filter.go:121-147 for a batch; enforcement is on (the host short-circuits
 // allow-all mode).
-__global__ __launch_bounds__(FILTER_THREADS) void filter_check_kernel(FilterArgs a)
+__global__ __launch_bounds__(FILTER_THREADS, 8) void filter_check_kernel(FilterArgs a)
 {
     extern __shared__ uint32_t lds[]; // bounds then meta (n_bounds + 1) when they fit, else unused
     const RuleIndexDev ri = a.rules;
@@ -204,13 +228,16 @@ __global__ __launch_bounds__(FILTER_THREADS) void filter_check_kernel(FilterArgs
                 mj = ri.meta[iv];
                 mn = ri.meta[iv + 1];
             }
+            // return traffic: remote = src, remotePort = srcPort, localPort = dstPort.
+            // The presence word is fetched alongside the rule list, not after it:
+            // most packets need both and the wave would wait twice.
+            const FlowSlot s = flow_slot(a.flows, h.src, h.sport, h.dport, h.proto);
+            const uint32_t pword = a.flows.present[s.bit >> 5];
             if (rules_match(ri, mj, mn, h.src, key)) {
                 pass = 1;
             } else {
-                // return traffic: remote = src, remotePort = srcPort, localPort = dstPort
-                const FlowSlot s = flow_slot(a.flows, h.src, h.sport, h.dport, h.proto);
                 // a clear bit means the key was never stored: no probe needed
-                const bool maybe = (a.flows.present[s.bit >> 5] >> (s.bit & 31u)) & 1u;
+                const bool maybe = (pword >> (s.bit & 31u)) & 1u;
                 for (uint32_t probe = 0; maybe && probe < a.flows.cap; probe++) {
                     FlowSlotMem *slot = a.flows.slots + s.base + ((s.start + probe) & (a.flows.cap - 1u));
                     // Keys only change in NoteOutbound batches, never during this

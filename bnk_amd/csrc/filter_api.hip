@@ -8,7 +8,7 @@ using namespace bnk;
 namespace bnk {
 
 static hipError_t flow_table_alloc(uint32_t cap, DevBuf &slots, DevBuf &counters, DevBuf &present,
-                                   FlowTableDev &ft, hipStream_t s)
+                                   DevBuf &present_small, FlowTableDev &ft, hipStream_t s)
 {
     const size_t n = (size_t)cap * FLOW_REGIONS;
     // the table is kept under half full, so 8 * cap bits see at most one key per 16 bits
@@ -17,6 +17,9 @@ static hipError_t flow_table_alloc(uint32_t cap, DevBuf &slots, DevBuf &counters
     if ((e = slots.reserve(n * sizeof(FlowSlotMem))) != hipSuccess) return e;
     if ((e = counters.reserve(FLOW_COUNTERS * 4)) != hipSuccess) return e;
     if ((e = present.reserve(bits / 8)) != hipSuccess) return e;
+    if ((e = present_small.reserve(SMALL_BITS / 8)) != hipSuccess) return e;
+    ft.present_small = present_small.as<uint32_t>();
+    ft.small_ok = 1;
     ft.slots = slots.as<FlowSlotMem>();
     ft.counters = counters.as<uint32_t>();
     ft.present = present.as<uint32_t>();
@@ -24,6 +27,7 @@ static hipError_t flow_table_alloc(uint32_t cap, DevBuf &slots, DevBuf &counters
     ft.present_mask = bits - 1u;
     if ((e = launch_flow_clear(ft.slots, (uint32_t)n, s)) != hipSuccess) return e;
     if ((e = launch_fill_u32(ft.present, bits / 32, 0, s)) != hipSuccess) return e;
+    if ((e = launch_fill_u32(ft.present_small, SMALL_BITS / 32, 0, s)) != hipSuccess) return e;
     return launch_fill_u32(ft.counters, FLOW_COUNTERS, 0, s);
 }
 
@@ -32,13 +36,9 @@ static hipError_t upload_rule_index(FilterState *f, const HostRuleIndex &h, hipS
     hipError_t e;
     const size_t nb = h.bounds.size();
     if ((e = f->bounds.reserve(std::max<size_t>(nb, 1) * 4)) != hipSuccess) return e;
-    if ((e = f->meta.reserve((nb + 1) * 4)) != hipSuccess) return e;
     if ((e = f->ranges.reserve(std::max<size_t>(h.ranges.size(), 1) * 4)) != hipSuccess) return e;
     if ((e = f->wide.reserve(std::max<size_t>(h.wide.size(), 1) * 16)) != hipSuccess) return e;
     if ((e = hipMemcpyAsync(f->bounds.p, h.bounds.data(), nb * 4, hipMemcpyHostToDevice, s)) != hipSuccess)
-        return e;
-    if ((e = hipMemcpyAsync(f->meta.p, h.meta.data(), (nb + 1) * 4, hipMemcpyHostToDevice, s)) !=
-        hipSuccess)
         return e;
     if (!h.ranges.empty() &&
         (e = hipMemcpyAsync(f->ranges.p, h.ranges.data(), h.ranges.size() * 4, hipMemcpyHostToDevice,
@@ -51,7 +51,6 @@ static hipError_t upload_rule_index(FilterState *f, const HostRuleIndex &h, hipS
     // the host vectors die with the caller's frame
     if ((e = hipStreamSynchronize(s)) != hipSuccess) return e;
     f->ridx.bounds = f->bounds.as<uint32_t>();
-    f->ridx.meta = f->meta.as<uint32_t>();
     f->ridx.ranges = f->ranges.as<uint32_t>();
     f->ridx.wide = f->wide.as<uint4>();
     f->ridx.n_bounds = (uint32_t)nb;
@@ -73,7 +72,7 @@ FilterState *filter_create(hipStream_t s, int cu_count)
     HostRuleIndex h;
     std::string err;
     build_rule_index(nullptr, 0, h, err);
-    if (flow_table_alloc(FLOW_CAP_INITIAL, f->slots, f->counters, f->present, f->flows, s) != hipSuccess ||
+    if (flow_table_alloc(FLOW_CAP_INITIAL, f->slots, f->counters, f->present, f->present_small, f->flows, s) != hipSuccess ||
         upload_rule_index(f, h, s) != hipSuccess) {
         filter_destroy(f);
         return nullptr;
@@ -100,6 +99,7 @@ int flows_reserve(bnk_ctx *ctx, uint32_t n_new)
     const uint64_t half = f->flows.cap / 2;
     if (f->claimed_upper + n_new <= half) {
         f->claimed_upper += n_new;
+        f->flows.small_ok = f->claimed_upper <= SMALL_KEYS_MAX;
         return BNK_OK;
     }
     uint32_t c[FLOW_COUNTERS];
@@ -108,26 +108,28 @@ int flows_reserve(bnk_ctx *ctx, uint32_t n_new)
     f->claimed_upper = c[FLOW_CLAIMED];
     if (f->claimed_upper + n_new <= half) {
         f->claimed_upper += n_new;
+        f->flows.small_ok = f->claimed_upper <= SMALL_KEYS_MAX;
         return BNK_OK;
     }
     uint64_t need = 4ull * ((uint64_t)c[FLOW_LIVE] + n_new); // at most a quarter full afterwards
     uint64_t cap = FLOW_CAP_INITIAL;
     while (cap < need) cap *= 2;
     if (cap > FLOW_CAP_MAX) return fail(ctx, BNK_E_NOMEM, "flow table would exceed its maximum size");
-    DevBuf ns, nc, np;
+    DevBuf ns, nc, np, nps;
     FlowTableDev nt{};
-    hipError_t e = flow_table_alloc((uint32_t)cap, ns, nc, np, nt, ctx->stream);
+    hipError_t e = flow_table_alloc((uint32_t)cap, ns, nc, np, nps, nt, ctx->stream);
     if (e == hipSuccess)
         e = launch_flow_rehash(f->flows, nt, ctx->d_status, f->max_blocks, ctx->stream);
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
     if (e != hipSuccess) {
-        ns.release(); nc.release(); np.release();
+        ns.release(); nc.release(); np.release(); nps.release();
         return fail_hip(ctx, "flow table growth", e);
     }
-    f->slots.release(); f->counters.release(); f->present.release();
-    f->slots = ns; f->counters = nc; f->present = np;
+    f->slots.release(); f->counters.release(); f->present.release(); f->present_small.release();
+    f->slots = ns; f->counters = nc; f->present = np; f->present_small = nps;
     f->flows = nt;
     f->claimed_upper = (uint64_t)c[FLOW_LIVE] + n_new;
+    f->flows.small_ok = f->claimed_upper <= SMALL_KEYS_MAX;
     return BNK_OK;
 }
 

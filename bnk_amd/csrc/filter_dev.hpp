@@ -21,23 +21,33 @@ struct FlowTableDev {
     uint32_t *counters; // [FLOW_COUNTERS]: entries in the map, slots ever claimed, sweep flag
     uint32_t *present;  // [present_bits / 32] one hashed bit per key ever stored in this table:
                         // small enough to stay in L2, it answers most misses without a probe
+    uint32_t *present_small; // [SMALL_BITS / 32] two hashed bits per key (a Bloom filter) in a
+                             // size a workgroup can hold in LDS beside the cut points: with
+                             // few enough keys the check kernel asks this one and never
+                             // leaves the CU for a packet without a flow
     uint32_t cap;       // slots per region, a power of two
     uint32_t present_mask; // present_bits - 1 (a power of two)
+    uint32_t small_ok;  // host's call: few enough keys for present_small to be worth reading
 };
 
-// A key is class << 16 | port with class < 3, so key_lo 0x3FFFF never occurs.
+constexpr uint32_t SMALL_BITS = 44u * 1024u * 8u; // 44 KiB: leaves 36 KiB of a workgroup's 80 for cut points
+constexpr uint32_t SMALL_KEYS_MAX = 3u << 16;     // beyond this a clear answer gets too rare (false
+                                                  // positives pass 43 %) and the large bitmap is asked
+
+// A key is class << 16 | port with class < 3, so key_lo 0x3FFFF and 0x3FFFE never occur.
 constexpr uint32_t RANGE_PAD = 0x3FFFFu << 14;
+constexpr uint32_t RANGE_LONG = 0x3FFFEu << 14;      // first word of a block that only points on
 constexpr uint32_t RANGE_MAX_SPAN = (1u << 14) - 1u; // largest key_hi - key_lo one entry holds
 constexpr uint32_t RANGE_BLOCK = 16;                 // entries per 64-byte block
 
 struct RuleIndexDev {
     const uint32_t *bounds; // [n_bounds] ascending starts of the elementary source intervals
-    const uint32_t *meta;   // [n_bounds + 1] (first 64-byte block of the interval's list) << 8 |
-                            // min(entries, 255); the last element only carries the block count
-    const uint32_t *ranges; // per interval: sorted disjoint key ranges, one word each
+    const uint32_t *ranges; // 64-byte blocks of RANGE_BLOCK one-word key ranges
                             // (key_lo << 14 | key_hi - key_lo; wider ranges are cut into
-                            // pieces), padded to a multiple of 16 entries (one 64-byte block)
-                            // with RANGE_PAD, which contains no key
+                            // pieces), sorted, disjoint, padded with RANGE_PAD.  Block j is
+                            // interval j's list, so finding the interval finds the list.  A
+                            // list of more than RANGE_BLOCK pieces lives in blocks past the
+                            // first n_bounds, and block j is {RANGE_LONG, first block, blocks}
     const uint4 *wide;      // [n_wide] (net, mask, key_lo, key_hi) scanned by every packet
     uint32_t n_bounds;
     uint32_t top_step;      // largest power of two < n_bounds (0 when n_bounds == 1)
@@ -54,6 +64,7 @@ struct FilterArgs {
     int64_t now;
     uint32_t n, stride, len;
     uint32_t trim;        // bytes at the end of each packet that are not payload
+    uint32_t small_in_lds; // set by the launcher: presence questions go to the folded bitmap in LDS
     RuleIndexDev rules;
     FlowTableDev flows;
 };

@@ -12,14 +12,14 @@
 namespace bnk {
 
 struct HostRuleIndex {
-    std::vector<uint32_t> bounds, meta;
+    std::vector<uint32_t> bounds;
     std::vector<uint32_t> ranges;
     std::vector<uint4> wide;
 };
 
 // Upper limit on expanded (interval, key range) entries; rules that would push
 // the total beyond it are kept in the wide list instead.
-constexpr size_t RULE_EXPANSION_BUDGET = size_t(1) << 22; // keeps block numbers within 24 bits
+constexpr size_t RULE_EXPANSION_BUDGET = size_t(1) << 22;
 
 // Compiles bnk_rule tuples (each one prefix x one port range of an
 // acl.CompiledRule, internal/acl/acl.go:33-42) into the interval index the
@@ -107,12 +107,12 @@ inline bool build_rule_index(const bnk_rule *rules, uint32_t n, HostRuleIndex &o
         if (!t.wide)
             for (uint32_t j = t.a; j < t.b; j++) raw[fill[j]++] = make_uint2(t.klo, t.khi);
     // per interval: sort by key_lo, merge overlapping or adjacent key ranges,
-    // cut what is left into one-word pieces, pad the list to whole 64-byte blocks
-    out.meta.assign(nb + 1, 0);
-    out.ranges.clear();
+    // cut what is left into one-word pieces; block j takes interval j's pieces,
+    // or points at blocks appended behind the first nb when there are too many
+    out.ranges.assign((size_t)nb * RANGE_BLOCK, RANGE_PAD);
     std::vector<uint2> merged;
+    std::vector<uint32_t> pieces;
     for (uint32_t j = 0; j < nb; j++) {
-        const size_t first = out.ranges.size();
         auto lo = raw.begin() + raw_start[j], hi = raw.begin() + raw_start[j + 1];
         std::sort(lo, hi, [](const uint2 &x, const uint2 &y) { return x.x < y.x; });
         merged.clear();
@@ -123,31 +123,40 @@ inline bool build_rule_index(const bnk_rule *rules, uint32_t n, HostRuleIndex &o
                 merged.push_back(*it);
             }
         }
+        pieces.clear();
         for (const uint2 &r : merged)
             for (uint32_t at = r.x;; at += RANGE_MAX_SPAN + 1u) {
                 const uint32_t span = std::min(r.y - at, RANGE_MAX_SPAN);
-                out.ranges.push_back(at << 14 | span);
+                pieces.push_back(at << 14 | span);
                 if (at + span == r.y) break;
             }
-        const size_t cnt = out.ranges.size() - first;
-        while (out.ranges.size() % RANGE_BLOCK) out.ranges.push_back(RANGE_PAD);
-        out.meta[j] = (uint32_t)(first / RANGE_BLOCK) << 8 | (uint32_t)std::min<size_t>(cnt, 255);
+        uint32_t *blk = out.ranges.data() + (size_t)j * RANGE_BLOCK;
+        if (pieces.size() <= RANGE_BLOCK) {
+            std::copy(pieces.begin(), pieces.end(), blk);
+        } else {
+            const size_t first = out.ranges.size() / RANGE_BLOCK;
+            out.ranges.insert(out.ranges.end(), pieces.begin(), pieces.end());
+            while (out.ranges.size() % RANGE_BLOCK) out.ranges.push_back(RANGE_PAD);
+            blk = out.ranges.data() + (size_t)j * RANGE_BLOCK; // the vector may have moved
+            blk[0] = RANGE_LONG;
+            blk[1] = (uint32_t)first;
+            blk[2] = (uint32_t)(out.ranges.size() / RANGE_BLOCK - first);
+        }
     }
-    out.meta[nb] = (uint32_t)(out.ranges.size() / RANGE_BLOCK) << 8;
     return true;
 }
 
 struct FilterState {
     bool enforce = false; // filter.New: allow-all until a policy arrives (filter.go:41-43)
-    DevBuf bounds, meta, ranges, wide;
+    DevBuf bounds, ranges, wide;
     RuleIndexDev ridx{};
-    DevBuf slots, counters, present;
+    DevBuf slots, counters, present, present_small;
     FlowTableDev flows{};
     uint64_t claimed_upper = 0; // host bound on slots ever claimed in the current table
     uint32_t max_blocks = 2048;
     void release()
     {
-        for (DevBuf *b : {&bounds, &meta, &ranges, &wide, &slots, &counters, &present}) b->release();
+        for (DevBuf *b : {&bounds, &ranges, &wide, &slots, &counters, &present, &present_small}) b->release();
     }
 };
 

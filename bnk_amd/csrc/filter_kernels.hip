@@ -109,11 +109,17 @@ BNK_DEV uint64_t mix64(uint64_t x)
     return x;
 }
 
+// The two positions of a key in the small presence bitmap (a Bloom filter with
+// two hash functions over SMALL_BITS bits, which is not a power of two).
+BNK_DEV uint32_t small_bit0(uint64_t hsh) { return __umulhi((uint32_t)(hsh >> 32), SMALL_BITS); }
+BNK_DEV uint32_t small_bit1(uint64_t hsh) { return __umulhi((uint32_t)hsh * 0x9E3779B1u, SMALL_BITS); }
+
 struct FlowSlot {
     uint64_t word;   // stored key word (never 0)
     uint32_t base;   // first slot of the region
     uint32_t start;  // probe start within the region
     uint32_t bit;    // this key's bit in the presence bitmap
+    uint32_t sbit0, sbit1; // and its two bits in the small one
 };
 
 BNK_DEV FlowSlot flow_slot(const FlowTableDev &ft, uint32_t remote, uint32_t rport, uint32_t lport,
@@ -126,6 +132,8 @@ BNK_DEV FlowSlot flow_slot(const FlowTableDev &ft, uint32_t remote, uint32_t rpo
     const uint64_t hsh = mix64(s.word ^ ((uint64_t)region << 59));
     s.start = (uint32_t)hsh & (ft.cap - 1u);
     s.bit = (uint32_t)(hsh >> 32) & ft.present_mask;
+    s.sbit0 = small_bit0(hsh);
+    s.sbit1 = small_bit1(hsh);
     return s;
 }
 
@@ -151,37 +159,30 @@ BNK_DEV bool quad_hit(uint4 v, uint32_t key)
     return in_range(v.x, key) || in_range(v.y, key) || in_range(v.z, key) || in_range(v.w, key);
 }
 
-// meta_j / meta_next: the interval's and the following interval's meta words.
-// The kernel is bound by the number of scattered load instructions a wave
-// issues (every lane reads a different line), and a wave waits for its slowest
-// lane: a list of up to 16 ranges is one 64-byte block read with as many
-// 16-byte loads as it has quads of entries, all issued together; longer lists
-// first find their block by its first key.
-BNK_DEV bool rules_match(const RuleIndexDev &ri, uint32_t meta_j, uint32_t meta_next, uint32_t src,
-                         uint32_t key)
+// iv: the packet's elementary source interval.  The kernel is bound by the
+// scattered 64-byte lines it pulls from L2 and beyond, so the interval's list
+// is a single such line (block iv), fetched with four 16-byte loads issued
+// together.  Only a list of more than 16 pieces goes through a second step,
+// finding its block by the block's first key.
+BNK_DEV bool rules_match(const RuleIndexDev &ri, uint32_t iv, uint32_t src, uint32_t key)
 {
-    const uint32_t nblk = (meta_next >> 8) - (meta_j >> 8);
-    const uint4 *blk = reinterpret_cast<const uint4 *>(ri.ranges + (size_t)(meta_j >> 8) * RANGE_BLOCK);
-    if (nblk == 1u) {
-        const uint32_t cnt = meta_j & 255u;
-        const uint4 pad = make_uint4(RANGE_PAD, RANGE_PAD, RANGE_PAD, RANGE_PAD);
-        const uint4 v0 = blk[0];
-        const uint4 v1 = cnt > 4u ? blk[1] : pad;
-        const uint4 v2 = cnt > 8u ? blk[2] : pad;
-        const uint4 v3 = cnt > 12u ? blk[3] : pad;
+    const uint4 *blk = reinterpret_cast<const uint4 *>(ri.ranges + (size_t)iv * RANGE_BLOCK);
+    const uint4 v0 = blk[0], v1 = blk[1], v2 = blk[2], v3 = blk[3];
+    if (v0.x != RANGE_LONG) {
         if (quad_hit(v0, key) || quad_hit(v1, key) || quad_hit(v2, key) || quad_hit(v3, key)) return true;
-    } else if (nblk > 1u) {
+    } else {
         // last block whose first key_lo <= key; the ranges are sorted and
         // disjoint, so only that block can hold the key
-        uint32_t lo = 0, hi = nblk;
+        const uint4 *ob = reinterpret_cast<const uint4 *>(ri.ranges + (size_t)v0.y * RANGE_BLOCK);
+        uint32_t lo = 0, hi = v0.z;
         while (hi - lo > 1u) {
             const uint32_t mid = (lo + hi) >> 1;
-            if ((blk[4u * mid].x >> 14) <= key) lo = mid;
+            if ((ob[4u * mid].x >> 14) <= key) lo = mid;
             else hi = mid;
         }
-        const uint4 *b = blk + 4u * lo;
-        const uint4 v0 = b[0], v1 = b[1], v2 = b[2], v3 = b[3];
-        if (quad_hit(v0, key) || quad_hit(v1, key) || quad_hit(v2, key) || quad_hit(v3, key)) return true;
+        const uint4 *b = ob + 4u * lo;
+        const uint4 w0 = b[0], w1 = b[1], w2 = b[2], w3 = b[3];
+        if (quad_hit(w0, key) || quad_hit(w1, key) || quad_hit(w2, key) || quad_hit(w3, key)) return true;
     }
     for (uint32_t w = 0; w < ri.n_wide; w++) {
         const uint4 r = ri.wide[w];
@@ -190,22 +191,24 @@ BNK_DEV bool rules_match(const RuleIndexDev &ri, uint32_t meta_j, uint32_t meta_
     return false;
 }
 
-constexpr uint32_t LDS_BOUNDS_MAX = 12288; // 96 KiB: cut points and meta words
+constexpr uint32_t LDS_BOUNDS_MAX = 24576; // 96 KiB of cut points
 constexpr uint32_t FILTER_THREADS = 1024; // one copy of the index serves 16 waves
 
 // filter.go:121-147 for a batch; enforcement is on (the host short-circuits
 // allow-all mode).
 __global__ __launch_bounds__(FILTER_THREADS, 8) void filter_check_kernel(FilterArgs a)
 {
-    extern __shared__ uint32_t lds[]; // bounds then meta (n_bounds + 1) when they fit, else unused
+    extern __shared__ uint32_t lds[]; // the cut points when they fit, then the small presence bitmap
     const RuleIndexDev ri = a.rules;
     const bool in_lds = ri.n_bounds <= LDS_BOUNDS_MAX;
-    uint32_t *lb = lds, *lm = lds + ri.n_bounds;
-    if (in_lds) {
+    const bool small = a.small_in_lds != 0u;
+    uint32_t *lb = lds, *lsmall = lds + (in_lds ? ri.n_bounds : 0u);
+    if (in_lds)
         for (uint32_t q = threadIdx.x; q < ri.n_bounds; q += FILTER_THREADS) lb[q] = ri.bounds[q];
-        for (uint32_t q = threadIdx.x; q <= ri.n_bounds; q += FILTER_THREADS) lm[q] = ri.meta[q];
-        __syncthreads();
-    }
+    if (small)
+        for (uint32_t q = threadIdx.x; q < SMALL_BITS / 32u; q += FILTER_THREADS)
+            lsmall[q] = a.flows.present_small[q];
+    __syncthreads();
     const uint32_t stride = gridDim.x * FILTER_THREADS;
     for (uint32_t i = blockIdx.x * FILTER_THREADS + threadIdx.x; i < a.n; i += stride) {
         if (a.gate && a.gate[i] == 0) {
@@ -218,26 +221,22 @@ __global__ __launch_bounds__(FILTER_THREADS, 8) void filter_check_kernel(FilterA
         uint8_t pass = 0;
         if (parse_packet(p, len - (len >= a.trim ? a.trim : len), h)) {
             const uint32_t key = proto_class(h.proto) << 16 | h.dport;
-            uint32_t mj, mn;
-            if (in_lds) {
-                const uint32_t iv = interval_of(lb, ri.n_bounds, ri.top_step, h.src);
-                mj = lm[iv];
-                mn = lm[iv + 1];
-            } else {
-                const uint32_t iv = interval_of(ri.bounds, ri.n_bounds, ri.top_step, h.src);
-                mj = ri.meta[iv];
-                mn = ri.meta[iv + 1];
-            }
+            const uint32_t iv = in_lds ? interval_of(lb, ri.n_bounds, ri.top_step, h.src)
+                                       : interval_of(ri.bounds, ri.n_bounds, ri.top_step, h.src);
             // return traffic: remote = src, remotePort = srcPort, localPort = dstPort.
-            // The presence word is fetched alongside the rule list, not after it:
-            // most packets need both and the wave would wait twice.
+            // A clear presence bit means the key was never stored: no probe
+            // needed.  The bits come from LDS when the small bitmap is in use;
+            // otherwise the word is fetched alongside the rule list, not after it.
             const FlowSlot s = flow_slot(a.flows, h.src, h.sport, h.dport, h.proto);
-            const uint32_t pword = a.flows.present[s.bit >> 5];
-            if (rules_match(ri, mj, mn, h.src, key)) {
+            bool maybe;
+            if (small) {
+                maybe = ((lsmall[s.sbit0 >> 5] >> (s.sbit0 & 31u)) & (lsmall[s.sbit1 >> 5] >> (s.sbit1 & 31u)) & 1u) != 0u;
+            } else {
+                maybe = ((a.flows.present[s.bit >> 5] >> (s.bit & 31u)) & 1u) != 0u;
+            }
+            if (rules_match(ri, iv, h.src, key)) {
                 pass = 1;
             } else {
-                // a clear bit means the key was never stored: no probe needed
-                const bool maybe = (pword >> (s.bit & 31u)) & 1u;
                 for (uint32_t probe = 0; maybe && probe < a.flows.cap; probe++) {
                     FlowSlotMem *slot = a.flows.slots + s.base + ((s.start + probe) & (a.flows.cap - 1u));
                     // Keys only change in NoteOutbound batches, never during this
@@ -289,6 +288,8 @@ __global__ __launch_bounds__(256) void filter_note_kernel(FilterArgs a)
             if (old == 0ULL) {
                 atomicAdd(&a.flows.counters[FLOW_CLAIMED], 1u);
                 atomicOr(&a.flows.present[s.bit >> 5], 1u << (s.bit & 31u));
+                atomicOr(&a.flows.present_small[s.sbit0 >> 5], 1u << (s.sbit0 & 31u));
+                atomicOr(&a.flows.present_small[s.sbit1 >> 5], 1u << (s.sbit1 & 31u));
             }
             if (old == 0ULL || old == s.word) {
                 unsigned long long *ep = reinterpret_cast<unsigned long long *>(&slot->exp);
@@ -350,6 +351,9 @@ __global__ __launch_bounds__(256) void flow_rehash_kernel(FlowTableDev from, Flo
             if (atomicCAS(kp, 0ULL, (unsigned long long)word) == 0ULL) {
                 to.slots[t].exp = e;
                 atomicOr(&to.present[bit >> 5], 1u << (bit & 31u));
+                const uint32_t b0 = small_bit0(hsh), b1 = small_bit1(hsh);
+                atomicOr(&to.present_small[b0 >> 5], 1u << (b0 & 31u));
+                atomicOr(&to.present_small[b1 >> 5], 1u << (b1 & 31u));
                 atomicAdd(&to.counters[FLOW_CLAIMED], 1u);
                 atomicAdd(&to.counters[FLOW_LIVE], 1u);
                 placed = true;
@@ -408,15 +412,19 @@ hipError_t launch_fill_u8(uint8_t *p, uint32_t n, uint8_t v, hipStream_t s)
     return hipGetLastError();
 }
 
-hipError_t launch_filter_check(const FilterArgs &a, uint32_t max_blocks, hipStream_t s)
+hipError_t launch_filter_check(const FilterArgs &args, uint32_t max_blocks, hipStream_t s)
 {
-    if (a.n == 0) return hipSuccess;
-    const uint32_t lds = a.rules.n_bounds <= LDS_BOUNDS_MAX ? (2u * a.rules.n_bounds + 1u) * 4u : 0u;
+    if (args.n == 0) return hipSuccess;
+    FilterArgs a = args;
+    uint32_t lds = a.rules.n_bounds <= LDS_BOUNDS_MAX ? a.rules.n_bounds * 4u : 0u;
+    // the small bitmap rides along while two workgroups still fit a CU's 160 KiB
+    a.small_in_lds = a.flows.small_ok && lds + SMALL_BITS / 8u <= 80u * 1024u ? 1u : 0u;
+    if (a.small_in_lds) lds += SMALL_BITS / 8u;
     if (lds > 48u * 1024u) {
         // more dynamic LDS than the default limit: opt in (gfx950 has 160 KiB per CU)
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(filter_check_kernel),
                                            hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           (int)((2u * LDS_BOUNDS_MAX + 1u) * 4u));
+                                           (int)(LDS_BOUNDS_MAX * 4u));
         if (e != hipSuccess) return e;
     }
     // one index copy per workgroup: as many workgroups per CU as their LDS allows, two at most

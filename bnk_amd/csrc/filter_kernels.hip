@@ -164,6 +164,8 @@ BNK_DEV bool quad_hit(uint4 v, uint32_t key)
 // is a single such line (block iv), fetched with four 16-byte loads issued
 // together.  Only a list of more than 16 pieces goes through a second step,
 // finding its block by the block's first key.
+// (Fetching only the quads a list occupies was tried and is slower: the
+// branches around the loads cost more than the loads they save.)
 BNK_DEV bool rules_match(const RuleIndexDev &ri, uint32_t iv, uint32_t src, uint32_t key)
 {
     const uint4 *blk = reinterpret_cast<const uint4 *>(ri.ranges + (size_t)iv * RANGE_BLOCK);
@@ -250,8 +252,16 @@ __global__ __launch_bounds__(FILTER_THREADS, 8) void filter_check_kernel(FilterA
                     if (e == FLOW_TOMB) break; // deleted earlier
                     if (a.now < e) {
                         // keep-alive on traffic (filter.go:141)
-                        __atomic_store_n(ep, (unsigned long long)(a.now + flow_ttl_ns(h.proto)),
-                                         __ATOMIC_RELAXED);
+                        // A plain store on purpose.  Every lane that refreshes this
+                        // flow in this batch writes the same value, a reader may see
+                        // the old expiry or the new one (both lie after `now`, so the
+                        // verdict is the same), and deletion cannot race with it: all
+                        // lanes see the same side of `now < e`.  An atomic store would
+                        // have to be visible across the eight L2s at once and is
+                        // pushed out to memory for it; this one waits for the end of
+                        // the kernel like any other store.
+                        // (`volatile` gets the same treatment as an atomic, hence not even that.)
+                        *ep = (unsigned long long)(a.now + flow_ttl_ns(h.proto));
                         pass = 1;
                     } else {
                         // expired: delete (filter.go:144); only the lane that

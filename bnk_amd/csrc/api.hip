@@ -7,99 +7,35 @@ using namespace bnk;
 
 namespace {
 
-// Chunked form of a host batch: while chunk k is computed, chunk k+1 is on its
-// way up and chunk k-1 on its way down (the link is full duplex).  Needs
-// packets laid out in ascending, non-overlapping order in both arenas, so that
-// a run of consecutive packets is one contiguous span.  Returns 1 when the
+// Chunked form of a host seal/open batch (see HostPipe).  Returns 1 when the
 // batch does not qualify and the caller should take the single-shot route.
-constexpr uint32_t PIPE_MAX_CHUNKS = 16;
-constexpr uint64_t PIPE_MIN_CHUNK_BYTES = 4ull << 20;
-
-bool ascending_layout(const bnk_batch *lay, const bnk_batch *src, int delta)
-{
-    const uint32_t n = src->n;
-    if (!lay->offsets) {
-        if (!src->lens) return (int64_t)src->len + delta <= (int64_t)lay->stride;
-        for (uint32_t i = 0; i < n; i++)
-            if ((int64_t)src->lens[i] + delta > (int64_t)lay->stride) return false;
-        return true;
-    }
-    uint64_t end = 0;
-    for (uint32_t i = 0; i < n; i++) {
-        const uint64_t off = lay->offsets[i];
-        int64_t len = (int64_t)(src->lens ? src->lens[i] : src->len) + delta;
-        if (len < 0) len = 0;
-        if (off < end) return false;
-        end = off + (uint64_t)len;
-    }
-    return true;
-}
-
-int ensure_pipe(bnk_ctx *ctx, uint32_t chunks)
-{
-    if (!ctx->s_up) HIPCHK(ctx, hipStreamCreateWithFlags(&ctx->s_up, hipStreamNonBlocking));
-    if (!ctx->s_down) HIPCHK(ctx, hipStreamCreateWithFlags(&ctx->s_down, hipStreamNonBlocking));
-    while (ctx->ev_up.size() < chunks + 1u) {
-        hipEvent_t e;
-        HIPCHK(ctx, hipEventCreateWithFlags(&e, hipEventDisableTiming));
-        ctx->ev_up.push_back(e);
-    }
-    while (ctx->ev_done.size() < chunks) {
-        hipEvent_t e;
-        HIPCHK(ctx, hipEventCreateWithFlags(&e, hipEventDisableTiming));
-        ctx->ev_done.push_back(e);
-    }
-    return BNK_OK;
-}
-
 int aead_batch_host_chunked(bnk_ctx *ctx, bool open, const bnk_batch *in, const bnk_batch *out,
                             uint8_t *verdict, AeadArgs a)
 {
     const uint32_t n = in->n;
     const int out_delta = open ? -16 : 16;
-    Span sin, sout;
-    int rc = scan_host_layout(ctx, in, in, 0, &sin, "in");
+    HostPipe hp;
+    hp.ctx = ctx;
+    hp.in = in;
+    hp.out = out;
+    hp.in_ext = [in](uint32_t i) { return (uint64_t)(in->lens ? in->lens[i] : in->len); };
+    hp.out_ext = [in, out_delta](uint32_t i) {
+        return (uint64_t)std::max<int64_t>((int64_t)(in->lens ? in->lens[i] : in->len) + out_delta, 0);
+    };
+    int rc = hp.plan(in->lens ? 0 : hp.out_ext(0));
     if (rc) return rc;
-    rc = scan_host_layout(ctx, out, in, out_delta, &sout, "out");
-    if (rc) return rc;
-    const uint32_t by_bytes = (uint32_t)std::min<uint64_t>(sin.size() / PIPE_MIN_CHUNK_BYTES, PIPE_MAX_CHUNKS);
-    if (by_bytes < 2 || n < 2u * 64u) return 1;
-    if (!ascending_layout(in, in, 0) || !ascending_layout(out, in, out_delta)) return 1;
     if (in->peer)
         for (uint32_t i = 0; i < n; i++)
             if (in->peer[i] >= a.n_peers)
                 return fail(ctx, BNK_E_RANGE, "peer index " + std::to_string(in->peer[i]) + " beyond the key table");
-    const uint32_t chunks = by_bytes;
-    const uint32_t per = ((n + chunks - 1u) / chunks + 63u) & ~63u; // whole waves per chunk
-    rc = ensure_pipe(ctx, chunks);
+    if (open) {
+        HIPCHK(ctx, ctx->verdict.reserve(n));
+        a.verdict = ctx->verdict.as<uint8_t>();
+        hp.add_result(verdict, a.verdict, 1);
+    }
+    rc = hp.begin();
     if (rc) return rc;
-    const bool in_place = same_layout(in, out);
-    if (in_place) {
-        sin.add(sout.lo, sout.hi);
-        sout = sin;
-    }
-    // a uniform output layout comes back row by row, so the gaps between its
-    // packets never need to be on the device; any other layout first takes the
-    // host's bytes up so that they come back unchanged
-    const bool rows_down = !in_place && !out->offsets && !in->lens;
-    // offsets staging, then verdict staging: a download into pageable memory
-    // would make the runtime wait for it and stall the pipeline
-    HIPCHK(ctx, ctx->pin.reserve((size_t)n * 17 + 64));
-    uint8_t *h_verdict = ctx->pin.as<uint8_t>() + (size_t)n * 16;
-    HIPCHK(ctx, ctx->in_arena.reserve(sin.size() + 16));
-    uint8_t *d_in = ctx->in_arena.as<uint8_t>(), *d_out = d_in;
-    if (!in_place) {
-        HIPCHK(ctx, ctx->out_arena.reserve(sout.size() + 16));
-        d_out = ctx->out_arena.as<uint8_t>();
-    }
     // per-packet arrays go up whole, ahead of everything, on the compute stream
-    rc = upload_offsets(ctx, in, n, sin.lo, &ctx->off_in, 0, &a.in_off);
-    if (rc) return rc;
-    if (in_place) a.out_off = a.in_off;
-    else {
-        rc = upload_offsets(ctx, out, n, sout.lo, &ctx->off_out, (size_t)n * 8, &a.out_off);
-        if (rc) return rc;
-    }
     auto up = [&](DevBuf *dst, const void *src, size_t bytes) -> hipError_t {
         hipError_t e = dst->reserve(bytes);
         if (e != hipSuccess) return e;
@@ -120,38 +56,17 @@ int aead_batch_host_chunked(bnk_ctx *ctx, bool open, const bnk_batch *in, const 
         HIPCHK(ctx, up(&ctx->counters, in->counters, (size_t)n * 8));
         a.counters = ctx->counters.as<uint64_t>();
     }
-    if (open) {
-        HIPCHK(ctx, ctx->verdict.reserve(n));
-        a.verdict = ctx->verdict.as<uint8_t>();
-    }
-    a.in = d_in;
-    a.out = d_out;
-    HIPCHK(ctx, hipEventRecord(ctx->ev_up[chunks], ctx->stream));
-    HIPCHK(ctx, hipStreamWaitEvent(ctx->s_up, ctx->ev_up[chunks], 0));
-
-    auto pkt_len = [&](uint32_t i) { return (uint64_t)(in->lens ? in->lens[i] : in->len); };
-    const uint8_t *h_in = (const uint8_t *)in->base;
-    uint8_t *h_out = (uint8_t *)out->base;
-    for (uint32_t k = 0; k < chunks; k++) {
-        const uint32_t lo = k * per, hi = std::min(n, lo + per);
-        if (lo >= hi) break;
-        // spans of this run of packets, relative to the staged arenas
-        const uint64_t i0 = pkt_off(in, lo), i1 = pkt_off(in, hi - 1) + pkt_len(hi - 1);
-        const int64_t last_out = std::max<int64_t>((int64_t)pkt_len(hi - 1) + out_delta, 0);
-        uint64_t o0 = pkt_off(out, lo), o1 = pkt_off(out, hi - 1) + (uint64_t)last_out;
-        uint64_t u0 = i0, u1 = i1;
-        if (in_place) {
-            u0 = std::min(i0, o0);
-            u1 = std::max(i1, o1);
-            o0 = u0;
-            o1 = u1;
-        }
-        if (u1 > u0)
-            HIPCHK(ctx, hipMemcpyAsync(d_in + (u0 - sin.lo), h_in + u0, u1 - u0, hipMemcpyHostToDevice, ctx->s_up));
-        if (!in_place && !rows_down && o1 > o0)
-            HIPCHK(ctx, hipMemcpyAsync(d_out + (o0 - sout.lo), h_out + o0, o1 - o0, hipMemcpyHostToDevice, ctx->s_up));
-        HIPCHK(ctx, hipEventRecord(ctx->ev_up[k], ctx->s_up));
-        HIPCHK(ctx, hipStreamWaitEvent(ctx->stream, ctx->ev_up[k], 0));
+    a.in = hp.d_in;
+    a.out = hp.d_out;
+    a.in_off = hp.d_in_off;
+    a.out_off = hp.d_out_off;
+    rc = hp.open_gate();
+    if (rc) return rc;
+    for (uint32_t k = 0; k < hp.chunks; k++) {
+        uint32_t lo, hi;
+        if (!hp.range(k, &lo, &hi)) break;
+        rc = hp.upload(k);
+        if (rc) return rc;
         AeadArgs c = a;
         c.first = lo;
         c.n = hi - lo;
@@ -161,21 +76,11 @@ int aead_batch_host_chunked(bnk_ctx *ctx, bool open, const bnk_batch *in, const 
             c.order = ctx->order.as<uint32_t>() + lo;
         }
         HIPCHK(ctx, open ? launch_aead_open(c, ctx->stream) : launch_aead_seal(c, ctx->stream));
-        HIPCHK(ctx, hipEventRecord(ctx->ev_done[k], ctx->stream));
-        HIPCHK(ctx, hipStreamWaitEvent(ctx->s_down, ctx->ev_done[k], 0));
-        if (rows_down) {
-            const uint64_t width = (uint64_t)std::max<int64_t>((int64_t)in->len + out_delta, 0);
-            if (width)
-                HIPCHK(ctx, hipMemcpy2DAsync(h_out + o0, out->stride, d_out + (o0 - sout.lo), out->stride, width,
-                                             hi - lo, hipMemcpyDeviceToHost, ctx->s_down));
-        } else if (o1 > o0) {
-            HIPCHK(ctx, hipMemcpyAsync(h_out + o0, d_out + (o0 - sout.lo), o1 - o0, hipMemcpyDeviceToHost, ctx->s_down));
-        }
-        if (open)
-            HIPCHK(ctx, hipMemcpyAsync(h_verdict + lo, a.verdict + lo, hi - lo, hipMemcpyDeviceToHost, ctx->s_down));
+        rc = hp.download(k);
+        if (rc) return rc;
     }
-    HIPCHK(ctx, hipStreamSynchronize(ctx->s_down));
-    if (open) memcpy(verdict, h_verdict, n);
+    rc = hp.finish();
+    if (rc) return rc;
     uint32_t status = 0;
     rc = take_status(ctx, &status);
     if (rc) return rc;

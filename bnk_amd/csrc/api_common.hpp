@@ -5,6 +5,7 @@
 #include <string.h>
 
 #include <algorithm>
+#include <functional>
 #include <new>
 #include <string>
 
@@ -203,6 +204,184 @@ inline int maybe_sort(bnk_ctx *ctx, const uint32_t *d_lens, uint32_t n, uint32_t
     *order = ctx->order.as<uint32_t>();
     return BNK_OK;
 }
+
+// ---------------------------------------------------------------------------
+// Chunked host batches.  While chunk k is computed, chunk k+1 is on its way up
+// and chunk k-1 on its way down (the link is full duplex): three streams, one
+// event pair per chunk.  Needs packets laid out in ascending, non-overlapping
+// order in both arenas, so that a run of consecutive packets is one contiguous
+// span.
+// ---------------------------------------------------------------------------
+constexpr uint32_t PIPE_MAX_CHUNKS = 16;
+constexpr uint64_t PIPE_MIN_CHUNK_BYTES = 4ull << 20;
+
+struct HostPipe {
+    bnk_ctx *ctx = nullptr;
+    const bnk_batch *in = nullptr, *out = nullptr;
+    uint32_t n = 0, chunks = 0, per = 0;
+    Span sin, sout;
+    bool in_place = false;
+    uint64_t row_width = 0; // > 0: the output comes back row by row (uniform layout, see plan)
+    uint8_t *d_in = nullptr, *d_out = nullptr;
+    const uint64_t *d_in_off = nullptr, *d_out_off = nullptr;
+
+    // Bytes packet i occupies from its offset in the input / output arena.
+    std::function<uint64_t(uint32_t)> in_ext, out_ext;
+
+    struct Result {
+        void *host;
+        const void *dev;
+        uint32_t elem;
+        size_t pin_off;
+    };
+    std::vector<Result> results;
+    size_t pin_used = 0;
+
+    // BNK_OK, an error code, or 1 when the batch does not qualify (too small, or
+    // not ascending) and the caller should take the single-shot route.
+    // uniform_out_width: the output extent when every packet has the same one
+    // and the layout is a uniform stride (then the gaps between output packets
+    // never need to be on the device), else 0.
+    int plan(uint64_t uniform_out_width)
+    {
+        n = in->n;
+        uint64_t in_end = 0, out_end = 0;
+        for (uint32_t i = 0; i < n; i++) {
+            const uint64_t io = pkt_off(in, i), ie = in_ext(i), oo = pkt_off(out, i), oe = out_ext(i);
+            if (io > in->bytes || ie > in->bytes - io)
+                return fail(ctx, BNK_E_INVAL, "in: packet " + std::to_string(i) + " lies outside the arena");
+            if (oo > out->bytes || oe > out->bytes - oo)
+                return fail(ctx, BNK_E_INVAL, "out: packet " + std::to_string(i) + " lies outside the arena");
+            if (io < in_end || oo < out_end) return 1;
+            in_end = io + ie;
+            out_end = oo + oe;
+            sin.add(io, io + ie);
+            sout.add(oo, oo + oe);
+        }
+        const uint32_t by_bytes =
+            (uint32_t)std::min<uint64_t>(std::max(sin.size(), sout.size()) / PIPE_MIN_CHUNK_BYTES, PIPE_MAX_CHUNKS);
+        if (by_bytes < 2 || n < 2u * 64u) return 1;
+        chunks = by_bytes;
+        per = ((n + chunks - 1u) / chunks + 63u) & ~63u; // whole waves per chunk
+        if (!ctx->s_up) HIPCHK(ctx, hipStreamCreateWithFlags(&ctx->s_up, hipStreamNonBlocking));
+        if (!ctx->s_down) HIPCHK(ctx, hipStreamCreateWithFlags(&ctx->s_down, hipStreamNonBlocking));
+        while (ctx->ev_up.size() < chunks + 1u || ctx->ev_done.size() < chunks) {
+            hipEvent_t a, b;
+            HIPCHK(ctx, hipEventCreateWithFlags(&a, hipEventDisableTiming));
+            ctx->ev_up.push_back(a);
+            HIPCHK(ctx, hipEventCreateWithFlags(&b, hipEventDisableTiming));
+            ctx->ev_done.push_back(b);
+        }
+        in_place = same_layout(in, out);
+        if (in_place) {
+            sin.add(sout.lo, sout.hi);
+            sout = sin;
+        }
+        row_width = (!in_place && !out->offsets) ? uniform_out_width : 0;
+        HIPCHK(ctx, ctx->in_arena.reserve(sin.size() + 16));
+        d_in = d_out = ctx->in_arena.as<uint8_t>();
+        if (!in_place) {
+            HIPCHK(ctx, ctx->out_arena.reserve(sout.size() + 16));
+            d_out = ctx->out_arena.as<uint8_t>();
+        }
+        pin_used = (size_t)n * 16; // the two rebased offset arrays
+        return BNK_OK;
+    }
+
+    // A per-packet result array that comes back chunk by chunk.  Downloads go
+    // through pinned staging: a copy into pageable memory would make the
+    // runtime wait for it and stall the pipeline.
+    void add_result(void *host, const void *dev, uint32_t elem)
+    {
+        results.push_back(Result{host, dev, elem, pin_used});
+        pin_used += ((size_t)n * elem + 15u) & ~size_t(15);
+    }
+
+    // Uploads the offset arrays (on the compute stream) and opens the pipeline.
+    int begin()
+    {
+        HIPCHK(ctx, ctx->pin.reserve(pin_used + 64));
+        int rc = upload_offsets(ctx, in, n, sin.lo, &ctx->off_in, 0, &d_in_off);
+        if (rc) return rc;
+        if (in_place) d_out_off = d_in_off;
+        else {
+            rc = upload_offsets(ctx, out, n, sout.lo, &ctx->off_out, (size_t)n * 8, &d_out_off);
+            if (rc) return rc;
+        }
+        return BNK_OK;
+    }
+    // After every other whole-batch upload has been queued on the compute stream.
+    int open_gate()
+    {
+        HIPCHK(ctx, hipEventRecord(ctx->ev_up[chunks], ctx->stream));
+        HIPCHK(ctx, hipStreamWaitEvent(ctx->s_up, ctx->ev_up[chunks], 0));
+        return BNK_OK;
+    }
+
+    bool range(uint32_t k, uint32_t *lo, uint32_t *hi) const
+    {
+        *lo = k * per;
+        *hi = std::min(n, *lo + per);
+        return *lo < *hi;
+    }
+
+    // Queues chunk k's upload and makes the compute stream wait for it.
+    int upload(uint32_t k)
+    {
+        uint32_t lo, hi;
+        if (!range(k, &lo, &hi)) return BNK_OK;
+        const uint8_t *h_in = (const uint8_t *)in->base;
+        const uint8_t *h_out = (const uint8_t *)out->base;
+        uint64_t u0 = pkt_off(in, lo), u1 = pkt_off(in, hi - 1) + in_ext(hi - 1);
+        const uint64_t o0 = pkt_off(out, lo), o1 = pkt_off(out, hi - 1) + out_ext(hi - 1);
+        if (in_place) {
+            u0 = std::min(u0, o0);
+            u1 = std::max(u1, o1);
+        }
+        if (u1 > u0)
+            HIPCHK(ctx, hipMemcpyAsync(d_in + (u0 - sin.lo), h_in + u0, u1 - u0, hipMemcpyHostToDevice, ctx->s_up));
+        // any layout that does not come back row by row first takes the host's
+        // output bytes up, so that what lies between packets comes back unchanged
+        if (!in_place && !row_width && o1 > o0)
+            HIPCHK(ctx, hipMemcpyAsync(d_out + (o0 - sout.lo), h_out + o0, o1 - o0, hipMemcpyHostToDevice, ctx->s_up));
+        HIPCHK(ctx, hipEventRecord(ctx->ev_up[k], ctx->s_up));
+        HIPCHK(ctx, hipStreamWaitEvent(ctx->stream, ctx->ev_up[k], 0));
+        return BNK_OK;
+    }
+
+    // After chunk k's kernels have been queued on the compute stream.
+    int download(uint32_t k)
+    {
+        uint32_t lo, hi;
+        if (!range(k, &lo, &hi)) return BNK_OK;
+        uint8_t *h_out = (uint8_t *)out->base;
+        HIPCHK(ctx, hipEventRecord(ctx->ev_done[k], ctx->stream));
+        HIPCHK(ctx, hipStreamWaitEvent(ctx->s_down, ctx->ev_done[k], 0));
+        uint64_t o0 = pkt_off(out, lo), o1 = pkt_off(out, hi - 1) + out_ext(hi - 1);
+        if (in_place) {
+            o0 = std::min(o0, pkt_off(in, lo));
+            o1 = std::max(o1, pkt_off(in, hi - 1) + in_ext(hi - 1));
+        }
+        if (row_width)
+            HIPCHK(ctx, hipMemcpy2DAsync(h_out + o0, out->stride, d_out + (o0 - sout.lo), out->stride, row_width,
+                                         hi - lo, hipMemcpyDeviceToHost, ctx->s_down));
+        else if (o1 > o0)
+            HIPCHK(ctx, hipMemcpyAsync(h_out + o0, d_out + (o0 - sout.lo), o1 - o0, hipMemcpyDeviceToHost, ctx->s_down));
+        for (const Result &r : results)
+            HIPCHK(ctx, hipMemcpyAsync(ctx->pin.as<uint8_t>() + r.pin_off + (size_t)lo * r.elem,
+                                       (const uint8_t *)r.dev + (size_t)lo * r.elem, (size_t)(hi - lo) * r.elem,
+                                       hipMemcpyDeviceToHost, ctx->s_down));
+        return BNK_OK;
+    }
+
+    // Waits for the last download and hands the result arrays over.
+    int finish()
+    {
+        HIPCHK(ctx, hipStreamSynchronize(ctx->s_down));
+        for (const Result &r : results) memcpy(r.host, ctx->pin.as<uint8_t>() + r.pin_off, (size_t)n * r.elem);
+        return BNK_OK;
+    }
+};
 
 // Reads and clears the device status word (waits for the stream).
 int take_status(bnk_ctx *ctx, uint32_t *status);

@@ -96,6 +96,10 @@ extern "C" int bnk_wg_encap_batch(bnk_ctx *ctx, const bnk_batch *slots, uint32_t
     if (!ctx->d_keys[BNK_KEYS_SEND] || ctx->n_keys[BNK_KEYS_SEND] < ctx->n_wg_peers)
         return fail(ctx, BNK_E_STATE, "send key table is smaller than the peer table");
     const bool host = slots->mem == BNK_MEM_HOST;
+    const auto slot_ext = [slots, mtu](uint32_t i) {
+        const uint32_t len = slots->lens ? slots->lens[i] : slots->len;
+        return 16ull + len + wg_padding_host(len, mtu) + 16ull;
+    };
 
     WgBatch b{};
     b.n = n;
@@ -104,25 +108,43 @@ extern "C" int bnk_wg_encap_batch(bnk_ctx *ctx, const bnk_batch *slots, uint32_t
     const uint32_t *d_peer = nullptr;
     uint32_t *d_wire_len = nullptr;
     Span span;
+    HostPipe hp;
+    bool chunked = false;
     if (host) {
-        for (uint32_t i = 0; i < n; i++) {
-            const uint64_t off = pkt_off(slots, i);
-            const uint32_t len = slots->lens ? slots->lens[i] : slots->len;
-            const uint64_t need = 16ull + len + wg_padding_host(len, mtu) + 16ull;
-            if (off > slots->bytes || need > slots->bytes - off)
-                return fail(ctx, BNK_E_INVAL, "slots: packet " + std::to_string(i) + " lies outside the arena");
-            if (slots->peer && slots->peer[i] >= ctx->n_wg_peers)
-                return fail(ctx, BNK_E_RANGE, "peer index " + std::to_string(slots->peer[i]) +
-                                                  " beyond the peer table");
-            span.add(off, off + need);
+        if (slots->peer)
+            for (uint32_t i = 0; i < n; i++)
+                if (slots->peer[i] >= ctx->n_wg_peers)
+                    return fail(ctx, BNK_E_RANGE, "peer index " + std::to_string(slots->peer[i]) +
+                                                      " beyond the peer table");
+        HIPCHK(ctx, ctx->wg_wirelen.reserve((size_t)n * 4));
+        d_wire_len = ctx->wg_wirelen.as<uint32_t>();
+        hp.ctx = ctx;
+        hp.in = hp.out = slots;
+        hp.in_ext = hp.out_ext = slot_ext;
+        rc = hp.plan(0);
+        if (rc != BNK_OK && rc != 1) return rc;
+        chunked = rc == BNK_OK;
+        if (chunked) {
+            hp.add_result(wire_len, d_wire_len, 4);
+            rc = hp.begin();
+            if (rc) return rc;
+            b.base = hp.d_in;
+            b.off = hp.d_in_off;
+        } else {
+            for (uint32_t i = 0; i < n; i++) {
+                const uint64_t off = pkt_off(slots, i), need = slot_ext(i);
+                if (off > slots->bytes || need > slots->bytes - off)
+                    return fail(ctx, BNK_E_INVAL, "slots: packet " + std::to_string(i) + " lies outside the arena");
+                span.add(off, off + need);
+            }
+            HIPCHK(ctx, ctx->pin.reserve((size_t)n * 16 + 64));
+            HIPCHK(ctx, ctx->in_arena.reserve(span.size() + 16));
+            HIPCHK(ctx, hipMemcpyAsync(ctx->in_arena.p, (const uint8_t *)slots->base + span.lo, span.size(),
+                                       hipMemcpyHostToDevice, ctx->stream));
+            b.base = ctx->in_arena.as<uint8_t>();
+            rc = upload_offsets(ctx, slots, n, span.lo, &ctx->off_in, 0, &b.off);
+            if (rc) return rc;
         }
-        HIPCHK(ctx, ctx->pin.reserve((size_t)n * 16 + 64));
-        HIPCHK(ctx, ctx->in_arena.reserve(span.size() + 16));
-        HIPCHK(ctx, hipMemcpyAsync(ctx->in_arena.p, (const uint8_t *)slots->base + span.lo, span.size(),
-                                   hipMemcpyHostToDevice, ctx->stream));
-        b.base = ctx->in_arena.as<uint8_t>();
-        rc = upload_offsets(ctx, slots, n, span.lo, &ctx->off_in, 0, &b.off);
-        if (rc) return rc;
         if (slots->lens) {
             rc = upload(ctx, &ctx->lens, slots->lens, (size_t)n * 4);
             if (rc) return rc;
@@ -133,12 +155,9 @@ extern "C" int bnk_wg_encap_batch(bnk_ctx *ctx, const bnk_batch *slots, uint32_t
             if (rc) return rc;
             d_peer = ctx->peer.as<uint32_t>();
         }
-        HIPCHK(ctx, ctx->wg_wirelen.reserve((size_t)n * 4));
-        d_wire_len = ctx->wg_wirelen.as<uint32_t>();
     } else {
         if (!slots->offsets && !slots->lens &&
-            (uint64_t)(n - 1) * slots->stride + 16ull + slots->len + wg_padding_host(slots->len, mtu) + 16ull >
-                slots->bytes)
+            (uint64_t)(n - 1) * slots->stride + slot_ext(0) > slots->bytes)
             return fail(ctx, BNK_E_INVAL, "slots: uniform layout exceeds the arena");
         b.base = (const uint8_t *)slots->base;
         b.off = slots->offsets;
@@ -153,43 +172,72 @@ extern "C" int bnk_wg_encap_batch(bnk_ctx *ctx, const bnk_batch *slots, uint32_t
     HIPCHK(ctx, ctx->wg_skip.reserve(n));
     const size_t tmp_bytes = relay_sort_tmp_bytes(n, ctx->n_wg_peers);
     HIPCHK(ctx, ctx->r_tmp.reserve(tmp_bytes + 16));
+    if (slots->lens) {
+        HIPCHK(ctx, ctx->order.reserve((size_t)n * 4));
+        HIPCHK(ctx, ctx->hist.reserve(LEN_BINS * 4));
+        HIPCHK(ctx, ctx->cursor.reserve(LEN_BINS * 4));
+    }
     const WgPeersDev pe = peers_view(ctx);
     uint64_t *d_ctr = ctx->r_ctr_out.as<uint64_t>();
     uint32_t *d_padded = ctx->wg_padded.as<uint32_t>();
     uint8_t *d_skip = ctx->wg_skip.as<uint8_t>();
 
-    // counters in batch order per peer, advancing the peers' send counters
+    // counters in batch order per peer, advancing the peers' send counters:
+    // needs the peer array only, so it runs ahead of the packet bytes
     HIPCHK(ctx, launch_wg_keys(d_peer, pe.n, n, ctx->r_keys.as<uint32_t>(), ctx->r_idx.as<uint32_t>(),
                                ctx->d_status, ctx->stream));
     HIPCHK(ctx, launch_peer_rank(ctx->r_keys.as<uint32_t>(), ctx->r_idx.as<uint32_t>(),
                                  ctx->r_skeys.as<uint32_t>(), ctx->r_sidx.as<uint32_t>(), ctx->r_tmp.p,
                                  tmp_bytes, pe.send_ctr, pe.n, n, d_ctr, true, ctx->stream));
-    HIPCHK(ctx, launch_wg_encap_prep(b, pe, d_peer, d_ctr, mtu, d_padded, d_wire_len, d_skip, ctx->stream));
 
-    AeadArgs se{};
-    se.keys = ctx->d_keys[BNK_KEYS_SEND];
-    se.n_peers = pe.n;
-    se.status = ctx->d_status;
-    se.n = n;
-    se.in = b.base;
-    se.out = const_cast<uint8_t *>(b.base);
-    se.in_off = se.out_off = b.off;
-    se.in_stride = se.out_stride = slots->stride;
-    se.in_skip = se.out_skip = 16;
-    se.lens = d_padded;
-    se.peer = d_peer;
-    se.counters = d_ctr;
-    se.skip = d_skip;
-    if (slots->lens) { // equal plaintext lengths pad to equal lengths
-        rc = maybe_sort(ctx, se.lens, n, 0, &se.order);
+    // header, padding and seal of packets [lo, hi)
+    auto run = [&](uint32_t lo, uint32_t hi) -> int {
+        WgBatch c = b;
+        c.first = lo;
+        c.n = hi - lo;
+        HIPCHK(ctx, launch_wg_encap_prep(c, pe, d_peer, d_ctr, mtu, d_padded, d_wire_len, d_skip, ctx->stream));
+        AeadArgs se{};
+        se.keys = ctx->d_keys[BNK_KEYS_SEND];
+        se.n_peers = pe.n;
+        se.status = ctx->d_status;
+        se.first = lo;
+        se.n = hi - lo;
+        se.in = b.base;
+        se.out = const_cast<uint8_t *>(b.base);
+        se.in_off = se.out_off = b.off;
+        se.in_stride = se.out_stride = slots->stride;
+        se.in_skip = se.out_skip = 16;
+        se.lens = d_padded;
+        se.peer = d_peer;
+        se.counters = d_ctr;
+        se.skip = d_skip;
+        if (slots->lens && se.n > 64) { // equal plaintext lengths pad to equal lengths
+            HIPCHK(ctx, launch_length_sort(d_padded + lo, se.n, 0, ctx->order.as<uint32_t>() + lo,
+                                           ctx->hist.as<uint32_t>(), ctx->cursor.as<uint32_t>(), ctx->stream));
+            se.order = ctx->order.as<uint32_t>() + lo;
+        }
+        HIPCHK(ctx, launch_aead_seal(se, ctx->stream));
+        return BNK_OK;
+    };
+
+    if (chunked) {
+        rc = hp.open_gate();
         if (rc) return rc;
+        for (uint32_t k = 0; k < hp.chunks; k++) {
+            uint32_t lo, hi;
+            if (!hp.range(k, &lo, &hi)) break;
+            if ((rc = hp.upload(k)) || (rc = run(lo, hi)) || (rc = hp.download(k))) return rc;
+        }
+        rc = hp.finish();
+        if (rc) return rc;
+    } else {
+        rc = run(0, n);
+        if (rc) return rc;
+        if (!host) return BNK_OK;
+        HIPCHK(ctx, hipMemcpyAsync((uint8_t *)slots->base + span.lo, ctx->in_arena.p, span.size(),
+                                   hipMemcpyDeviceToHost, ctx->stream));
+        HIPCHK(ctx, hipMemcpyAsync(wire_len, d_wire_len, (size_t)n * 4, hipMemcpyDeviceToHost, ctx->stream));
     }
-    HIPCHK(ctx, launch_aead_seal(se, ctx->stream));
-    if (!host) return BNK_OK;
-
-    HIPCHK(ctx, hipMemcpyAsync((uint8_t *)slots->base + span.lo, ctx->in_arena.p, span.size(),
-                               hipMemcpyDeviceToHost, ctx->stream));
-    HIPCHK(ctx, hipMemcpyAsync(wire_len, d_wire_len, (size_t)n * 4, hipMemcpyDeviceToHost, ctx->stream));
     uint32_t status = 0;
     rc = take_status(ctx, &status);
     if (rc) return rc;
@@ -223,17 +271,19 @@ extern "C" int bnk_wg_decap_batch(bnk_ctx *ctx, const bnk_batch *wire, const bnk
     uint32_t *d_out_len = nullptr, *d_peer = nullptr;
     uint64_t *d_counter = nullptr;
     Staged st;
+    HostPipe hp;
+    bool chunked = false;
+    bnk_batch w2 = *wire; // the sender's identity comes out of the datagrams, not in with them
+    w2.peer = nullptr;
+    w2.counters = nullptr;
+    // the pipeline keeps these until the call returns: they live at function scope
+    // and hold copies of what they need
+    const auto wire_ext = [wire](uint32_t i) { return (uint64_t)(wire->lens ? wire->lens[i] : wire->len); };
+    const auto plain_ext = [wire](uint32_t i) {
+        const uint64_t l = wire->lens ? wire->lens[i] : wire->len;
+        return l >= 32u ? l - 32u : (uint64_t)0;
+    };
     if (host) {
-        bnk_batch w2 = *wire;
-        w2.peer = nullptr;
-        w2.counters = nullptr;
-        rc = stage_host(ctx, &w2, out, -32, 0, &st);
-        if (rc) return rc;
-        wb.base = st.d_in;
-        wb.off = st.d_in_off;
-        wb.lens = st.d_lens;
-        ob.base = st.d_out;
-        ob.off = st.d_out_off;
         HIPCHK(ctx, ctx->wg_result.reserve(n));
         HIPCHK(ctx, ctx->wg_outlen.reserve((size_t)n * 4));
         HIPCHK(ctx, ctx->wg_peer.reserve((size_t)n * 4));
@@ -242,6 +292,39 @@ extern "C" int bnk_wg_decap_batch(bnk_ctx *ctx, const bnk_batch *wire, const bnk
         d_out_len = ctx->wg_outlen.as<uint32_t>();
         d_peer = ctx->wg_peer.as<uint32_t>();
         d_counter = ctx->wg_counter.as<uint64_t>();
+        hp.ctx = ctx;
+        hp.in = &w2;
+        hp.out = out;
+        hp.in_ext = wire_ext;
+        hp.out_ext = plain_ext;
+        rc = hp.plan(wire->lens ? 0 : plain_ext(0));
+        if (rc != BNK_OK && rc != 1) return rc;
+        chunked = rc == BNK_OK;
+        if (chunked) {
+            hp.add_result(result, d_result, 1);
+            hp.add_result(out_len, d_out_len, 4);
+            hp.add_result(peer, d_peer, 4);
+            hp.add_result(counter, d_counter, 8);
+            rc = hp.begin();
+            if (rc) return rc;
+            wb.base = hp.d_in;
+            wb.off = hp.d_in_off;
+            ob.base = hp.d_out;
+            ob.off = hp.d_out_off;
+            if (wire->lens) {
+                rc = upload(ctx, &ctx->lens, wire->lens, (size_t)n * 4);
+                if (rc) return rc;
+                wb.lens = ctx->lens.as<uint32_t>();
+            }
+        } else {
+            rc = stage_host(ctx, &w2, out, -32, 0, &st);
+            if (rc) return rc;
+            wb.base = st.d_in;
+            wb.off = st.d_in_off;
+            wb.lens = st.d_lens;
+            ob.base = st.d_out;
+            ob.off = st.d_out_off;
+        }
     } else {
         if (!wire->offsets && !wire->lens && (uint64_t)(n - 1) * wire->stride + wire->len > wire->bytes)
             return fail(ctx, BNK_E_INVAL, "wire: uniform layout exceeds the arena");
@@ -260,43 +343,70 @@ extern "C" int bnk_wg_decap_batch(bnk_ctx *ctx, const bnk_batch *wire, const bnk
     }
     HIPCHK(ctx, ctx->wg_ctlen.reserve((size_t)n * 4));
     HIPCHK(ctx, ctx->r_auth.reserve(n));
+    if (wire->lens) {
+        HIPCHK(ctx, ctx->order.reserve((size_t)n * 4));
+        HIPCHK(ctx, ctx->hist.reserve(LEN_BINS * 4));
+        HIPCHK(ctx, ctx->cursor.reserve(LEN_BINS * 4));
+    }
     uint32_t *d_ctlen = ctx->wg_ctlen.as<uint32_t>();
     uint8_t *d_auth = ctx->r_auth.as<uint8_t>();
     const WgPeersDev pe = peers_view(ctx);
 
-    HIPCHK(ctx, launch_wg_parse(wb, pe, d_peer, d_counter, d_ctlen, d_result, ctx->stream));
+    // parse, open and check packets [lo, hi)
+    auto run = [&](uint32_t lo, uint32_t hi) -> int {
+        WgBatch cw = wb, co = ob;
+        cw.first = co.first = lo;
+        cw.n = co.n = hi - lo;
+        HIPCHK(ctx, launch_wg_parse(cw, pe, d_peer, d_counter, d_ctlen, d_result, ctx->stream));
+        AeadArgs op{};
+        op.keys = ctx->d_keys[BNK_KEYS_RECV];
+        op.n_peers = pe.n;
+        op.status = ctx->d_status;
+        op.first = lo;
+        op.n = hi - lo;
+        op.in = wb.base;
+        op.in_off = wb.off;
+        op.in_stride = wire->stride;
+        op.in_skip = 16;
+        op.out = const_cast<uint8_t *>(ob.base);
+        op.out_off = ob.off;
+        op.out_stride = out->stride;
+        op.lens = d_ctlen;
+        op.peer = d_peer;
+        op.counters = d_counter;
+        op.verdict = d_auth;
+        op.skip = d_result; // BNK_WG_OK is 0: header failures are not opened
+        if (wire->lens && op.n > 64) {
+            HIPCHK(ctx, launch_length_sort(d_ctlen + lo, op.n, 16, ctx->order.as<uint32_t>() + lo,
+                                           ctx->hist.as<uint32_t>(), ctx->cursor.as<uint32_t>(), ctx->stream));
+            op.order = ctx->order.as<uint32_t>() + lo;
+        }
+        HIPCHK(ctx, launch_aead_open(op, ctx->stream));
+        HIPCHK(ctx, launch_wg_finish(co, 0, pe, d_peer, d_ctlen, d_auth, d_result, d_out_len, ctx->stream));
+        return BNK_OK;
+    };
 
-    AeadArgs op{};
-    op.keys = ctx->d_keys[BNK_KEYS_RECV];
-    op.n_peers = pe.n;
-    op.status = ctx->d_status;
-    op.n = n;
-    op.in = wb.base;
-    op.in_off = wb.off;
-    op.in_stride = wire->stride;
-    op.in_skip = 16;
-    op.out = const_cast<uint8_t *>(ob.base);
-    op.out_off = ob.off;
-    op.out_stride = out->stride;
-    op.lens = d_ctlen;
-    op.peer = d_peer;
-    op.counters = d_counter;
-    op.verdict = d_auth;
-    op.skip = d_result; // BNK_WG_OK is 0: header failures are not opened
-    if (wire->lens) {
-        rc = maybe_sort(ctx, op.lens, n, 16, &op.order);
+    if (chunked) {
+        rc = hp.open_gate();
         if (rc) return rc;
+        for (uint32_t k = 0; k < hp.chunks; k++) {
+            uint32_t lo, hi;
+            if (!hp.range(k, &lo, &hi)) break;
+            if ((rc = hp.upload(k)) || (rc = run(lo, hi)) || (rc = hp.download(k))) return rc;
+        }
+        rc = hp.finish();
+        if (rc) return rc;
+    } else {
+        rc = run(0, n);
+        if (rc) return rc;
+        if (!host) return BNK_OK;
+        HIPCHK(ctx, hipMemcpyAsync((uint8_t *)out->base + st.sout.lo, st.d_out, st.sout.size(),
+                                   hipMemcpyDeviceToHost, ctx->stream));
+        HIPCHK(ctx, hipMemcpyAsync(result, d_result, n, hipMemcpyDeviceToHost, ctx->stream));
+        HIPCHK(ctx, hipMemcpyAsync(out_len, d_out_len, (size_t)n * 4, hipMemcpyDeviceToHost, ctx->stream));
+        HIPCHK(ctx, hipMemcpyAsync(peer, d_peer, (size_t)n * 4, hipMemcpyDeviceToHost, ctx->stream));
+        HIPCHK(ctx, hipMemcpyAsync(counter, d_counter, (size_t)n * 8, hipMemcpyDeviceToHost, ctx->stream));
     }
-    HIPCHK(ctx, launch_aead_open(op, ctx->stream));
-    HIPCHK(ctx, launch_wg_finish(ob, 0, pe, d_peer, d_ctlen, d_auth, d_result, d_out_len, ctx->stream));
-    if (!host) return BNK_OK;
-
-    HIPCHK(ctx, hipMemcpyAsync((uint8_t *)out->base + st.sout.lo, st.d_out, st.sout.size(),
-                               hipMemcpyDeviceToHost, ctx->stream));
-    HIPCHK(ctx, hipMemcpyAsync(result, d_result, n, hipMemcpyDeviceToHost, ctx->stream));
-    HIPCHK(ctx, hipMemcpyAsync(out_len, d_out_len, (size_t)n * 4, hipMemcpyDeviceToHost, ctx->stream));
-    HIPCHK(ctx, hipMemcpyAsync(peer, d_peer, (size_t)n * 4, hipMemcpyDeviceToHost, ctx->stream));
-    HIPCHK(ctx, hipMemcpyAsync(counter, d_counter, (size_t)n * 8, hipMemcpyDeviceToHost, ctx->stream));
     uint32_t status = 0;
     rc = take_status(ctx, &status);
     if (rc) return rc;

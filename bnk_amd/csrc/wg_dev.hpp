@@ -19,6 +19,7 @@ struct WgBatch {
     const uint64_t *off;  // or nullptr: i * stride
     const uint32_t *lens; // or nullptr: len
     uint32_t n, stride, len;
+    uint32_t first; // the launch covers packets first .. first+n-1 of the arrays
 };
 
 hipError_t launch_wg_parse(const WgBatch &b, const WgPeersDev &pe, uint32_t *peer, uint64_t *counter,

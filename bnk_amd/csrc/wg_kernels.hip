@@ -36,8 +36,9 @@ __global__ __launch_bounds__(256) void wg_parse_kernel(WgBatch b, WgPeersDev pe,
                                                        uint64_t *counter, uint32_t *ct_len,
                                                        uint8_t *result)
 {
-    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
-    if (i >= b.n) return;
+    const uint32_t t = blockIdx.x * 256u + threadIdx.x;
+    if (t >= b.n) return;
+    const uint32_t i = b.first + t;
     const uint8_t *w = b.base + (b.off ? b.off[i] : (uint64_t)i * b.stride);
     const uint32_t len = b.lens ? b.lens[i] : b.len;
     peer[i] = 0xFFFFFFFFu;
@@ -70,8 +71,9 @@ __global__ __launch_bounds__(256) void wg_finish_kernel(WgBatch out, uint32_t ou
                                                         const uint8_t *auth, uint8_t *result,
                                                         uint32_t *out_len)
 {
-    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
-    if (i >= out.n) return;
+    const uint32_t t = blockIdx.x * 256u + threadIdx.x;
+    if (t >= out.n) return;
+    const uint32_t i = out.first + t;
     out_len[i] = 0;
     if (result[i] != BNK_WG_OK) return;
     if (!auth[i]) {
@@ -126,8 +128,9 @@ __global__ __launch_bounds__(256) void wg_encap_prep_kernel(WgBatch b, WgPeersDe
                                                             uint32_t *padded_len, uint32_t *wire_len,
                                                             uint8_t *skip)
 {
-    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
-    if (i >= b.n) return;
+    const uint32_t t = blockIdx.x * 256u + threadIdx.x;
+    if (t >= b.n) return;
+    const uint32_t i = b.first + t;
     const uint32_t pr = peer ? peer[i] : 0u;
     const uint32_t len = b.lens ? b.lens[i] : b.len;
     if (pr >= pe.n) {

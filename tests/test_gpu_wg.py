@@ -319,6 +319,86 @@ def test_encap_then_decap_round_trip_full_size():
     rx.close()
 
 
+def test_large_host_rings_take_the_chunked_route():
+    """Host rings of several chunks' worth (pinned, as a tunnel would use them):
+    encapsulate in place and decapsulate chunk by chunk with upload, kernels
+    and download overlapped; results equal the device-resident path's and a
+    sample equals the oracle."""
+    import torch
+    from bnk_amd import lib
+    from oracle import binding as O
+    rng = np.random.default_rng(31)
+    n, n_peers, stride = 24000, 64, 1536
+    keys = rng.integers(0, 256, (n_peers, 32), dtype=np.uint8)
+    idx_a = (np.arange(n_peers, dtype=np.uint32) * 7919 + 3).astype(np.uint32)
+    idx_b = (np.arange(n_peers, dtype=np.uint32) * 104729 + 11).astype(np.uint32)
+    addr = (0x64400000 + np.arange(n_peers, dtype=np.uint32)).astype(np.uint32)
+    full = np.full(n_peers, 0xFFFFFFFF, np.uint32)
+    peer = rng.integers(0, n_peers, n).astype(np.uint32)
+    lens = rng.choice([28, 60, 576, 1300, 1420], n).astype(np.uint32)
+    tx, rx = lib.Context(0), lib.Context(0)
+    tx.keys_set(lib.KEYS_SEND, keys)
+    tx.wg_peers_set(np.stack([idx_a, idx_b, addr, full], 1))
+    rx.keys_set(lib.KEYS_RECV, keys)
+    rx.wg_peers_set(np.stack([idx_b, idx_a, addr, full], 1))
+    ring = tx.ring_alloc(n * stride)
+    assert ring.nbytes > 8 * (4 << 20)
+    ring[:] = 0xEE
+    slots = ring.reshape(n, stride)
+    plain = rng.integers(0, 256, (n, 1420), dtype=np.uint8)
+    plain[:, 0] = 0x45
+    plain[:, 2] = (lens >> 8).astype(np.uint8)
+    plain[:, 3] = (lens & 0xFF).astype(np.uint8)
+    for k in range(4):
+        plain[:, 12 + k] = ((addr[peer] >> (24 - 8 * k)) & 0xFF).astype(np.uint8)
+    for L in np.unique(lens):
+        rows = np.flatnonzero(lens == L)
+        slots[rows, 16:16 + L] = plain[rows, :L]
+    wl = np.zeros(n, np.uint32)
+    tx.wg_encap(lib.make_batch(ring, ring.nbytes, n, lib.MEM_HOST, stride=stride, lens=lens, peer=peer),
+                MTU, wl)
+    pad = np.minimum((lens.astype(np.int64) + 15) // 16 * 16, MTU) - lens  # never beyond the MTU
+    assert np.array_equal(wl, (16 + lens + pad + 16).astype(np.uint32))
+    rank = np.zeros(n, np.uint64)
+    seen = np.zeros(n_peers, np.uint64)
+    for i in range(n):
+        rank[i] = seen[peer[i]]
+        seen[peer[i]] += 1
+    assert np.array_equal(tx.wg_send_counters(n_peers), seen)
+    for i in rng.choice(n, 48, replace=False):
+        p = int(peer[i])
+        w = O.wg_encap(plain[i, :lens[i]].tobytes(), MTU, keys[p].tobytes(), int(idx_b[p]), int(rank[i]))
+        assert slots[i, :len(w)].tobytes() == w
+        assert (slots[i, len(w):] == 0xEE).all()  # the rest of the slot came back untouched
+    # receive side: same ring as the wire, plaintext into a second ring
+    out = rx.ring_alloc(n * stride)
+    out[:] = 0x77
+    res = np.full(n, 99, np.uint8)
+    olen = np.zeros(n, np.uint32)
+    gp = np.zeros(n, np.uint32)
+    gc = np.zeros(n, np.uint64)
+    ring.reshape(n, stride)[5, 40] ^= 1  # one forged datagram
+    rx.wg_decap(lib.make_batch(ring, ring.nbytes, n, lib.MEM_HOST, stride=stride, lens=wl),
+                lib.make_batch(out[16:], out.nbytes - 16, n, lib.MEM_HOST, stride=stride),
+                res, olen, gp, gc)
+    want_res = np.zeros(n, np.uint8)
+    want_res[5] = O.WG_AUTH_FAIL
+    assert np.array_equal(res, want_res)
+    ok = res == 0
+    assert np.array_equal(olen[ok], lens[ok]) and olen[5] == 0
+    assert np.array_equal(gp, peer) and np.array_equal(gc, rank)
+    o2 = out.reshape(n, stride)
+    for L in np.unique(lens):
+        rows = np.flatnonzero((lens == L) & ok)
+        assert np.array_equal(o2[rows, 16:16 + L], plain[rows, :L])
+    assert (o2[:, :16] == 0x77).all()  # bytes between packets survive
+    assert not o2[5, 16:16 + int(wl[5]) - 32].any()  # a failed open leaves zeros
+    tx.ring_free(ring)
+    rx.ring_free(out)
+    tx.close()
+    rx.close()
+
+
 def test_wg_argument_errors():
     from bnk_amd import lib
     ctx = lib.Context(0)

@@ -377,7 +377,8 @@ def bench_host(args) -> dict:
     ctx.keys_set(lib.KEYS_RECV, key)
     nbytes = n * STRIDE
     plain, sealed, opened = (ctx.ring_alloc(nbytes) for _ in range(3))
-    plain.reshape(n, STRIDE)[:, :L] = W.rand_bytes(W.stream_seed(2, 1), n * L).reshape(n, L)
+    plain_copy = W.rand_bytes(W.stream_seed(2, 1), n * L).reshape(n, L)
+    plain.reshape(n, STRIDE)[:, :L] = plain_copy
     verdict = np.zeros(n, np.uint8)
     b_plain = lib.make_batch(plain, nbytes, n, lib.MEM_HOST, stride=STRIDE, length=L)
     b_sealed_out = lib.make_batch(sealed, nbytes, n, lib.MEM_HOST, stride=STRIDE)
@@ -397,6 +398,52 @@ def bench_host(args) -> dict:
     assert verdict.all() and np.array_equal(opened.reshape(n, STRIDE)[:, :L], plain.reshape(n, STRIDE)[:, :L])
     for r in (plain, sealed, opened):
         ctx.ring_free(r)
+    # the same through the framing entry points: encapsulate in place, decapsulate into a second ring
+    n_peers, wstride = 256, 1456
+    keys = W.rand_bytes(W.stream_seed(2, 40), n_peers * 32).reshape(n_peers, 32)
+    ia = (np.arange(n_peers, dtype=np.uint32) * 7919 + 3).astype(np.uint32)
+    ib = (np.arange(n_peers, dtype=np.uint32) * 104729 + 11).astype(np.uint32)
+    addr = (0x64400000 + np.arange(n_peers, dtype=np.uint32)).astype(np.uint32)
+    full = np.full(n_peers, 0xFFFFFFFF, np.uint32)
+    peer = W.rand_below(W.stream_seed(2, 41), n, n_peers).astype(np.uint32)
+    ctx.keys_set(lib.KEYS_SEND, keys)
+    ctx.wg_peers_set(np.stack([ia, ib, addr, full], 1))
+    rx = lib.Context(0)
+    rx.keys_set(lib.KEYS_RECV, keys)
+    rx.wg_peers_set(np.stack([ib, ia, addr, full], 1))
+    ring, out = ctx.ring_alloc(n * wstride), rx.ring_alloc(n * wstride + 16)
+    slots = ring.reshape(n, wstride)
+    slots[:, 16:16 + L] = plain_copy
+    slots[:, 16] = 0x45
+    slots[:, 18] = L >> 8
+    slots[:, 19] = L & 0xFF
+    for k in range(4):
+        slots[:, 28 + k] = ((addr[peer] >> (24 - 8 * k)) & 0xFF).astype(np.uint8)
+    wl = np.zeros(n, np.uint32)
+    res = np.zeros(n, np.uint8)
+    olen = np.zeros(n, np.uint32)
+    gp = np.zeros(n, np.uint32)
+    gc = np.zeros(n, np.uint64)
+    b_slots = lib.make_batch(ring, n * wstride, n, lib.MEM_HOST, stride=wstride, length=L, peer=peer)
+    b_wire = lib.make_batch(ring, n * wstride, n, lib.MEM_HOST, stride=wstride, length=L + 32)
+    b_out = lib.make_batch(out[16:], n * wstride, n, lib.MEM_HOST, stride=wstride)
+    wg_ms = []
+    for it in range(args.warmup + args.steps):
+        # the header fields the receive side checks were encrypted by the last round (untimed)
+        slots[:, 16] = 0x45
+        slots[:, 18] = L >> 8
+        slots[:, 19] = L & 0xFF
+        for k in range(4):
+            slots[:, 28 + k] = ((addr[peer] >> (24 - 8 * k)) & 0xFF).astype(np.uint8)
+        t0 = time.perf_counter()
+        ctx.wg_encap(b_slots, L, wl)
+        rx.wg_decap(b_wire, b_out, res, olen, gp, gc)
+        wg_ms.append((time.perf_counter() - t0) * 1e3)
+    assert (res == 0).all() and (olen == L).all() and np.array_equal(gp, peer)
+    wg = sum(wg_ms[args.warmup:]) / args.steps
+    ctx.ring_free(ring)
+    rx.ring_free(out)
+    rx.close()
     ctx.close()
     moved = 2 * (n * STRIDE + n * STRIDE)  # per step: arena up and arena down, twice
     return {
@@ -407,6 +454,10 @@ def bench_host(args) -> dict:
         "config": {"workload": "cfg2 through BNK_MEM_HOST: seal+open of %d packets x %d B from pinned host "
                                "rings, upload and download inside every call" % (n, L), "packets": n},
         "host_link_gb_per_s": round(moved / (ms * 1e-3) / 1e9, 1),
+        "framing": {"metric": "wg_encap_decap_gbit_per_s_host_memory",
+                    "value": round(n * L * 8 / (wg * 1e-3) / 1e9, 1), "ms_per_step": round(wg, 3),
+                    "workload": "encapsulate in place + decapsulate of the same packets through pinned "
+                                "rings, %d peers" % n_peers},
     }
 
 

@@ -159,38 +159,72 @@ BNK_DEV bool quad_hit(uint4 v, uint32_t key)
     return in_range(v.x, key) || in_range(v.y, key) || in_range(v.z, key) || in_range(v.w, key);
 }
 
-// iv: the packet's elementary source interval.  The kernel is bound by the
-// scattered 64-byte lines it pulls from L2 and beyond, so the interval's list
-// is a single such line (block iv), fetched with four 16-byte loads issued
-// together.  Only a list of more than 16 pieces goes through a second step,
-// finding its block by the block's first key.
-// (Fetching only the quads a list occupies was tried and is slower: the
-// branches around the loads cost more than the loads they save.)
-BNK_DEV bool rules_match(const RuleIndexDev &ri, uint32_t iv, uint32_t src, uint32_t key)
+// Value of x in lane J of this lane's quad (lanes 4k .. 4k+3).
+template <int J>
+BNK_DEV uint32_t quad_bcast(uint32_t x)
 {
-    const uint4 *blk = reinterpret_cast<const uint4 *>(ri.ranges + (size_t)iv * RANGE_BLOCK);
-    const uint4 v0 = blk[0], v1 = blk[1], v2 = blk[2], v3 = blk[3];
-    if (v0.x != RANGE_LONG) {
-        if (quad_hit(v0, key) || quad_hit(v1, key) || quad_hit(v2, key) || quad_hit(v3, key)) return true;
-    } else {
-        // last block whose first key_lo <= key; the ranges are sorted and
-        // disjoint, so only that block can hold the key
-        const uint4 *ob = reinterpret_cast<const uint4 *>(ri.ranges + (size_t)v0.y * RANGE_BLOCK);
-        uint32_t lo = 0, hi = v0.z;
-        while (hi - lo > 1u) {
-            const uint32_t mid = (lo + hi) >> 1;
-            if ((ob[4u * mid].x >> 14) <= key) lo = mid;
-            else hi = mid;
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, J | J << 2 | J << 4 | J << 6, 0xF, 0xF, true);
+}
+
+// A list of more than 16 pieces: head is the first quad of the interval's own
+// block, {RANGE_LONG, first block, blocks}.  Finds the block by its first key
+// (the ranges are sorted and disjoint, so only that block can hold the key).
+BNK_DEV bool long_list_hit(const RuleIndexDev &ri, uint32_t first, uint32_t nblk, uint32_t key)
+{
+    const uint4 *ob = reinterpret_cast<const uint4 *>(ri.ranges + (size_t)first * RANGE_BLOCK);
+    uint32_t lo = 0, hi = nblk;
+    while (hi - lo > 1u) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if ((ob[4u * mid].x >> 14) <= key) lo = mid;
+        else hi = mid;
+    }
+    const uint4 *b = ob + 4u * lo;
+    const uint4 w0 = b[0], w1 = b[1], w2 = b[2], w3 = b[3];
+    return quad_hit(w0, key) || quad_hit(w1, key) || quad_hit(w2, key) || quad_hit(w3, key);
+}
+
+// Rule lookup for the four packets of a quad of lanes at once; every lane of the
+// wave must call it (lanes without a packet pass iv 0 and ignore the answer).
+// The kernel is bound by the cache lookups its scattered loads cause, one per
+// distinct line per load instruction.  A lane fetching its own 64-byte block
+// with four 16-byte loads causes four; here the four lanes of a quad fetch one
+// packet's block together, 16 bytes each, which the memory pipeline sees as a
+// single 64-byte access, and do that for each of their four packets in turn.
+// Each lane tests its 16 bytes against the key of the packet they belong to and
+// the verdicts are gathered per quad with a wave-wide vote.
+BNK_DEV bool rules_match_quad(const RuleIndexDev &ri, uint32_t lane, uint32_t iv, uint32_t src, uint32_t key)
+{
+    const uint32_t part = lane & 3u, qshift = lane & ~3u;
+    const uint32_t *mine = ri.ranges + part * 4u;
+    const uint32_t iv0 = quad_bcast<0>(iv), iv1 = quad_bcast<1>(iv), iv2 = quad_bcast<2>(iv), iv3 = quad_bcast<3>(iv);
+    const uint4 p0 = *reinterpret_cast<const uint4 *>(mine + (size_t)iv0 * RANGE_BLOCK);
+    const uint4 p1 = *reinterpret_cast<const uint4 *>(mine + (size_t)iv1 * RANGE_BLOCK);
+    const uint4 p2 = *reinterpret_cast<const uint4 *>(mine + (size_t)iv2 * RANGE_BLOCK);
+    const uint4 p3 = *reinterpret_cast<const uint4 *>(mine + (size_t)iv3 * RANGE_BLOCK);
+    const unsigned long long h0 = __ballot(quad_hit(p0, quad_bcast<0>(key)));
+    const unsigned long long h1 = __ballot(quad_hit(p1, quad_bcast<1>(key)));
+    const unsigned long long h2 = __ballot(quad_hit(p2, quad_bcast<2>(key)));
+    const unsigned long long h3 = __ballot(quad_hit(p3, quad_bcast<3>(key)));
+    const unsigned long long hm = part == 0u ? h0 : part == 1u ? h1 : part == 2u ? h2 : h3;
+    bool hit = ((hm >> qshift) & 0xFull) != 0ull;
+    // a long list shows in the first word of its block, which the quad's first
+    // lane holds for round j as p<j>; the votes are taken by all lanes together
+    const unsigned long long l0 = __ballot(part == 0u && p0.x == RANGE_LONG);
+    const unsigned long long l1 = __ballot(part == 0u && p1.x == RANGE_LONG);
+    const unsigned long long l2 = __ballot(part == 0u && p2.x == RANGE_LONG);
+    const unsigned long long l3 = __ballot(part == 0u && p3.x == RANGE_LONG);
+    const unsigned long long lm = part == 0u ? l0 : part == 1u ? l1 : part == 2u ? l2 : l3;
+    if ((lm >> qshift) & 1ull) {
+        // rare: fetch the pointer words myself (the line is in L1 by now)
+        const uint4 head = *reinterpret_cast<const uint4 *>(ri.ranges + (size_t)iv * RANGE_BLOCK);
+        hit = long_list_hit(ri, head.y, head.z, key);
+    }
+    if (!hit)
+        for (uint32_t w = 0; w < ri.n_wide; w++) {
+            const uint4 r = ri.wide[w];
+            if ((src & r.y) == r.x && key >= r.z && key <= r.w) hit = true;
         }
-        const uint4 *b = ob + 4u * lo;
-        const uint4 w0 = b[0], w1 = b[1], w2 = b[2], w3 = b[3];
-        if (quad_hit(w0, key) || quad_hit(w1, key) || quad_hit(w2, key) || quad_hit(w3, key)) return true;
-    }
-    for (uint32_t w = 0; w < ri.n_wide; w++) {
-        const uint4 r = ri.wide[w];
-        if ((src & r.y) == r.x && key >= r.z && key <= r.w) return true;
-    }
-    return false;
+    return hit;
 }
 
 constexpr uint32_t LDS_BOUNDS_MAX = 24576; // 96 KiB of cut points
@@ -212,68 +246,73 @@ __global__ __launch_bounds__(FILTER_THREADS, 8) void filter_check_kernel(FilterA
             lsmall[q] = a.flows.present_small[q];
     __syncthreads();
     const uint32_t stride = gridDim.x * FILTER_THREADS;
-    for (uint32_t i = blockIdx.x * FILTER_THREADS + threadIdx.x; i < a.n; i += stride) {
-        if (a.gate && a.gate[i] == 0) {
-            a.verdict[i] = 0;
-            continue;
+    const uint32_t lane = threadIdx.x & 63u;
+    // whole waves stay in the loop together: the rule lookup is a joint effort
+    for (uint32_t i0 = blockIdx.x * FILTER_THREADS + (threadIdx.x & ~63u); i0 < a.n; i0 += stride) {
+        const uint32_t i = i0 + lane;
+        bool valid = i < a.n && !(a.gate && a.gate[i] == 0);
+        Parsed h{};
+        if (valid) {
+            const uint8_t *p = a.pkts + (a.off ? a.off[i] : (uint64_t)i * a.stride);
+            const uint32_t len = a.lens ? a.lens[i] : a.len;
+            valid = parse_packet(p, len - (len >= a.trim ? a.trim : len), h);
         }
-        const uint8_t *p = a.pkts + (a.off ? a.off[i] : (uint64_t)i * a.stride);
-        const uint32_t len = a.lens ? a.lens[i] : a.len;
-        Parsed h;
-        uint8_t pass = 0;
-        if (parse_packet(p, len - (len >= a.trim ? a.trim : len), h)) {
-            const uint32_t key = proto_class(h.proto) << 16 | h.dport;
-            const uint32_t iv = in_lds ? interval_of(lb, ri.n_bounds, ri.top_step, h.src)
-                                       : interval_of(ri.bounds, ri.n_bounds, ri.top_step, h.src);
+        uint32_t key = 0, iv = 0;
+        bool maybe = false;
+        FlowSlot s{};
+        if (valid) {
+            key = proto_class(h.proto) << 16 | h.dport;
+            iv = in_lds ? interval_of(lb, ri.n_bounds, ri.top_step, h.src)
+                        : interval_of(ri.bounds, ri.n_bounds, ri.top_step, h.src);
             // return traffic: remote = src, remotePort = srcPort, localPort = dstPort.
             // A clear presence bit means the key was never stored: no probe
             // needed.  The bits come from LDS when the small bitmap is in use;
             // otherwise the word is fetched alongside the rule list, not after it.
-            const FlowSlot s = flow_slot(a.flows, h.src, h.sport, h.dport, h.proto);
-            bool maybe;
+            s = flow_slot(a.flows, h.src, h.sport, h.dport, h.proto);
             if (small) {
                 maybe = ((lsmall[s.sbit0 >> 5] >> (s.sbit0 & 31u)) & (lsmall[s.sbit1 >> 5] >> (s.sbit1 & 31u)) & 1u) != 0u;
             } else {
                 maybe = ((a.flows.present[s.bit >> 5] >> (s.bit & 31u)) & 1u) != 0u;
             }
-            if (rules_match(ri, iv, h.src, key)) {
-                pass = 1;
-            } else {
-                for (uint32_t probe = 0; maybe && probe < a.flows.cap; probe++) {
-                    FlowSlotMem *slot = a.flows.slots + s.base + ((s.start + probe) & (a.flows.cap - 1u));
-                    // Keys only change in NoteOutbound batches, never during this
-                    // kernel.  An expiry that another lane is refreshing may be seen
-                    // old or new: both are values this batch's single `now` allows.
-                    const ulonglong2 cur = *reinterpret_cast<const ulonglong2 *>(slot);
-                    if (cur.x == 0) break; // miss
-                    if (cur.x != s.word) continue;
-                    unsigned long long *ep = reinterpret_cast<unsigned long long *>(&slot->exp);
-                    const int64_t e = (int64_t)cur.y;
-                    if (e == FLOW_TOMB) break; // deleted earlier
-                    if (a.now < e) {
-                        // keep-alive on traffic (filter.go:141)
-                        // A plain store on purpose.  Every lane that refreshes this
-                        // flow in this batch writes the same value, a reader may see
-                        // the old expiry or the new one (both lie after `now`, so the
-                        // verdict is the same), and deletion cannot race with it: all
-                        // lanes see the same side of `now < e`.  An atomic store would
-                        // have to be visible across the eight L2s at once and is
-                        // pushed out to memory for it; this one waits for the end of
-                        // the kernel like any other store.
-                        // (`volatile` gets the same treatment as an atomic, hence not even that.)
-                        *ep = (unsigned long long)(a.now + flow_ttl_ns(h.proto));
-                        pass = 1;
-                    } else {
-                        // expired: delete (filter.go:144); only the lane that
-                        // turns it into a tombstone adjusts the entry count
-                        const int64_t prev = (int64_t)atomicExch(ep, (unsigned long long)FLOW_TOMB);
-                        if (prev != FLOW_TOMB) atomicSub(&a.flows.counters[FLOW_LIVE], 1u);
-                    }
-                    break;
+        }
+        uint8_t pass = 0;
+        if (rules_match_quad(ri, lane, iv, h.src, key)) {
+            pass = valid ? 1 : 0;
+        } else if (valid) {
+            for (uint32_t probe = 0; maybe && probe < a.flows.cap; probe++) {
+                FlowSlotMem *slot = a.flows.slots + s.base + ((s.start + probe) & (a.flows.cap - 1u));
+                // Keys only change in NoteOutbound batches, never during this
+                // kernel.  An expiry that another lane is refreshing may be seen
+                // old or new: both are values this batch's single `now` allows.
+                const ulonglong2 cur = *reinterpret_cast<const ulonglong2 *>(slot);
+                if (cur.x == 0) break; // miss
+                if (cur.x != s.word) continue;
+                unsigned long long *ep = reinterpret_cast<unsigned long long *>(&slot->exp);
+                const int64_t e = (int64_t)cur.y;
+                if (e == FLOW_TOMB) break; // deleted earlier
+                if (a.now < e) {
+                    // keep-alive on traffic (filter.go:141)
+                    // A plain store on purpose.  Every lane that refreshes this
+                    // flow in this batch writes the same value, a reader may see
+                    // the old expiry or the new one (both lie after `now`, so the
+                    // verdict is the same), and deletion cannot race with it: all
+                    // lanes see the same side of `now < e`.  An atomic store would
+                    // have to be visible across the eight L2s at once and is
+                    // pushed out to memory for it; this one waits for the end of
+                    // the kernel like any other store.
+                    // (`volatile` gets the same treatment as an atomic, hence not even that.)
+                    *ep = (unsigned long long)(a.now + flow_ttl_ns(h.proto));
+                    pass = 1;
+                } else {
+                    // expired: delete (filter.go:144); only the lane that
+                    // turns it into a tombstone adjusts the entry count
+                    const int64_t prev = (int64_t)atomicExch(ep, (unsigned long long)FLOW_TOMB);
+                    if (prev != FLOW_TOMB) atomicSub(&a.flows.counters[FLOW_LIVE], 1u);
                 }
+                break;
             }
         }
-        a.verdict[i] = pass;
+        if (i < a.n) a.verdict[i] = pass;
     }
 }
 

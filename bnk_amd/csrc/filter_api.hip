@@ -36,9 +36,14 @@ static hipError_t upload_rule_index(FilterState *f, const HostRuleIndex &h, hipS
     hipError_t e;
     const size_t nb = h.bounds.size();
     if ((e = f->bounds.reserve(std::max<size_t>(nb, 1) * 4)) != hipSuccess) return e;
+    if ((e = f->jump.reserve((JUMP_BUCKETS + 2) * 2)) != hipSuccess) return e;
     if ((e = f->ranges.reserve(std::max<size_t>(h.ranges.size(), 1) * 4)) != hipSuccess) return e;
     if ((e = f->wide.reserve(std::max<size_t>(h.wide.size(), 1) * 16)) != hipSuccess) return e;
     if ((e = hipMemcpyAsync(f->bounds.p, h.bounds.data(), nb * 4, hipMemcpyHostToDevice, s)) != hipSuccess)
+        return e;
+    if (!h.jump.empty() &&
+        (e = hipMemcpyAsync(f->jump.p, h.jump.data(), h.jump.size() * 2, hipMemcpyHostToDevice, s)) !=
+            hipSuccess)
         return e;
     if (!h.ranges.empty() &&
         (e = hipMemcpyAsync(f->ranges.p, h.ranges.data(), h.ranges.size() * 4, hipMemcpyHostToDevice,
@@ -51,6 +56,9 @@ static hipError_t upload_rule_index(FilterState *f, const HostRuleIndex &h, hipS
     // the host vectors die with the caller's frame
     if ((e = hipStreamSynchronize(s)) != hipSuccess) return e;
     f->ridx.bounds = f->bounds.as<uint32_t>();
+    f->ridx.jump = h.jump.empty() ? nullptr : f->jump.as<uint16_t>();
+    f->ridx.jump_lo = h.jump_lo;
+    f->ridx.jump_shift = h.jump_shift;
     f->ridx.ranges = f->ranges.as<uint32_t>();
     f->ridx.wide = f->wide.as<uint4>();
     f->ridx.n_bounds = (uint32_t)nb;

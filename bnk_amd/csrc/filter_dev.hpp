@@ -38,7 +38,8 @@ constexpr uint32_t SMALL_KEYS_MAX = 3u << 16;     // beyond this a clear answer 
 constexpr uint32_t RANGE_PAD = 0x3FFFFu << 14;
 constexpr uint32_t RANGE_LONG = 0x3FFFEu << 14;      // first word of a block that only points on
 constexpr uint32_t RANGE_MAX_SPAN = (1u << 14) - 1u; // largest key_hi - key_lo one entry holds
-constexpr uint32_t RANGE_BLOCK = 16;                 // entries per 64-byte block
+constexpr uint32_t RANGE_BLOCK = 16;
+constexpr uint32_t JUMP_BUCKETS = 1024;                 // entries per 64-byte block
 
 struct RuleIndexDev {
     const uint32_t *bounds; // [n_bounds] ascending starts of the elementary source intervals
@@ -49,6 +50,12 @@ struct RuleIndexDev {
                             // list of more than RANGE_BLOCK pieces lives in blocks past the
                             // first n_bounds, and block j is {RANGE_LONG, first block, blocks}
     const uint4 *wide;      // [n_wide] (net, mask, key_lo, key_hi) scanned by every packet
+    const uint16_t *jump;   // [JUMP_BUCKETS + 1] when n_bounds fits 16 bits, else null: the cut
+                            // points from bounds[1] up are spread over equal address buckets
+                            // and jump[b] is the last cut point at or below bucket b's start,
+                            // so a search only has to look between jump[b] and jump[b + 1]
+    uint32_t jump_lo;       // bounds[1]
+    uint32_t jump_shift;    // bucket of src = (src - jump_lo) >> jump_shift
     uint32_t n_bounds;
     uint32_t top_step;      // largest power of two < n_bounds (0 when n_bounds == 1)
     uint32_t n_wide;

@@ -13,6 +13,8 @@ namespace bnk {
 
 struct HostRuleIndex {
     std::vector<uint32_t> bounds;
+    std::vector<uint16_t> jump; // see RuleIndexDev::jump; empty when not applicable
+    uint32_t jump_lo = 0, jump_shift = 0;
     std::vector<uint32_t> ranges;
     std::vector<uint4> wide;
 };
@@ -109,6 +111,21 @@ inline bool build_rule_index(const bnk_rule *rules, uint32_t n, HostRuleIndex &o
     // per interval: sort by key_lo, merge overlapping or adjacent key ranges,
     // cut what is left into one-word pieces; block j takes interval j's pieces,
     // or points at blocks appended behind the first nb when there are too many
+    // jump table over the populated part of the address space
+    out.jump.clear();
+    if (nb >= 2 && nb <= 0xFFFFu) {
+        out.jump_lo = B[1];
+        const uint32_t span = B[nb - 1] - B[1];
+        out.jump_shift = 0;
+        while ((span >> out.jump_shift) >= JUMP_BUCKETS) out.jump_shift++;
+        out.jump.resize(JUMP_BUCKETS + 1);
+        uint32_t j = 1;
+        for (uint32_t b = 0; b <= JUMP_BUCKETS; b++) {
+            const uint64_t start = (uint64_t)B[1] + ((uint64_t)b << out.jump_shift);
+            while (j + 1 < nb && (uint64_t)B[j + 1] <= start) j++;
+            out.jump[b] = (uint16_t)j;
+        }
+    }
     out.ranges.assign((size_t)nb * RANGE_BLOCK, RANGE_PAD);
     std::vector<uint2> merged;
     std::vector<uint32_t> pieces;
@@ -148,7 +165,7 @@ inline bool build_rule_index(const bnk_rule *rules, uint32_t n, HostRuleIndex &o
 
 struct FilterState {
     bool enforce = false; // filter.New: allow-all until a policy arrives (filter.go:41-43)
-    DevBuf bounds, ranges, wide;
+    DevBuf bounds, jump, ranges, wide;
     RuleIndexDev ridx{};
     DevBuf slots, counters, present, present_small;
     FlowTableDev flows{};
@@ -156,7 +173,7 @@ struct FilterState {
     uint32_t max_blocks = 2048;
     void release()
     {
-        for (DevBuf *b : {&bounds, &ranges, &wide, &slots, &counters, &present, &present_small}) b->release();
+        for (DevBuf *b : {&bounds, &jump, &ranges, &wide, &slots, &counters, &present, &present_small}) b->release();
     }
 };
 

@@ -102,7 +102,7 @@ def bench_filter(args) -> dict:
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
                      # FETCH_SIZE x2 + WRITE_SIZE under rocprofv3 --pmc for this launch
                      # (profiles/filter_check_kernel_cfg4.md); not re-measured by this run
-                     "traffic": 232.8e6 if n == 1 << 22 else None, "bytes_per_launch": alg_bytes,
+                     "traffic": 234.8e6 if n == 1 << 22 else None, "bytes_per_launch": alg_bytes,
                      "avg_launch_ms": round(kern_ms, 4)},
     }
     if not args.no_cpu_baseline:

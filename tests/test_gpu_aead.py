@@ -342,3 +342,67 @@ def test_device_resident_large_batch_properties(ctx):
     ctx.sync()
     assert bool(((ct[:, :L] ^ ct2[:, :L]) == 0x3C).all())
     assert not torch.equal(ct[:, L:L + 16], ct2[:, L:L + 16])
+
+
+def test_cfg3_full_size_imix_with_forged_tags(ctx):
+    """Configuration 3 at full size (2^20 IMIX packets, 256 peers, 1 % of the
+    tags with one seeded bit flipped), device resident: rejects are exactly the
+    forged packets and their plaintext is zero, every other packet opens to what
+    was sealed, nothing between packets is written, and a sample of sealed
+    packets is bit-exact against the oracle."""
+    import torch
+    from bnk_amd import lib
+    from oracle import binding as O
+    n = 1 << 20
+    b = W.aead_imix(3, n, n_peers=256, payload=False)
+    dev = torch.device("cuda:0")
+    total = b.meta["total"]
+    plain = W.imix_plain_torch(b, dev)
+    d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)  # noqa: E731
+    d_off, d_peer, d_ctr = d(b.off.astype(np.int64)), d(b.peer.astype(np.int32)), d(b.counters.astype(np.int64))
+    d_lens, d_ctl = d(b.lens.astype(np.int32)), d((b.lens + 16).astype(np.int32))
+    sealed = torch.full((total,), 0x5A, dtype=torch.uint8, device=dev)
+    back = torch.full((total,), 0xA5, dtype=torch.uint8, device=dev)
+    v = torch.full((n,), 7, dtype=torch.uint8, device=dev)
+    torch.cuda.synchronize()
+    keys = np.ascontiguousarray(b.keys)
+    ctx.keys_set(lib.KEYS_SEND, keys)
+    ctx.keys_set(lib.KEYS_RECV, keys)
+    ctx.seal(lib.make_batch(plain, total, n, lib.MEM_DEVICE, offsets=d_off, lens=d_lens, peer=d_peer,
+                            counters=d_ctr),
+             lib.make_batch(sealed, total, n, lib.MEM_DEVICE, offsets=d_off))
+    ctx.sync()
+    # sample against the oracle, all three sizes
+    for L in W.IMIX_SIZES:
+        for i in np.flatnonzero(b.lens == L)[[0, 1, -1]]:
+            o = int(b.off[i])
+            pt = plain[o:o + L].cpu().numpy().tobytes()
+            want = O.aead_seal(keys[b.peer[i]].tobytes(), O.wg_nonce(int(b.counters[i])), pt)
+            assert sealed[o:o + L + 16].cpu().numpy().tobytes() == want
+    # forge 1 % of the tags
+    k = int(0.01 * n)
+    which = W.permutation(W.stream_seed(3, 5), n)[:k].astype(np.int64)
+    bit = W.rand_below(W.stream_seed(3, 6), k, 128)
+    pos = b.off[which].astype(np.int64) + b.lens[which].astype(np.int64) + (bit >> 3).astype(np.int64)
+    sealed[d(pos)] ^= d((1 << (bit & 7)).astype(np.uint8))
+    torch.cuda.synchronize()
+    ctx.open(lib.make_batch(sealed, total, n, lib.MEM_DEVICE, offsets=d_off, lens=d_ctl, peer=d_peer,
+                            counters=d_ctr),
+             lib.make_batch(back, total, n, lib.MEM_DEVICE, offsets=d_off), v)
+    ctx.sync()
+    forged = np.zeros(n, bool)
+    forged[which] = True
+    assert k == 10485 and np.array_equal(v.cpu().numpy() == 0, forged)
+    # byte-level expectation: packet bytes = plaintext (zeros where forged), everything else untouched
+    is_pkt = torch.zeros(total + 1, dtype=torch.int32, device=dev)
+    is_pkt.index_add_(0, d_off, torch.ones(n, dtype=torch.int32, device=dev))
+    is_pkt.index_add_(0, d_off + d_lens.long(), -torch.ones(n, dtype=torch.int32, device=dev))
+    inside = torch.cumsum(is_pkt[:total], 0) > 0
+    zero = torch.zeros(total + 1, dtype=torch.int32, device=dev)
+    f_off, f_len = d_off[d(which)], d_lens.long()[d(which)]
+    zero.index_add_(0, f_off, torch.ones(k, dtype=torch.int32, device=dev))
+    zero.index_add_(0, f_off + f_len, -torch.ones(k, dtype=torch.int32, device=dev))
+    zeroed = torch.cumsum(zero[:total], 0) > 0
+    want = torch.where(inside, torch.where(zeroed, torch.zeros_like(plain), plain),
+                       torch.full_like(plain, 0xA5))
+    assert torch.equal(back, want)

@@ -207,8 +207,8 @@ BNK_DEV void body_generic(uint8_t *tile, uint32_t lane, const uint8_t *src, uint
 
 template <bool OPEN>
 BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_t *dst, uint32_t len,
-                        const uint32_t (&k)[8], uint32_t n1, uint32_t n2, Poly32 &mac,
-                        uint32_t (&x)[16])
+                        const uint8_t *safe, const uint32_t (&k)[8], uint32_t n1, uint32_t n2,
+                        Poly32 &mac, uint32_t (&x)[16])
 {
     // Cells are 16 bytes; a packet's cell kc sits at stream position c0 + kc,
     // where the stream starts at the 128-byte line holding the packet's first
@@ -259,11 +259,19 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
     uint8_t *mycell = tile + (lane >> 3) * RING_ROW;
 #define BNK_INSIDE(q, m) (8u * (m) + sub >= cfirst[q] && 8u * (m) + sub < cend[q])
 #define BNK_SLOT(q, m) reinterpret_cast<uint4 *>(mycell + 8u * q * RING_ROW + (((8u * (m) + sub) & 15u) << 4))
-#define BNK_ISSUE(q, m) if (BNK_INSIDE(q, m)) pre##q = ld16a(csrc[q] + 128u * (m))
+    // Boundary lines: a load under a branch makes the wave wait for it before the
+    // branch closes, eight times per line; loading unconditionally from a harmless
+    // address instead keeps all eight in flight (cells outside the packet are
+    // fetched from `safe` and never leave their register).
+#define BNK_ISSUE(q, m) pre##q = ld16a(BNK_INSIDE(q, m) ? csrc[q] + 128u * (m) : safe)
 #define BNK_ISSUE_ALL(q, m) pre##q = ld16a(csrc[q] + 128u * (m))
 #define BNK_COMMIT(q, m) if (BNK_INSIDE(q, m)) *BNK_SLOT(q, m) = pre##q
 #define BNK_COMMIT_ALL(q, m) *BNK_SLOT(q, m) = pre##q
-#define BNK_STORE(q, m) if (BNK_INSIDE(q, m)) st16a(cdst[q] + 128u * (m), *BNK_SLOT(q, m))
+#define BNK_STORE(q, m)                                                                     \
+    do {                                                                                    \
+        const uint4 out_##q = *BNK_SLOT(q, m); /* read first, unconditionally: same reason */ \
+        if (BNK_INSIDE(q, m)) st16a(cdst[q] + 128u * (m), out_##q);                         \
+    } while (0)
 #define BNK_STORE_ALL(q, m) st16a(cdst[q] + 128u * (m), *BNK_SLOT(q, m))
 #define BNK_EIGHT(OP, m)                                                                    \
     do {                                                                                    \
@@ -390,7 +398,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
     const bool lane_lines = (((uintptr_t)src | (uintptr_t)dst) & 15u) == 0 &&
                             (((uintptr_t)src ^ (uintptr_t)dst) & 127u) == 0;
-    if (__ballot(!lane_lines) == 0ull) body_lines<OPEN>(tile, lane, src, dst, len, k, n1, n2, mac, x);
+    if (__ballot(!lane_lines) == 0ull) body_lines<OPEN>(tile, lane, src, dst, len, reinterpret_cast<const uint8_t *>(a.keys), k, n1, n2, mac, x);
     else body_generic<OPEN>(tile, lane, src, dst, len, k, n1, n2, mac, x);
 
     bool reject = false;

@@ -31,11 +31,25 @@ BNK_DEV uint32_t wg_padding(uint32_t len, uint32_t mtu)
     return padded - last;
 }
 
-// Header checks and receiver-index lookup of received datagrams.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef u32x4 __attribute__((aligned(1))) u32x4_unaligned;
+
+constexpr uint32_t WG_LDS_PEERS_MAX = 8192; // 64 KiB of (index, peer) pairs
+
+// Header checks and receiver-index lookup of received datagrams.  The sorted
+// index table is searched in LDS when it fits (ten dependent reads per packet
+// would otherwise each go out to L2); the header comes in with one load.
 __global__ __launch_bounds__(256) void wg_parse_kernel(WgBatch b, WgPeersDev pe, uint32_t *peer,
                                                        uint64_t *counter, uint32_t *ct_len,
                                                        uint8_t *result)
 {
+    extern __shared__ uint2 ltab[];
+    const bool in_lds = pe.n <= WG_LDS_PEERS_MAX;
+    if (in_lds) {
+        for (uint32_t q = threadIdx.x; q < pe.n; q += 256u) ltab[q] = pe.index_sorted[q];
+        __syncthreads();
+    }
+    const uint2 *tab = in_lds ? ltab : pe.index_sorted;
     const uint32_t t = blockIdx.x * 256u + threadIdx.x;
     if (t >= b.n) return;
     const uint32_t i = b.first + t;
@@ -44,23 +58,28 @@ __global__ __launch_bounds__(256) void wg_parse_kernel(WgBatch b, WgPeersDev pe,
     peer[i] = 0xFFFFFFFFu;
     counter[i] = 0;
     ct_len[i] = 0;
-    if (len < 32u || wg_ld32(w) != 4u) {
+    if (len < 32u) {
         result[i] = BNK_WG_BAD_HEADER;
         return;
     }
-    const uint32_t idx = wg_ld32(w + 4);
+    const u32x4 h = *reinterpret_cast<const u32x4_unaligned *>(w);
+    if (h.x != 4u) {
+        result[i] = BNK_WG_BAD_HEADER;
+        return;
+    }
+    const uint32_t idx = h.y;
     uint32_t lo = 0, hi = pe.n;
     while (lo < hi) {
         const uint32_t mid = (lo + hi) >> 1;
-        if (pe.index_sorted[mid].x < idx) lo = mid + 1;
+        if (tab[mid].x < idx) lo = mid + 1;
         else hi = mid;
     }
-    if (lo >= pe.n || pe.index_sorted[lo].x != idx) {
+    if (lo >= pe.n || tab[lo].x != idx) {
         result[i] = BNK_WG_UNKNOWN_INDEX;
         return;
     }
-    peer[i] = pe.index_sorted[lo].y;
-    counter[i] = (uint64_t)wg_ld32(w + 8) | (uint64_t)wg_ld32(w + 12) << 32;
+    peer[i] = tab[lo].y;
+    counter[i] = (uint64_t)h.z | (uint64_t)h.w << 32;
     ct_len[i] = len - 16u;
     result[i] = BNK_WG_OK; // so far
 }
@@ -86,12 +105,20 @@ __global__ __launch_bounds__(256) void wg_finish_kernel(WgBatch out, uint32_t ou
         return;
     }
     const uint8_t *p = out.base + (out.off ? out.off[i] : (uint64_t)i * out.stride) + out_skip;
-    const uint32_t version = p[0] >> 4;
+    if (plen < 16u) {
+        // too short for either header; only the version nibble could matter and
+        // every version is refused at this length
+        result[i] = BNK_WG_BAD_IP;
+        return;
+    }
+    // the first 16 bytes hold every field looked at below, in one load
+    const u32x4 hw = *reinterpret_cast<const u32x4_unaligned *>(p);
+    const uint32_t version = (hw.x >> 4) & 0xFu;
     if (version == 4u) {
         if (plen < 20u) { result[i] = BNK_WG_BAD_IP; return; }
-        const uint32_t total = (uint32_t)p[2] << 8 | p[3];
+        const uint32_t total = __builtin_bswap32(hw.x) & 0xFFFFu;
         if (total > plen || total < 20u) { result[i] = BNK_WG_BAD_IP; return; }
-        const uint32_t src = __builtin_bswap32(wg_ld32(p + 12));
+        const uint32_t src = __builtin_bswap32(hw.w);
         const uint2 al = pe.allowed[peer[i]];
         if ((src & al.y) != (al.x & al.y)) { result[i] = BNK_WG_NOT_ALLOWED; return; }
         out_len[i] = total;
@@ -99,7 +126,7 @@ __global__ __launch_bounds__(256) void wg_finish_kernel(WgBatch out, uint32_t ou
     }
     if (version == 6u) {
         if (plen < 40u) { result[i] = BNK_WG_BAD_IP; return; }
-        const uint32_t total = ((uint32_t)p[4] << 8 | p[5]) + 40u;
+        const uint32_t total = (__builtin_bswap32(hw.y) >> 16) + 40u;
         result[i] = total > plen ? BNK_WG_BAD_IP : BNK_WG_NOT_ALLOWED; // peers own IPv4 addresses only
         return;
     }
@@ -142,10 +169,8 @@ __global__ __launch_bounds__(256) void wg_encap_prep_kernel(WgBatch b, WgPeersDe
     uint8_t *w = const_cast<uint8_t *>(b.base) + (b.off ? b.off[i] : (uint64_t)i * b.stride);
     const uint32_t pad = wg_padding(len, mtu);
     const uint64_t c = counter[i];
-    wg_st32(w, 4u);
-    wg_st32(w + 4, pe.remote_index[pr]);
-    wg_st32(w + 8, (uint32_t)c);
-    wg_st32(w + 12, (uint32_t)(c >> 32));
+    const u32x4 hdr = {4u, pe.remote_index[pr], (uint32_t)c, (uint32_t)(c >> 32)};
+    *reinterpret_cast<u32x4_unaligned *>(w) = hdr;
     for (uint32_t k = 0; k < pad; k++) w[16u + len + k] = 0;
     skip[i] = 0;
     padded_len[i] = len + pad;
@@ -158,7 +183,14 @@ hipError_t launch_wg_parse(const WgBatch &b, const WgPeersDev &pe, uint32_t *pee
                            uint32_t *ct_len, uint8_t *result, hipStream_t s)
 {
     if (b.n == 0) return hipSuccess;
-    hipLaunchKernelGGL(wg_parse_kernel, grid_of(b.n), dim3(256), 0, s, b, pe, peer, counter, ct_len, result);
+    const uint32_t lds = pe.n <= WG_LDS_PEERS_MAX ? pe.n * 8u : 0u;
+    if (lds > 48u * 1024u) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(wg_parse_kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)(WG_LDS_PEERS_MAX * 8u));
+        if (e != hipSuccess) return e;
+    }
+    hipLaunchKernelGGL(wg_parse_kernel, grid_of(b.n), dim3(256), lds, s, b, pe, peer, counter, ct_len, result);
     return hipGetLastError();
 }
 

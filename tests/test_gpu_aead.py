@@ -406,3 +406,44 @@ def test_cfg3_full_size_imix_with_forged_tags(ctx):
     want = torch.where(inside, torch.where(zeroed, torch.zeros_like(plain), plain),
                        torch.full_like(plain, 0xA5))
     assert torch.equal(back, want)
+
+
+def test_concurrent_callers_share_one_context(ctx):
+    """wireguard-go calls Seal from one goroutine per peer: entry points on one
+    context may be called from several threads at once and are serialised
+    inside the library; every caller gets its own correct result."""
+    import threading
+    from bnk_amd import lib
+    b0 = W.aead_imix(21, 3000, n_peers=8)
+    keys = np.ascontiguousarray(b0.keys)
+    ctx.keys_set(lib.KEYS_SEND, keys)
+    ctx.keys_set(lib.KEYS_RECV, keys)
+    want = _oracle_seal(b0)
+    errors = []
+
+    def worker(tid):
+        try:
+            for it in range(6):
+                out = np.zeros_like(b0.plain)
+                ctx.seal(lib.make_batch(b0.plain, b0.plain.nbytes, b0.n, lib.MEM_HOST, offsets=b0.off,
+                                        lens=b0.lens, peer=b0.peer, counters=b0.counters),
+                         lib.make_batch(out, out.nbytes, b0.n, lib.MEM_HOST, offsets=b0.off))
+                if not np.array_equal(out, want):
+                    errors.append((tid, it, "seal"))
+                back = np.zeros_like(b0.plain)
+                v = np.zeros(b0.n, np.uint8)
+                ctx.open(lib.make_batch(out, out.nbytes, b0.n, lib.MEM_HOST, offsets=b0.off,
+                                        lens=(b0.lens + 16).astype(np.uint32), peer=b0.peer,
+                                        counters=b0.counters),
+                         lib.make_batch(back, back.nbytes, b0.n, lib.MEM_HOST, offsets=b0.off), v)
+                if not (v.all() and _packets_equal(back, b0.plain, b0.off, b0.lens) == -1):
+                    errors.append((tid, it, "open"))
+        except Exception as e:  # noqa: BLE001
+            errors.append((tid, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(6)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors[:3]

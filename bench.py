@@ -461,6 +461,59 @@ def bench_host(args) -> dict:
     }
 
 
+def bench_latency(args) -> dict:
+    """What one call costs at the batch sizes the reference's interfaces hand over
+    (wireguard-go passes at most 128 packets per Read/Write): host-memory seal,
+    open and filter check, one call at a time, median of many."""
+    import numpy as np
+    from bnk_amd import lib, workloads as W
+    ctx = lib.Context(0)
+    key = W.rand_bytes(W.stream_seed(2, 0), 32).reshape(1, 32)
+    ctx.keys_set(lib.KEYS_SEND, key)
+    ctx.keys_set(lib.KEYS_RECV, key)
+    ctx.filter_set_rules([([(W.CGNAT_BASE | 7, 32)], "tcp", [(22, 22)])])
+    out = {}
+    reps = max(args.steps, 5) * 10
+    for n in (1, 128, 1024, 8192):
+        nbytes = n * STRIDE
+        plain, sealed, opened = (ctx.ring_alloc(nbytes) for _ in range(3))
+        plain.reshape(n, STRIDE)[:, :L] = W.rand_bytes(W.stream_seed(2, 1), n * L).reshape(n, L)
+        plain.reshape(n, STRIDE)[:, 0] = 0x45
+        plain.reshape(n, STRIDE)[:, 9] = 6
+        v = np.zeros(n, np.uint8)
+        b_plain = lib.make_batch(plain, nbytes, n, lib.MEM_HOST, stride=STRIDE, length=L)
+        b_so = lib.make_batch(sealed, nbytes, n, lib.MEM_HOST, stride=STRIDE)
+        b_si = lib.make_batch(sealed, nbytes, n, lib.MEM_HOST, stride=STRIDE, length=L + 16)
+        b_op = lib.make_batch(opened, nbytes, n, lib.MEM_HOST, stride=STRIDE)
+        t = {"seal": [], "open": [], "filter": []}
+        for it in range(reps + 5):
+            t0 = time.perf_counter()
+            ctx.seal(b_plain, b_so)
+            t1 = time.perf_counter()
+            ctx.open(b_si, b_op, v)
+            t2 = time.perf_counter()
+            ctx.filter_check_inbound(b_plain, 1_700_000_000_000_000_000, v)
+            t3 = time.perf_counter()
+            if it >= 5:
+                t["seal"].append(t1 - t0)
+                t["open"].append(t2 - t1)
+                t["filter"].append(t3 - t2)
+        out[str(n)] = {k: round(float(np.median(x)) * 1e6, 1) for k, x in t.items()}
+        for r in (plain, sealed, opened):
+            ctx.ring_free(r)
+    ctx.close()
+    return {
+        "metric": "call_latency_us_host_memory", "value": out["128"]["seal"], "unit": "us", "n_gpus": 1,
+        "steps": reps, "warmup": 5, "ms_per_step": round(out["128"]["seal"] / 1e3, 4),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "u32",
+        "data": "synthetic",
+        "config": {"workload": "median microseconds per call (upload + kernel + download + wait) for "
+                               "batches of 1 / 128 / 1024 / 8192 packets x %d B in pinned rings; value is "
+                               "seal at 128 packets" % L},
+        "per_batch_size_us": out,
+    }
+
+
 def bench_copy(args) -> dict:
     """Plain device-to-device copy of 1 GiB: the measured HBM ceiling and the
     known-size launch the FETCH_SIZE / WRITE_SIZE counters are scaled by."""
@@ -481,9 +534,9 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--packets", type=int, default=1 << 20)
-    ap.add_argument("--workload", default="aead", choices=["aead", "filter", "imix", "relay", "wg", "host", "copy"],
+    ap.add_argument("--workload", default="aead", choices=["aead", "filter", "imix", "relay", "wg", "host", "latency", "copy"],
                     help="aead (default, the headline line, with the ACL filter rate as an extra); "
-                         "filter / imix / relay / wg / host / copy print one line for that workload alone")
+                         "filter / imix / relay / wg / host / latency / copy print one line for that workload alone")
     ap.add_argument("--serial", action="store_true",
                     help="wg: wait for the send side before starting the receive side, so a kernel "
                          "trace shows undisturbed durations (the two sides use separate streams)")
@@ -505,7 +558,7 @@ def main() -> int:
         return 2
     if args.workload != "aead":
         out = {"filter": bench_filter, "imix": bench_imix, "relay": bench_relay,
-               "wg": bench_wg, "host": bench_host, "copy": bench_copy}[args.workload](args)
+               "wg": bench_wg, "host": bench_host, "latency": bench_latency, "copy": bench_copy}[args.workload](args)
         print(json.dumps(out))
         return 0
     n = args.packets

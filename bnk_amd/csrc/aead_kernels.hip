@@ -8,6 +8,8 @@
 // one-time key; data uses blocks 1..; the MAC covers the zero-padded
 // ciphertext and one length block.
 #include "aead_lane.hpp"
+#include <algorithm>
+
 #include "kernels.hpp"
 
 namespace bnk {
@@ -345,6 +347,51 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
 #undef BNK_COMMIT_LINE
 }
 
+// Tag and verdict of each lane's packet once its bytes have gone through the
+// MAC, and the zero-fill of rejected plaintexts.
+template <bool OPEN>
+BNK_DEV void lane_finish(const AeadArgs &a, uint32_t lane, bool have, uint32_t i, uint32_t len,
+                         const uint8_t *src, uint8_t *dst, Poly32 &mac)
+{
+    bool reject = false;
+    if (have) {
+        // LE64(len(aad) = 0) || LE64(len(ciphertext))
+        mac.block(0, 0, len, 0);
+        uint32_t tag[4];
+        mac.finish(tag);
+        if (!OPEN) {
+            st16(dst + len, make_uint4(tag[0], tag[1], tag[2], tag[3]));
+        } else {
+            const uint4 tg = ld16(src + len);
+            // all 16 bytes are compared, no early exit
+            const uint32_t diff = (tg.x ^ tag[0]) | (tg.y ^ tag[1]) | (tg.z ^ tag[2]) |
+                                  (tg.w ^ tag[3]);
+            reject = diff != 0;
+            a.verdict[i] = reject ? 0 : 1;
+        }
+    }
+    if (OPEN) {
+        unsigned long long rej = __ballot(reject);
+        if (rej != 0ull) {
+            // the plaintext cells were stored by other lanes of this wave: wait
+            // until those stores have been acknowledged (a workgroup-scope
+            // release is just that wait; a wider fence would write back the
+            // whole L2), then the wave clears each rejected packet together
+            // (chacha20poly1305.Open leaves zeros behind)
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+            while (rej != 0ull) {
+                const int r = __ffsll((long long)rej) - 1;
+                rej &= rej - 1ull;
+                uint8_t *d = reinterpret_cast<uint8_t *>(shfl64((uint64_t)(uintptr_t)dst, r));
+                const uint32_t L = (uint32_t)__shfl((int)len, r, 64);
+                for (uint32_t pos = 16u * lane; pos + 16u <= L; pos += 1024u)
+                    st16(d + pos, make_uint4(0, 0, 0, 0));
+                if (lane < (L & 15u)) st8(d + (L & ~15u) + lane, 0);
+            }
+        }
+    }
+}
+
 template <bool OPEN>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void aead_wave_kernel(AeadArgs a)
 {
@@ -401,56 +448,157 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     if (__ballot(!lane_lines) == 0ull) body_lines<OPEN>(tile, lane, src, dst, len, reinterpret_cast<const uint8_t *>(a.keys), k, n1, n2, mac, x);
     else body_generic<OPEN>(tile, lane, src, dst, len, k, n1, n2, mac, x);
 
-    bool reject = false;
-    if (have) {
-        // LE64(len(aad) = 0) || LE64(len(ciphertext))
-        mac.block(0, 0, len, 0);
-        uint32_t tag[4];
-        mac.finish(tag);
-        if (!OPEN) {
-            st16(dst + len, make_uint4(tag[0], tag[1], tag[2], tag[3]));
-        } else {
-            const uint4 tg = ld16(src + len);
-            // all 16 bytes are compared, no early exit
-            const uint32_t diff = (tg.x ^ tag[0]) | (tg.y ^ tag[1]) | (tg.z ^ tag[2]) |
-                                  (tg.w ^ tag[3]);
-            reject = diff != 0;
-            a.verdict[i] = reject ? 0 : 1;
+    lane_finish<OPEN>(a, lane, have, i, len, src, dst, mac);
+}
+
+// One wave = one packet, for batches too small to fill the chip with a packet
+// per lane (there a call lasts as long as one lane needs for a whole packet:
+// about 85 us at 1420 bytes, however few the packets).  Lane 0 computes
+// ChaCha20 block 0 and owns the length block, lane l >= 1 computes block l and
+// moves bytes [64(l-1), 64l) of the packet; the tag is the sum of the lanes'
+// terms (aead_lane.hpp).  All loads of a packet are issued before any store,
+// and a lane stores only what it loaded, so sealing in place is safe.  A
+// packet longer than 63 blocks is done by lane 0 alone, the per-lane way.
+template <bool OPEN>
+__global__ __launch_bounds__(256) void aead_spread_kernel(AeadArgs a)
+{
+    __shared__ __attribute__((aligned(16))) uint8_t tile_all[WAVES_PER_BLOCK][64 * LDS_ROW];
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t w = blockIdx.x * WAVES_PER_BLOCK + (threadIdx.x >> 6);
+    if (w >= a.n) return;
+    // everything up to the per-lane work below is uniform across the wave
+    const uint32_t i = a.first + w;
+    uint32_t len = a.lens ? a.lens[i] : a.len;
+    if (!OPEN) len = len >= a.trim ? len - a.trim : 0u;
+    const uint32_t pr = a.peer ? a.peer[i] : 0u;
+    if (a.skip && a.skip[i] != 0) return;
+    if (pr >= a.n_peers) {
+        if (lane == 0) {
+            atomicOr(a.status, STATUS_PEER_RANGE);
+            if (OPEN) a.verdict[i] = 0;
         }
+        return;
     }
-    if (OPEN) {
-        unsigned long long rej = __ballot(reject);
-        if (rej != 0ull) {
-            // the plaintext cells were stored by other lanes of this wave: wait
-            // until those stores have been acknowledged (a workgroup-scope
-            // release is just that wait; a wider fence would write back the
-            // whole L2), then the wave clears each rejected packet together
-            // (chacha20poly1305.Open leaves zeros behind)
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-            while (rej != 0ull) {
-                const int r = __ffsll((long long)rej) - 1;
-                rej &= rej - 1ull;
-                uint8_t *d = reinterpret_cast<uint8_t *>(shfl64((uint64_t)(uintptr_t)dst, r));
-                const uint32_t L = (uint32_t)__shfl((int)len, r, 64);
-                for (uint32_t pos = 16u * lane; pos + 16u <= L; pos += 1024u)
-                    st16(d + pos, make_uint4(0, 0, 0, 0));
-                if (lane < (L & 15u)) st8(d + (L & ~15u) + lane, 0);
-            }
-        }
+    if (OPEN && len < 16u) {
+        if (lane == 0) a.verdict[i] = 0;
+        return;
+    }
+    if (OPEN) len -= 16u;
+    const uint8_t *src = a.in + (a.in_off ? a.in_off[i] : (uint64_t)i * a.in_stride) + a.in_skip;
+    uint8_t *dst = a.out + (a.out_off ? a.out_off[i] : (uint64_t)i * a.out_stride) + a.out_skip;
+    uint32_t k[8];
+    {
+        const uint4 *kp = reinterpret_cast<const uint4 *>(a.keys + 8u * pr);
+        const uint4 k0 = kp[0], k1 = kp[1];
+        k[0] = k0.x; k[1] = k0.y; k[2] = k0.z; k[3] = k0.w;
+        k[4] = k1.x; k[5] = k1.y; k[6] = k1.z; k[7] = k1.w;
+    }
+    const uint64_t ctr = a.counters ? a.counters[i] : a.counter0 + i;
+    const uint32_t n1 = (uint32_t)ctr, n2 = (uint32_t)(ctr >> 32);
+    uint32_t x[16];
+
+    if (len > SPREAD_MAX_LEN) {
+        const bool have = lane == 0;
+        Poly32 mac;
+        body_generic<OPEN>(tile_all[threadIdx.x >> 6], lane, have ? src : nullptr, have ? dst : nullptr,
+                           have ? len : 0u, k, n1, n2, mac, x);
+        lane_finish<OPEN>(a, lane, have, i, len, have ? src : nullptr, have ? dst : nullptr, mac);
+        return;
+    }
+
+    // ---- my 64 bytes: loads first, they fly while the block is computed ----
+    const uint32_t at = 64u * (lane - 1u);
+    const uint32_t mine = (lane == 0 || at >= len) ? 0u : min(len - at, 64u);
+    uint32_t m[16];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (mine >= 16u * (j + 1)) v = ld16(src + at + 16 * j);
+        else if (mine > 16u * j) v = ld_partial(src + at + 16 * j, mine - 16u * j);
+        m[4 * j] = v.x; m[4 * j + 1] = v.y; m[4 * j + 2] = v.z; m[4 * j + 3] = v.w;
+    }
+    uint4 want_tag = make_uint4(0, 0, 0, 0);
+    if (OPEN) want_tag = ld16(src + len);
+
+    chacha_block(k, lane, n1, n2, x);
+    // the one-time key is lane 0's block
+    const Fe26 r = fe_clamped_r((uint32_t)__builtin_amdgcn_readlane((int)x[0], 0),
+                                (uint32_t)__builtin_amdgcn_readlane((int)x[1], 0),
+                                (uint32_t)__builtin_amdgcn_readlane((int)x[2], 0),
+                                (uint32_t)__builtin_amdgcn_readlane((int)x[3], 0));
+    const uint32_t pad[4] = {(uint32_t)__builtin_amdgcn_readlane((int)x[4], 0),
+                             (uint32_t)__builtin_amdgcn_readlane((int)x[5], 0),
+                             (uint32_t)__builtin_amdgcn_readlane((int)x[6], 0),
+                             (uint32_t)__builtin_amdgcn_readlane((int)x[7], 0)};
+
+    // ---- crypt: o = m ^ keystream; the MAC reads the ciphertext side ----
+    uint32_t o[16];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        uint4 v = make_uint4(m[4 * j] ^ x[4 * j], m[4 * j + 1] ^ x[4 * j + 1], m[4 * j + 2] ^ x[4 * j + 2],
+                             m[4 * j + 3] ^ x[4 * j + 3]);
+        const uint32_t have_b = mine > 16u * j ? min(mine - 16u * j, 16u) : 0u;
+        v = keep_bytes(v, have_b);
+        o[4 * j] = v.x; o[4 * j + 1] = v.y; o[4 * j + 2] = v.z; o[4 * j + 3] = v.w;
+    }
+    if (lane == 0) {
+        // LE64(len(aad) = 0) || LE64(len(ciphertext)) as my only cell
+        m[0] = 0; m[1] = 0; m[2] = len; m[3] = 0;
+        o[0] = 0; o[1] = 0; o[2] = len; o[3] = 0;
+    }
+    const SpreadShare sh = spread_share(lane, len);
+    const Fe26 term = spread_term(r, OPEN ? m : o, sh.k, sh.e, spread_e_max(len));
+
+    // ---- add the 64 terms: 32 lanes fit 32 bits per limb, the last step is wider ----
+    uint32_t t32[5] = {term.v0, term.v1, term.v2, term.v3, term.v4};
+#pragma unroll
+    for (int step = 1; step < 32; step <<= 1)
+#pragma unroll
+        for (int q = 0; q < 5; q++) t32[q] += (uint32_t)__shfl_xor((int)t32[q], step, 64);
+    uint64_t sum[5];
+#pragma unroll
+    for (int q = 0; q < 5; q++) sum[q] = (uint64_t)t32[q] + (uint32_t)__shfl_xor((int)t32[q], 32, 64);
+    uint32_t tag[4];
+    spread_finish(sum, pad, tag);
+
+    bool reject = false;
+    if (!OPEN) {
+        if (lane == 0) st16(dst + len, make_uint4(tag[0], tag[1], tag[2], tag[3]));
+    } else {
+        // all 16 bytes are compared, no early exit
+        reject = ((want_tag.x ^ tag[0]) | (want_tag.y ^ tag[1]) | (want_tag.z ^ tag[2]) |
+                  (want_tag.w ^ tag[3])) != 0;
+        if (lane == 0) a.verdict[i] = reject ? 0 : 1;
+    }
+    // ---- my bytes out; a rejected packet leaves zeros (chacha20poly1305.Open) ----
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const uint4 v = reject ? make_uint4(0, 0, 0, 0)
+                               : make_uint4(o[4 * j], o[4 * j + 1], o[4 * j + 2], o[4 * j + 3]);
+        if (mine >= 16u * (j + 1)) st16(dst + at + 16 * j, v);
+        else if (mine > 16u * j) st_partial(dst + at + 16 * j, v, mine - 16u * j);
     }
 }
 
 hipError_t launch_aead_seal(const AeadArgs &a, hipStream_t s)
 {
     if (a.n == 0) return hipSuccess;
-    hipLaunchKernelGGL(aead_wave_kernel<false>, dim3((a.n + 255u) / 256u), dim3(256), 0, s, a);
+    if (a.n <= a.spread_max)
+        hipLaunchKernelGGL(aead_spread_kernel<false>, dim3((a.n + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK),
+                           dim3(256), 0, s, a);
+    else
+        hipLaunchKernelGGL(aead_wave_kernel<false>, dim3((a.n + 255u) / 256u), dim3(256), 0, s, a);
     return hipGetLastError();
 }
 
 hipError_t launch_aead_open(const AeadArgs &a, hipStream_t s)
 {
     if (a.n == 0) return hipSuccess;
-    hipLaunchKernelGGL(aead_wave_kernel<true>, dim3((a.n + 255u) / 256u), dim3(256), 0, s, a);
+    if (a.n <= a.spread_max)
+        hipLaunchKernelGGL(aead_spread_kernel<true>, dim3((a.n + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK),
+                           dim3(256), 0, s, a);
+    else
+        hipLaunchKernelGGL(aead_wave_kernel<true>, dim3((a.n + 255u) / 256u), dim3(256), 0, s, a);
     return hipGetLastError();
 }
 
@@ -588,6 +736,35 @@ hipError_t launch_fill_u32(uint32_t *p, uint32_t n, uint32_t v, hipStream_t s)
 {
     if (n == 0) return hipSuccess;
     hipLaunchKernelGGL(fill_u32_kernel, dim3((n + 255u) / 256u), dim3(256), 0, s, p, n, v);
+    return hipGetLastError();
+}
+
+// Copies `bytes` bytes from src to dst, which must share their alignment
+// within 16 bytes: every lane moves one aligned 16-byte piece, so a span in
+// pinned host memory crosses the link in one round trip instead of one per
+// ChaCha20 line.  The ragged ends go byte by byte.
+__global__ __launch_bounds__(256) void pull_kernel(const uint8_t *src, uint8_t *dst, uint64_t bytes)
+{
+    const uint64_t head = min((uint64_t)((16u - (uint32_t)((uintptr_t)src & 15u)) & 15u), bytes);
+    const uint64_t n16 = (bytes - head) >> 4;
+    const uint64_t tail = head + (n16 << 4);
+    const uint64_t stride = (uint64_t)gridDim.x * 256u;
+    for (uint64_t i = (uint64_t)blockIdx.x * 256u + threadIdx.x; i < n16; i += stride)
+        st16a(dst + head + (i << 4), ld16a(src + head + (i << 4)));
+    if (blockIdx.x == 0) {
+        if (threadIdx.x < head) st8(dst + threadIdx.x, ld8(src + threadIdx.x));
+        const uint32_t t = threadIdx.x - 64u;
+        if (threadIdx.x >= 64u && tail + t < bytes) st8(dst + tail + t, ld8(src + tail + t));
+    }
+}
+
+hipError_t launch_pull(const void *src, void *dst, uint64_t bytes, hipStream_t s)
+{
+    if (bytes == 0) return hipSuccess;
+    if ((((uintptr_t)src ^ (uintptr_t)dst) & 15u) != 0) return hipErrorInvalidValue;
+    const uint64_t blocks = std::min<uint64_t>((bytes / 16 + 255) / 256 + 1, 2048);
+    hipLaunchKernelGGL(pull_kernel, dim3((uint32_t)blocks), dim3(256), 0, s, (const uint8_t *)src,
+                       (uint8_t *)dst, bytes);
     return hipGetLastError();
 }
 

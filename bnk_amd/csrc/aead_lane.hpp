@@ -222,4 +222,145 @@ struct Poly32 {
     }
 };
 
+// ---------------------------------------------------------------------------
+// One packet spread over the lanes of a wave (small batches, where a packet
+// per lane would leave the chip empty and a call would last as long as one
+// lane takes for a whole packet).  Lane 0 runs ChaCha20 block 0 (the one-time
+// key) and owns the AEAD length block, lane l >= 1 owns keystream block l and
+// its four 16-byte cells.  With C MAC cells m_0 .. m_{C-1} the tag is
+// sum m_j r^(C-j) + s: each lane evaluates its own cells by Horner's rule,
+// lifts the result by r^(cells after its last one), and the lanes' terms are
+// added.  General multipliers (powers of r are not clamped) need the radix
+// 2^26 form.
+// ---------------------------------------------------------------------------
+
+// Element of GF(2^130 - 5), five limbs of 26 bits; arithmetic keeps limbs
+// below 2^27 and accepts limbs below 2^28 in the left operand of fe_mul.
+struct Fe26 {
+    uint32_t v0, v1, v2, v3, v4;
+};
+
+BNK_DEV Fe26 fe_small(uint32_t x) { return Fe26{x, 0, 0, 0, 0}; }
+
+// A 16-byte cell (little-endian words) with bit 128 set.
+BNK_DEV Fe26 fe_cell(uint32_t w0, uint32_t w1, uint32_t w2, uint32_t w3)
+{
+    return Fe26{w0 & 0x3ffffffu, funnel(w1, w0, 26) & 0x3ffffffu, funnel(w2, w1, 20) & 0x3ffffffu,
+                funnel(w3, w2, 14) & 0x3ffffffu, (w3 >> 8) | (1u << 24)};
+}
+
+// r from the first four words of ChaCha20 block 0, clamped.
+BNK_DEV Fe26 fe_clamped_r(uint32_t x0, uint32_t x1, uint32_t x2, uint32_t x3)
+{
+    Fe26 r = fe_cell(x0 & 0x0fffffffu, x1 & 0x0ffffffcu, x2 & 0x0ffffffcu, x3 & 0x0ffffffcu);
+    r.v4 &= 0xffffffu; // no bit 128
+    return r;
+}
+
+BNK_DEV Fe26 fe_add(const Fe26 &a, const Fe26 &b)
+{
+    return Fe26{a.v0 + b.v0, a.v1 + b.v1, a.v2 + b.v2, a.v3 + b.v3, a.v4 + b.v4};
+}
+
+BNK_DEV Fe26 fe_select(bool take_a, const Fe26 &a, const Fe26 &b)
+{
+    return Fe26{take_a ? a.v0 : b.v0, take_a ? a.v1 : b.v1, take_a ? a.v2 : b.v2,
+                take_a ? a.v3 : b.v3, take_a ? a.v4 : b.v4};
+}
+
+// a * b mod 2^130 - 5.  a's limbs below 2^28, b's below 2^27: a product is
+// below 2^28 * 5 * 2^27 < 2^58 and five of them stay below 2^61.
+BNK_DEV Fe26 fe_mul(const Fe26 &a, const Fe26 &b)
+{
+    const uint32_t s1 = b.v1 * 5, s2 = b.v2 * 5, s3 = b.v3 * 5, s4 = b.v4 * 5;
+    uint64_t d0 = (uint64_t)a.v0 * b.v0 + (uint64_t)a.v1 * s4 + (uint64_t)a.v2 * s3 +
+                  (uint64_t)a.v3 * s2 + (uint64_t)a.v4 * s1;
+    uint64_t d1 = (uint64_t)a.v0 * b.v1 + (uint64_t)a.v1 * b.v0 + (uint64_t)a.v2 * s4 +
+                  (uint64_t)a.v3 * s3 + (uint64_t)a.v4 * s2;
+    uint64_t d2 = (uint64_t)a.v0 * b.v2 + (uint64_t)a.v1 * b.v1 + (uint64_t)a.v2 * b.v0 +
+                  (uint64_t)a.v3 * s4 + (uint64_t)a.v4 * s3;
+    uint64_t d3 = (uint64_t)a.v0 * b.v3 + (uint64_t)a.v1 * b.v2 + (uint64_t)a.v2 * b.v1 +
+                  (uint64_t)a.v3 * b.v0 + (uint64_t)a.v4 * s4;
+    uint64_t d4 = (uint64_t)a.v0 * b.v4 + (uint64_t)a.v1 * b.v3 + (uint64_t)a.v2 * b.v2 +
+                  (uint64_t)a.v3 * b.v1 + (uint64_t)a.v4 * b.v0;
+    Fe26 o;
+    uint64_t c;
+    c = d0 >> 26; o.v0 = (uint32_t)d0 & 0x3ffffffu; d1 += c;
+    c = d1 >> 26; o.v1 = (uint32_t)d1 & 0x3ffffffu; d2 += c;
+    c = d2 >> 26; o.v2 = (uint32_t)d2 & 0x3ffffffu; d3 += c;
+    c = d3 >> 26; o.v3 = (uint32_t)d3 & 0x3ffffffu; d4 += c;
+    c = d4 >> 26; o.v4 = (uint32_t)d4 & 0x3ffffffu;
+    // c < 2^36: times five it still fits 64 bits, and two more carries settle it
+    c = (uint64_t)o.v0 + c * 5;
+    o.v0 = (uint32_t)c & 0x3ffffffu;
+    c = (uint64_t)o.v1 + (c >> 26);
+    o.v1 = (uint32_t)c & 0x3ffffffu;
+    o.v2 += (uint32_t)(c >> 26);
+    return o;
+}
+
+// One lane's share of the tag polynomial: its k (0..4) cells m[4t .. 4t+3]
+// evaluated as sum_t m_t r^(k-t), times r^e.  e_max bounds e over the wave
+// (it only limits the length of the square-and-multiply loop, so every lane
+// of a wave runs the same trip count).
+BNK_DEV Fe26 spread_term(const Fe26 &r, const uint32_t (&m)[16], uint32_t k, uint32_t e, uint32_t e_max)
+{
+    Fe26 acc = fe_small(0);
+#pragma unroll
+    for (uint32_t t = 0; t < 4; t++) {
+        const Fe26 nx = fe_mul(fe_add(acc, fe_cell(m[4 * t], m[4 * t + 1], m[4 * t + 2], m[4 * t + 3])), r);
+        acc = fe_select(t < k, nx, acc);
+    }
+    Fe26 lift = fe_small(1), pw = r;
+#pragma unroll 1
+    for (uint32_t b = 0; (1u << b) <= e_max; b++) {
+        const Fe26 nl = fe_mul(lift, pw);
+        lift = fe_select(((e >> b) & 1u) != 0, nl, lift);
+        pw = fe_mul(pw, pw);
+    }
+    return fe_mul(acc, lift);
+}
+
+// Tag from the limb-wise sum of the lanes' terms (each sum below 2^34) and the
+// second half of the one-time key.
+BNK_DEV void spread_finish(const uint64_t (&sum)[5], const uint32_t (&pad)[4], uint32_t (&tag)[4])
+{
+    uint64_t t0 = sum[0], t1 = sum[1], t2 = sum[2], t3 = sum[3], t4 = sum[4];
+#pragma unroll
+    for (int pass = 0; pass < 2; pass++) {
+        t1 += t0 >> 26; t0 &= 0x3ffffffu;
+        t2 += t1 >> 26; t1 &= 0x3ffffffu;
+        t3 += t2 >> 26; t2 &= 0x3ffffffu;
+        t4 += t3 >> 26; t3 &= 0x3ffffffu;
+        t0 += (t4 >> 26) * 5; t4 &= 0x3ffffffu;
+    }
+    Poly26 p;
+    p.h0 = (uint32_t)t0; p.h1 = (uint32_t)t1; p.h2 = (uint32_t)t2; p.h3 = (uint32_t)t3; p.h4 = (uint32_t)t4;
+    p.pad0 = pad[0]; p.pad1 = pad[1]; p.pad2 = pad[2]; p.pad3 = pad[3];
+    p.finish(tag);
+}
+
+// Which cells lane l owns in a packet of `len` ciphertext bytes, and how far
+// its term is lifted.  Lane 0: the length block, last in the MAC input, so it
+// is lifted by nothing.  Lane l >= 1: data cells 4(l-1) .. of ceil(len/16).
+struct SpreadShare {
+    uint32_t k, e;
+};
+BNK_DEV SpreadShare spread_share(uint32_t lane, uint32_t len)
+{
+    const uint32_t cd = (len + 15u) >> 4;
+    if (lane == 0) return SpreadShare{1u, 0u};
+    const uint32_t first = 4u * (lane - 1u);
+    if (first >= cd) return SpreadShare{0u, 0u};
+    const uint32_t k = cd - first < 4u ? cd - first : 4u;
+    return SpreadShare{k, cd - first - k + 1u}; // the cells after mine, and the length block
+}
+// Largest lift in the wave: lane 1's.
+BNK_DEV uint32_t spread_e_max(uint32_t len)
+{
+    const uint32_t cd = (len + 15u) >> 4;
+    return cd > 4u ? cd - 3u : 1u;
+}
+constexpr uint32_t SPREAD_MAX_LEN = 63u * 64u; // data blocks on lanes 1..63
+
 } // namespace bnk

@@ -87,6 +87,80 @@ int aead_batch_host_chunked(bnk_ctx *ctx, bool open, const bnk_batch *in, const 
     return status_to_rc(ctx, status);
 }
 
+// Small batches whose arenas lie in the context's pinned rings: kernels read
+// and write the rings over the link themselves and the per-packet arrays sit
+// in pinned staging, so a call is host bookkeeping, two launches and one wait,
+// with no copy-engine transfer.  Returns 1 when the batch does not qualify.
+int aead_batch_host_direct(bnk_ctx *ctx, bool open, const bnk_batch *in, const bnk_batch *out,
+                           uint8_t *verdict, AeadArgs a)
+{
+    const uint32_t n = in->n;
+    if (n > DIRECT_MAX_PACKETS) return 1;
+    uint8_t *d_in = ring_device_ptr(ctx, in->base, in->bytes);
+    uint8_t *d_out = ring_device_ptr(ctx, out->base, out->bytes);
+    if (!d_in || !d_out) return 1;
+    Span sin, sout;
+    int rc = scan_host_layout(ctx, in, in, 0, &sin, "in");
+    if (rc) return rc;
+    rc = scan_host_layout(ctx, out, in, open ? -16 : 16, &sout, "out");
+    if (rc) return rc;
+    if (sin.size() > DIRECT_MAX_BYTES) return 1;
+    if (in->peer)
+        for (uint32_t i = 0; i < n; i++)
+            if (in->peer[i] >= a.n_peers)
+                return fail(ctx, BNK_E_RANGE, "peer index " + std::to_string(in->peer[i]) + " beyond the key table");
+
+    // pinned staging: three 8-byte arrays, three 4-byte arrays, verdict bytes
+    HIPCHK(ctx, ctx->pin.reserve((size_t)n * 37 + 64));
+    uint8_t *pin = ctx->pin.as<uint8_t>();
+    uint64_t *p_in_off = (uint64_t *)pin, *p_out_off = p_in_off + n, *p_ctr = p_out_off + n;
+    uint32_t *p_lens = (uint32_t *)(p_ctr + n), *p_peer = p_lens + n, *p_order = p_peer + n;
+    uint8_t *p_verdict = (uint8_t *)(p_order + n);
+    // The input span is fetched into device memory by one wide copy kernel
+    // (every 16 bytes in flight at once); the AEAD kernel then writes its
+    // output straight into the ring, where stores need no round trip.
+    const uint32_t mis = (uint32_t)((uintptr_t)(d_in + sin.lo) & 15u);
+    HIPCHK(ctx, ctx->in_arena.reserve(sin.size() + 32));
+    HIPCHK(ctx, launch_pull(d_in + sin.lo, ctx->in_arena.as<uint8_t>() + mis, sin.size(), ctx->stream));
+    a.in = ctx->in_arena.as<uint8_t>() + mis;
+    a.out = d_out;
+    if (in->offsets) {
+        for (uint32_t i = 0; i < n; i++) p_in_off[i] = in->offsets[i] - sin.lo;
+        a.in_off = ctx->pin.dev(p_in_off);
+    }
+    if (out->offsets) { memcpy(p_out_off, out->offsets, (size_t)n * 8); a.out_off = ctx->pin.dev(p_out_off); }
+    if (in->counters) { memcpy(p_ctr, in->counters, (size_t)n * 8); a.counters = ctx->pin.dev(p_ctr); }
+    if (in->peer) { memcpy(p_peer, in->peer, (size_t)n * 4); a.peer = ctx->pin.dev(p_peer); }
+    if (in->lens) {
+        memcpy(p_lens, in->lens, (size_t)n * 4);
+        a.lens = ctx->pin.dev(p_lens);
+        if (n > 64) {
+            // lanes of a wave should run equal block counts: longest first
+            const uint32_t tag = open ? 16 : 0;
+            auto blocks = [&](uint32_t i) {
+                const uint32_t len = in->lens[i];
+                return ((len >= tag ? len - tag : 0u) + 63u) >> 6;
+            };
+            uint32_t most = 0;
+            for (uint32_t i = 0; i < n; i++) most = std::max(most, blocks(i));
+            if (most <= 65535) {
+                std::vector<uint32_t> at(most + 2, 0);
+                for (uint32_t i = 0; i < n; i++) at[most - blocks(i) + 1]++;
+                for (uint32_t b = 0; b <= most; b++) at[b + 1] += at[b];
+                for (uint32_t i = 0; i < n; i++) p_order[at[most - blocks(i)]++] = i;
+                a.order = ctx->pin.dev(p_order);
+            }
+        }
+    }
+    if (open) a.verdict = ctx->pin.dev(p_verdict);
+    HIPCHK(ctx, open ? launch_aead_open(a, ctx->stream) : launch_aead_seal(a, ctx->stream));
+    // host batches have had their peer indices checked above, so the kernel
+    // has nothing to report through the status word
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    if (open) memcpy(verdict, p_verdict, n);
+    return BNK_OK;
+}
+
 int aead_batch(bnk_ctx *ctx, bool open, const bnk_batch *in, const bnk_batch *out,
                uint8_t *verdict)
 {
@@ -104,6 +178,8 @@ int aead_batch(bnk_ctx *ctx, bool open, const bnk_batch *in, const bnk_batch *ou
     if (!in->peer && ctx->n_keys[which] < 1) return fail(ctx, BNK_E_RANGE, "empty key table");
 
     AeadArgs a{};
+
+    a.spread_max = ctx->spread_max;
     a.keys = ctx->d_keys[which];
     a.n_peers = ctx->n_keys[which];
     a.status = ctx->d_status;
@@ -137,6 +213,8 @@ int aead_batch(bnk_ctx *ctx, bool open, const bnk_batch *in, const bnk_batch *ou
         return BNK_OK;
     }
 
+    rc = aead_batch_host_direct(ctx, open, in, out, verdict, a);
+    if (rc != 1) return rc;
     rc = aead_batch_host_chunked(ctx, open, in, out, verdict, a);
     if (rc != 1) return rc;
     Staged st;
@@ -173,8 +251,9 @@ namespace bnk {
 // Reads and clears the device status word; the stream must be idle.
 int take_status(bnk_ctx *ctx, uint32_t *status)
 {
-    HIPCHK(ctx, hipMemcpyAsync(status, ctx->d_status, 4, hipMemcpyDeviceToHost, ctx->stream));
+    HIPCHK(ctx, hipMemcpyAsync(ctx->h_status, ctx->d_status, 4, hipMemcpyDeviceToHost, ctx->stream));
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    *status = *ctx->h_status;
     if (*status) HIPCHK(ctx, launch_fill_u32(ctx->d_status, 1, 0, ctx->stream));
     return BNK_OK;
 }
@@ -222,6 +301,8 @@ int bnk_init(int device_ordinal, bnk_ctx **out)
     if ((e = hipEventCreate(&ctx->ev0)) != hipSuccess) return bail("hipEventCreate", e);
     if ((e = hipEventCreate(&ctx->ev1)) != hipSuccess) return bail("hipEventCreate", e);
     if ((e = hipMalloc((void **)&ctx->d_status, 256)) != hipSuccess) return bail("hipMalloc", e);
+    if ((e = hipHostMalloc((void **)&ctx->h_status, 64, hipHostMallocDefault)) != hipSuccess)
+        return bail("hipHostMalloc", e);
     if ((e = launch_fill_u32(ctx->d_status, 64, 0, ctx->stream)) != hipSuccess)
         return bail("status clear", e);
     ctx->filter = filter_create(ctx->stream, prop.multiProcessorCount);
@@ -254,6 +335,7 @@ void bnk_shutdown(bnk_ctx *ctx)
         for (int w = 0; w < 2; w++)
             if (ctx->d_keys[w]) (void)hipFree(ctx->d_keys[w]);
         if (ctx->d_status) (void)hipFree(ctx->d_status);
+        if (ctx->h_status) (void)hipHostFree(ctx->h_status);
         if (ctx->filter) filter_destroy(ctx->filter);
         for (hipEvent_t e : ctx->ev_up) (void)hipEventDestroy(e);
         for (hipEvent_t e : ctx->ev_done) (void)hipEventDestroy(e);
@@ -274,6 +356,11 @@ int bnk_ring_alloc(bnk_ctx *ctx, size_t bytes, void **host_pinned)
     if (g.rc) return g.rc;
     if (!host_pinned || bytes == 0) return fail(ctx, BNK_E_INVAL, "bad ring request");
     HIPCHK(ctx, hipHostMalloc(host_pinned, bytes, hipHostMallocDefault));
+    void *dev = nullptr;
+    if (hipHostGetDevicePointer(&dev, *host_pinned, 0) == hipSuccess && dev)
+        ctx->rings.push_back({(uintptr_t)*host_pinned, (uint8_t *)dev, bytes});
+    else
+        (void)hipGetLastError(); // the ring still works through the copying routes
     return BNK_OK;
 }
 
@@ -283,7 +370,20 @@ int bnk_ring_free(bnk_ctx *ctx, void *host_pinned)
     if (g.rc) return g.rc;
     if (!host_pinned) return BNK_OK;
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    for (size_t i = 0; i < ctx->rings.size(); i++)
+        if (ctx->rings[i].host == (uintptr_t)host_pinned) {
+            ctx->rings.erase(ctx->rings.begin() + i);
+            break;
+        }
     HIPCHK(ctx, hipHostFree(host_pinned));
+    return BNK_OK;
+}
+
+int bnk_set_spread_max_packets(bnk_ctx *ctx, uint32_t max_packets)
+{
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    ctx->spread_max = max_packets;
     return BNK_OK;
 }
 

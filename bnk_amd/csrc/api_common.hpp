@@ -89,6 +89,21 @@ inline int check_batch_common(bnk_ctx *ctx, const bnk_batch *b, const char *name
 }
 
 
+// Host batches up to this size run in place when their arenas are pinned rings
+// of the context (no staging copies): above it the copy engines win.
+constexpr uint32_t DIRECT_MAX_PACKETS = 2048;
+constexpr uint64_t DIRECT_MAX_BYTES = 1ull << 20;
+
+// Device address of [p, p + bytes) when it lies inside one of the context's
+// pinned rings, else null.
+inline uint8_t *ring_device_ptr(const bnk_ctx *ctx, const void *p, uint64_t bytes)
+{
+    const uintptr_t a = (uintptr_t)p;
+    for (const bnk_ctx::Ring &r : ctx->rings)
+        if (a >= r.host && bytes <= r.bytes && a - r.host <= r.bytes - bytes) return r.dev + (a - r.host);
+    return nullptr;
+}
+
 // Host-resident view of a batch staged on the device.
 struct Staged {
     uint8_t *d_in = nullptr, *d_out = nullptr;

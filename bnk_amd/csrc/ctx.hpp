@@ -51,8 +51,15 @@ struct PinBuf {
         void *np = nullptr;
         hipError_t e = hipHostMalloc(&np, want, hipHostMallocDefault);
         if (e != hipSuccess) return e;
+        void *nd = nullptr;
+        e = hipHostGetDevicePointer(&nd, np, 0);
+        if (e != hipSuccess) {
+            (void)hipHostFree(np);
+            return e;
+        }
         if (p) (void)hipHostFree(p);
         p = np;
+        d = static_cast<uint8_t *>(nd);
         cap = want;
         return hipSuccess;
     }
@@ -60,8 +67,15 @@ struct PinBuf {
     {
         if (p) (void)hipHostFree(p);
         p = nullptr;
+        d = nullptr;
         cap = 0;
     }
+    // The address a kernel uses for a host address inside the buffer.
+    template <class T> T *dev(T *host) const
+    {
+        return reinterpret_cast<T *>(d + ((uint8_t *)host - static_cast<uint8_t *>(p)));
+    }
+    uint8_t *d = nullptr;
     template <class T> T *as() const { return static_cast<T *>(p); }
 };
 
@@ -88,6 +102,12 @@ struct bnk_ctx {
     bnk::DevBuf in_arena, out_arena, off_in, off_out, lens, peer, counters, verdict;
     bnk::DevBuf order, hist, cursor, misc;
     bnk::PinBuf pin;
+    // Pinned rings handed out by bnk_ring_alloc: kernels may read and write
+    // them in place (small host batches skip the copies).
+    struct Ring { uintptr_t host; uint8_t *dev; size_t bytes; };
+    std::vector<Ring> rings;
+    uint32_t *h_status = nullptr; // pinned landing word for d_status
+    uint32_t spread_max = bnk::SPREAD_MAX_PACKETS; // see AeadArgs::spread_max
     // fused relay: plaintext scratch, per-packet flags, sort buffers, staged arrays
     bnk::DevBuf r_plain, r_auth, r_pass, r_keys, r_idx, r_skeys, r_sidx, r_tmp;
     bnk::DevBuf r_peer_out, r_ctr_base, r_ctr_out, r_verdict;

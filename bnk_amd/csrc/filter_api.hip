@@ -146,11 +146,14 @@ int flows_reserve(bnk_ctx *ctx, uint32_t n_new)
 // stride into pinned staging and only that is uploaded.
 constexpr uint32_t HDR_BYTES = 64;
 
+// Small batches skip the upload: the kernel reads the pinned staging in place
+// and writes its verdicts there (*h_verdict, null when the batch was uploaded).
 template <class GetPtr, class GetLen>
-int stage_headers(bnk_ctx *ctx, uint32_t n, GetPtr ptr_of, GetLen len_of, FilterArgs *a)
+int stage_headers(bnk_ctx *ctx, uint32_t n, GetPtr ptr_of, GetLen len_of, FilterArgs *a,
+                  uint8_t **h_verdict)
 {
     const size_t hdr_bytes = (size_t)n * HDR_BYTES, len_bytes = (size_t)n * 4;
-    HIPCHK(ctx, ctx->pin.reserve(hdr_bytes + len_bytes));
+    HIPCHK(ctx, ctx->pin.reserve(hdr_bytes + len_bytes + n));
     uint8_t *hp = ctx->pin.as<uint8_t>();
     uint32_t *hl = reinterpret_cast<uint32_t *>(hp + hdr_bytes);
     for (uint32_t i = 0; i < n; i++) {
@@ -159,15 +162,48 @@ int stage_headers(bnk_ctx *ctx, uint32_t n, GetPtr ptr_of, GetLen len_of, Filter
         const uint32_t c = len < HDR_BYTES ? len : HDR_BYTES;
         if (c) memcpy(hp + (size_t)i * HDR_BYTES, ptr_of(i), c);
     }
+    a->off = nullptr;
+    a->stride = HDR_BYTES;
+    if (n <= DIRECT_MAX_PACKETS) {
+        a->pkts = ctx->pin.dev(hp);
+        a->lens = ctx->pin.dev(hl);
+        *h_verdict = hp + hdr_bytes + len_bytes;
+        return BNK_OK;
+    }
+    *h_verdict = nullptr;
     HIPCHK(ctx, ctx->in_arena.reserve(hdr_bytes));
     HIPCHK(ctx, ctx->lens.reserve(len_bytes));
     HIPCHK(ctx, hipMemcpyAsync(ctx->in_arena.p, hp, hdr_bytes, hipMemcpyHostToDevice, ctx->stream));
     HIPCHK(ctx, hipMemcpyAsync(ctx->lens.p, hl, len_bytes, hipMemcpyHostToDevice, ctx->stream));
     a->pkts = ctx->in_arena.as<uint8_t>();
-    a->off = nullptr;
-    a->stride = HDR_BYTES;
     a->lens = ctx->lens.as<uint32_t>();
     return BNK_OK;
+}
+
+// Runs a staged host batch and brings the verdicts (check) or the overflow
+// flag (note) back.
+int run_staged(bnk_ctx *ctx, bool check, FilterArgs &a, uint8_t *h_verdict, uint8_t *verdict)
+{
+    FilterState *f = ctx->filter;
+    if (!check) {
+        HIPCHK(ctx, launch_filter_note(a, f->max_blocks, ctx->stream));
+    } else if (h_verdict) {
+        // CheckInbound reports nothing through the status word
+        a.verdict = ctx->pin.dev(h_verdict);
+        HIPCHK(ctx, launch_filter_check(a, f->max_blocks, ctx->stream));
+        HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+        memcpy(verdict, h_verdict, a.n);
+        return BNK_OK;
+    } else {
+        HIPCHK(ctx, ctx->verdict.reserve(a.n));
+        a.verdict = ctx->verdict.as<uint8_t>();
+        HIPCHK(ctx, launch_filter_check(a, f->max_blocks, ctx->stream));
+        HIPCHK(ctx, hipMemcpyAsync(verdict, a.verdict, a.n, hipMemcpyDeviceToHost, ctx->stream));
+    }
+    uint32_t status = 0;
+    int rc = take_status(ctx, &status);
+    if (rc) return rc;
+    return status_to_rc(ctx, status);
 }
 
 void base_args(bnk_ctx *ctx, uint32_t n, int64_t now_ns, FilterArgs *a)
@@ -226,22 +262,12 @@ int filter_batch(bnk_ctx *ctx, bool check, const bnk_batch *pkts, int64_t now_ns
     rc = scan_host_layout(ctx, pkts, pkts, 0, &span, "pkts");
     if (rc) return rc;
     const uint8_t *base = (const uint8_t *)pkts->base;
+    uint8_t *h_verdict = nullptr;
     rc = stage_headers(
         ctx, n, [&](uint32_t i) { return base + pkt_off(pkts, i); },
-        [&](uint32_t i) { return pkts->lens ? pkts->lens[i] : pkts->len; }, &a);
+        [&](uint32_t i) { return pkts->lens ? pkts->lens[i] : pkts->len; }, &a, &h_verdict);
     if (rc) return rc;
-    if (check) {
-        HIPCHK(ctx, ctx->verdict.reserve(n));
-        a.verdict = ctx->verdict.as<uint8_t>();
-        HIPCHK(ctx, launch_filter_check(a, f->max_blocks, ctx->stream));
-        HIPCHK(ctx, hipMemcpyAsync(verdict, a.verdict, n, hipMemcpyDeviceToHost, ctx->stream));
-    } else {
-        HIPCHK(ctx, launch_filter_note(a, f->max_blocks, ctx->stream));
-    }
-    uint32_t status = 0;
-    rc = take_status(ctx, &status);
-    if (rc) return rc;
-    return status_to_rc(ctx, status);
+    return run_staged(ctx, check, a, h_verdict, verdict);
 }
 
 int filter_ptrs(bnk_ctx *ctx, bool check, const uint8_t *const *pkts, const uint32_t *lens,
@@ -264,21 +290,11 @@ int filter_ptrs(bnk_ctx *ctx, bool check, const uint8_t *const *pkts, const uint
     }
     FilterArgs a;
     base_args(ctx, n, now_ns, &a);
+    uint8_t *h_verdict = nullptr;
     rc = stage_headers(
-        ctx, n, [&](uint32_t i) { return pkts[i]; }, [&](uint32_t i) { return lens[i]; }, &a);
+        ctx, n, [&](uint32_t i) { return pkts[i]; }, [&](uint32_t i) { return lens[i]; }, &a, &h_verdict);
     if (rc) return rc;
-    if (check) {
-        HIPCHK(ctx, ctx->verdict.reserve(n));
-        a.verdict = ctx->verdict.as<uint8_t>();
-        HIPCHK(ctx, launch_filter_check(a, f->max_blocks, ctx->stream));
-        HIPCHK(ctx, hipMemcpyAsync(verdict, a.verdict, n, hipMemcpyDeviceToHost, ctx->stream));
-    } else {
-        HIPCHK(ctx, launch_filter_note(a, f->max_blocks, ctx->stream));
-    }
-    uint32_t status = 0;
-    rc = take_status(ctx, &status);
-    if (rc) return rc;
-    return status_to_rc(ctx, status);
+    return run_staged(ctx, check, a, h_verdict, verdict);
 }
 
 } // namespace

@@ -28,7 +28,12 @@ struct AeadArgs {
     uint32_t trim;             // seal only: lens[i] - trim is the plaintext length
     uint32_t in_skip, out_skip; // bytes between a packet's offset and its AEAD data
     uint32_t first;            // the launch covers packets first .. first+n-1; order[] is relative to first
+    uint32_t spread_max;       // launches of at most this many packets run one wave per packet
 };
+
+// Below this many packets a wave per packet finishes sooner than a lane per
+// packet (which needs 64 packets per wave and about 130 000 to fill the chip).
+constexpr uint32_t SPREAD_MAX_PACKETS = 4096;
 
 enum : uint32_t { STATUS_PEER_RANGE = 1u, STATUS_FLOWS_FULL = 2u };
 
@@ -64,6 +69,11 @@ hipError_t launch_relay_assign(const uint8_t *auth, const uint8_t *pass, const u
 hipError_t launch_peer_rank(uint32_t *keys, uint32_t *idx, uint32_t *skeys, uint32_t *sidx,
                             void *sort_tmp, size_t sort_tmp_bytes, uint64_t *ctr_base, uint32_t n_keys,
                             uint32_t n, uint64_t *ctr_out, bool advance, hipStream_t s);
+
+// Copy of a byte span whose two ends share their alignment within 16 bytes,
+// one aligned 16-byte piece per lane (used to fetch small spans of pinned
+// host memory).
+hipError_t launch_pull(const void *src, void *dst, uint64_t bytes, hipStream_t s);
 
 // VALU throughput probe; out receives one word per thread so nothing is
 // optimised away.

@@ -30,6 +30,7 @@ extern "C" int bnk_relay_fused_batch(bnk_ctx *ctx, const bnk_batch *in, const ui
 
     // ---- where everything lives on the device ----
     AeadArgs op{};
+    op.spread_max = ctx->spread_max;
     op.keys = ctx->d_keys[BNK_KEYS_RECV];
     op.n_peers = ctx->n_keys[BNK_KEYS_RECV];
     op.status = ctx->d_status;
@@ -139,6 +140,7 @@ extern "C" int bnk_relay_fused_batch(bnk_ctx *ctx, const bnk_batch *in, const ui
 
     // ---- 4. re-seal the survivors under the outbound keys ----
     AeadArgs se{};
+    se.spread_max = ctx->spread_max;
     se.keys = ctx->d_keys[BNK_KEYS_SEND];
     se.n_peers = n_peers_out;
     se.status = ctx->d_status;

@@ -197,6 +197,7 @@ extern "C" int bnk_wg_encap_batch(bnk_ctx *ctx, const bnk_batch *slots, uint32_t
         c.n = hi - lo;
         HIPCHK(ctx, launch_wg_encap_prep(c, pe, d_peer, d_ctr, mtu, d_padded, d_wire_len, d_skip, ctx->stream));
         AeadArgs se{};
+        se.spread_max = ctx->spread_max;
         se.keys = ctx->d_keys[BNK_KEYS_SEND];
         se.n_peers = pe.n;
         se.status = ctx->d_status;
@@ -359,6 +360,7 @@ extern "C" int bnk_wg_decap_batch(bnk_ctx *ctx, const bnk_batch *wire, const bnk
         cw.n = co.n = hi - lo;
         HIPCHK(ctx, launch_wg_parse(cw, pe, d_peer, d_counter, d_ctlen, d_result, ctx->stream));
         AeadArgs op{};
+        op.spread_max = ctx->spread_max;
         op.keys = ctx->d_keys[BNK_KEYS_RECV];
         op.n_peers = pe.n;
         op.status = ctx->d_status;

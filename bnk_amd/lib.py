@@ -210,6 +210,11 @@ class Context:
         self._rings[arr.ctypes.data] = p.value
         return arr
 
+    def set_spread_max_packets(self, max_packets: int) -> None:
+        """Batches of at most this many packets run one wave per packet
+        (0: always one lane per packet).  A tuning knob, results are the same."""
+        self._chk(self._lib.bnk_set_spread_max_packets(self._h, C.c_uint32(max_packets)))
+
     def ring_free(self, arr: np.ndarray) -> None:
         p = self._rings.pop(arr.ctypes.data)
         self._chk(self._lib.bnk_ring_free(self._h, C.c_void_p(p)))

@@ -113,6 +113,84 @@ template <class P> static void run_poly(const char *name)
     }
 }
 
+// The tag of `len` ciphertext bytes the way a wave computes it when one packet
+// is spread over its lanes: 64 lane terms, each evaluated independently.
+static void spread_tag(const uint32_t (&otk)[16], const uint8_t *ct, uint32_t len, uint32_t (&tag)[4])
+{
+    const Fe26 r = fe_clamped_r(otk[0], otk[1], otk[2], otk[3]);
+    const uint32_t e_max = spread_e_max(len);
+    uint64_t sum[5] = {0, 0, 0, 0, 0};
+    for (uint32_t lane = 0; lane < 64; lane++) {
+        uint32_t m[16] = {0};
+        if (lane == 0) {
+            m[2] = len;
+        } else {
+            uint8_t buf[64] = {0};
+            const uint32_t at = 64 * (lane - 1);
+            if (at < len) memcpy(buf, ct + at, len - at < 64 ? len - at : 64);
+            for (int i = 0; i < 16; i++) m[i] = ld32(buf + 4 * i);
+        }
+        const SpreadShare sh = spread_share(lane, len);
+        const Fe26 t = spread_term(r, m, sh.k, sh.e, e_max);
+        sum[0] += t.v0; sum[1] += t.v1; sum[2] += t.v2; sum[3] += t.v3; sum[4] += t.v4;
+    }
+    const uint32_t pad[4] = {otk[4], otk[5], otk[6], otk[7]};
+    spread_finish(sum, pad, tag);
+}
+
+// The same tag serially: zero-padded cells, then the length block.
+static void serial_tag(const uint32_t (&otk)[16], const uint8_t *ct, uint32_t len, uint32_t (&tag)[4])
+{
+    Poly32 mac;
+    mac.init(otk);
+    for (uint32_t o = 0; o < len; o += 16) {
+        uint8_t cell[16] = {0};
+        memcpy(cell, ct + o, len - o < 16 ? len - o : 16);
+        mac.block(ld32(cell), ld32(cell + 4), ld32(cell + 8), ld32(cell + 12));
+    }
+    mac.block(0, 0, len, 0);
+    mac.finish(tag);
+}
+
+static void run_spread()
+{
+    uint64_t st = 777;
+    auto rnd = [&]() { st ^= st << 13; st ^= st >> 7; st ^= st << 17; return st; };
+    std::vector<uint8_t> ct(SPREAD_MAX_LEN);
+    int bad = 0, cases = 0;
+    auto check = [&](const uint32_t (&otk)[16], uint32_t len) {
+        uint32_t a[4], b[4];
+        spread_tag(otk, ct.data(), len, a);
+        serial_tag(otk, ct.data(), len, b);
+        cases++;
+        if (memcmp(a, b, 16) != 0) bad++;
+    };
+    // every length class around cell, block and lane boundaries, random keys
+    for (uint32_t len = 0; len <= SPREAD_MAX_LEN; len += (len < 300 || len > SPREAD_MAX_LEN - 80) ? 1 : 37) {
+        uint32_t otk[16];
+        for (auto &w : otk) w = (uint32_t)rnd();
+        for (auto &b : ct) b = (uint8_t)rnd();
+        check(otk, len);
+    }
+    // extreme limbs: r with every clamped bit set, all-ones and all-zero data
+    // (drives the carries of the limb products and of the lane sum to their
+    // largest), and the RFC 8439 A.3 keys r = 1, 2 with s = 0 or all ones
+    for (int data = 0; data < 3; data++)
+        for (int key = 0; key < 4; key++) {
+            uint32_t otk[16] = {0};
+            if (key == 0) { otk[0] = 0x0fffffffu; otk[1] = otk[2] = otk[3] = 0x0ffffffcu; }
+            if (key == 1) otk[0] = 1;
+            if (key == 2) { otk[0] = 2; otk[4] = otk[5] = otk[6] = otk[7] = 0xffffffffu; }
+            if (key == 3) { otk[0] = 0x0fffffffu; otk[1] = otk[2] = otk[3] = 0x0ffffffcu;
+                            otk[4] = otk[5] = otk[6] = otk[7] = 0xffffffffu; }
+            for (auto &b : ct) b = data == 0 ? 0xff : data == 1 ? 0x00 : (uint8_t)rnd();
+            for (uint32_t len : {0u, 1u, 15u, 16u, 17u, 63u, 64u, 65u, 256u, 1420u, 1436u, 4000u, 4031u, 4032u})
+                check(otk, len);
+        }
+    printf("spread tags: %d cases, %d differ from the serial form\n", cases, bad);
+    expect(bad == 0, "one packet spread over the lanes of a wave");
+}
+
 int main()
 {
     // ChaCha20 block, RFC 8439 2.3.2 through the WireGuard-shaped state
@@ -136,6 +214,7 @@ int main()
     }
     run_poly<Poly26>("Poly26");
     run_poly<Poly32>("Poly32");
+    run_spread();
     printf(failures ? "FAILED %d\n" : "PASS lane arithmetic (%d failures)\n", failures);
     return failures;
 }

@@ -20,6 +20,16 @@ def ctx():
     c.close()
 
 
+@pytest.fixture(params=["wave_per_packet", "lane_per_packet"])
+def small_ctx(request, ctx):
+    """Small batches run one wave per packet by default; with the threshold at
+    zero they take the lane-per-packet kernel the large batches use.  Tests of
+    small batches run both ways."""
+    ctx.set_spread_max_packets(4096 if request.param == "wave_per_packet" else 0)
+    yield ctx
+    ctx.set_spread_max_packets(4096)
+
+
 def _oracle_seal(b):
     from oracle import binding as O
     out = np.zeros_like(b.plain)
@@ -71,7 +81,8 @@ def _packets_equal(a, b, off, lens, extra=0):
     return -1
 
 
-def test_cfg1_against_oracle_and_openssl_fixture(ctx):
+def test_cfg1_against_oracle_and_openssl_fixture(small_ctx):
+    ctx = small_ctx
     b = W.aead_uniform(1, 128, 1420)
     got = _gpu_seal_host(ctx, b, uniform=True)
     want = _oracle_seal(b)
@@ -96,7 +107,8 @@ EDGE_LENS = [0, 1, 3, 4, 15, 16, 17, 31, 32, 33, 47, 48, 49, 63, 64, 65, 79, 80,
              255, 256, 575, 576, 1419, 1420, 1421, 1424, 1500, 4096, 9000]
 
 
-def test_edge_lengths_and_high_counters(ctx):
+def test_edge_lengths_and_high_counters(small_ctx):
+    ctx = small_ctx
     lens = np.array(EDGE_LENS * 3, np.uint32)
     b = W.aead_imix(11, len(lens), n_peers=5, lens=lens)
     # counters straddling 2^32 and the top of the 64-bit range
@@ -112,7 +124,8 @@ def test_edge_lengths_and_high_counters(ctx):
 
 
 @pytest.mark.parametrize("n", [64, 128, 100])
-def test_unsorted_mixed_lengths_within_a_wave(ctx, n):
+def test_unsorted_mixed_lengths_within_a_wave(small_ctx, n):
+    ctx = small_ctx
     """Up to 64 packets are not grouped by length, so one wave holds long and
     short packets at once: the lines inside every packet of the wave take the
     unchecked route, the others the bounds-checked one, and a partly filled
@@ -136,7 +149,8 @@ def test_unsorted_mixed_lengths_within_a_wave(ctx, n):
     assert np.array_equal(back, oback)
 
 
-def test_imix_multi_peer_with_forged_tags(ctx):
+def test_imix_multi_peer_with_forged_tags(small_ctx):
+    ctx = small_ctx
     from oracle import binding as O
     b = W.aead_imix(3, 6000, n_peers=256)
     got = _gpu_seal_host(ctx, b, uniform=False)
@@ -156,7 +170,8 @@ def test_imix_multi_peer_with_forged_tags(ctx):
     assert not back[o:o + L].any()
 
 
-def test_maximum_packet_sizes(ctx):
+def test_maximum_packet_sizes(small_ctx):
+    ctx = small_ctx
     """Jumbo frames and the largest length a 16-bit IP total-length field can
     name (65,535), next to minimum-size packets: more ChaCha20 blocks than the
     length grouping has bins, in both memory paths' batch sizes."""
@@ -235,7 +250,76 @@ def test_large_host_batches_take_the_chunked_route(ctx, layout):
     assert np.array_equal(back, oback)
 
 
-def test_in_place_and_unaligned_slots(ctx):
+@pytest.mark.parametrize("layout", ["offsets", "reversed", "in_place", "uniform"])
+@pytest.mark.parametrize("n", [1, 70, 2048, 2049])
+def test_small_batches_in_pinned_rings(small_ctx, layout, n):
+    """Small host batches whose arenas are pinned rings of the context are read
+    and written in place by the kernel (no staging copies); one packet more
+    than that route takes and the batch is staged again.  Same bar either way:
+    oracle-exact bytes, verdicts, zero-filled rejects and untouched gaps."""
+    ctx = small_ctx
+    from bnk_amd import lib
+    from oracle import binding as O
+    if layout == "uniform":
+        b = W.aead_uniform(15, n, 333, stride=352, counter0=(1 << 40) + 5)
+    else:
+        b = W.aead_imix(15, n, n_peers=8)
+    off, peer, counters, lens = b.off, b.peer, b.counters, b.lens
+    if layout == "reversed":
+        perm = np.arange(n)[::-1].copy()
+        off, peer, counters, lens = off[perm].copy(), peer[perm].copy(), counters[perm].copy(), lens[perm].copy()
+    keys = np.ascontiguousarray(b.keys)
+    ctx.keys_set(lib.KEYS_SEND, keys)
+    ctx.keys_set(lib.KEYS_RECV, keys)
+    want = np.full_like(b.plain, 0x5A)
+    O.seal_batch(keys, peer, counters, b.plain, off, lens, want, off, 4)
+    ct_lens = (lens + 16).astype(np.uint32)
+    nbytes = b.plain.nbytes
+    rings = [ctx.ring_alloc(nbytes + 64) for _ in range(3)]
+    # arenas that start inside a ring, not at its base
+    src, got, back = (r[32:32 + nbytes] for r in rings)
+
+    def batch(buf, ln, with_meta=True):
+        if layout == "uniform":
+            return lib.make_batch(buf, nbytes, n, lib.MEM_HOST, stride=b.stride,
+                                  length=int(ln[0]) if with_meta else 0, counter0=(1 << 40) + 5)
+        return lib.make_batch(buf, nbytes, n, lib.MEM_HOST, offsets=off,
+                              lens=ln if with_meta else None, peer=peer if with_meta else None,
+                              counters=counters if with_meta else None)
+
+    try:
+        if layout == "in_place":
+            got[:] = b.plain
+            ctx.seal(batch(got, lens), batch(got, lens, False))
+            assert _packets_equal(got, want, off, lens, 16) == -1
+            mask = np.ones(got.size, bool)
+            for o, l in zip(off.astype(np.int64), lens.astype(np.int64)):
+                mask[o:o + l + 16] = False
+            assert np.array_equal(got[mask], b.plain[mask])
+        else:
+            src[:] = b.plain
+            got[:] = 0x5A
+            ctx.seal(batch(src, lens), batch(got, lens, False))
+            assert np.array_equal(got, want)
+        forged = W.forge_tags(15, got, off, lens, 0.1) if n > 1 else np.zeros(1, bool)
+        back[:] = 0xEE
+        verdict = np.full(n, 7, np.uint8)
+        ctx.open(batch(got, ct_lens), batch(back, lens, False), verdict)
+        oback = np.full_like(b.plain, 0xEE)
+        overdict = O.open_batch(keys, peer, counters, np.array(got), off, ct_lens, oback, off, 4)
+        assert np.array_equal(verdict, overdict)
+        assert np.array_equal(verdict == 0, forged)
+        assert np.array_equal(back, oback)
+        # a ring that has been freed is staged like any other host memory
+        spare = ctx.ring_alloc(nbytes)
+        ctx.ring_free(spare)
+    finally:
+        for r in rings:
+            ctx.ring_free(r)
+
+
+def test_in_place_and_unaligned_slots(small_ctx):
+    ctx = small_ctx
     """WireGuard seals in place at offset 16 of its buffers; slots need not be
     16-byte aligned."""
     from bnk_amd import lib
@@ -265,7 +349,8 @@ def test_in_place_and_unaligned_slots(ctx):
     assert np.array_equal(wv.reshape(n, stride)[:, :L], view.reshape(n, stride)[:, :L])
 
 
-def test_short_and_error_paths(ctx):
+def test_short_and_error_paths(small_ctx):
+    ctx = small_ctx
     from bnk_amd import lib
     b = W.aead_uniform(13, 4, 32)
     ctx.keys_set(lib.KEYS_SEND, b.keys)

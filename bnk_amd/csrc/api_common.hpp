@@ -90,9 +90,10 @@ inline int check_batch_common(bnk_ctx *ctx, const bnk_batch *b, const char *name
 
 
 // Host batches up to this size run in place when their arenas are pinned rings
-// of the context (no staging copies): above it the copy engines win.
-constexpr uint32_t DIRECT_MAX_PACKETS = 2048;
-constexpr uint64_t DIRECT_MAX_BYTES = 1ull << 20;
+// of the context (no staging copies).  Measured against the chunked copy-engine
+// route the crossover lies at about 8 MB of packets, whatever their size.
+constexpr uint32_t DIRECT_MAX_PACKETS = 1u << 16;
+constexpr uint64_t DIRECT_MAX_BYTES = 8ull << 20;
 
 // Device address of [p, p + bytes) when it lies inside one of the context's
 // pinned rings, else null.

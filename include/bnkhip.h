@@ -118,7 +118,8 @@ void *bnk_stream(bnk_ctx *ctx);
 /* Tuning: seal/open batches of at most max_packets packets give each packet
  * a whole wave instead of one lane (a lane needs about 85 us for a 1420-byte
  * packet however small the batch; a wave about a tenth of that).  Default
- * 4096; 0 always uses a lane per packet.  Results do not depend on it.  No
+ * 4096, scaled by the packet length when the batch has one common length; 0
+ * always uses a lane per packet.  Results do not depend on it.  No
  * counterpart in the reference. */
 int bnk_set_spread_max_packets(bnk_ctx *ctx, uint32_t max_packets);
 

@@ -584,7 +584,7 @@ __global__ __launch_bounds__(256) void aead_spread_kernel(AeadArgs a)
 // however few packets there are, a wave per packet about 20 us + 4 ns per
 // packet: with the common length known the crossover is near 10 packets per
 // byte, without it the caller's threshold stands alone.
-static bool use_spread(const AeadArgs &a)
+bool aead_runs_spread(const AeadArgs &a)
 {
     if (a.lens) return a.n <= a.spread_max;
     const uint64_t by_len = std::max<uint64_t>(10ull * a.len, a.spread_max / 4);
@@ -594,7 +594,7 @@ static bool use_spread(const AeadArgs &a)
 hipError_t launch_aead_seal(const AeadArgs &a, hipStream_t s)
 {
     if (a.n == 0) return hipSuccess;
-    if (use_spread(a))
+    if (aead_runs_spread(a))
         hipLaunchKernelGGL(aead_spread_kernel<false>, dim3((a.n + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK),
                            dim3(256), 0, s, a);
     else
@@ -605,7 +605,7 @@ hipError_t launch_aead_seal(const AeadArgs &a, hipStream_t s)
 hipError_t launch_aead_open(const AeadArgs &a, hipStream_t s)
 {
     if (a.n == 0) return hipSuccess;
-    if (use_spread(a))
+    if (aead_runs_spread(a))
         hipLaunchKernelGGL(aead_spread_kernel<true>, dim3((a.n + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK),
                            dim3(256), 0, s, a);
     else

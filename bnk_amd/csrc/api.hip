@@ -119,8 +119,10 @@ int aead_batch_host_direct(bnk_ctx *ctx, bool open, const bnk_batch *in, const b
     // The input span is fetched into device memory by one wide copy kernel
     // (every 16 bytes in flight at once); the AEAD kernel then writes its
     // output straight into the ring, where stores need no round trip.
-    const uint32_t mis = (uint32_t)((uintptr_t)(d_in + sin.lo) & 15u);
-    HIPCHK(ctx, ctx->in_arena.reserve(sin.size() + 32));
+    // the copy keeps the span's position within a 128-byte line, which is what
+    // lets the lane-per-packet kernel move whole lines
+    const uint32_t mis = (uint32_t)((uintptr_t)(d_in + sin.lo) & 127u);
+    HIPCHK(ctx, ctx->in_arena.reserve(sin.size() + 160));
     HIPCHK(ctx, launch_pull(d_in + sin.lo, ctx->in_arena.as<uint8_t>() + mis, sin.size(), ctx->stream));
     a.in = ctx->in_arena.as<uint8_t>() + mis;
     a.out = d_out;
@@ -134,7 +136,7 @@ int aead_batch_host_direct(bnk_ctx *ctx, bool open, const bnk_batch *in, const b
     if (in->lens) {
         memcpy(p_lens, in->lens, (size_t)n * 4);
         a.lens = ctx->pin.dev(p_lens);
-        if (n > 64) {
+        if (n > 64 && !aead_runs_spread(a)) {
             // lanes of a wave should run equal block counts: longest first
             const uint32_t tag = open ? 16 : 0;
             auto blocks = [&](uint32_t i) {
@@ -207,7 +209,7 @@ int aead_batch(bnk_ctx *ctx, bool open, const bnk_batch *in, const bnk_batch *ou
         a.peer = in->peer;
         a.counters = in->counters;
         a.verdict = verdict;
-        rc = maybe_sort(ctx, a.lens, n, open ? 16 : 0, &a.order);
+        rc = maybe_sort(ctx, &a, open ? 16 : 0);
         if (rc) return rc;
         HIPCHK(ctx, open ? launch_aead_open(a, ctx->stream) : launch_aead_seal(a, ctx->stream));
         return BNK_OK;
@@ -231,7 +233,7 @@ int aead_batch(bnk_ctx *ctx, bool open, const bnk_batch *in, const bnk_batch *ou
         HIPCHK(ctx, ctx->verdict.reserve(n));
         a.verdict = ctx->verdict.as<uint8_t>();
     }
-    rc = maybe_sort(ctx, a.lens, n, open ? 16 : 0, &a.order);
+    rc = maybe_sort(ctx, &a, open ? 16 : 0);
     if (rc) return rc;
     HIPCHK(ctx, open ? launch_aead_open(a, ctx->stream) : launch_aead_seal(a, ctx->stream));
     HIPCHK(ctx, hipMemcpyAsync((uint8_t *)out->base + st.sout.lo, st.d_out, st.sout.size(),

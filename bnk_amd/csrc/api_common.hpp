@@ -206,18 +206,18 @@ inline int stage_host(bnk_ctx *ctx, const bnk_batch *in, const bnk_batch *out, i
 
 // Lanes of a wave should run the same number of ChaCha20 blocks: when lengths
 // vary, hand packets to lanes in length order.
-inline int maybe_sort(bnk_ctx *ctx, const uint32_t *d_lens, uint32_t n, uint32_t tag_bytes,
-               const uint32_t **order)
+// A launch that gives every packet its own wave has no use for the order.
+inline int maybe_sort(bnk_ctx *ctx, AeadArgs *a, uint32_t tag_bytes)
 {
-    *order = nullptr;
-    if (!d_lens || n <= 64) return BNK_OK;
-    HIPCHK(ctx, ctx->order.reserve((size_t)n * 4));
+    a->order = nullptr;
+    if (!a->lens || a->n <= 64 || aead_runs_spread(*a)) return BNK_OK;
+    HIPCHK(ctx, ctx->order.reserve((size_t)a->n * 4));
     HIPCHK(ctx, ctx->hist.reserve(LEN_BINS * 4));
     HIPCHK(ctx, ctx->cursor.reserve(LEN_BINS * 4));
-    HIPCHK(ctx, launch_length_sort(d_lens, n, tag_bytes, ctx->order.as<uint32_t>(),
+    HIPCHK(ctx, launch_length_sort(a->lens, a->n, tag_bytes, ctx->order.as<uint32_t>(),
                                    ctx->hist.as<uint32_t>(), ctx->cursor.as<uint32_t>(),
                                    ctx->stream));
-    *order = ctx->order.as<uint32_t>();
+    a->order = ctx->order.as<uint32_t>();
     return BNK_OK;
 }
 

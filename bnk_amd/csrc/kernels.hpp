@@ -37,6 +37,9 @@ constexpr uint32_t SPREAD_MAX_PACKETS = 4096;
 
 enum : uint32_t { STATUS_PEER_RANGE = 1u, STATUS_FLOWS_FULL = 2u };
 
+// True when the launch will run one wave per packet (then order[] is not used
+// and callers need not build it).
+bool aead_runs_spread(const AeadArgs &a);
 hipError_t launch_aead_seal(const AeadArgs &a, hipStream_t s);
 hipError_t launch_aead_open(const AeadArgs &a, hipStream_t s);
 
@@ -74,6 +77,13 @@ hipError_t launch_peer_rank(uint32_t *keys, uint32_t *idx, uint32_t *skeys, uint
 // one aligned 16-byte piece per lane (used to fetch small spans of pinned
 // host memory).
 hipError_t launch_pull(const void *src, void *dst, uint64_t bytes, hipStream_t s);
+
+// launch_wg_keys + launch_peer_rank for at most PEER_RANK_SMALL_MAX packets in
+// one launch, straight from the peer array (null: every packet is peer 0).  A
+// peer index beyond the table sets STATUS_PEER_RANGE and gets no counter.
+constexpr uint32_t PEER_RANK_SMALL_MAX = 1024;
+hipError_t launch_peer_rank_small(const uint32_t *peer, uint32_t n_keys, uint32_t n, uint64_t *ctr_base,
+                                  uint64_t *ctr_out, bool advance, uint32_t *status, hipStream_t s);
 
 // VALU throughput probe; out receives one word per thread so nothing is
 // optimised away.

@@ -104,7 +104,7 @@ extern "C" int bnk_relay_fused_batch(bnk_ctx *ctx, const bnk_batch *in, const ui
     op.out_off = op.in_off;
     op.out_stride = in->stride;
     op.verdict = ctx->r_auth.as<uint8_t>();
-    rc = maybe_sort(ctx, op.lens, n, 16, &op.order);
+    rc = maybe_sort(ctx, &op, 16);
     if (rc) return rc;
     HIPCHK(ctx, launch_aead_open(op, ctx->stream));
 

@@ -115,6 +115,51 @@ hipError_t launch_relay_assign(const uint8_t *auth, const uint8_t *pass, const u
                             const_cast<uint64_t *>(ctr_base_out), n_peers_out, n, ctr_out, false, s);
 }
 
+// Batch-order counters for a small batch in one launch of one block, straight
+// from the peer array: every thread compares its packet with all the others
+// in LDS.  The last packet of each peer moves the peer's base.
+__global__ __launch_bounds__(1024) void peer_rank_small_kernel(const uint32_t *peer, uint32_t n_keys,
+                                                               uint32_t n, uint64_t *ctr_base,
+                                                               uint64_t *ctr_out, int advance,
+                                                               uint32_t *status)
+{
+    __shared__ uint32_t pk[PEER_RANK_SMALL_MAX];
+    const uint32_t i = threadIdx.x;
+    uint32_t p = NO_PEER;
+    if (i < n) {
+        p = peer ? peer[i] : 0u;
+        if (p >= n_keys) {
+            atomicOr(status, STATUS_PEER_RANGE);
+            p = NO_PEER;
+        }
+    }
+    pk[i] = p;
+    __syncthreads();
+    uint32_t before = 0, after = 0;
+    uint64_t base = 0;
+    if (p != NO_PEER) {
+        for (uint32_t j = 0; j < n; j++) {
+            const bool same = pk[j] == p;
+            before += (same && j < i) ? 1u : 0u;
+            after += (same && j > i) ? 1u : 0u;
+        }
+        base = ctr_base[p];
+        ctr_out[i] = base + before;
+    }
+    __syncthreads(); // every base has been read
+    if (advance && p != NO_PEER && after == 0) ctr_base[p] = base + before + 1u;
+}
+
+hipError_t launch_peer_rank_small(const uint32_t *peer, uint32_t n_keys, uint32_t n, uint64_t *ctr_base,
+                                  uint64_t *ctr_out, bool advance, uint32_t *status, hipStream_t s)
+{
+    if (n == 0) return hipSuccess;
+    if (n > PEER_RANK_SMALL_MAX) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(peer_rank_small_kernel, dim3(1), dim3(1024), 0, s, peer, n_keys, n, ctr_base, ctr_out,
+                       advance ? 1 : 0, status);
+    return hipGetLastError();
+}
+
 hipError_t launch_peer_rank(uint32_t *keys, uint32_t *idx, uint32_t *skeys, uint32_t *sidx,
                             void *sort_tmp, size_t sort_tmp_bytes, uint64_t *ctr_base, uint32_t n_keys,
                             uint32_t n, uint64_t *ctr_out, bool advance, hipStream_t s)

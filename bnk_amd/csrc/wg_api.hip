@@ -110,12 +110,48 @@ extern "C" int bnk_wg_encap_batch(bnk_ctx *ctx, const bnk_batch *slots, uint32_t
     Span span;
     HostPipe hp;
     bool chunked = false;
+    // direct route (small batches in a pinned ring): the plaintexts are fetched
+    // by a copy kernel, headers and sealed packets go straight into the ring
+    uint8_t *ring_out = nullptr;
+    uint32_t *h_wire_len = nullptr;
     if (host) {
         if (slots->peer)
             for (uint32_t i = 0; i < n; i++)
                 if (slots->peer[i] >= ctx->n_wg_peers)
                     return fail(ctx, BNK_E_RANGE, "peer index " + std::to_string(slots->peer[i]) +
                                                       " beyond the peer table");
+        uint8_t *d_ring = n <= DIRECT_MAX_PACKETS ? ring_device_ptr(ctx, slots->base, slots->bytes) : nullptr;
+        if (d_ring) {
+            Span sp;
+            for (uint32_t i = 0; i < n; i++) {
+                const uint64_t off = pkt_off(slots, i), need = slot_ext(i);
+                if (off > slots->bytes || need > slots->bytes - off)
+                    return fail(ctx, BNK_E_INVAL, "slots: packet " + std::to_string(i) + " lies outside the arena");
+                sp.add(off, off + need);
+            }
+            if (sp.size() <= DIRECT_MAX_BYTES) {
+                span = sp;
+                ring_out = d_ring + span.lo;
+            }
+        }
+    }
+    if (ring_out) {
+        HIPCHK(ctx, ctx->pin.reserve((size_t)n * 20 + 64));
+        uint64_t *p_off = ctx->pin.as<uint64_t>();
+        uint32_t *p_lens = (uint32_t *)(p_off + n), *p_peer = p_lens + n;
+        h_wire_len = p_peer + n;
+        const uint32_t mis = (uint32_t)((uintptr_t)ring_out & 127u);
+        HIPCHK(ctx, ctx->in_arena.reserve(span.size() + 160));
+        HIPCHK(ctx, launch_pull(ring_out, ctx->in_arena.as<uint8_t>() + mis, span.size(), ctx->stream));
+        b.base = ctx->in_arena.as<uint8_t>() + mis;
+        if (slots->offsets) {
+            for (uint32_t i = 0; i < n; i++) p_off[i] = slots->offsets[i] - span.lo;
+            b.off = ctx->pin.dev(p_off);
+        }
+        if (slots->lens) { memcpy(p_lens, slots->lens, (size_t)n * 4); b.lens = ctx->pin.dev(p_lens); }
+        if (slots->peer) { memcpy(p_peer, slots->peer, (size_t)n * 4); d_peer = ctx->pin.dev(p_peer); }
+        d_wire_len = ctx->pin.dev(h_wire_len);
+    } else if (host) {
         HIPCHK(ctx, ctx->wg_wirelen.reserve((size_t)n * 4));
         d_wire_len = ctx->wg_wirelen.as<uint32_t>();
         hp.ctx = ctx;
@@ -184,18 +220,23 @@ extern "C" int bnk_wg_encap_batch(bnk_ctx *ctx, const bnk_batch *slots, uint32_t
 
     // counters in batch order per peer, advancing the peers' send counters:
     // needs the peer array only, so it runs ahead of the packet bytes
-    HIPCHK(ctx, launch_wg_keys(d_peer, pe.n, n, ctx->r_keys.as<uint32_t>(), ctx->r_idx.as<uint32_t>(),
-                               ctx->d_status, ctx->stream));
-    HIPCHK(ctx, launch_peer_rank(ctx->r_keys.as<uint32_t>(), ctx->r_idx.as<uint32_t>(),
-                                 ctx->r_skeys.as<uint32_t>(), ctx->r_sidx.as<uint32_t>(), ctx->r_tmp.p,
-                                 tmp_bytes, pe.send_ctr, pe.n, n, d_ctr, true, ctx->stream));
+    if (n <= PEER_RANK_SMALL_MAX) {
+        HIPCHK(ctx, launch_peer_rank_small(d_peer, pe.n, n, pe.send_ctr, d_ctr, true, ctx->d_status, ctx->stream));
+    } else {
+        HIPCHK(ctx, launch_wg_keys(d_peer, pe.n, n, ctx->r_keys.as<uint32_t>(), ctx->r_idx.as<uint32_t>(),
+                                   ctx->d_status, ctx->stream));
+        HIPCHK(ctx, launch_peer_rank(ctx->r_keys.as<uint32_t>(), ctx->r_idx.as<uint32_t>(),
+                                     ctx->r_skeys.as<uint32_t>(), ctx->r_sidx.as<uint32_t>(), ctx->r_tmp.p,
+                                     tmp_bytes, pe.send_ctr, pe.n, n, d_ctr, true, ctx->stream));
+    }
 
     // header, padding and seal of packets [lo, hi)
     auto run = [&](uint32_t lo, uint32_t hi) -> int {
         WgBatch c = b;
         c.first = lo;
         c.n = hi - lo;
-        HIPCHK(ctx, launch_wg_encap_prep(c, pe, d_peer, d_ctr, mtu, d_padded, d_wire_len, d_skip, ctx->stream));
+        uint8_t *sealed = ring_out ? ring_out : const_cast<uint8_t *>(b.base);
+        HIPCHK(ctx, launch_wg_encap_prep(c, sealed, pe, d_peer, d_ctr, mtu, d_padded, d_wire_len, d_skip, ctx->stream));
         AeadArgs se{};
         se.spread_max = ctx->spread_max;
         se.keys = ctx->d_keys[BNK_KEYS_SEND];
@@ -204,7 +245,7 @@ extern "C" int bnk_wg_encap_batch(bnk_ctx *ctx, const bnk_batch *slots, uint32_t
         se.first = lo;
         se.n = hi - lo;
         se.in = b.base;
-        se.out = const_cast<uint8_t *>(b.base);
+        se.out = sealed;
         se.in_off = se.out_off = b.off;
         se.in_stride = se.out_stride = slots->stride;
         se.in_skip = se.out_skip = 16;
@@ -212,7 +253,7 @@ extern "C" int bnk_wg_encap_batch(bnk_ctx *ctx, const bnk_batch *slots, uint32_t
         se.peer = d_peer;
         se.counters = d_ctr;
         se.skip = d_skip;
-        if (slots->lens && se.n > 64) { // equal plaintext lengths pad to equal lengths
+        if (slots->lens && se.n > 64 && !aead_runs_spread(se)) { // equal plaintext lengths pad to equal lengths
             HIPCHK(ctx, launch_length_sort(d_padded + lo, se.n, 0, ctx->order.as<uint32_t>() + lo,
                                            ctx->hist.as<uint32_t>(), ctx->cursor.as<uint32_t>(), ctx->stream));
             se.order = ctx->order.as<uint32_t>() + lo;
@@ -235,6 +276,12 @@ extern "C" int bnk_wg_encap_batch(bnk_ctx *ctx, const bnk_batch *slots, uint32_t
         rc = run(0, n);
         if (rc) return rc;
         if (!host) return BNK_OK;
+        if (ring_out) {
+            // peer indices were checked above: nothing comes back through the status word
+            HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+            memcpy(wire_len, h_wire_len, (size_t)n * 4);
+            return BNK_OK;
+        }
         HIPCHK(ctx, hipMemcpyAsync((uint8_t *)slots->base + span.lo, ctx->in_arena.p, span.size(),
                                    hipMemcpyDeviceToHost, ctx->stream));
         HIPCHK(ctx, hipMemcpyAsync(wire_len, d_wire_len, (size_t)n * 4, hipMemcpyDeviceToHost, ctx->stream));
@@ -284,7 +331,50 @@ extern "C" int bnk_wg_decap_batch(bnk_ctx *ctx, const bnk_batch *wire, const bnk
         const uint64_t l = wire->lens ? wire->lens[i] : wire->len;
         return l >= 32u ? l - 32u : (uint64_t)0;
     };
-    if (host) {
+    // direct route (small batches in pinned rings): datagrams fetched by a copy
+    // kernel, plaintexts written straight into the out ring, per-packet results
+    // into pinned staging
+    bool direct = false;
+    uint8_t *h_result = nullptr;
+    uint32_t *h_out_len = nullptr, *h_peer = nullptr;
+    uint64_t *h_counter = nullptr;
+    if (host && n <= DIRECT_MAX_PACKETS) {
+        uint8_t *d_wire = ring_device_ptr(ctx, wire->base, wire->bytes);
+        uint8_t *d_outr = ring_device_ptr(ctx, out->base, out->bytes);
+        if (d_wire && d_outr) {
+            Span sin, sout;
+            rc = scan_host_layout(ctx, &w2, &w2, 0, &sin, "in");
+            if (rc) return rc;
+            rc = scan_host_layout(ctx, out, &w2, -32, &sout, "out");
+            if (rc) return rc;
+            if (sin.size() <= DIRECT_MAX_BYTES) {
+                direct = true;
+                HIPCHK(ctx, ctx->pin.reserve((size_t)n * 37 + 64));
+                uint64_t *p_in_off = ctx->pin.as<uint64_t>(), *p_out_off = p_in_off + n;
+                h_counter = p_out_off + n;
+                uint32_t *p_lens = (uint32_t *)(h_counter + n);
+                h_out_len = p_lens + n;
+                h_peer = h_out_len + n;
+                h_result = (uint8_t *)(h_peer + n);
+                const uint32_t mis = (uint32_t)((uintptr_t)(d_wire + sin.lo) & 127u);
+                HIPCHK(ctx, ctx->in_arena.reserve(sin.size() + 160));
+                HIPCHK(ctx, launch_pull(d_wire + sin.lo, ctx->in_arena.as<uint8_t>() + mis, sin.size(), ctx->stream));
+                wb.base = ctx->in_arena.as<uint8_t>() + mis;
+                if (wire->offsets) {
+                    for (uint32_t i = 0; i < n; i++) p_in_off[i] = wire->offsets[i] - sin.lo;
+                    wb.off = ctx->pin.dev(p_in_off);
+                }
+                if (wire->lens) { memcpy(p_lens, wire->lens, (size_t)n * 4); wb.lens = ctx->pin.dev(p_lens); }
+                ob.base = d_outr;
+                if (out->offsets) { memcpy(p_out_off, out->offsets, (size_t)n * 8); ob.off = ctx->pin.dev(p_out_off); }
+                d_result = ctx->pin.dev(h_result);
+                d_out_len = ctx->pin.dev(h_out_len);
+                d_peer = ctx->pin.dev(h_peer);
+                d_counter = ctx->pin.dev(h_counter);
+            }
+        }
+    }
+    if (host && !direct) {
         HIPCHK(ctx, ctx->wg_result.reserve(n));
         HIPCHK(ctx, ctx->wg_outlen.reserve((size_t)n * 4));
         HIPCHK(ctx, ctx->wg_peer.reserve((size_t)n * 4));
@@ -326,7 +416,7 @@ extern "C" int bnk_wg_decap_batch(bnk_ctx *ctx, const bnk_batch *wire, const bnk
             ob.base = st.d_out;
             ob.off = st.d_out_off;
         }
-    } else {
+    } else if (!host) {
         if (!wire->offsets && !wire->lens && (uint64_t)(n - 1) * wire->stride + wire->len > wire->bytes)
             return fail(ctx, BNK_E_INVAL, "wire: uniform layout exceeds the arena");
         if (!out->offsets && !wire->lens &&
@@ -378,7 +468,7 @@ extern "C" int bnk_wg_decap_batch(bnk_ctx *ctx, const bnk_batch *wire, const bnk
         op.counters = d_counter;
         op.verdict = d_auth;
         op.skip = d_result; // BNK_WG_OK is 0: header failures are not opened
-        if (wire->lens && op.n > 64) {
+        if (wire->lens && op.n > 64 && !aead_runs_spread(op)) {
             HIPCHK(ctx, launch_length_sort(d_ctlen + lo, op.n, 16, ctx->order.as<uint32_t>() + lo,
                                            ctx->hist.as<uint32_t>(), ctx->cursor.as<uint32_t>(), ctx->stream));
             op.order = ctx->order.as<uint32_t>() + lo;
@@ -402,6 +492,16 @@ extern "C" int bnk_wg_decap_batch(bnk_ctx *ctx, const bnk_batch *wire, const bnk
         rc = run(0, n);
         if (rc) return rc;
         if (!host) return BNK_OK;
+        if (direct) {
+            // the peer index of every opened packet comes from the table lookup:
+            // nothing comes back through the status word
+            HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+            memcpy(result, h_result, n);
+            memcpy(out_len, h_out_len, (size_t)n * 4);
+            memcpy(peer, h_peer, (size_t)n * 4);
+            memcpy(counter, h_counter, (size_t)n * 8);
+            return BNK_OK;
+        }
         HIPCHK(ctx, hipMemcpyAsync((uint8_t *)out->base + st.sout.lo, st.d_out, st.sout.size(),
                                    hipMemcpyDeviceToHost, ctx->stream));
         HIPCHK(ctx, hipMemcpyAsync(result, d_result, n, hipMemcpyDeviceToHost, ctx->stream));

@@ -29,7 +29,7 @@ hipError_t launch_wg_finish(const WgBatch &out, uint32_t out_skip, const WgPeers
                             uint8_t *result, uint32_t *out_len, hipStream_t s);
 hipError_t launch_wg_keys(const uint32_t *peer, uint32_t n_peers, uint32_t n, uint32_t *keys,
                           uint32_t *idx, uint32_t *status, hipStream_t s);
-hipError_t launch_wg_encap_prep(const WgBatch &b, const WgPeersDev &pe, const uint32_t *peer,
+hipError_t launch_wg_encap_prep(const WgBatch &b, uint8_t *hdr_base, const WgPeersDev &pe, const uint32_t *peer,
                                 const uint64_t *counter, uint32_t mtu, uint32_t *padded_len,
                                 uint32_t *wire_len, uint8_t *skip, hipStream_t s);
 

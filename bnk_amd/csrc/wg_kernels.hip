@@ -149,8 +149,10 @@ __global__ __launch_bounds__(256) void wg_keys_kernel(const uint32_t *peer, uint
 }
 
 // Writes the transport header into the slot's headroom, zero-pads the
-// plaintext, and reports the padded and wire lengths.
-__global__ __launch_bounds__(256) void wg_encap_prep_kernel(WgBatch b, WgPeersDev pe, const uint32_t *peer,
+// plaintext, and reports the padded and wire lengths.  The header goes to
+// hdr_base (same offsets as b.base): the arena the sealed packet is written
+// to, when that is not the one the plaintext is read from.
+__global__ __launch_bounds__(256) void wg_encap_prep_kernel(WgBatch b, uint8_t *hdr_base, WgPeersDev pe, const uint32_t *peer,
                                                             const uint64_t *counter, uint32_t mtu,
                                                             uint32_t *padded_len, uint32_t *wire_len,
                                                             uint8_t *skip)
@@ -166,11 +168,12 @@ __global__ __launch_bounds__(256) void wg_encap_prep_kernel(WgBatch b, WgPeersDe
         wire_len[i] = 0;
         return;
     }
-    uint8_t *w = const_cast<uint8_t *>(b.base) + (b.off ? b.off[i] : (uint64_t)i * b.stride);
+    const uint64_t at = b.off ? b.off[i] : (uint64_t)i * b.stride;
+    uint8_t *w = const_cast<uint8_t *>(b.base) + at;
     const uint32_t pad = wg_padding(len, mtu);
     const uint64_t c = counter[i];
     const u32x4 hdr = {4u, pe.remote_index[pr], (uint32_t)c, (uint32_t)(c >> 32)};
-    *reinterpret_cast<u32x4_unaligned *>(w) = hdr;
+    *reinterpret_cast<u32x4_unaligned *>(hdr_base + at) = hdr;
     for (uint32_t k = 0; k < pad; k++) w[16u + len + k] = 0;
     skip[i] = 0;
     padded_len[i] = len + pad;
@@ -212,12 +215,12 @@ hipError_t launch_wg_keys(const uint32_t *peer, uint32_t n_peers, uint32_t n, ui
     return hipGetLastError();
 }
 
-hipError_t launch_wg_encap_prep(const WgBatch &b, const WgPeersDev &pe, const uint32_t *peer,
+hipError_t launch_wg_encap_prep(const WgBatch &b, uint8_t *hdr_base, const WgPeersDev &pe, const uint32_t *peer,
                                 const uint64_t *counter, uint32_t mtu, uint32_t *padded_len,
                                 uint32_t *wire_len, uint8_t *skip, hipStream_t s)
 {
     if (b.n == 0) return hipSuccess;
-    hipLaunchKernelGGL(wg_encap_prep_kernel, grid_of(b.n), dim3(256), 0, s, b, pe, peer, counter, mtu,
+    hipLaunchKernelGGL(wg_encap_prep_kernel, grid_of(b.n), dim3(256), 0, s, b, hdr_base, pe, peer, counter, mtu,
                        padded_len, wire_len, skip);
     return hipGetLastError();
 }

@@ -63,16 +63,19 @@ def _ctx(peers, keys_send=None, keys_recv=None):
     return ctx
 
 
-@pytest.mark.parametrize("mem", ["host", "device"])
+@pytest.mark.parametrize("mem", ["host", "ring", "device"])
 @pytest.mark.parametrize("misalign", [False, True])
-def test_encap_matches_oracle(mem, misalign):
+@pytest.mark.parametrize("n", [3000, 700])
+def test_encap_matches_oracle(mem, misalign, n):
+    """"ring": the slots lie in a pinned ring of the context, which small
+    batches seal in place without staging copies.  700 packets also take the
+    one-launch counter assignment, 3000 the sorted one."""
     import torch
     from bnk_amd import lib
     from oracle import binding as O
     rng = np.random.default_rng(11 + misalign)
     peers = _peers(rng)
     keys = rng.integers(0, 256, (N_PEERS, 32), dtype=np.uint8)
-    n = 3000
     lens = rng.choice([0, 1, 15, 16, 17, 20, 40, 63, 64, 65, 127, 128, 129, 576, 1399, 1408, 1419, 1420],
                       n).astype(np.uint32)
     lens[:200] = rng.integers(0, MTU + 1, 200)
@@ -101,6 +104,15 @@ def test_encap_matches_oracle(mem, misalign):
             got_len = np.zeros(n, np.uint32)
             ctx.wg_encap(lib.make_batch(got, got.nbytes, n, lib.MEM_HOST, offsets=off, lens=lens, peer=peer),
                          MTU, got_len)
+        elif mem == "ring":
+            ring = ctx.ring_alloc(arena.nbytes + 48)
+            view = ring[48:]  # an arena that starts inside the ring
+            view[:] = arena
+            got_len = np.zeros(n, np.uint32)
+            ctx.wg_encap(lib.make_batch(view, arena.nbytes, n, lib.MEM_HOST, offsets=off, lens=lens, peer=peer),
+                         MTU, got_len)
+            got = np.array(view)
+            ctx.ring_free(ring)
         else:
             dev = torch.device("cuda:0")
             d_arena = torch.from_numpy(arena).to(dev)
@@ -167,7 +179,7 @@ def _decap_cases(rng, peers, keys, n):
     return wires, np.array(kinds)
 
 
-@pytest.mark.parametrize("mem", ["host", "device"])
+@pytest.mark.parametrize("mem", ["host", "ring", "device"])
 @pytest.mark.parametrize("aligned", [True, False])
 def test_decap_matches_oracle(mem, aligned):
     import torch
@@ -212,6 +224,20 @@ def test_decap_matches_oracle(mem, aligned):
         ctx.wg_decap(lib.make_batch(arena, arena.nbytes, n, lib.MEM_HOST, offsets=off, lens=lens),
                      lib.make_batch(got_out, got_out.nbytes, n, lib.MEM_HOST, offsets=out_off),
                      res, olen, gp, gc)
+    elif mem == "ring":
+        r_in, r_out = ctx.ring_alloc(arena.nbytes + 80), ctx.ring_alloc(total + 16)
+        r_in[80:] = arena
+        r_out[:] = 0x77
+        res = np.full(n, 99, np.uint8)
+        olen = np.full(n, 99, np.uint32)
+        gp = np.full(n, 99, np.uint32)
+        gc = np.full(n, 99, np.uint64)
+        ctx.wg_decap(lib.make_batch(r_in[80:], arena.nbytes, n, lib.MEM_HOST, offsets=off, lens=lens),
+                     lib.make_batch(r_out, total + 16, n, lib.MEM_HOST, offsets=out_off),
+                     res, olen, gp, gc)
+        got_out = np.array(r_out)
+        ctx.ring_free(r_in)
+        ctx.ring_free(r_out)
     else:
         dev = torch.device("cuda:0")
         d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)  # noqa: E731

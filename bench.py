@@ -501,6 +501,46 @@ def bench_latency(args) -> dict:
         out[str(n)] = {k: round(float(np.median(x)) * 1e6, 1) for k, x in t.items()}
         for r in (plain, sealed, opened):
             ctx.ring_free(r)
+    # WireGuard framing around the AEAD, the calls a wireguard-go bind would make
+    P = 16
+    keys = W.rand_bytes(W.stream_seed(2, 3), 32 * P).reshape(P, 32)
+    ctx.keys_set(lib.KEYS_SEND, keys)
+    ctx.keys_set(lib.KEYS_RECV, keys)
+    ctx.wg_peers_set([(100 + i, 100 + i, W.CGNAT_BASE | (i + 1), 0xFFFFFFFF) for i in range(P)])
+    slot, inner = 1504, 1400
+    for n in (1, 128, 1024):
+        ring, back = ctx.ring_alloc(n * slot), ctx.ring_alloc(n * slot)
+        off = np.arange(n, dtype=np.uint64) * slot
+        lens = np.full(n, inner, np.uint32)
+        peer = (np.arange(n) % P).astype(np.uint32)
+        src = (W.CGNAT_BASE | (peer + 1)).astype(np.uint32)
+        rows = ring.reshape(n, slot)
+        wl, res, ol = np.zeros(n, np.uint32), np.zeros(n, np.uint8), np.zeros(n, np.uint32)
+        gp, gc = np.zeros(n, np.uint32), np.zeros(n, np.uint64)
+        te, td = [], []
+        for it in range(reps + 5):
+            rows[:, 16:36] = 0
+            rows[:, 16] = 0x45
+            rows[:, 18] = inner >> 8
+            rows[:, 19] = inner & 255
+            for k in range(4):
+                rows[:, 28 + k] = (src >> (24 - 8 * k)) & 255
+            t0 = time.perf_counter()
+            ctx.wg_encap(lib.make_batch(ring, n * slot, n, lib.MEM_HOST, offsets=off, lens=lens, peer=peer),
+                         1420, wl)
+            t1 = time.perf_counter()
+            ctx.wg_decap(lib.make_batch(ring, n * slot, n, lib.MEM_HOST, offsets=off, lens=wl),
+                         lib.make_batch(back, n * slot, n, lib.MEM_HOST, offsets=off), res, ol, gp, gc)
+            t2 = time.perf_counter()
+            if it >= 5:
+                te.append(t1 - t0)
+                td.append(t2 - t1)
+        if int((res != 0).sum()) != 0:
+            raise SystemExit("framing round trip rejected packets")
+        out[str(n)]["wg_encap"] = round(float(np.median(te)) * 1e6, 1)
+        out[str(n)]["wg_decap"] = round(float(np.median(td)) * 1e6, 1)
+        ctx.ring_free(ring)
+        ctx.ring_free(back)
     ctx.close()
     return {
         "metric": "call_latency_us_host_memory", "value": out["128"]["seal"], "unit": "us", "n_gpus": 1,
@@ -508,8 +548,9 @@ def bench_latency(args) -> dict:
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "u32",
         "data": "synthetic",
         "config": {"workload": "median microseconds per call (upload + kernel + download + wait) for "
-                               "batches of 1 / 128 / 1024 / 8192 packets x %d B in pinned rings; value is "
-                               "seal at 128 packets" % L},
+                               "batches of 1 / 128 / 1024 / 8192 packets x %d B in pinned rings, and for "
+                               "WireGuard encapsulation / decapsulation of 1400-byte inner packets; value "
+                               "is seal at 128 packets" % L},
         "per_batch_size_us": out,
     }
 

@@ -101,6 +101,10 @@ size_t relay_sort_tmp_bytes(uint32_t n, uint32_t n_keys)
     return std::max(bytes, (size_t)n_keys * 4);
 }
 
+__global__ void peer_rank_small_kernel(const uint32_t *peer, uint32_t n_keys, uint32_t n, uint64_t *ctr_base,
+                                       uint64_t *ctr_out, int advance, int no_peer_ok, unsigned bits,
+                                       uint32_t *status);
+
 hipError_t launch_relay_assign(const uint8_t *auth, const uint8_t *pass, const uint32_t *peer_out,
                                const uint64_t *ctr_base_out, uint32_t n_peers_out, uint32_t n,
                                uint32_t *keys, uint32_t *idx, uint32_t *skeys, uint32_t *sidx,
@@ -111,43 +115,59 @@ hipError_t launch_relay_assign(const uint8_t *auth, const uint8_t *pass, const u
     const dim3 grid((n + 255u) / 256u);
     hipLaunchKernelGGL(relay_verdict_kernel, grid, dim3(256), 0, s, auth, pass, peer_out, n_peers_out,
                        n, keys, idx, verdict, ctr_out, status);
+    if (n <= PEER_RANK_SMALL_MAX) {
+        // keys[] is the peer of each survivor and all ones for the rest
+        hipLaunchKernelGGL(peer_rank_small_kernel, dim3(1), dim3(PEER_RANK_SMALL_MAX), 0, s, keys, n_peers_out,
+                           n, const_cast<uint64_t *>(ctr_base_out), ctr_out, 0, 1, key_bits(n_peers_out), status);
+        return hipGetLastError();
+    }
     return launch_peer_rank(keys, idx, skeys, sidx, sort_tmp, sort_tmp_bytes,
                             const_cast<uint64_t *>(ctr_base_out), n_peers_out, n, ctr_out, false, s);
 }
 
 // Batch-order counters for a small batch in one launch of one block, straight
-// from the peer array: every thread compares its packet with all the others
-// in LDS.  The last packet of each peer moves the peer's base.
-__global__ __launch_bounds__(1024) void peer_rank_small_kernel(const uint32_t *peer, uint32_t n_keys,
-                                                               uint32_t n, uint64_t *ctr_base,
-                                                               uint64_t *ctr_out, int advance,
-                                                               uint32_t *status)
+// from the peer array: a stable block-wide radix sort of (peer, position)
+// brings each peer's packets together in batch order; a packet's rank is its
+// distance from the head of its run, and the last packet of a run moves the
+// peer's base.
+__global__ __launch_bounds__(PEER_RANK_SMALL_MAX) void peer_rank_small_kernel(
+    const uint32_t *peer, uint32_t n_keys, uint32_t n, uint64_t *ctr_base, uint64_t *ctr_out,
+    int advance, int no_peer_ok, unsigned bits, uint32_t *status)
 {
-    __shared__ uint32_t pk[PEER_RANK_SMALL_MAX];
-    const uint32_t i = threadIdx.x;
-    uint32_t p = NO_PEER;
-    if (i < n) {
-        p = peer ? peer[i] : 0u;
-        if (p >= n_keys) {
-            atomicOr(status, STATUS_PEER_RANGE);
-            p = NO_PEER;
+    using Sort = rocprim::block_radix_sort<uint32_t, PEER_RANK_SMALL_MAX, 1, uint32_t>;
+    using Scan = rocprim::block_scan<uint32_t, PEER_RANK_SMALL_MAX>;
+    __shared__ union {
+        typename Sort::storage_type sort;
+        typename Scan::storage_type scan;
+    } tmp;
+    __shared__ uint32_t sk[PEER_RANK_SMALL_MAX + 1];
+    const uint32_t t = threadIdx.x;
+    uint32_t key[1] = {NO_PEER}, pos[1] = {t};
+    if (t < n) {
+        key[0] = peer ? peer[t] : 0u;
+        if (key[0] >= n_keys) {
+            if (!(no_peer_ok && key[0] == NO_PEER)) atomicOr(status, STATUS_PEER_RANGE);
+            key[0] = NO_PEER;
         }
     }
-    pk[i] = p;
+    // valid keys are below n_keys < 2^bits and "no peer" is all ones, so the low
+    // bits order them the way the full word does, "no peer" last
+    Sort().sort(key, pos, tmp.sort, 0, bits);
+    sk[t] = key[0];
+    if (t == 0) sk[PEER_RANK_SMALL_MAX] = NO_PEER;
     __syncthreads();
-    uint32_t before = 0, after = 0;
-    uint64_t base = 0;
-    if (p != NO_PEER) {
-        for (uint32_t j = 0; j < n; j++) {
-            const bool same = pk[j] == p;
-            before += (same && j < i) ? 1u : 0u;
-            after += (same && j > i) ? 1u : 0u;
-        }
-        base = ctr_base[p];
-        ctr_out[i] = base + before;
+    const bool valid = key[0] != NO_PEER;
+    const bool head = t == 0 || sk[t - 1] != key[0];
+    const bool last = sk[t + 1] != key[0];
+    uint32_t start = 0;
+    Scan().inclusive_scan(head ? t : 0u, start, tmp.scan, rocprim::maximum<uint32_t>());
+    uint64_t mine = 0;
+    if (valid) {
+        mine = ctr_base[key[0]] + (t - start);
+        ctr_out[pos[0]] = mine;
     }
     __syncthreads(); // every base has been read
-    if (advance && p != NO_PEER && after == 0) ctr_base[p] = base + before + 1u;
+    if (advance && valid && last) ctr_base[key[0]] = mine + 1u;
 }
 
 hipError_t launch_peer_rank_small(const uint32_t *peer, uint32_t n_keys, uint32_t n, uint64_t *ctr_base,
@@ -155,8 +175,8 @@ hipError_t launch_peer_rank_small(const uint32_t *peer, uint32_t n_keys, uint32_
 {
     if (n == 0) return hipSuccess;
     if (n > PEER_RANK_SMALL_MAX) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(peer_rank_small_kernel, dim3(1), dim3(1024), 0, s, peer, n_keys, n, ctr_base, ctr_out,
-                       advance ? 1 : 0, status);
+    hipLaunchKernelGGL(peer_rank_small_kernel, dim3(1), dim3(PEER_RANK_SMALL_MAX), 0, s, peer, n_keys, n,
+                       ctr_base, ctr_out, advance ? 1 : 0, 0, key_bits(n_keys), status);
     return hipGetLastError();
 }
 

@@ -19,10 +19,15 @@ def _note(ctx, ora, w):
     ctx.filter_note_outbound(lib.make_batch(buf, buf.nbytes, m, lib.MEM_HOST, stride=32, length=28), now)
 
 
-def test_relay_matches_oracle_host_path():
+@pytest.mark.parametrize("mem", ["host", "ring"])
+@pytest.mark.parametrize("n", [12000, 900])
+def test_relay_matches_oracle_host_path(mem, n):
+    """"ring": both arenas lie in pinned rings of the context, which batches of
+    a few megabytes relay in place without staging copies.  900 packets also
+    take the wave-per-packet kernels and the one-launch counter assignment."""
     from bnk_amd import lib
     from oracle import binding as O
-    w = W.relay_workload(n=12000, n_peers=64, n_rules=512)
+    w = W.relay_workload(n=n, n_peers=64, n_rules=512)
     b = w.batch
     keys_in = np.ascontiguousarray(b.keys)
     keys_out = np.ascontiguousarray(w.keys_out)
@@ -43,7 +48,15 @@ def test_relay_matches_oracle_host_path():
     want_v, want_c = ora.relay_fused_batch(keys_in, b.peer, b.counters, keys_out, w.peer_out,
                                            w.ctr_base_out, sealed, b.off, ct_lens, want_out, b.off,
                                            w.now_ns)
-    got_out = np.full_like(b.plain, 0x77)
+    rings = []
+    if mem == "ring":
+        rings = [ctx.ring_alloc(sealed.nbytes + 32), ctx.ring_alloc(sealed.nbytes)]
+        rings[0][32:] = sealed
+        sealed = rings[0][32:]
+        got_out = rings[1]
+        got_out[:] = 0x77
+    else:
+        got_out = np.full_like(b.plain, 0x77)
     got_v = np.full(b.n, 9, np.uint8)
     got_c = np.full(b.n, 123, np.uint64)
     ctx.relay_fused(
@@ -66,6 +79,8 @@ def test_relay_matches_oracle_host_path():
         w.peer_out, w.ctr_base_out, len(w.ctr_base_out), w.now_ns,
         lib.make_batch(got_out, got_out.nbytes, b.n, lib.MEM_HOST, offsets=b.off), got_v, got_c)
     assert np.array_equal(got_v == 1, expect == 1) and not (got_v == 2).any()
+    for r in rings:
+        ctx.ring_free(r)
     ctx.close()
 
 

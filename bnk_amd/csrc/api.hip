@@ -116,15 +116,21 @@ int aead_batch_host_direct(bnk_ctx *ctx, bool open, const bnk_batch *in, const b
     uint64_t *p_in_off = (uint64_t *)pin, *p_out_off = p_in_off + n, *p_ctr = p_out_off + n;
     uint32_t *p_lens = (uint32_t *)(p_ctr + n), *p_peer = p_lens + n, *p_order = p_peer + n;
     uint8_t *p_verdict = (uint8_t *)(p_order + n);
-    // The input span is fetched into device memory by one wide copy kernel
-    // (every 16 bytes in flight at once); the AEAD kernel then writes its
-    // output straight into the ring, where stores need no round trip.
-    // the copy keeps the span's position within a 128-byte line, which is what
-    // lets the lane-per-packet kernel move whole lines
-    const uint32_t mis = (uint32_t)((uintptr_t)(d_in + sin.lo) & 127u);
-    HIPCHK(ctx, ctx->in_arena.reserve(sin.size() + 160));
-    HIPCHK(ctx, launch_pull(d_in + sin.lo, ctx->in_arena.as<uint8_t>() + mis, sin.size(), ctx->stream));
-    a.in = ctx->in_arena.as<uint8_t>() + mis;
+    // A wave per packet loads each byte once, all loads in flight together, so
+    // it reads the ring itself.  A lane per packet walks its packet line by
+    // line, a round trip over the link each: for it the span is first fetched
+    // into device memory by one wide copy kernel, at the same position within a
+    // 128-byte line so that whole lines can be moved.  Either way the output
+    // goes straight into the ring, where stores need no round trip.
+    a.lens = in->lens ? ctx->pin.dev(p_lens) : nullptr;
+    if (aead_runs_spread(a)) {
+        a.in = d_in + sin.lo;
+    } else {
+        const uint32_t mis = (uint32_t)((uintptr_t)(d_in + sin.lo) & 127u);
+        HIPCHK(ctx, ctx->in_arena.reserve(sin.size() + 160));
+        HIPCHK(ctx, launch_pull(d_in + sin.lo, ctx->in_arena.as<uint8_t>() + mis, sin.size(), ctx->stream));
+        a.in = ctx->in_arena.as<uint8_t>() + mis;
+    }
     a.out = d_out;
     if (in->offsets) {
         for (uint32_t i = 0; i < n; i++) p_in_off[i] = in->offsets[i] - sin.lo;

@@ -78,15 +78,20 @@ extern "C" int bnk_relay_fused_batch(bnk_ctx *ctx, const bnk_batch *in, const ui
                 uint64_t *p_base = h_ctr_out + n;
                 uint32_t *p_lens = (uint32_t *)(p_base + n_peers_out), *p_peer = p_lens + n, *p_peer_out = p_peer + n;
                 h_verdict = (uint8_t *)(p_peer_out + n);
+                if (in->lens) { memcpy(p_lens, in->lens, (size_t)n * 4); op.lens = ctx->pin.dev(p_lens); }
                 const uint32_t mis = (uint32_t)((uintptr_t)(d_ring_in + sin.lo) & 127u);
-                HIPCHK(ctx, ctx->in_arena.reserve(sin.size() + 160));
-                HIPCHK(ctx, launch_pull(d_ring_in + sin.lo, ctx->in_arena.as<uint8_t>() + mis, sin.size(), ctx->stream));
-                op.in = ctx->in_arena.as<uint8_t>() + mis;
+                if (aead_runs_spread(op)) {
+                    // a wave per packet reads the ring itself (see aead_batch_host_direct)
+                    op.in = d_ring_in + sin.lo;
+                } else {
+                    HIPCHK(ctx, ctx->in_arena.reserve(sin.size() + 160));
+                    HIPCHK(ctx, launch_pull(d_ring_in + sin.lo, ctx->in_arena.as<uint8_t>() + mis, sin.size(), ctx->stream));
+                    op.in = ctx->in_arena.as<uint8_t>() + mis;
+                }
                 if (in->offsets) {
                     for (uint32_t i = 0; i < n; i++) p_in_off[i] = in->offsets[i] - sin.lo;
                     op.in_off = ctx->pin.dev(p_in_off);
                 }
-                if (in->lens) { memcpy(p_lens, in->lens, (size_t)n * 4); op.lens = ctx->pin.dev(p_lens); }
                 if (in->peer) { memcpy(p_peer, in->peer, (size_t)n * 4); op.peer = ctx->pin.dev(p_peer); }
                 if (in->counters) { memcpy(p_ctr, in->counters, (size_t)n * 8); op.counters = ctx->pin.dev(p_ctr); }
                 d_out = d_ring_out;

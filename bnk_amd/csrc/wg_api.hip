@@ -140,10 +140,15 @@ extern "C" int bnk_wg_encap_batch(bnk_ctx *ctx, const bnk_batch *slots, uint32_t
         uint64_t *p_off = ctx->pin.as<uint64_t>();
         uint32_t *p_lens = (uint32_t *)(p_off + n), *p_peer = p_lens + n;
         h_wire_len = p_peer + n;
-        const uint32_t mis = (uint32_t)((uintptr_t)ring_out & 127u);
-        HIPCHK(ctx, ctx->in_arena.reserve(span.size() + 160));
-        HIPCHK(ctx, launch_pull(ring_out, ctx->in_arena.as<uint8_t>() + mis, span.size(), ctx->stream));
-        b.base = ctx->in_arena.as<uint8_t>() + mis;
+        if (n <= ctx->spread_max) {
+            // a wave per packet reads the ring itself (see aead_batch_host_direct)
+            b.base = ring_out;
+        } else {
+            const uint32_t mis = (uint32_t)((uintptr_t)ring_out & 127u);
+            HIPCHK(ctx, ctx->in_arena.reserve(span.size() + 160));
+            HIPCHK(ctx, launch_pull(ring_out, ctx->in_arena.as<uint8_t>() + mis, span.size(), ctx->stream));
+            b.base = ctx->in_arena.as<uint8_t>() + mis;
+        }
         if (slots->offsets) {
             for (uint32_t i = 0; i < n; i++) p_off[i] = slots->offsets[i] - span.lo;
             b.off = ctx->pin.dev(p_off);
@@ -356,10 +361,15 @@ extern "C" int bnk_wg_decap_batch(bnk_ctx *ctx, const bnk_batch *wire, const bnk
                 h_out_len = p_lens + n;
                 h_peer = h_out_len + n;
                 h_result = (uint8_t *)(h_peer + n);
-                const uint32_t mis = (uint32_t)((uintptr_t)(d_wire + sin.lo) & 127u);
-                HIPCHK(ctx, ctx->in_arena.reserve(sin.size() + 160));
-                HIPCHK(ctx, launch_pull(d_wire + sin.lo, ctx->in_arena.as<uint8_t>() + mis, sin.size(), ctx->stream));
-                wb.base = ctx->in_arena.as<uint8_t>() + mis;
+                if (n <= ctx->spread_max) {
+                    // a wave per packet reads the ring itself (see aead_batch_host_direct)
+                    wb.base = d_wire + sin.lo;
+                } else {
+                    const uint32_t mis = (uint32_t)((uintptr_t)(d_wire + sin.lo) & 127u);
+                    HIPCHK(ctx, ctx->in_arena.reserve(sin.size() + 160));
+                    HIPCHK(ctx, launch_pull(d_wire + sin.lo, ctx->in_arena.as<uint8_t>() + mis, sin.size(), ctx->stream));
+                    wb.base = ctx->in_arena.as<uint8_t>() + mis;
+                }
                 if (wire->offsets) {
                     for (uint32_t i = 0; i < n; i++) p_in_off[i] = wire->offsets[i] - sin.lo;
                     wb.off = ctx->pin.dev(p_in_off);

@@ -44,9 +44,11 @@ enum {
 
 /* Where the pointers of a bnk_batch live. */
 enum {
-    BNK_MEM_HOST = 0,  /* host memory (pinned rings from bnk_ring_alloc copy
-                          fastest); the call stages, runs and copies back
-                          before it returns */
+    BNK_MEM_HOST = 0,  /* host memory; the call stages, runs and copies back
+                          before it returns.  Arenas inside pinned rings from
+                          bnk_ring_alloc are fastest: batches of up to 8 MB
+                          are read and written in place by the kernels, larger
+                          ones are copied in overlapped chunks */
     BNK_MEM_DEVICE = 1 /* device memory of the context's GPU; the call only
                           enqueues work on the context stream (bnk_sync waits) */
 };
@@ -102,7 +104,9 @@ void bnk_shutdown(bnk_ctx *ctx);
  * ctx is NULL).  Valid until the next call on the context. */
 const char *bnk_last_error(bnk_ctx *ctx);
 
-/* Pinned host packet ring for wireguard-go style buffer pools. */
+/* Pinned host packet ring for wireguard-go style buffer pools.  The GPU can
+ * address it: small batches whose arenas lie inside a ring of the same context
+ * need no staging copies. */
 int bnk_ring_alloc(bnk_ctx *ctx, size_t bytes, void **host_pinned);
 int bnk_ring_free(bnk_ctx *ctx, void *host_pinned);
 /* Device memory for callers that keep batches resident (BNK_MEM_DEVICE). */

@@ -10,6 +10,7 @@
 #include "aead_lane.hpp"
 #include <algorithm>
 
+#include "../../include/bnkhip.h"
 #include "kernels.hpp"
 
 namespace bnk {
@@ -459,7 +460,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 // terms (aead_lane.hpp).  All loads of a packet are issued before any store,
 // and a lane stores only what it loaded, so sealing in place is safe.  A
 // packet longer than 63 blocks is done by lane 0 alone, the per-lane way.
-template <bool OPEN>
+//
+// With WG set the wave also does the packet's WireGuard framing (a.wg): on the
+// way out it writes the transport header and treats the bytes between the
+// plaintext and its padded length as zeros without their being in memory; on
+// the way in it checks the header, finds the sender by its receiver index (a
+// 64-way search of the sorted table, the lanes probing together), and after
+// the tag check looks at the inner IP header while it is still in registers.
+// Same results as wg_parse_kernel / wg_encap_prep_kernel / wg_finish_kernel
+// around a plain launch.
+template <bool OPEN, bool WG>
 __global__ __launch_bounds__(256) void aead_spread_kernel(AeadArgs a)
 {
     __shared__ __attribute__((aligned(16))) uint8_t tile_all[WAVES_PER_BLOCK][64 * LDS_ROW];
@@ -470,22 +480,85 @@ __global__ __launch_bounds__(256) void aead_spread_kernel(AeadArgs a)
     const uint32_t i = a.first + w;
     uint32_t len = a.lens ? a.lens[i] : a.len;
     if (!OPEN) len = len >= a.trim ? len - a.trim : 0u;
-    const uint32_t pr = a.peer ? a.peer[i] : 0u;
-    if (a.skip && a.skip[i] != 0) return;
-    if (pr >= a.n_peers) {
-        if (lane == 0) {
-            atomicOr(a.status, STATUS_PEER_RANGE);
-            if (OPEN) a.verdict[i] = 0;
-        }
-        return;
-    }
-    if (OPEN && len < 16u) {
-        if (lane == 0) a.verdict[i] = 0;
-        return;
-    }
-    if (OPEN) len -= 16u;
+    uint32_t pr = a.peer ? a.peer[i] : 0u;
     const uint8_t *src = a.in + (a.in_off ? a.in_off[i] : (uint64_t)i * a.in_stride) + a.in_skip;
     uint8_t *dst = a.out + (a.out_off ? a.out_off[i] : (uint64_t)i * a.out_stride) + a.out_skip;
+    uint32_t present = len; // bytes of src that exist in memory; the rest up to len read as zero
+    uint64_t ctr = 0;
+    if (!WG) {
+        if (a.skip && a.skip[i] != 0) return;
+        if (pr >= a.n_peers) {
+            if (lane == 0) {
+                atomicOr(a.status, STATUS_PEER_RANGE);
+                if (OPEN) a.verdict[i] = 0;
+            }
+            return;
+        }
+        if (OPEN && len < 16u) {
+            if (lane == 0) a.verdict[i] = 0;
+            return;
+        }
+        if (OPEN) len -= 16u;
+        present = len;
+        ctr = a.counters ? a.counters[i] : a.counter0 + i;
+    } else if (!OPEN) {
+        // ---- encapsulate: header into the headroom, padding as implied zeros ----
+        if (pr >= a.wg.n_peers || len + 15u > WG_FUSE_MAX_LEN) {
+            if (lane == 0) a.wg.wire_len[i] = 0;
+            return;
+        }
+        ctr = a.counters[i];
+        present = len;
+        len += wg_padding(len, a.wg.mtu);
+        if (lane == 0) {
+            st16(dst, make_uint4(4u, a.wg.remote_index[pr], (uint32_t)ctr, (uint32_t)(ctr >> 32)));
+            a.wg.wire_len[i] = 16u + len + 16u;
+        }
+        src += 16;
+        dst += 16;
+    } else {
+        // ---- decapsulate: header checks and the receiver-index lookup ----
+        uint8_t res = BNK_WG_OK;
+        uint4 h = make_uint4(0, 0, 0, 0);
+        if (len < 32u || len - 32u > WG_FUSE_MAX_LEN) res = BNK_WG_BAD_HEADER;
+        else h = ld16(src);
+        if (res == BNK_WG_OK && h.x != 4u) res = BNK_WG_BAD_HEADER;
+        if (res == BNK_WG_OK) {
+            // narrow [lo, hi) to at most 64 entries, 64 probes at a time
+            uint32_t lo = 0, hi = a.wg.n_peers;
+            while (hi - lo > 64u) {
+                const uint32_t step = (hi - lo + 63u) / 64u;
+                const uint32_t at = min(lo + lane * step, hi - 1u);
+                const bool le = a.wg.index_sorted[at].x <= h.y;
+                const unsigned long long m = __ballot(le);
+                // lanes probe ascending positions: those at or below the index form a prefix
+                const uint32_t below = (uint32_t)__popcll(m);
+                if (below == 0u) { hi = lo; break; }
+                const uint32_t nlo = min(lo + (below - 1u) * step, hi - 1u);
+                hi = min(nlo + step, hi);
+                lo = nlo;
+            }
+            uint2 e = make_uint2(0, 0);
+            const bool mine = lo + lane < hi;
+            if (mine) e = a.wg.index_sorted[lo + lane];
+            const unsigned long long hit = __ballot(mine && e.x == h.y);
+            if (hit == 0ull) res = BNK_WG_UNKNOWN_INDEX;
+            else pr = (uint32_t)__shfl((int)e.y, __ffsll((long long)hit) - 1, 64);
+        }
+        if (res != BNK_WG_OK) {
+            if (lane == 0) {
+                a.wg.result[i] = res;
+                a.wg.out_len[i] = 0;
+                a.wg.peer_out[i] = 0xFFFFFFFFu;
+                a.wg.counter_out[i] = 0;
+            }
+            return;
+        }
+        ctr = (uint64_t)h.z | (uint64_t)h.w << 32;
+        len -= 32u; // header and tag
+        present = len;
+        src += 16;
+    }
     uint32_t k[8];
     {
         const uint4 *kp = reinterpret_cast<const uint4 *>(a.keys + 8u * pr);
@@ -493,11 +566,10 @@ __global__ __launch_bounds__(256) void aead_spread_kernel(AeadArgs a)
         k[0] = k0.x; k[1] = k0.y; k[2] = k0.z; k[3] = k0.w;
         k[4] = k1.x; k[5] = k1.y; k[6] = k1.z; k[7] = k1.w;
     }
-    const uint64_t ctr = a.counters ? a.counters[i] : a.counter0 + i;
     const uint32_t n1 = (uint32_t)ctr, n2 = (uint32_t)(ctr >> 32);
     uint32_t x[16];
 
-    if (len > SPREAD_MAX_LEN) {
+    if (!WG && len > SPREAD_MAX_LEN) {
         const bool have = lane == 0;
         Poly32 mac;
         body_generic<OPEN>(tile_all[threadIdx.x >> 6], lane, have ? src : nullptr, have ? dst : nullptr,
@@ -509,12 +581,13 @@ __global__ __launch_bounds__(256) void aead_spread_kernel(AeadArgs a)
     // ---- my 64 bytes: loads first, they fly while the block is computed ----
     const uint32_t at = 64u * (lane - 1u);
     const uint32_t mine = (lane == 0 || at >= len) ? 0u : min(len - at, 64u);
+    const uint32_t there = (lane == 0 || at >= present) ? 0u : min(present - at, 64u);
     uint32_t m[16];
 #pragma unroll
     for (int j = 0; j < 4; j++) {
         uint4 v = make_uint4(0, 0, 0, 0);
-        if (mine >= 16u * (j + 1)) v = ld16(src + at + 16 * j);
-        else if (mine > 16u * j) v = ld_partial(src + at + 16 * j, mine - 16u * j);
+        if (there >= 16u * (j + 1)) v = ld16(src + at + 16 * j);
+        else if (there > 16u * j) v = ld_partial(src + at + 16 * j, there - 16u * j);
         m[4 * j] = v.x; m[4 * j + 1] = v.y; m[4 * j + 2] = v.z; m[4 * j + 3] = v.w;
     }
     uint4 want_tag = make_uint4(0, 0, 0, 0);
@@ -568,7 +641,40 @@ __global__ __launch_bounds__(256) void aead_spread_kernel(AeadArgs a)
         // all 16 bytes are compared, no early exit
         reject = ((want_tag.x ^ tag[0]) | (want_tag.y ^ tag[1]) | (want_tag.z ^ tag[2]) |
                   (want_tag.w ^ tag[3])) != 0;
-        if (lane == 0) a.verdict[i] = reject ? 0 : 1;
+        if (!WG && lane == 0) a.verdict[i] = reject ? 0 : 1;
+    }
+    if (WG && OPEN) {
+        // ---- what wireguard-go checks once a packet is authentic: keepalive, IP
+        // version, length fields, source inside the sender's allowed prefix.  The
+        // first 16 plaintext bytes (lane 1's first cell) hold every field used.
+        const uint32_t w0 = (uint32_t)__builtin_amdgcn_readlane((int)o[0], 1);
+        const uint32_t w1 = (uint32_t)__builtin_amdgcn_readlane((int)o[1], 1);
+        const uint32_t w3 = (uint32_t)__builtin_amdgcn_readlane((int)o[3], 1);
+        uint8_t res = BNK_WG_OK;
+        uint32_t inner = 0;
+        const uint32_t version = (w0 >> 4) & 0xFu;
+        if (reject) res = BNK_WG_AUTH_FAIL;
+        else if (len == 0u) res = BNK_WG_KEEPALIVE;
+        else if (len < 16u) res = BNK_WG_BAD_IP;
+        else if (version == 4u) {
+            const uint32_t total = __builtin_bswap32(w0) & 0xFFFFu;
+            const uint2 al = a.wg.allowed[pr];
+            if (len < 20u || total > len || total < 20u) res = BNK_WG_BAD_IP;
+            else if ((__builtin_bswap32(w3) & al.y) != (al.x & al.y)) res = BNK_WG_NOT_ALLOWED;
+            else inner = total;
+        } else if (version == 6u) {
+            // peers own IPv4 addresses only
+            const uint32_t total = (__builtin_bswap32(w1) >> 16) + 40u;
+            res = (len < 40u || total > len) ? BNK_WG_BAD_IP : BNK_WG_NOT_ALLOWED;
+        } else {
+            res = BNK_WG_BAD_IP;
+        }
+        if (lane == 0) {
+            a.wg.result[i] = res;
+            a.wg.out_len[i] = inner;
+            a.wg.peer_out[i] = pr;
+            a.wg.counter_out[i] = ctr;
+        }
     }
     // ---- my bytes out; a rejected packet leaves zeros (chacha20poly1305.Open) ----
 #pragma unroll
@@ -594,9 +700,12 @@ bool aead_runs_spread(const AeadArgs &a)
 hipError_t launch_aead_seal(const AeadArgs &a, hipStream_t s)
 {
     if (a.n == 0) return hipSuccess;
-    if (aead_runs_spread(a))
-        hipLaunchKernelGGL(aead_spread_kernel<false>, dim3((a.n + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK),
-                           dim3(256), 0, s, a);
+    const dim3 waves((a.n + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK);
+    if (a.wg.mode != WG_FUSE_OFF) {
+        if (a.wg.mode != WG_FUSE_ENCAP || !aead_runs_spread(a)) return hipErrorInvalidValue;
+        hipLaunchKernelGGL((aead_spread_kernel<false, true>), waves, dim3(256), 0, s, a);
+    } else if (aead_runs_spread(a))
+        hipLaunchKernelGGL((aead_spread_kernel<false, false>), waves, dim3(256), 0, s, a);
     else
         hipLaunchKernelGGL(aead_wave_kernel<false>, dim3((a.n + 255u) / 256u), dim3(256), 0, s, a);
     return hipGetLastError();
@@ -605,9 +714,12 @@ hipError_t launch_aead_seal(const AeadArgs &a, hipStream_t s)
 hipError_t launch_aead_open(const AeadArgs &a, hipStream_t s)
 {
     if (a.n == 0) return hipSuccess;
-    if (aead_runs_spread(a))
-        hipLaunchKernelGGL(aead_spread_kernel<true>, dim3((a.n + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK),
-                           dim3(256), 0, s, a);
+    const dim3 waves((a.n + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK);
+    if (a.wg.mode != WG_FUSE_OFF) {
+        if (a.wg.mode != WG_FUSE_DECAP || !aead_runs_spread(a)) return hipErrorInvalidValue;
+        hipLaunchKernelGGL((aead_spread_kernel<true, true>), waves, dim3(256), 0, s, a);
+    } else if (aead_runs_spread(a))
+        hipLaunchKernelGGL((aead_spread_kernel<true, false>), waves, dim3(256), 0, s, a);
     else
         hipLaunchKernelGGL(aead_wave_kernel<true>, dim3((a.n + 255u) / 256u), dim3(256), 0, s, a);
     return hipGetLastError();

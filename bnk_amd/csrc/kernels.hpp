@@ -6,6 +6,39 @@
 
 namespace bnk {
 
+// WireGuard pads the plaintext with zeros to a multiple of 16, never beyond the
+// MTU (a packet longer than the MTU pads its remainder).
+__host__ __device__ inline uint32_t wg_padding(uint32_t len, uint32_t mtu)
+{
+    uint32_t last = len;
+    if (mtu == 0) return ((last + 15u) & ~15u) - last;
+    if (last > mtu) last %= mtu;
+    uint32_t padded = (last + 15u) & ~15u;
+    if (padded > mtu) padded = mtu;
+    return padded - last;
+}
+
+// WireGuard transport framing done by a wave-per-packet AEAD launch itself
+// (small batches only; larger ones run the framing kernels of wg_kernels.hip
+// around the launch).  in/out offsets then address the slot or datagram, not
+// the AEAD data inside it, and every packet must be at most WG_FUSE_MAX_LEN
+// bytes long, padding included.
+struct WgFuse {
+    uint32_t mode;               // WG_FUSE_*
+    uint32_t n_peers;            // rows of the peer tables
+    uint32_t mtu;                // encapsulate: padding cap
+    const uint2 *index_sorted;   // decapsulate: (receiver index, peer), ascending
+    const uint2 *allowed;        // decapsulate: (net, mask) per peer
+    const uint32_t *remote_index; // encapsulate: index the peer expects
+    uint8_t *result;             // decapsulate: BNK_WG_* per packet
+    uint32_t *out_len;           // decapsulate: inner packet length
+    uint32_t *peer_out;          // decapsulate: sender
+    uint64_t *counter_out;       // decapsulate: its counter
+    uint32_t *wire_len;          // encapsulate: datagram length
+};
+enum : uint32_t { WG_FUSE_OFF = 0, WG_FUSE_ENCAP = 1, WG_FUSE_DECAP = 2 };
+constexpr uint32_t WG_FUSE_MAX_LEN = 63u * 64u;
+
 // Device-side view of one AEAD launch.  All pointers are device pointers.
 struct AeadArgs {
     const uint8_t *in;
@@ -29,6 +62,7 @@ struct AeadArgs {
     uint32_t in_skip, out_skip; // bytes between a packet's offset and its AEAD data
     uint32_t first;            // the launch covers packets first .. first+n-1; order[] is relative to first
     uint32_t spread_max;       // launches of at most this many packets run one wave per packet
+    WgFuse wg;                 // only with aead_runs_spread(); mode 0: plain AEAD
 };
 
 // Below this many packets a wave per packet finishes sooner than a lane per

@@ -9,16 +9,6 @@ using namespace bnk;
 
 namespace {
 
-uint32_t wg_padding_host(uint32_t len, uint32_t mtu)
-{
-    uint32_t last = len;
-    if (mtu == 0) return ((last + 15u) & ~15u) - last;
-    if (last > mtu) last %= mtu;
-    uint32_t padded = (last + 15u) & ~15u;
-    if (padded > mtu) padded = mtu;
-    return padded - last;
-}
-
 WgPeersDev peers_view(bnk_ctx *ctx)
 {
     WgPeersDev pe{};
@@ -98,7 +88,7 @@ extern "C" int bnk_wg_encap_batch(bnk_ctx *ctx, const bnk_batch *slots, uint32_t
     const bool host = slots->mem == BNK_MEM_HOST;
     const auto slot_ext = [slots, mtu](uint32_t i) {
         const uint32_t len = slots->lens ? slots->lens[i] : slots->len;
-        return 16ull + len + wg_padding_host(len, mtu) + 16ull;
+        return 16ull + len + wg_padding(len, mtu) + 16ull;
     };
 
     WgBatch b{};
@@ -235,12 +225,49 @@ extern "C" int bnk_wg_encap_batch(bnk_ctx *ctx, const bnk_batch *slots, uint32_t
                                      tmp_bytes, pe.send_ctr, pe.n, n, d_ctr, true, ctx->stream));
     }
 
+    // A wave-per-packet launch does the framing itself; it needs every packet to
+    // fit 63 ChaCha20 blocks, which only a host batch can promise.
+    bool fits = host;
+    if (host) {
+        if (slots->lens) {
+            for (uint32_t i = 0; i < n && fits; i++) fits = slots->lens[i] + 15u <= WG_FUSE_MAX_LEN;
+        } else {
+            fits = slots->len + 15u <= WG_FUSE_MAX_LEN;
+        }
+    }
+
     // header, padding and seal of packets [lo, hi)
     auto run = [&](uint32_t lo, uint32_t hi) -> int {
         WgBatch c = b;
         c.first = lo;
         c.n = hi - lo;
         uint8_t *sealed = ring_out ? ring_out : const_cast<uint8_t *>(b.base);
+        if (fits) {
+            AeadArgs se{};
+            se.spread_max = ctx->spread_max;
+            se.keys = ctx->d_keys[BNK_KEYS_SEND];
+            se.n_peers = pe.n;
+            se.status = ctx->d_status;
+            se.first = lo;
+            se.n = hi - lo;
+            se.in = b.base;
+            se.out = sealed;
+            se.in_off = se.out_off = b.off;
+            se.in_stride = se.out_stride = slots->stride;
+            se.lens = b.lens;
+            se.len = slots->len;
+            se.peer = d_peer;
+            se.counters = d_ctr;
+            if (aead_runs_spread(se)) {
+                se.wg.mode = WG_FUSE_ENCAP;
+                se.wg.n_peers = pe.n;
+                se.wg.mtu = mtu;
+                se.wg.remote_index = pe.remote_index;
+                se.wg.wire_len = d_wire_len;
+                HIPCHK(ctx, launch_aead_seal(se, ctx->stream));
+                return BNK_OK;
+            }
+        }
         HIPCHK(ctx, launch_wg_encap_prep(c, sealed, pe, d_peer, d_ctr, mtu, d_padded, d_wire_len, d_skip, ctx->stream));
         AeadArgs se{};
         se.spread_max = ctx->spread_max;
@@ -453,11 +480,51 @@ extern "C" int bnk_wg_decap_batch(bnk_ctx *ctx, const bnk_batch *wire, const bnk
     uint8_t *d_auth = ctx->r_auth.as<uint8_t>();
     const WgPeersDev pe = peers_view(ctx);
 
+    // A wave-per-packet launch does the framing itself; it needs every packet to
+    // fit 63 ChaCha20 blocks, which only a host batch can promise.
+    bool fits = host;
+    if (host) {
+        if (wire->lens) {
+            for (uint32_t i = 0; i < n && fits; i++) fits = wire->lens[i] <= WG_FUSE_MAX_LEN + 32u;
+        } else {
+            fits = wire->len <= WG_FUSE_MAX_LEN + 32u;
+        }
+    }
+
     // parse, open and check packets [lo, hi)
     auto run = [&](uint32_t lo, uint32_t hi) -> int {
         WgBatch cw = wb, co = ob;
         cw.first = co.first = lo;
         cw.n = co.n = hi - lo;
+        if (fits) {
+            AeadArgs op{};
+            op.spread_max = ctx->spread_max;
+            op.keys = ctx->d_keys[BNK_KEYS_RECV];
+            op.n_peers = pe.n;
+            op.status = ctx->d_status;
+            op.first = lo;
+            op.n = hi - lo;
+            op.in = wb.base;
+            op.in_off = wb.off;
+            op.in_stride = wire->stride;
+            op.out = const_cast<uint8_t *>(ob.base);
+            op.out_off = ob.off;
+            op.out_stride = out->stride;
+            op.lens = wb.lens;
+            op.len = wire->len;
+            if (aead_runs_spread(op)) {
+                op.wg.mode = WG_FUSE_DECAP;
+                op.wg.n_peers = pe.n;
+                op.wg.index_sorted = pe.index_sorted;
+                op.wg.allowed = pe.allowed;
+                op.wg.result = d_result;
+                op.wg.out_len = d_out_len;
+                op.wg.peer_out = d_peer;
+                op.wg.counter_out = d_counter;
+                HIPCHK(ctx, launch_aead_open(op, ctx->stream));
+                return BNK_OK;
+            }
+        }
         HIPCHK(ctx, launch_wg_parse(cw, pe, d_peer, d_counter, d_ctlen, d_result, ctx->stream));
         AeadArgs op{};
         op.spread_max = ctx->spread_max;

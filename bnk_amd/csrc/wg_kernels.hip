@@ -6,6 +6,7 @@
 // internal/dataplane/engine.go:51, and gives every peer one /32 allowed IP,
 // engine.go:292-299).
 #include "../../include/bnkhip.h"
+#include "kernels.hpp"
 #include "wg_dev.hpp"
 
 namespace bnk {
@@ -20,16 +21,6 @@ BNK_DEV uint32_t wg_ld32(const uint8_t *p)
 }
 
 BNK_DEV void wg_st32(uint8_t *p, uint32_t v) { __builtin_memcpy(p, &v, 4); }
-
-BNK_DEV uint32_t wg_padding(uint32_t len, uint32_t mtu)
-{
-    uint32_t last = len;
-    if (mtu == 0) return ((last + 15u) & ~15u) - last;
-    if (last > mtu) last %= mtu;
-    uint32_t padded = (last + 15u) & ~15u;
-    if (padded > mtu) padded = mtu;
-    return padded - last;
-}
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef u32x4 __attribute__((aligned(1))) u32x4_unaligned;

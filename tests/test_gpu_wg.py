@@ -66,10 +66,14 @@ def _ctx(peers, keys_send=None, keys_recv=None):
 @pytest.mark.parametrize("mem", ["host", "ring", "device"])
 @pytest.mark.parametrize("misalign", [False, True])
 @pytest.mark.parametrize("n", [3000, 700])
-def test_encap_matches_oracle(mem, misalign, n):
+@pytest.mark.parametrize("fused", [True, False])
+def test_encap_matches_oracle(mem, misalign, n, fused):
     """"ring": the slots lie in a pinned ring of the context, which small
     batches seal in place without staging copies.  700 packets also take the
-    one-launch counter assignment, 3000 the sorted one."""
+    one-launch counter assignment, 3000 the sorted one.  fused: host batches
+    this small are framed by the wave-per-packet AEAD launch itself; with the
+    threshold at zero the framing kernels run around a lane-per-packet launch,
+    as they do for large batches."""
     import torch
     from bnk_amd import lib
     from oracle import binding as O
@@ -89,6 +93,8 @@ def test_encap_matches_oracle(mem, misalign, n):
         plains.append(pt)
         arena[int(off[i]) + 16:int(off[i]) + 16 + len(pt)] = np.frombuffer(pt, np.uint8)
     ctx = _ctx(peers, keys_send=keys)
+    if not fused:
+        ctx.set_spread_max_packets(0)
     next_ctr = np.zeros(N_PEERS, np.uint64)
     for round_ in range(2):  # the second batch continues the peers' counters
         want = arena.copy()
@@ -181,7 +187,8 @@ def _decap_cases(rng, peers, keys, n):
 
 @pytest.mark.parametrize("mem", ["host", "ring", "device"])
 @pytest.mark.parametrize("aligned", [True, False])
-def test_decap_matches_oracle(mem, aligned):
+@pytest.mark.parametrize("fused", [True, False])
+def test_decap_matches_oracle(mem, aligned, fused):
     import torch
     from bnk_amd import lib
     from oracle import binding as O
@@ -215,6 +222,8 @@ def test_decap_matches_oracle(mem, aligned):
             want_out[int(out_off[i]):int(out_off[i]) + plen] = np.frombuffer(body, np.uint8)
     assert len(set(want[:, 0].tolist())) == 7  # every result class occurs
     ctx = _ctx(peers, keys_recv=keys)
+    if not fused:
+        ctx.set_spread_max_packets(0)
     if mem == "host":
         got_out = np.full(total + 16, 0x77, np.uint8)
         res = np.full(n, 99, np.uint8)
@@ -264,6 +273,59 @@ def test_decap_matches_oracle(mem, aligned):
     assert np.array_equal(gc, want[:, 3])
     bad = np.flatnonzero(got_out != want_out)
     assert bad.size == 0, f"first differing byte at {bad[:5]}"
+    ctx.close()
+
+
+@pytest.mark.parametrize("n_peers", [65, 4097, 70000])
+@pytest.mark.parametrize("fused", [True, False])
+def test_receiver_index_lookup_in_large_peer_tables(n_peers, fused):
+    """The sender is found by its receiver index in a sorted table: searched 64
+    entries at a time by the lanes of a wave (small batches), or by binary
+    search per packet (70000 peers do not fit the LDS copy and are searched in
+    memory).  Indices at both ends of the table, unknown ones below, between
+    and above: results, peers and counters against the oracle."""
+    from bnk_amd import lib
+    from oracle import binding as O
+    rng = np.random.default_rng(n_peers)
+    local = (rng.permutation(1 << 22)[:n_peers].astype(np.uint64) * 1021 + 5).astype(np.uint32)
+    peers = [(int(local[i]), i, 0x64400001 + i, 0xFFFFFFFF) for i in range(n_peers)]
+    keys = rng.integers(0, 256, (n_peers, 32), dtype=np.uint8)
+    srt = np.sort(local)
+    n = 600 if n_peers < 10000 else 200  # the oracle rebuilds its table per packet
+    who = rng.integers(0, n_peers, n)
+    who[:4] = [int(np.argmin(local)), int(np.argmax(local)), 0, n_peers - 1]
+    wires = []
+    for i in range(n):
+        p = int(who[i])
+        pt = bytearray(rng.integers(0, 256, 48, dtype=np.uint8).tobytes())
+        pt[0] = 0x45
+        pt[2:4] = struct.pack(">H", 48)
+        pt[12:16] = struct.pack(">I", peers[p][2])
+        w = bytearray(O.wg_encap(bytes(pt), MTU, keys[p].tobytes(), peers[p][0], 1000 + i))
+        if i % 5 == 4:  # an index nobody owns
+            bogus = [int(srt[0]) - 1, int(srt[-1]) + 1, int(srt[len(srt) // 2]) + 1, 0, 0xFFFFFFFF][(i // 5) % 5]
+            w[4:8] = struct.pack("<I", bogus & 0xFFFFFFFF)
+        wires.append(bytes(w))
+    lens = np.array([len(w) for w in wires], np.uint32)
+    off = np.arange(n, dtype=np.uint64) * 128
+    arena = np.zeros(n * 128, np.uint8)
+    for i, w in enumerate(wires):
+        arena[i * 128:i * 128 + len(w)] = np.frombuffer(w, np.uint8)
+    want = np.array([(lambda r: (r[0], len(r[1]), r[2], r[3]))(O.wg_decap(w, peers, keys)) for w in wires],
+                    np.uint64)
+    assert (want[:, 0] == O.WG_UNKNOWN_INDEX).sum() >= n // 5 - 1 and (want[:, 0] == 0).sum() >= n // 2
+    ctx = _ctx(peers, keys_recv=keys)
+    if not fused:
+        ctx.set_spread_max_packets(0)
+    out = np.zeros(n * 128, np.uint8)
+    res, olen = np.full(n, 99, np.uint8), np.full(n, 99, np.uint32)
+    gp, gc = np.full(n, 99, np.uint32), np.full(n, 99, np.uint64)
+    ctx.wg_decap(lib.make_batch(arena, arena.nbytes, n, lib.MEM_HOST, offsets=off, lens=lens),
+                 lib.make_batch(out, out.nbytes, n, lib.MEM_HOST, offsets=off), res, olen, gp, gc)
+    assert np.array_equal(res, want[:, 0].astype(np.uint8))
+    assert np.array_equal(olen, want[:, 1].astype(np.uint32))
+    assert np.array_equal(gp, want[:, 2].astype(np.uint32))
+    assert np.array_equal(gc, want[:, 3])
     ctx.close()
 
 

@@ -148,11 +148,9 @@ BNK_DEV void crypt_tail(Poly32 &mac, const uint32_t (&x)[16], int j, const uint8
 
 template <bool OPEN>
 BNK_DEV void body_generic(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_t *dst,
-                          uint32_t len, const uint32_t (&k)[8], uint32_t n1, uint32_t n2,
-                          Poly32 &mac, uint32_t (&x)[16])
+                          uint32_t len, const uint8_t *safe, const uint32_t (&k)[8], uint32_t n1,
+                          uint32_t n2, Poly32 &mac, uint32_t (&x)[16])
 {
-    chacha_block(k, 0, n1, n2, x);
-    mac.init(x);
     const uint32_t nfull = len >> 6, rem = len & 63u;
     const uint32_t steps = nfull + (rem ? 1u : 0u);
     // the four (packet, 16-byte column) cells this lane moves per step
@@ -167,17 +165,27 @@ BNK_DEV void body_generic(uint8_t *tile, uint32_t lane, const uint8_t *src, uint
         cdst[j] = reinterpret_cast<uint8_t *>(shfl64((uint64_t)(uintptr_t)dst, owner)) + 16u * col;
         clen[j] = (uint32_t)__shfl((int)len, owner, 64);
     }
+    // The cells of step b+1 are fetched into registers while step b is
+    // computed.  Every lane loads every time, from a harmless address (`safe`,
+    // 16 readable bytes) when the cell is not a packet's: a load under a branch
+    // would make the wave wait for it before the branch closes.
+    uint4 pre[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) pre[j] = ld16(16u * col + 16u <= clen[j] ? csrc[j] : safe);
+    chacha_block(k, 0, n1, n2, x);
+    mac.init(x);
     for (uint32_t b = 0; __ballot(b < steps) != 0ull; b++) {
         const uint32_t pos = 64u * b + 16u * col;
-        // global -> LDS, all 64 lanes, only 16-byte cells that lie fully inside a packet
+        // registers -> LDS, all 64 lanes, only 16-byte cells that lie fully inside a packet
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            if (pos + 16u <= clen[j]) {
-                const uint4 v = ld16(csrc[j] + 64u * b);
-                *reinterpret_cast<uint4 *>(tile + (16u * j + (lane >> 2)) * LDS_ROW + 16u * col) = v;
-            }
+            if (pos + 16u <= clen[j])
+                *reinterpret_cast<uint4 *>(tile + (16u * j + (lane >> 2)) * LDS_ROW + 16u * col) = pre[j];
         }
         wave_sync();
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            pre[j] = ld16(pos + 64u + 16u <= clen[j] ? csrc[j] + 64u * (b + 1u) : safe);
         if (b < steps) {
             chacha_block(k, b + 1, n1, n2, x);
             uint8_t *row = tile + lane * LDS_ROW;
@@ -447,7 +455,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const bool lane_lines = (((uintptr_t)src | (uintptr_t)dst) & 15u) == 0 &&
                             (((uintptr_t)src ^ (uintptr_t)dst) & 127u) == 0;
     if (__ballot(!lane_lines) == 0ull) body_lines<OPEN>(tile, lane, src, dst, len, reinterpret_cast<const uint8_t *>(a.keys), k, n1, n2, mac, x);
-    else body_generic<OPEN>(tile, lane, src, dst, len, k, n1, n2, mac, x);
+    else body_generic<OPEN>(tile, lane, src, dst, len, reinterpret_cast<const uint8_t *>(a.keys), k, n1, n2, mac, x);
 
     lane_finish<OPEN>(a, lane, have, i, len, src, dst, mac);
 }
@@ -573,7 +581,7 @@ __global__ __launch_bounds__(256) void aead_spread_kernel(AeadArgs a)
         const bool have = lane == 0;
         Poly32 mac;
         body_generic<OPEN>(tile_all[threadIdx.x >> 6], lane, have ? src : nullptr, have ? dst : nullptr,
-                           have ? len : 0u, k, n1, n2, mac, x);
+                           have ? len : 0u, reinterpret_cast<const uint8_t *>(a.keys), k, n1, n2, mac, x);
         lane_finish<OPEN>(a, lane, have, i, len, have ? src : nullptr, have ? dst : nullptr, mac);
         return;
     }

@@ -582,6 +582,9 @@ def main() -> int:
                     help="wg: wait for the send side before starting the receive side, so a kernel "
                          "trace shows undisturbed durations (the two sides use separate streams)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="aead: leave out the packed-layout leg and the ACL filter extra, so that a "
+                         "kernel trace of the run holds the timed launches only")
     ap.add_argument("--cpu-sample", type=int, default=0,
                     help="packets in the CPU baseline sample (0 = sized for ~10 s)")
     args = ap.parse_args()
@@ -709,6 +712,10 @@ def main() -> int:
     # the same packets packed back to back (plaintexts at a 1420-byte stride,
     # sealed packets at 1436): no slot is 16-byte aligned, so the kernel moves
     # them 64 bytes at a time at any alignment instead of whole 128-byte lines
+    if args.no_extras:
+        ctx.close()
+        print(json.dumps(out))
+        return 0
     pk_plain = plain[:, :L].contiguous().view(-1)
     pk_sealed = torch.zeros(n * (L + 16), dtype=torch.uint8, device=dev)
     pk_opened = torch.zeros(n * L, dtype=torch.uint8, device=dev)

@@ -123,6 +123,49 @@ def test_edge_lengths_and_high_counters(small_ctx):
     assert _packets_equal(back, b.plain, b.off, b.lens) == -1
 
 
+@pytest.mark.parametrize("half", [0, 1])
+@pytest.mark.parametrize("misalign", [False, True])
+def test_every_length_through_one_wave_and_beyond(small_ctx, half, misalign):
+    """Every plaintext length from 0 to 4200 bytes: all the shapes of a packet
+    spread over a wave (cells, blocks, lanes partly filled, the 63-block limit
+    at 4032 bytes and the single-lane fallback beyond it), at aligned and at
+    arbitrary byte offsets, forged tags among them."""
+    from bnk_amd import lib
+    from oracle import binding as O
+    ctx = small_ctx
+    lens = np.arange(half, 4201, 2, dtype=np.uint32)
+    n = len(lens)
+    rng = np.random.default_rng(40 + half + 2 * misalign)
+    rng.shuffle(lens)
+    gaps = rng.integers(0, 16, n) if misalign else np.zeros(n, np.int64)
+    room = ((lens.astype(np.int64) + 16 + 15) & ~15) + 16
+    off = (np.concatenate([[0], np.cumsum(room)[:-1]]) + gaps).astype(np.uint64)
+    total = int(room.sum()) + 16
+    plain = rng.integers(0, 256, total, dtype=np.uint8)
+    keys = rng.integers(0, 256, (3, 32), dtype=np.uint8)
+    peer = rng.integers(0, 3, n).astype(np.uint32)
+    counters = rng.integers(0, 1 << 63, n, dtype=np.uint64)
+    ctx.keys_set(lib.KEYS_SEND, keys)
+    ctx.keys_set(lib.KEYS_RECV, keys)
+    want = np.full(total, 0x5A, np.uint8)
+    O.seal_batch(keys, peer, counters, plain, off, lens, want, off, 4)
+    got = np.full(total, 0x5A, np.uint8)
+    ctx.seal(lib.make_batch(plain, total, n, lib.MEM_HOST, offsets=off, lens=lens, peer=peer, counters=counters),
+             lib.make_batch(got, total, n, lib.MEM_HOST, offsets=off))
+    bad = np.flatnonzero(got != want)
+    assert bad.size == 0, f"first differing byte at {bad[:3]}"
+    forged = W.forge_tags(41, got, off, lens, 0.05)
+    ct_lens = (lens + 16).astype(np.uint32)
+    back = np.full(total, 0xEE, np.uint8)
+    verdict = np.full(n, 7, np.uint8)
+    ctx.open(lib.make_batch(got, total, n, lib.MEM_HOST, offsets=off, lens=ct_lens, peer=peer, counters=counters),
+             lib.make_batch(back, total, n, lib.MEM_HOST, offsets=off), verdict)
+    oback = np.full(total, 0xEE, np.uint8)
+    overdict = O.open_batch(keys, peer, counters, got, off, ct_lens, oback, off, 4)
+    assert np.array_equal(verdict, overdict) and np.array_equal(verdict == 0, forged)
+    assert np.array_equal(back, oback)
+
+
 @pytest.mark.parametrize("n", [64, 128, 100])
 def test_unsorted_mixed_lengths_within_a_wave(small_ctx, n):
     ctx = small_ctx

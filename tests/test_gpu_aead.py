@@ -392,15 +392,20 @@ def test_in_place_and_unaligned_slots(small_ctx):
     assert np.array_equal(wv.reshape(n, stride)[:, :L], view.reshape(n, stride)[:, :L])
 
 
-def test_short_and_error_paths(small_ctx):
+@pytest.mark.parametrize("mem", ["pageable", "ring"])
+def test_short_and_error_paths(small_ctx, mem):
     ctx = small_ctx
     from bnk_amd import lib
     b = W.aead_uniform(13, 4, 32)
     ctx.keys_set(lib.KEYS_SEND, b.keys)
     ctx.keys_set(lib.KEYS_RECV, b.keys)
     # ciphertext shorter than a tag: verdict 0, nothing written
-    buf = np.zeros(64, np.uint8)
-    out = np.full(64, 0xEE, np.uint8)
+    rings = [ctx.ring_alloc(64) for _ in range(3)] if mem == "ring" else []
+    buf, out, ka = rings if rings else (np.zeros(64, np.uint8), np.zeros(64, np.uint8), np.zeros(32, np.uint8))
+    buf[:] = 0
+    out[:] = 0xEE
+    ka = ka[:32]
+    ka[:] = 0
     v = np.full(2, 9, np.uint8)
     inb = lib.make_batch(buf, 64, 2, lib.MEM_HOST, stride=32, length=15)
     outb = lib.make_batch(out, 64, 2, lib.MEM_HOST, stride=32)
@@ -420,7 +425,6 @@ def test_short_and_error_paths(small_ctx):
                  lib.make_batch(out, 64, 2, lib.MEM_HOST, stride=32))
     assert ei.value.code == lib.E_RANGE
     # keepalive: empty plaintext seals to just a tag, and opens
-    ka = np.zeros(32, np.uint8)
     ctx.seal(lib.make_batch(ka, 32, 2, lib.MEM_HOST, stride=16, length=0, counter0=9),
              lib.make_batch(ka, 32, 2, lib.MEM_HOST, stride=16))
     from oracle import binding as O
@@ -429,6 +433,8 @@ def test_short_and_error_paths(small_ctx):
     ctx.open(lib.make_batch(ka, 32, 2, lib.MEM_HOST, stride=16, length=16, counter0=9),
              lib.make_batch(ka, 32, 2, lib.MEM_HOST, stride=16), v)
     assert v.tolist() == [1, 1]
+    for r in rings:
+        ctx.ring_free(r)
 
 
 def test_device_resident_large_batch_properties(ctx):

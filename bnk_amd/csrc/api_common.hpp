@@ -152,8 +152,9 @@ inline int stage_host(bnk_ctx *ctx, const bnk_batch *in, const bnk_batch *out, i
             if (in->peer[i] >= n_keys)
                 return fail(ctx, BNK_E_RANGE, "peer index " + std::to_string(in->peer[i]) +
                                                   " beyond the key table");
-    // pinned staging for the two rebased offset arrays
-    HIPCHK(ctx, ctx->pin.reserve((size_t)n * 16 + 64));
+    // pinned staging for the two rebased offset arrays, and behind them room for
+    // one result byte per packet (a copy into pageable memory is slow)
+    HIPCHK(ctx, ctx->pin.reserve((size_t)n * 17 + 64));
 
     st->in_place = same_layout(in, out);
     if (st->in_place) {

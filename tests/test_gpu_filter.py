@@ -41,10 +41,13 @@ def _flat(rec):
             np.full(n, 28, np.uint32))
 
 
-def test_cfg4_small_verdicts_and_flow_table_match_oracle():
+@pytest.mark.parametrize("n", [1 << 15, 70000])
+def test_cfg4_small_verdicts_and_flow_table_match_oracle(n):
+    """Host batches: up to 65,536 packets the kernel reads the gathered headers
+    from pinned staging in place, above that they are uploaded first."""
     from bnk_amd import lib
     from oracle import binding as O
-    w = W.acl_workload(n=1 << 15)
+    w = W.acl_workload(n=n)
     ctx = lib.Context(0)
     ora = O.Filter()
     ctx.filter_set_rules(w.rules_ref)

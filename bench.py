@@ -517,7 +517,7 @@ def bench_latency(args) -> dict:
         rows = ring.reshape(n, slot)
         wl, res, ol = np.zeros(n, np.uint32), np.zeros(n, np.uint8), np.zeros(n, np.uint32)
         gp, gc = np.zeros(n, np.uint32), np.zeros(n, np.uint64)
-        te, td = [], []
+        te, td, tne, tdf = [], [], [], []
         for it in range(reps + 5):
             rows[:, 16:36] = 0
             rows[:, 16] = 0x45
@@ -532,13 +532,34 @@ def bench_latency(args) -> dict:
             ctx.wg_decap(lib.make_batch(ring, n * slot, n, lib.MEM_HOST, offsets=off, lens=wl),
                          lib.make_batch(back, n * slot, n, lib.MEM_HOST, offsets=off), res, ol, gp, gc)
             t2 = time.perf_counter()
+            if int((res != 0).sum()) != 0:
+                raise SystemExit("framing round trip rejected packets")
+            # the same with the filter inside the call: NoteOutbound before the
+            # encapsulation, CheckInbound after the decapsulation
+            rows[:, 16:36] = 0
+            rows[:, 16] = 0x45
+            rows[:, 18] = inner >> 8
+            rows[:, 19] = inner & 255
+            rows[:, 25] = 17
+            for k in range(4):
+                rows[:, 28 + k] = (src >> (24 - 8 * k)) & 255
+            t3 = time.perf_counter()
+            ctx.wg_note_encap(lib.make_batch(ring, n * slot, n, lib.MEM_HOST, offsets=off, lens=lens, peer=peer),
+                              1420, 1_700_000_000_000_000_000, wl)
+            t4 = time.perf_counter()
+            ctx.wg_decap_filter(lib.make_batch(ring, n * slot, n, lib.MEM_HOST, offsets=off, lens=wl),
+                                lib.make_batch(back, n * slot, n, lib.MEM_HOST, offsets=off),
+                                1_700_000_000_000_000_000, res, ol, gp, gc)
+            t5 = time.perf_counter()
             if it >= 5:
                 te.append(t1 - t0)
                 td.append(t2 - t1)
-        if int((res != 0).sum()) != 0:
-            raise SystemExit("framing round trip rejected packets")
+                tne.append(t4 - t3)
+                tdf.append(t5 - t4)
         out[str(n)]["wg_encap"] = round(float(np.median(te)) * 1e6, 1)
         out[str(n)]["wg_decap"] = round(float(np.median(td)) * 1e6, 1)
+        out[str(n)]["wg_note_encap"] = round(float(np.median(tne)) * 1e6, 1)
+        out[str(n)]["wg_decap_filter"] = round(float(np.median(tdf)) * 1e6, 1)
         ctx.ring_free(ring)
         ctx.ring_free(back)
     ctx.close()

@@ -97,7 +97,7 @@ void filter_destroy(FilterState *f)
 
 } // namespace bnk
 
-namespace {
+namespace bnk {
 
 // Makes room for n_new more distinct flows: open addressing stays below half
 // full per region, growing (and dropping tombstones) when it would not.
@@ -140,6 +140,10 @@ int flows_reserve(bnk_ctx *ctx, uint32_t n_new)
     f->flows.small_ok = f->claimed_upper <= SMALL_KEYS_MAX;
     return BNK_OK;
 }
+
+} // namespace bnk
+
+namespace {
 
 // The filter reads at most the first 64 bytes of a packet (IPv4 header of up
 // to 60 bytes, then 4 port bytes): host packets are gathered at a 64-byte

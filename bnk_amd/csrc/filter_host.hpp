@@ -181,6 +181,9 @@ constexpr uint32_t FLOW_CAP_INITIAL = 8192;      // slots per region
 constexpr uint32_t FLOW_CAP_MAX = 1u << 26;
 
 FilterState *filter_create(hipStream_t s, int cu_count);
+// Makes room for n_new more distinct flows before a NoteOutbound launch (may
+// rehash the table, which waits for the context's stream).
+int flows_reserve(bnk_ctx *ctx, uint32_t n_new);
 void filter_destroy(FilterState *f);
 
 } // namespace bnk

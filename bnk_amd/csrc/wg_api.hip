@@ -3,6 +3,7 @@
 #include <vector>
 
 #include "api_common.hpp"
+#include "filter_host.hpp"
 #include "wg_dev.hpp"
 
 using namespace bnk;
@@ -73,10 +74,11 @@ extern "C" int bnk_wg_send_counters(bnk_ctx *ctx, uint64_t *out, uint32_t n)
     return BNK_OK;
 }
 
-extern "C" int bnk_wg_encap_batch(bnk_ctx *ctx, const bnk_batch *slots, uint32_t mtu, uint32_t *wire_len)
+// bnk_wg_encap_batch, with NoteOutbound at *note_now on the plaintexts first
+// when note_now is given.
+static int wg_encap_impl(bnk_ctx *ctx, const bnk_batch *slots, uint32_t mtu, uint32_t *wire_len,
+                         const int64_t *note_now)
 {
-    Guard g(ctx);
-    if (g.rc) return g.rc;
     int rc = check_batch_common(ctx, slots, "slots");
     if (rc) return rc;
     const uint32_t n = slots->n;
@@ -236,12 +238,34 @@ extern "C" int bnk_wg_encap_batch(bnk_ctx *ctx, const bnk_batch *slots, uint32_t
         }
     }
 
-    // header, padding and seal of packets [lo, hi)
+    // filter.go:192-194: NoteOutbound does nothing in allow-all mode
+    const bool note = note_now != nullptr && ctx->filter->enforce;
+    if (note) {
+        rc = flows_reserve(ctx, n);
+        if (rc) return rc;
+    }
+
+    // NoteOutbound, then header, padding and seal of packets [lo, hi)
     auto run = [&](uint32_t lo, uint32_t hi) -> int {
         WgBatch c = b;
         c.first = lo;
         c.n = hi - lo;
         uint8_t *sealed = ring_out ? ring_out : const_cast<uint8_t *>(b.base);
+        if (note) {
+            FilterState *f = ctx->filter;
+            FilterArgs fa{};
+            fa.pkts = b.base + 16 + (b.off ? 0 : (uint64_t)lo * slots->stride);
+            fa.off = b.off ? b.off + lo : nullptr;
+            fa.lens = b.lens ? b.lens + lo : nullptr;
+            fa.stride = slots->stride;
+            fa.len = slots->len;
+            fa.status = ctx->d_status;
+            fa.now = *note_now;
+            fa.n = hi - lo;
+            fa.rules = f->ridx;
+            fa.flows = f->flows;
+            HIPCHK(ctx, launch_filter_note(fa, f->max_blocks, ctx->stream));
+        }
         if (fits) {
             AeadArgs se{};
             se.spread_max = ctx->spread_max;
@@ -309,10 +333,17 @@ extern "C" int bnk_wg_encap_batch(bnk_ctx *ctx, const bnk_batch *slots, uint32_t
         if (rc) return rc;
         if (!host) return BNK_OK;
         if (ring_out) {
-            // peer indices were checked above: nothing comes back through the status word
-            HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+            // peer indices were checked above: only a flow table overflow could come
+            // back through the status word
+            uint32_t status = 0;
+            if (note) {
+                rc = take_status(ctx, &status);
+                if (rc) return rc;
+            } else {
+                HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+            }
             memcpy(wire_len, h_wire_len, (size_t)n * 4);
-            return BNK_OK;
+            return status_to_rc(ctx, status);
         }
         HIPCHK(ctx, hipMemcpyAsync((uint8_t *)slots->base + span.lo, ctx->in_arena.p, span.size(),
                                    hipMemcpyDeviceToHost, ctx->stream));
@@ -324,11 +355,26 @@ extern "C" int bnk_wg_encap_batch(bnk_ctx *ctx, const bnk_batch *slots, uint32_t
     return status_to_rc(ctx, status);
 }
 
-extern "C" int bnk_wg_decap_batch(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *out,
-                                  uint8_t *result, uint32_t *out_len, uint32_t *peer, uint64_t *counter)
+extern "C" int bnk_wg_encap_batch(bnk_ctx *ctx, const bnk_batch *slots, uint32_t mtu, uint32_t *wire_len)
 {
     Guard g(ctx);
     if (g.rc) return g.rc;
+    return wg_encap_impl(ctx, slots, mtu, wire_len, nullptr);
+}
+
+extern "C" int bnk_wg_note_encap_batch(bnk_ctx *ctx, const bnk_batch *slots, uint32_t mtu, int64_t now_ns,
+                                       uint32_t *wire_len)
+{
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    return wg_encap_impl(ctx, slots, mtu, wire_len, &now_ns);
+}
+
+// bnk_wg_decap_batch, with CheckInbound at *check_now on the delivered
+// packets afterwards when check_now is given.
+static int wg_decap_impl(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *out, uint8_t *result,
+                         uint32_t *out_len, uint32_t *peer, uint64_t *counter, const int64_t *check_now)
+{
     int rc = check_batch_common(ctx, wire, "wire");
     if (rc) return rc;
     rc = check_batch_common(ctx, out, "out");
@@ -491,6 +537,32 @@ extern "C" int bnk_wg_decap_batch(bnk_ctx *ctx, const bnk_batch *wire, const bnk
         }
     }
 
+    // filter.go:124-126: CheckInbound passes everything in allow-all mode
+    const bool check = check_now != nullptr && ctx->filter->enforce;
+    if (check) HIPCHK(ctx, ctx->r_pass.reserve(n));
+
+    // CheckInbound of what packets [lo, hi) delivered: a packet that was not
+    // delivered has length 0 here, which the filter refuses without a side effect
+    auto filter_range = [&](uint32_t lo, uint32_t hi) -> int {
+        if (!check) return BNK_OK;
+        FilterState *f = ctx->filter;
+        uint8_t *d_pass = ctx->r_pass.as<uint8_t>();
+        FilterArgs fa{};
+        fa.pkts = ob.base + (ob.off ? 0 : (uint64_t)lo * out->stride);
+        fa.off = ob.off ? ob.off + lo : nullptr;
+        fa.lens = d_out_len + lo;
+        fa.stride = out->stride;
+        fa.verdict = d_pass + lo;
+        fa.status = ctx->d_status;
+        fa.now = *check_now;
+        fa.n = hi - lo;
+        fa.rules = f->ridx;
+        fa.flows = f->flows;
+        HIPCHK(ctx, launch_filter_check(fa, f->max_blocks, ctx->stream));
+        HIPCHK(ctx, launch_wg_mark_filtered(d_result + lo, d_pass + lo, hi - lo, ctx->stream));
+        return BNK_OK;
+    };
+
     // parse, open and check packets [lo, hi)
     auto run = [&](uint32_t lo, uint32_t hi) -> int {
         WgBatch cw = wb, co = ob;
@@ -522,7 +594,7 @@ extern "C" int bnk_wg_decap_batch(bnk_ctx *ctx, const bnk_batch *wire, const bnk
                 op.wg.peer_out = d_peer;
                 op.wg.counter_out = d_counter;
                 HIPCHK(ctx, launch_aead_open(op, ctx->stream));
-                return BNK_OK;
+                return filter_range(lo, hi);
             }
         }
         HIPCHK(ctx, launch_wg_parse(cw, pe, d_peer, d_counter, d_ctlen, d_result, ctx->stream));
@@ -552,7 +624,7 @@ extern "C" int bnk_wg_decap_batch(bnk_ctx *ctx, const bnk_batch *wire, const bnk
         }
         HIPCHK(ctx, launch_aead_open(op, ctx->stream));
         HIPCHK(ctx, launch_wg_finish(co, 0, pe, d_peer, d_ctlen, d_auth, d_result, d_out_len, ctx->stream));
-        return BNK_OK;
+        return filter_range(lo, hi);
     };
 
     if (chunked) {
@@ -590,4 +662,21 @@ extern "C" int bnk_wg_decap_batch(bnk_ctx *ctx, const bnk_batch *wire, const bnk
     rc = take_status(ctx, &status);
     if (rc) return rc;
     return status_to_rc(ctx, status);
+}
+
+extern "C" int bnk_wg_decap_batch(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *out,
+                                  uint8_t *result, uint32_t *out_len, uint32_t *peer, uint64_t *counter)
+{
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    return wg_decap_impl(ctx, wire, out, result, out_len, peer, counter, nullptr);
+}
+
+extern "C" int bnk_wg_decap_filter_batch(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *out,
+                                         int64_t now_ns, uint8_t *result, uint32_t *out_len,
+                                         uint32_t *peer, uint64_t *counter)
+{
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    return wg_decap_impl(ctx, wire, out, result, out_len, peer, counter, &now_ns);
 }

@@ -33,4 +33,7 @@ hipError_t launch_wg_encap_prep(const WgBatch &b, uint8_t *hdr_base, const WgPee
                                 const uint64_t *counter, uint32_t mtu, uint32_t *padded_len,
                                 uint32_t *wire_len, uint8_t *skip, hipStream_t s);
 
+// result[i] = BNK_WG_FILTERED where it was BNK_WG_OK and pass[i] == 0.
+hipError_t launch_wg_mark_filtered(uint8_t *result, const uint8_t *pass, uint32_t n, hipStream_t s);
+
 } // namespace bnk

@@ -40,6 +40,7 @@ class Batch(C.Structure):
 
 WG_OK, WG_KEEPALIVE, WG_BAD_HEADER, WG_UNKNOWN_INDEX, WG_AUTH_FAIL, WG_BAD_IP, \
     WG_NOT_ALLOWED = range(7)
+WG_FILTERED = 7
 
 
 class Rule(C.Structure):
@@ -343,6 +344,16 @@ class Context:
         self._chk(self._lib.bnk_wg_decap_batch(
             self._h, C.byref(wire), C.byref(outb), C.c_void_p(_ptr(result)),
             C.c_void_p(_ptr(out_len)), C.c_void_p(_ptr(peer)), C.c_void_p(_ptr(counter))))
+
+    def wg_decap_filter(self, wire: Batch, outb: Batch, now_ns: int, result, out_len, peer,
+                        counter) -> None:
+        self._chk(self._lib.bnk_wg_decap_filter_batch(
+            self._h, C.byref(wire), C.byref(outb), C.c_int64(now_ns), C.c_void_p(_ptr(result)),
+            C.c_void_p(_ptr(out_len)), C.c_void_p(_ptr(peer)), C.c_void_p(_ptr(counter))))
+
+    def wg_note_encap(self, slots: Batch, mtu: int, now_ns: int, wire_len) -> None:
+        self._chk(self._lib.bnk_wg_note_encap_batch(self._h, C.byref(slots), C.c_uint32(mtu),
+                                                    C.c_int64(now_ns), C.c_void_p(_ptr(wire_len))))
 
     # ---- measurement ----
     def probe_valu(self, op: str | int, iters: int = 2000) -> float:

@@ -229,7 +229,9 @@ enum {
     BNK_WG_UNKNOWN_INDEX = 3, /* no peer owns the receiver index */
     BNK_WG_AUTH_FAIL = 4,     /* tag mismatch */
     BNK_WG_BAD_IP = 5,        /* not IPv4/IPv6 or length fields beyond the plaintext */
-    BNK_WG_NOT_ALLOWED = 6    /* inner source outside the peer's allowed IP */
+    BNK_WG_NOT_ALLOWED = 6,   /* inner source outside the peer's allowed IP */
+    BNK_WG_FILTERED = 7       /* bnk_wg_decap_filter_batch only: delivered by
+                                 WireGuard, dropped by the inbound filter */
 };
 
 typedef struct bnk_wg_peer {
@@ -265,6 +267,24 @@ int bnk_wg_encap_batch(bnk_ctx *ctx, const bnk_batch *slots, uint32_t mtu,
 int bnk_wg_decap_batch(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *out,
                        uint8_t *result, uint32_t *out_len, uint32_t *peer,
                        uint64_t *counter);
+
+/* The receive path of a tunnel in one call: bnk_wg_decap_batch, then
+ * CheckInbound (internal/filter/filter.go:121-147) with one now_ns on every
+ * packet that came out BNK_WG_OK, as filteredTUN.Write (filter.go:171-186)
+ * does with what wireguard-go hands it.  A packet the filter denies reports
+ * BNK_WG_FILTERED; everything else about it (plaintext in its slot, out_len,
+ * peer, counter) is as for BNK_WG_OK, because wireguard-go runs the replay
+ * window before the write that filters: feed its counter to the window too.
+ * In allow-all mode nothing is filtered.  Same arguments as
+ * bnk_wg_decap_batch otherwise. */
+int bnk_wg_decap_filter_batch(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *out,
+                              int64_t now_ns, uint8_t *result, uint32_t *out_len,
+                              uint32_t *peer, uint64_t *counter);
+/* The send path in one call: NoteOutbound (filter.go:189-209) with one
+ * now_ns on every plaintext, as filteredTUN.Read (filter.go:160-167) does
+ * with what the TUN hands it, then bnk_wg_encap_batch. */
+int bnk_wg_note_encap_batch(bnk_ctx *ctx, const bnk_batch *slots, uint32_t mtu,
+                            int64_t now_ns, uint32_t *wire_len);
 
 /* ---- fused relay ------------------------------------------------------- */
 

@@ -329,6 +329,210 @@ def test_receiver_index_lookup_in_large_peer_tables(n_peers, fused):
     ctx.close()
 
 
+def _filter_setup(rng, peers):
+    """Rules that let some peers reach some ports, and a few recorded outbound
+    flows whose replies must pass without a rule."""
+    rules = [([(peers[p][2], 32)], "tcp", [(22, 22), (8000, 8100)]) for p in range(0, N_PEERS, 3)]
+    rules += [([(0x64400000, 16)], "udp", [(53, 53)]), ([(peers[1][2], 32)], "icmp", [])]
+    local = 0x64700001
+    noted = [W.udp(local, peers[p][2], 4000 + p, 9000 + p) for p in range(2, N_PEERS, 4)]
+    noted += [W.tcp(local, peers[p][2], 5000 + p, 443) for p in range(3, N_PEERS, 5)]
+    return rules, local, noted
+
+
+@pytest.mark.parametrize("mem", ["host", "ring", "device"])
+@pytest.mark.parametrize("fused", [True, False])
+def test_decap_with_the_inbound_filter_in_one_call(mem, fused):
+    """bnk_wg_decap_filter_batch = decapsulate, then CheckInbound with one `now`
+    on what was delivered: results (FILTERED for the denied), plaintexts,
+    peers, counters and the flow table afterwards against the oracle's two
+    steps, and against the library's own two calls."""
+    import torch
+    from bnk_amd import lib
+    from oracle import binding as O
+    rng = np.random.default_rng(77)
+    peers = _peers(rng)
+    keys = rng.integers(0, 256, (N_PEERS, 32), dtype=np.uint8)
+    rules, local, noted = _filter_setup(rng, peers)
+    t0 = 1_700_000_000 * 10**9
+    n = 1500
+    wires = []
+    for i in range(n):
+        p = int(rng.integers(0, N_PEERS))
+        src = peers[p][2]
+        kind = int(rng.integers(0, 8))
+        if kind == 0:
+            pt = W.tcp(src, local, 40000 + i, int(rng.choice([22, 23, 8000, 8100, 8101, 443])))
+        elif kind == 1:
+            pt = W.udp(src, local, int(rng.choice([53, 9000 + p])), int(rng.choice([53, 4000 + p, 4001])))
+        elif kind == 2:
+            pt = W.tcp(src, local, 443, 5000 + p, syn=False)      # reply to a recorded flow, or not
+        elif kind == 3:
+            pt = W.icmp_echo(src, local)
+        elif kind == 4:
+            pt = W.udp(src ^ 0x00010000, local, 53, 53)           # not the peer's address
+        elif kind == 5:
+            pt = b""                                              # keepalive
+        elif kind == 6:
+            pt = W.tcp(src, local, 1, 22) + bytes(int(rng.integers(0, 40)))  # trailing bytes beyond the IP length
+        else:
+            pt = W.ipv4(47, src, local, bytes(8))                 # a protocol the filter does not parse
+        w = bytearray(O.wg_encap(pt, MTU, keys[p].tobytes(), peers[p][0], 100 + i))
+        if i % 19 == 0:
+            w[-1] ^= 1
+        wires.append(bytes(w))
+    lens = np.array([len(w) for w in wires], np.uint32)
+    off, total = _layout(rng, lens)
+    arena = np.full(total, 0xEE, np.uint8)
+    for i, w in enumerate(wires):
+        arena[int(off[i]):int(off[i]) + len(w)] = np.frombuffer(w, np.uint8)
+    out_off = off + np.uint64(16)
+
+    # the oracle's two steps
+    ora = O.Filter()
+    ora.set_rules(rules)
+    for pkt in noted:
+        ora.note_outbound(pkt, t0 - 10**9)
+    want = np.zeros((n, 4), np.uint64)
+    for i, w in enumerate(wires):
+        rc, pt, p, c = O.wg_decap(w, peers, keys)
+        if rc == O.WG_OK and not ora.check_inbound(pt, t0):
+            rc = lib.WG_FILTERED
+        want[i] = (rc, len(pt), p, c)
+    assert {0, 1, 4, 6, 7} <= set(want[:, 0].tolist())
+    assert 0.2 < (want[:, 0] == 7).mean() < 0.7 and (want[:, 0] == 0).mean() > 0.1
+
+    def fresh_ctx():
+        ctx = _ctx(peers, keys_recv=keys)
+        if not fused:
+            ctx.set_spread_max_packets(0)
+        ctx.filter_set_rules(rules)
+        for pkt in noted:
+            ctx.filter_note_outbound_ptrs([pkt], t0 - 10**9)
+        return ctx
+
+    ctx = fresh_ctx()
+    res, olen = np.full(n, 99, np.uint8), np.full(n, 99, np.uint32)
+    gp, gc = np.full(n, 99, np.uint32), np.full(n, 99, np.uint64)
+    if mem == "device":
+        dev = torch.device("cuda:0")
+        d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)  # noqa: E731
+        d_arena, d_off, d_lens, d_ooff = d(arena), d(off.astype(np.int64)), d(lens.astype(np.int32)), d(out_off.astype(np.int64))
+        d_out = torch.full((total + 16,), 0x77, dtype=torch.uint8, device=dev)
+        d_res = torch.full((n,), 99, dtype=torch.uint8, device=dev)
+        d_olen, d_gp = torch.zeros(n, dtype=torch.int32, device=dev), torch.zeros(n, dtype=torch.int32, device=dev)
+        d_gc = torch.zeros(n, dtype=torch.int64, device=dev)
+        torch.cuda.synchronize()
+        ctx.wg_decap_filter(lib.make_batch(d_arena, d_arena.numel(), n, lib.MEM_DEVICE, offsets=d_off, lens=d_lens),
+                            lib.make_batch(d_out, d_out.numel(), n, lib.MEM_DEVICE, offsets=d_ooff),
+                            t0, d_res, d_olen, d_gp, d_gc)
+        ctx.sync()
+        got_out = d_out.cpu().numpy()
+        res, olen = d_res.cpu().numpy(), d_olen.cpu().numpy().astype(np.uint32)
+        gp, gc = d_gp.cpu().numpy().astype(np.uint32), d_gc.cpu().numpy().astype(np.uint64)
+    else:
+        rings = []
+        if mem == "ring":
+            rings = [ctx.ring_alloc(arena.nbytes), ctx.ring_alloc(total + 16)]
+            rings[0][:] = arena
+            src, got_out = rings
+        else:
+            src, got_out = arena, np.zeros(total + 16, np.uint8)
+        got_out[:] = 0x77
+        ctx.wg_decap_filter(lib.make_batch(src, arena.nbytes, n, lib.MEM_HOST, offsets=off, lens=lens),
+                            lib.make_batch(got_out, total + 16, n, lib.MEM_HOST, offsets=out_off),
+                            t0, res, olen, gp, gc)
+        got_out = np.array(got_out)
+        for r in rings:
+            ctx.ring_free(r)
+    assert np.array_equal(res, want[:, 0].astype(np.uint8))
+    assert np.array_equal(olen, want[:, 1].astype(np.uint32))
+    assert np.array_equal(gp, want[:, 2].astype(np.uint32))
+    assert np.array_equal(gc, want[:, 3])
+    assert ctx.filter_flows() == ora.flows()
+
+    # the library's own two calls leave the same plaintexts and the same table
+    ctx2 = fresh_ctx()
+    out2 = np.full(total + 16, 0x77, np.uint8)
+    r2, l2 = np.zeros(n, np.uint8), np.zeros(n, np.uint32)
+    p2, c2 = np.zeros(n, np.uint32), np.zeros(n, np.uint64)
+    ctx2.wg_decap(lib.make_batch(arena, arena.nbytes, n, lib.MEM_HOST, offsets=off, lens=lens),
+                  lib.make_batch(out2, out2.nbytes, n, lib.MEM_HOST, offsets=out_off), r2, l2, p2, c2)
+    v2 = np.zeros(n, np.uint8)
+    ctx2.filter_check_inbound(lib.make_batch(out2, out2.nbytes, n, lib.MEM_HOST, offsets=out_off, lens=l2), t0, v2)
+    assert np.array_equal(got_out, out2)
+    assert np.array_equal(np.where((r2 == 0) & (v2 == 0), 7, r2), res)
+    assert ctx2.filter_flows() == ctx.filter_flows()
+    # allow-all: nothing is filtered
+    ctx2.filter_set_allow_all()
+    ctx2.wg_decap_filter(lib.make_batch(arena, arena.nbytes, n, lib.MEM_HOST, offsets=off, lens=lens),
+                         lib.make_batch(out2, out2.nbytes, n, lib.MEM_HOST, offsets=out_off), t0, r2, l2, p2, c2)
+    assert not (r2 == 7).any() and np.array_equal(r2 == 0, np.isin(res, (0, 7)))
+    ctx.close()
+    ctx2.close()
+
+
+@pytest.mark.parametrize("mem", ["host", "ring"])
+@pytest.mark.parametrize("n", [900, 3000])
+def test_note_outbound_and_encap_in_one_call(mem, n):
+    """bnk_wg_note_encap_batch = NoteOutbound with one `now` on every
+    plaintext, then encapsulate: the datagrams of bnk_wg_encap_batch and the
+    flow table of bnk_filter_note_outbound_batch, both against the oracle."""
+    from bnk_amd import lib
+    from oracle import binding as O
+    rng = np.random.default_rng(5 + n)
+    peers = _peers(rng)
+    keys = rng.integers(0, 256, (N_PEERS, 32), dtype=np.uint8)
+    t0 = 1_700_000_000 * 10**9
+    local = 0x64700001
+    peer = rng.integers(0, N_PEERS, n).astype(np.uint32)
+    plains = []
+    for i in range(n):
+        dst = peers[int(peer[i])][2]
+        kind = i % 5
+        if kind == 0:
+            plains.append(W.tcp(local, dst, 30000 + (i % 2000), 443))
+        elif kind == 1:
+            plains.append(W.udp(local, dst, 30000 + (i % 500), 53))
+        elif kind == 2:
+            plains.append(W.icmp_echo(local, dst))
+        elif kind == 3:
+            plains.append(bytes(int(rng.integers(0, 19))))       # too short to be noted
+        else:
+            plains.append(W.tcp(local, dst, 1234, 80) + bytes(int(rng.integers(0, 600))))
+    lens = np.array([len(p) for p in plains], np.uint32)
+    room = 16 + lens.astype(np.int64) + 15 + 16
+    off, total = _layout(rng, room)
+    arena = np.full(total, 0xEE, np.uint8)
+    for i, pt in enumerate(plains):
+        arena[int(off[i]) + 16:int(off[i]) + 16 + len(pt)] = np.frombuffer(pt, np.uint8)
+    ora = O.Filter()
+    ora.set_rules([])
+    want = arena.copy()
+    want_len = np.zeros(n, np.uint32)
+    next_ctr = np.zeros(N_PEERS, np.uint64)
+    for i, pt in enumerate(plains):
+        ora.note_outbound(pt, t0)
+        p = int(peer[i])
+        w = O.wg_encap(pt, MTU, keys[p].tobytes(), peers[p][1], int(next_ctr[p]))
+        next_ctr[p] += 1
+        want[int(off[i]):int(off[i]) + len(w)] = np.frombuffer(w, np.uint8)
+        want_len[i] = len(w)
+    ctx = _ctx(peers, keys_send=keys)
+    ctx.filter_set_rules([])
+    ring = ctx.ring_alloc(total) if mem == "ring" else None
+    got = ring if mem == "ring" else arena.copy()
+    got[:] = arena
+    got_len = np.zeros(n, np.uint32)
+    ctx.wg_note_encap(lib.make_batch(got, total, n, lib.MEM_HOST, offsets=off, lens=lens, peer=peer), MTU, t0, got_len)
+    assert np.array_equal(got_len, want_len)
+    assert np.array_equal(np.array(got), want)
+    assert ctx.filter_flows() == ora.flows() and ora.flow_count() > n // 4
+    if ring is not None:
+        ctx.ring_free(ring)
+    ctx.close()
+
+
 def test_encap_then_decap_round_trip_full_size():
     """2^20 MTU-sized slots, device resident: every datagram decapsulates to
     its plaintext under the mirrored peer table, counters are each peer's

@@ -361,6 +361,51 @@ def test_small_batches_in_pinned_rings(small_ctx, layout, n):
             ctx.ring_free(r)
 
 
+def test_random_shapes_through_pinned_rings(ctx):
+    """Three hundred batches of random size (1 to 5000 packets), length mix,
+    alignment and kernel choice, one after the other through the same rings
+    and the same context: every sealed byte and every gap against the oracle,
+    every packet back."""
+    from bnk_amd import lib
+    from oracle import binding as O
+    rng = np.random.default_rng(2026)
+    n_keys = 9
+    keys = rng.integers(0, 256, (n_keys, 32), dtype=np.uint8)
+    ctx.keys_set(lib.KEYS_SEND, keys)
+    ctx.keys_set(lib.KEYS_RECV, keys)
+    rings = [ctx.ring_alloc(9 << 20) for _ in range(3)]
+    try:
+        for it in range(300):
+            n = int(rng.choice([1, 2, 63, 64, 65, 128, 500, 1024, 3000, 5000]))
+            lens = rng.integers(0, int(rng.choice([64, 200, 1500])) + 1, n).astype(np.uint32)
+            room = ((lens.astype(np.int64) + 16 + 15) & ~15) + 16
+            gaps = rng.integers(0, 16, n) if rng.integers(0, 2) else np.zeros(n, np.int64)
+            off = (np.concatenate([[0], np.cumsum(room)[:-1]]) + gaps).astype(np.uint64)
+            total = int(room.sum()) + 16
+            ctx.set_spread_max_packets(int(rng.choice([0, 4096])))
+            plain = rng.integers(0, 256, total, dtype=np.uint8)
+            peer = rng.integers(0, n_keys, n).astype(np.uint32)
+            counters = rng.integers(0, 1 << 63, n, dtype=np.uint64)
+            want = np.full(total, 0x5A, np.uint8)
+            O.seal_batch(keys, peer, counters, plain, off, lens, want, off, 4)
+            a, b, c = (r[:total] for r in rings)
+            a[:] = plain
+            b[:] = 0x5A
+            c[:] = 0xEE
+            ctx.seal(lib.make_batch(a, total, n, lib.MEM_HOST, offsets=off, lens=lens, peer=peer, counters=counters),
+                     lib.make_batch(b, total, n, lib.MEM_HOST, offsets=off))
+            assert np.array_equal(b, want), f"batch {it}: {n} packets"
+            verdict = np.zeros(n, np.uint8)
+            ctx.open(lib.make_batch(b, total, n, lib.MEM_HOST, offsets=off, lens=(lens + 16).astype(np.uint32),
+                                    peer=peer, counters=counters),
+                     lib.make_batch(c, total, n, lib.MEM_HOST, offsets=off), verdict)
+            assert verdict.all() and _packets_equal(c, plain, off, lens) == -1, f"batch {it}: {n} packets"
+    finally:
+        ctx.set_spread_max_packets(4096)
+        for r in rings:
+            ctx.ring_free(r)
+
+
 def test_in_place_and_unaligned_slots(small_ctx):
     ctx = small_ctx
     """WireGuard seals in place at offset 16 of its buffers; slots need not be

@@ -441,7 +441,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const uint4 *kp = reinterpret_cast<const uint4 *>(a.keys + 8u * (bad_peer ? 0u : pr));
     const uint4 k0 = kp[0], k1 = kp[1];
     if (in_batch && !skipped && (bad_peer || too_short)) {
-        if (bad_peer) atomicOr(a.status, STATUS_PEER_RANGE);
+        if (bad_peer) status_raise(a.status, STATUS_PEER_RANGE);
         if (OPEN) a.verdict[i] = 0;
     }
     if (OPEN) len -= 16u;
@@ -502,7 +502,7 @@ __global__ __launch_bounds__(256) void aead_spread_kernel(AeadArgs a)
         if (a.skip && a.skip[i] != 0) return;
         if (pr >= a.n_peers) {
             if (lane == 0) {
-                atomicOr(a.status, STATUS_PEER_RANGE);
+                status_raise(a.status, STATUS_PEER_RANGE);
                 if (OPEN) a.verdict[i] = 0;
             }
             return;

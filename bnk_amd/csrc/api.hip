@@ -258,13 +258,16 @@ int aead_batch(bnk_ctx *ctx, bool open, const bnk_batch *in, const bnk_batch *ou
 
 namespace bnk {
 
-// Reads and clears the device status word; the stream must be idle.
+// Waits for the stream, then reads and clears the status words.
 int take_status(bnk_ctx *ctx, uint32_t *status)
 {
-    HIPCHK(ctx, hipMemcpyAsync(ctx->h_status, ctx->d_status, 4, hipMemcpyDeviceToHost, ctx->stream));
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
-    *status = *ctx->h_status;
-    if (*status) HIPCHK(ctx, launch_fill_u32(ctx->d_status, 1, 0, ctx->stream));
+    volatile uint32_t *h = ctx->h_status;
+    *status = (h[STATUS_PEER_RANGE] ? STATUS_PEER_RANGE : 0u) | (h[STATUS_FLOWS_FULL] ? STATUS_FLOWS_FULL : 0u);
+    if (*status) {
+        h[STATUS_PEER_RANGE] = 0;
+        h[STATUS_FLOWS_FULL] = 0;
+    }
     return BNK_OK;
 }
 
@@ -310,11 +313,11 @@ int bnk_init(int device_ordinal, bnk_ctx **out)
         return bail("hipStreamCreate", e);
     if ((e = hipEventCreate(&ctx->ev0)) != hipSuccess) return bail("hipEventCreate", e);
     if ((e = hipEventCreate(&ctx->ev1)) != hipSuccess) return bail("hipEventCreate", e);
-    if ((e = hipMalloc((void **)&ctx->d_status, 256)) != hipSuccess) return bail("hipMalloc", e);
     if ((e = hipHostMalloc((void **)&ctx->h_status, 64, hipHostMallocDefault)) != hipSuccess)
         return bail("hipHostMalloc", e);
-    if ((e = launch_fill_u32(ctx->d_status, 64, 0, ctx->stream)) != hipSuccess)
-        return bail("status clear", e);
+    memset(ctx->h_status, 0, 64);
+    if ((e = hipHostGetDevicePointer((void **)&ctx->d_status, ctx->h_status, 0)) != hipSuccess)
+        return bail("hipHostGetDevicePointer", e);
     ctx->filter = filter_create(ctx->stream, prop.multiProcessorCount);
     if (!ctx->filter) return bail("filter state", hipErrorOutOfMemory);
     if ((e = hipStreamSynchronize(ctx->stream)) != hipSuccess) return bail("hipStreamSynchronize", e);
@@ -344,7 +347,6 @@ void bnk_shutdown(bnk_ctx *ctx)
         ctx->pin.release();
         for (int w = 0; w < 2; w++)
             if (ctx->d_keys[w]) (void)hipFree(ctx->d_keys[w]);
-        if (ctx->d_status) (void)hipFree(ctx->d_status);
         if (ctx->h_status) (void)hipHostFree(ctx->h_status);
         if (ctx->filter) filter_destroy(ctx->filter);
         for (hipEvent_t e : ctx->ev_up) (void)hipEventDestroy(e);

@@ -96,7 +96,7 @@ struct bnk_ctx {
 
     uint32_t *d_keys[2] = {nullptr, nullptr};
     uint32_t n_keys[2] = {0, 0};
-    uint32_t *d_status = nullptr; // one word, see STATUS_*
+    uint32_t *d_status = nullptr; // the device's address of h_status, see STATUS_*
 
     // staging for BNK_MEM_HOST batches and scratch for the length sort
     bnk::DevBuf in_arena, out_arena, off_in, off_out, lens, peer, counters, verdict;
@@ -106,7 +106,7 @@ struct bnk_ctx {
     // them in place (small host batches skip the copies).
     struct Ring { uintptr_t host; uint8_t *dev; size_t bytes; };
     std::vector<Ring> rings;
-    uint32_t *h_status = nullptr; // pinned landing word for d_status
+    uint32_t *h_status = nullptr; // pinned status words the kernels write
     uint32_t spread_max = bnk::SPREAD_MAX_PACKETS; // see AeadArgs::spread_max
     // fused relay: plaintext scratch, per-packet flags, sort buffers, staged arrays
     bnk::DevBuf r_plain, r_auth, r_pass, r_keys, r_idx, r_skeys, r_sidx, r_tmp;

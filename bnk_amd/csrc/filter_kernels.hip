@@ -380,7 +380,7 @@ __global__ __launch_bounds__(256) void filter_note_kernel(FilterArgs a)
                 break;
             }
         }
-        if (!placed) atomicOr(a.status, STATUS_FLOWS_FULL);
+        if (!placed) status_raise(a.status, STATUS_FLOWS_FULL);
     }
 }
 
@@ -438,7 +438,7 @@ __global__ __launch_bounds__(256) void flow_rehash_kernel(FlowTableDev from, Flo
                 break;
             }
         }
-        if (!placed) atomicOr(status, STATUS_FLOWS_FULL);
+        if (!placed) status_raise(status, STATUS_FLOWS_FULL);
     }
 }
 

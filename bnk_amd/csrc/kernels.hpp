@@ -69,7 +69,19 @@ struct AeadArgs {
 // packet (which needs 64 packets per wave and about 130 000 to fill the chip).
 constexpr uint32_t SPREAD_MAX_PACKETS = 4096;
 
+// What kernels report besides their results.  The status words live in pinned
+// host memory that the GPU can write: one word per condition, raised with a
+// plain store of 1 (the same store from every lane that has the news, so no
+// atomic is needed), and read by the host after it has waited for the stream,
+// with no copy.
 enum : uint32_t { STATUS_PEER_RANGE = 1u, STATUS_FLOWS_FULL = 2u };
+constexpr uint32_t STATUS_WORDS = 4; // word [bit value] holds that condition
+#if defined(__HIPCC__)
+__device__ inline void status_raise(uint32_t *status, uint32_t condition)
+{
+    __hip_atomic_store(&status[condition], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+#endif
 
 // True when the launch will run one wave per packet (then order[] is not used
 // and callers need not build it).

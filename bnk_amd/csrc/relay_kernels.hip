@@ -30,7 +30,7 @@ __global__ __launch_bounds__(256) void relay_verdict_kernel(
     if (v == BNK_RELAY_OK) {
         key = peer_out[i];
         if (key >= n_peers_out) {
-            atomicOr(status, STATUS_PEER_RANGE);
+            status_raise(status, STATUS_PEER_RANGE);
             v = BNK_RELAY_DENIED;
             key = NO_PEER;
         }
@@ -146,7 +146,7 @@ __global__ __launch_bounds__(PEER_RANK_SMALL_MAX) void peer_rank_small_kernel(
     if (t < n) {
         key[0] = peer ? peer[t] : 0u;
         if (key[0] >= n_keys) {
-            if (!(no_peer_ok && key[0] == NO_PEER)) atomicOr(status, STATUS_PEER_RANGE);
+            if (!(no_peer_ok && key[0] == NO_PEER)) status_raise(status, STATUS_PEER_RANGE);
             key[0] = NO_PEER;
         }
     }

@@ -132,7 +132,7 @@ __global__ __launch_bounds__(256) void wg_keys_kernel(const uint32_t *peer, uint
     if (i >= n) return;
     uint32_t k = peer ? peer[i] : 0u;
     if (k >= n_peers) {
-        atomicOr(status, 1u); // STATUS_PEER_RANGE
+        status_raise(status, STATUS_PEER_RANGE);
         k = 0xFFFFFFFFu;
     }
     keys[i] = k;

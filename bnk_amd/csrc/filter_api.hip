@@ -190,7 +190,7 @@ int run_staged(bnk_ctx *ctx, bool check, FilterArgs &a, uint8_t *h_verdict, uint
 {
     FilterState *f = ctx->filter;
     if (!check) {
-        HIPCHK(ctx, launch_filter_note(a, f->max_blocks, ctx->stream));
+        HIPCHK(ctx, launch_filter_note(a, f->max_blocks, f->claimed_upper > 4096, ctx->stream));
     } else if (h_verdict) {
         // CheckInbound reports nothing through the status word
         a.verdict = ctx->pin.dev(h_verdict);
@@ -259,7 +259,7 @@ int filter_batch(bnk_ctx *ctx, bool check, const bnk_batch *pkts, int64_t now_ns
         a.len = pkts->len;
         a.verdict = verdict;
         HIPCHK(ctx, check ? launch_filter_check(a, f->max_blocks, ctx->stream)
-                          : launch_filter_note(a, f->max_blocks, ctx->stream));
+                          : launch_filter_note(a, f->max_blocks, f->claimed_upper > 4096, ctx->stream));
         return BNK_OK;
     }
     Span span;

@@ -81,7 +81,10 @@ hipError_t launch_flow_clear(FlowSlotMem *p, uint32_t n, hipStream_t s);
 hipError_t launch_fill_u8(uint8_t *p, uint32_t n, uint8_t v, hipStream_t s);
 hipError_t launch_filter_check(const FilterArgs &a, uint32_t max_blocks, hipStream_t s);
 // inserts, then the reference's conditional expiry sweep
-hipError_t launch_filter_note(const FilterArgs &a, uint32_t max_blocks, hipStream_t s);
+// may_sweep: the table may hold more than 4096 entries after this batch (the
+// host's upper bound on claimed slots says so); otherwise the expiry sweep
+// cannot fire and its two launches are left out.
+hipError_t launch_filter_note(const FilterArgs &a, uint32_t max_blocks, bool may_sweep, hipStream_t s);
 hipError_t launch_flow_rehash(const FlowTableDev &from, const FlowTableDev &to, uint32_t *status,
                               uint32_t max_blocks, hipStream_t s);
 

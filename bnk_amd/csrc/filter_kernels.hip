@@ -516,10 +516,12 @@ hipError_t launch_filter_check(const FilterArgs &args, uint32_t max_blocks, hipS
     return hipGetLastError();
 }
 
-hipError_t launch_filter_note(const FilterArgs &a, uint32_t max_blocks, hipStream_t s)
+hipError_t launch_filter_note(const FilterArgs &a, uint32_t max_blocks, bool may_sweep, hipStream_t s)
 {
     if (a.n == 0) return hipSuccess;
     hipLaunchKernelGGL(filter_note_kernel, dim3(grid_for(a.n, max_blocks)), dim3(256), 0, s, a);
+    // filter.go:202: no sweep while the map holds at most 4096 entries
+    if (!may_sweep) return hipGetLastError();
     hipLaunchKernelGGL(flow_sweep_flag_kernel, dim3(1), dim3(64), 0, s, a.flows);
     hipLaunchKernelGGL(flow_sweep_kernel, dim3(grid_for(a.flows.cap * FLOW_REGIONS, max_blocks)),
                        dim3(256), 0, s, a.flows, a.now);

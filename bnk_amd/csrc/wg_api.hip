@@ -264,7 +264,7 @@ static int wg_encap_impl(bnk_ctx *ctx, const bnk_batch *slots, uint32_t mtu, uin
             fa.n = hi - lo;
             fa.rules = f->ridx;
             fa.flows = f->flows;
-            HIPCHK(ctx, launch_filter_note(fa, f->max_blocks, ctx->stream));
+            HIPCHK(ctx, launch_filter_note(fa, f->max_blocks, f->claimed_upper > 4096, ctx->stream));
         }
         if (fits) {
             AeadArgs se{};

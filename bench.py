@@ -485,7 +485,7 @@ def bench_latency(args) -> dict:
         b_so = lib.make_batch(sealed, nbytes, n, lib.MEM_HOST, stride=STRIDE)
         b_si = lib.make_batch(sealed, nbytes, n, lib.MEM_HOST, stride=STRIDE, length=L + 16)
         b_op = lib.make_batch(opened, nbytes, n, lib.MEM_HOST, stride=STRIDE)
-        t = {"seal": [], "open": [], "filter": []}
+        t = {"seal": [], "open": [], "filter": [], "note": []}
         for it in range(reps + 5):
             t0 = time.perf_counter()
             ctx.seal(b_plain, b_so)
@@ -494,10 +494,13 @@ def bench_latency(args) -> dict:
             t2 = time.perf_counter()
             ctx.filter_check_inbound(b_plain, 1_700_000_000_000_000_000, v)
             t3 = time.perf_counter()
+            ctx.filter_note_outbound(b_plain, 1_700_000_000_000_000_000)
+            t4 = time.perf_counter()
             if it >= 5:
                 t["seal"].append(t1 - t0)
                 t["open"].append(t2 - t1)
                 t["filter"].append(t3 - t2)
+                t["note"].append(t4 - t3)
         out[str(n)] = {k: round(float(np.median(x)) * 1e6, 1) for k, x in t.items()}
         for r in (plain, sealed, opened):
             ctx.ring_free(r)

@@ -239,6 +239,7 @@ struct HostPipe {
     Span sin, sout;
     bool in_place = false;
     uint64_t row_width = 0; // > 0: the output comes back row by row (uniform layout, see plan)
+    uint32_t max_chunks = PIPE_MAX_CHUNKS;
     uint8_t *d_in = nullptr, *d_out = nullptr;
     const uint64_t *d_in_off = nullptr, *d_out_off = nullptr;
 
@@ -276,7 +277,7 @@ struct HostPipe {
             sout.add(oo, oo + oe);
         }
         const uint32_t by_bytes =
-            (uint32_t)std::min<uint64_t>(std::max(sin.size(), sout.size()) / PIPE_MIN_CHUNK_BYTES, PIPE_MAX_CHUNKS);
+            (uint32_t)std::min<uint64_t>(std::max(sin.size(), sout.size()) / PIPE_MIN_CHUNK_BYTES, max_chunks);
         if (by_bytes < 2 || n < 2u * 64u) return 1;
         chunks = by_bytes;
         per = ((n + chunks - 1u) / chunks + 63u) & ~63u; // whole waves per chunk

@@ -103,12 +103,14 @@ hipError_t launch_fill_u32(uint32_t *p, uint32_t n, uint32_t v, hipStream_t s);
 // Fused relay bookkeeping (relay_kernels.hip).  After open (auth[i]) and the
 // filter (pass[i]): verdicts, then per-peer batch-order counters for the
 // survivors.  sort_tmp holds sort_tmp_bytes of scratch (relay_sort_tmp_bytes).
+// With advance set, ctr_base_out (then writable) moves past the counters
+// handed out, so that the next part of the same batch continues them.
 size_t relay_sort_tmp_bytes(uint32_t n, uint32_t n_keys);
 hipError_t launch_relay_assign(const uint8_t *auth, const uint8_t *pass, const uint32_t *peer_out,
                                const uint64_t *ctr_base_out, uint32_t n_peers_out, uint32_t n,
                                uint32_t *keys, uint32_t *idx, uint32_t *skeys, uint32_t *sidx,
                                void *sort_tmp, size_t sort_tmp_bytes, uint8_t *verdict,
-                               uint64_t *ctr_out, uint32_t *status, hipStream_t s);
+                               uint64_t *ctr_out, uint32_t *status, bool advance, hipStream_t s);
 
 // Batch-order counters per peer: ctr_out[i] = ctr_base[keys[i]] + (number of
 // earlier i' with the same key), for keys[i] < n_keys; other keys must be

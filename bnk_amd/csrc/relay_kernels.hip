@@ -109,7 +109,7 @@ hipError_t launch_relay_assign(const uint8_t *auth, const uint8_t *pass, const u
                                const uint64_t *ctr_base_out, uint32_t n_peers_out, uint32_t n,
                                uint32_t *keys, uint32_t *idx, uint32_t *skeys, uint32_t *sidx,
                                void *sort_tmp, size_t sort_tmp_bytes, uint8_t *verdict,
-                               uint64_t *ctr_out, uint32_t *status, hipStream_t s)
+                               uint64_t *ctr_out, uint32_t *status, bool advance, hipStream_t s)
 {
     if (n == 0) return hipSuccess;
     const dim3 grid((n + 255u) / 256u);
@@ -118,11 +118,12 @@ hipError_t launch_relay_assign(const uint8_t *auth, const uint8_t *pass, const u
     if (n <= PEER_RANK_SMALL_MAX) {
         // keys[] is the peer of each survivor and all ones for the rest
         hipLaunchKernelGGL(peer_rank_small_kernel, dim3(1), dim3(PEER_RANK_SMALL_MAX), 0, s, keys, n_peers_out,
-                           n, const_cast<uint64_t *>(ctr_base_out), ctr_out, 0, 1, key_bits(n_peers_out), status);
+                           n, const_cast<uint64_t *>(ctr_base_out), ctr_out, advance ? 1 : 0, 1,
+                           key_bits(n_peers_out), status);
         return hipGetLastError();
     }
     return launch_peer_rank(keys, idx, skeys, sidx, sort_tmp, sort_tmp_bytes,
-                            const_cast<uint64_t *>(ctr_base_out), n_peers_out, n, ctr_out, false, s);
+                            const_cast<uint64_t *>(ctr_base_out), n_peers_out, n, ctr_out, advance, s);
 }
 
 // Batch-order counters for a small batch in one launch of one block, straight

@@ -20,11 +20,13 @@ def _note(ctx, ora, w):
 
 
 @pytest.mark.parametrize("mem", ["host", "ring"])
-@pytest.mark.parametrize("n", [12000, 900])
+@pytest.mark.parametrize("n", [12000, 900, 40000])
 def test_relay_matches_oracle_host_path(mem, n):
     """"ring": both arenas lie in pinned rings of the context, which batches of
     a few megabytes relay in place without staging copies.  900 packets also
-    take the wave-per-packet kernels and the one-launch counter assignment."""
+    take the wave-per-packet kernels and the one-launch counter assignment;
+    40000 (14 MB) go through in overlapped chunks, each continuing the
+    counters of the one before."""
     from bnk_amd import lib
     from oracle import binding as O
     w = W.relay_workload(n=n, n_peers=64, n_rules=512)

@@ -601,15 +601,22 @@ def test_concurrent_callers_share_one_context(ctx):
     errors = []
 
     def worker(tid):
+        rings = []
         try:
+            # odd threads keep their packets in pinned rings of the shared context
+            # (allocated, used in place and freed while the others are calling)
+            if tid % 2:
+                rings = [ctx.ring_alloc(b0.plain.nbytes) for _ in range(2)]
             for it in range(6):
-                out = np.zeros_like(b0.plain)
+                out = rings[0] if rings else np.zeros_like(b0.plain)
+                out[:] = 0
                 ctx.seal(lib.make_batch(b0.plain, b0.plain.nbytes, b0.n, lib.MEM_HOST, offsets=b0.off,
                                         lens=b0.lens, peer=b0.peer, counters=b0.counters),
                          lib.make_batch(out, out.nbytes, b0.n, lib.MEM_HOST, offsets=b0.off))
                 if not np.array_equal(out, want):
                     errors.append((tid, it, "seal"))
-                back = np.zeros_like(b0.plain)
+                back = rings[1] if rings else np.zeros_like(b0.plain)
+                back[:] = 0
                 v = np.zeros(b0.n, np.uint8)
                 ctx.open(lib.make_batch(out, out.nbytes, b0.n, lib.MEM_HOST, offsets=b0.off,
                                         lens=(b0.lens + 16).astype(np.uint32), peer=b0.peer,
@@ -619,6 +626,9 @@ def test_concurrent_callers_share_one_context(ctx):
                     errors.append((tid, it, "open"))
         except Exception as e:  # noqa: BLE001
             errors.append((tid, repr(e)))
+        finally:
+            for r in rings:
+                ctx.ring_free(r)
 
     threads = [threading.Thread(target=worker, args=(t,)) for t in range(6)]
     for t in threads:

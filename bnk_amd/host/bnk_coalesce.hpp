@@ -7,6 +7,12 @@
 // leader, waits until the window is full or its time is up, runs one batch for
 // everyone and hands each caller its own verdicts.  No background thread.
 //
+// A caller that has been alone lately should not pay the whole window for
+// company that is not coming: when the previous window held a single call, the
+// next leader waits only solo_wait (SetSoloWait; by default the full window).
+// A follower that turns up within that time is merged as usual and restores
+// the full window for the next round.
+//
 // What changes against calling the filter directly: the packets of one window
 // share one `now` (the leader's clock at flush time, at most max_wait later
 // than a caller's own), and NoteOutbound calls of a window are applied before
@@ -42,8 +48,15 @@ public:
     BatchCoalescer(Executor exec, size_t max_packets, std::chrono::microseconds max_wait,
                    Clock clock = nullptr)
         : exec_(std::move(exec)), max_packets_(max_packets ? max_packets : 1), max_wait_(max_wait),
-          clock_(std::move(clock))
+          solo_wait_(max_wait), clock_(std::move(clock))
     {
+    }
+
+    // How long a leader waits when the window before its own held one call only.
+    void SetSoloWait(std::chrono::microseconds solo_wait)
+    {
+        std::lock_guard<std::mutex> lk(mu_);
+        solo_wait_ = solo_wait < max_wait_ ? solo_wait : max_wait_;
     }
 
     // Blocks until the window this call joined has run.  verdict may be null
@@ -59,6 +72,7 @@ public:
         w->ptrs.insert(w->ptrs.end(), ptrs, ptrs + n);
         w->lens.insert(w->lens.end(), lens, lens + n);
         w->note.insert(w->note.end(), n, note ? 1 : 0);
+        w->callers++;
         stats_.calls++;
         stats_.packets += n;
         if (w->ptrs.size() >= max_packets_) {
@@ -68,8 +82,9 @@ public:
             w->cv.notify_all();
         }
         if (leader) {
-            w->cv.wait_for(lk, max_wait_, [&] { return w->full; });
+            w->cv.wait_for(lk, last_callers_ >= 2 ? max_wait_ : solo_wait_, [&] { return w->full; });
             if (open_ == w) open_.reset();
+            last_callers_ = w->callers;
             if (w->full) stats_.full_flushes++;
             stats_.batches++;
             if (w->ptrs.size() > stats_.largest_batch) stats_.largest_batch = w->ptrs.size();
@@ -110,6 +125,7 @@ private:
         std::vector<const uint8_t *> ptrs;
         std::vector<uint32_t> lens;
         std::vector<uint8_t> note, verdict;
+        uint32_t callers = 0;
         bool full = false, done = false;
         std::exception_ptr error;
         std::condition_variable cv;
@@ -118,6 +134,8 @@ private:
     Executor exec_;
     const size_t max_packets_;
     const std::chrono::microseconds max_wait_;
+    std::chrono::microseconds solo_wait_;
+    uint32_t last_callers_ = 2; // the first window waits in full
     Clock clock_;
     std::mutex mu_;
     std::shared_ptr<Window> open_;

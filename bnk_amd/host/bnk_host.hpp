@@ -193,15 +193,19 @@ private:
 // A Filter behind a BatchCoalescer: calls from many threads (one per peer in
 // wireguard-go) that arrive within max_wait of each other become one GPU
 // batch.  The `now_ns` arguments are ignored: a merged batch takes the clock
-// when it is flushed.
+// when it is flushed.  A caller that was alone in the previous window waits
+// only solo_wait for company (a call by itself costs about 20 us, so a lone
+// peer should not pay a 200 us window on every write).
 class CoalescedFilter : public PacketFilter {
 public:
     CoalescedFilter(Filter *f, size_t max_packets = 8192,
-                    std::chrono::microseconds max_wait = std::chrono::microseconds(200))
+                    std::chrono::microseconds max_wait = std::chrono::microseconds(200),
+                    std::chrono::microseconds solo_wait = std::chrono::microseconds(10))
         : f_(f), co_([this](const uint8_t *const *ptrs, const uint32_t *lens, const uint8_t *note,
                             uint32_t n, int64_t now, uint8_t *verdict) { Run(ptrs, lens, note, n, now, verdict); },
                      max_packets, max_wait)
     {
+        co_.SetSoloWait(solo_wait);
     }
     bool CheckInbound(ByteSlice pkt)
     {

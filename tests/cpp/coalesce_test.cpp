@@ -94,6 +94,48 @@ static void lone_caller_waits_at_most_the_window()
     EXPECT(full.Stats().full_flushes == 1, "counted as a full flush");
 }
 
+static void lone_callers_stop_waiting_for_company()
+{
+    std::atomic<uint64_t> execs{0};
+    BatchCoalescer co([&](const uint8_t *const *, const uint32_t *, const uint8_t *, uint32_t n, int64_t,
+                          uint8_t *v) { execs++; for (uint32_t i = 0; i < n; i++) v[i] = 1; },
+                      1000, microseconds(40000));
+    co.SetSoloWait(microseconds(200));
+    uint8_t pkt[1] = {0};
+    const uint8_t *p = pkt;
+    const uint32_t len = 1;
+    uint8_t v = 0;
+    auto timed = [&] {
+        const auto t0 = steady_clock::now();
+        co.Submit(&p, &len, 1, false, &v);
+        return std::chrono::duration_cast<microseconds>(steady_clock::now() - t0).count();
+    };
+    const auto first = timed();  // nothing is known yet: the full window
+    const auto second = timed(); // the window before held one call
+    const auto third = timed();
+    EXPECT(first >= 35000, "the first window waits in full");
+    EXPECT(second < 20000 && third < 20000, "a caller that was alone waits the short time only");
+    // two callers at once: the follower is merged, and the next window waits in full again
+    std::thread other([&] {
+        uint8_t q[1] = {1};
+        const uint8_t *qp = q;
+        uint8_t qv = 0;
+        std::this_thread::sleep_for(microseconds(5000));
+        co.Submit(&qp, &len, 1, false, &qv);
+    });
+    BatchCoalescer *c = &co;
+    c->SetSoloWait(microseconds(39000)); // long enough for the other thread to turn up
+    const uint64_t before = execs;
+    (void)timed();
+    other.join();
+    EXPECT(execs == before + 1, "the follower rode the leader's window");
+    c->SetSoloWait(microseconds(200));
+    const auto after_pair = timed();
+    EXPECT(after_pair >= 35000, "after a shared window the next one waits in full");
+    const auto alone_again = timed();
+    EXPECT(alone_again < 20000, "and alone again it does not");
+}
+
 static void failures_reach_every_caller()
 {
     BatchCoalescer co([](const uint8_t *const *, const uint32_t *, const uint8_t *, uint32_t, int64_t,
@@ -121,6 +163,7 @@ int main()
 {
     many_threads_get_their_own_verdicts();
     lone_caller_waits_at_most_the_window();
+    lone_callers_stop_waiting_for_company();
     failures_reach_every_caller();
     if (failures) {
         printf("%d failure(s)\n", failures);

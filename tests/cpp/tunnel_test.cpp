@@ -133,7 +133,7 @@ int main()
     // A socket buffer holds a few hundred datagrams at most: send in rounds and
     // drain each round before the next.
     constexpr uint32_t ROUND = 25; // datagrams per spoke per round
-    uint32_t total = 0, batches = 0, sent_so_far = 0, next_seq = 0;
+    uint32_t total = 0, batches = 0, sent_so_far = 0, next_seq = 0, last_batch = 0;
     while (total < N) {
         if (total == sent_so_far && next_seq < PER_SPOKE) {
             const uint32_t upto = next_seq + ROUND < PER_SPOKE ? next_seq + ROUND : PER_SPOKE;
@@ -185,6 +185,7 @@ int main()
             delivered.insert({sp, seq});
         }
         total += k;
+        last_batch = k;
     }
     EXPECT(total == N && delivered.size() == N, "every packet delivered exactly once");
     // a replayed datagram still authenticates and is then refused by the window
@@ -205,6 +206,45 @@ int main()
                                 counter.data()));
         EXPECT(result[0] == BNK_WG_OK, "the replayed datagram is authentic");
         EXPECT(!replay[by_index[0]].ValidateCounter(counter[0]), "and the window refuses it");
+    }
+    // the receive path with the inbound filter in the same call: the hub admits
+    // UDP from the even spokes only; the last batch is still in the ring
+    {
+        std::vector<bnk_rule> rules;
+        for (uint32_t sp = 0; sp < SPOKES; sp += 2) {
+            bnk_rule r{};
+            r.src_net = 0x64400001u + sp;
+            r.src_mask = 0xFFFFFFFFu;
+            r.port_first = 0;
+            r.port_last = 65535;
+            r.proto = 17;
+            rules.push_back(r);
+        }
+        MUST(bnk_filter_set_rules(rx, rules.data(), (uint32_t)rules.size()));
+        const uint32_t k = last_batch;
+        bnk_batch wire{}, out{};
+        wire.base = recv_ring;
+        wire.bytes = ring.bytes;
+        wire.n = k;
+        wire.mem = BNK_MEM_HOST;
+        wire.stride = STRIDE;
+        wire.lens = sizes.data();
+        out.base = plain_ring + 16;
+        out.bytes = ring.bytes - 16;
+        out.n = k;
+        out.mem = BNK_MEM_HOST;
+        out.stride = STRIDE;
+        MUST(bnk_wg_decap_filter_batch(rx, &wire, &out, 1700000000000000000LL, result.data(), out_len.data(),
+                                       by_index.data(), counter.data()));
+        uint32_t passed = 0, filtered = 0;
+        for (uint32_t i = 0; i < k; i++) {
+            const bool even = (by_index[i] & 1u) == 0;
+            EXPECT(result[i] == (even ? BNK_WG_OK : BNK_WG_FILTERED), "the filter admits the even spokes only");
+            passed += result[i] == BNK_WG_OK;
+            filtered += result[i] == BNK_WG_FILTERED;
+        }
+        EXPECT(k > 0 && passed > 0 && filtered > 0, "both kinds occurred");
+        MUST(bnk_filter_set_allow_all(rx));
     }
     printf("%u datagrams in %u receive batches\n", total, batches);
     bnk_ring_free(tx, send_ring);

@@ -139,6 +139,47 @@ def test_encap_matches_oracle(mem, misalign, n, fused):
     ctx.close()
 
 
+@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("length,mtu", [(100, 1420), (1500, 1420), (1413, 1420), (37, 0), (0, 1420), (2839, 1420)])
+def test_encap_uniform_slots_one_peer_and_padding_rules(fused, length, mtu):
+    """Uniform slots without length or peer arrays (everything goes to peer 0),
+    and the padding rule at its corners: a packet longer than the MTU pads its
+    remainder, one just below the MTU pads up to it and no further, mtu 0 means
+    no cap, an empty packet is a keepalive."""
+    from bnk_amd import lib
+    from oracle import binding as O
+    rng = np.random.default_rng(length * 7 + mtu)
+    peers = _peers(rng)
+    keys = rng.integers(0, 256, (N_PEERS, 32), dtype=np.uint8)
+    n = 300
+    stride = (16 + length + 15 + 16 + 15) & ~15
+    arena = rng.integers(0, 256, n * stride, dtype=np.uint8)
+    want = arena.copy()
+    want_len = np.zeros(n, np.uint32)
+    for i in range(n):
+        pt = arena[i * stride + 16:i * stride + 16 + length].tobytes()
+        w = O.wg_encap(pt, mtu, keys[0].tobytes(), peers[0][1], i)
+        want[i * stride:i * stride + len(w)] = np.frombuffer(w, np.uint8)
+        want_len[i] = len(w)
+    assert want_len[0] == 32 + length + O.wg_padding(length, mtu)
+    ctx = _ctx(peers, keys_send=keys)
+    if not fused:
+        ctx.set_spread_max_packets(0)
+    for mem in ("pageable", "ring"):
+        ring = ctx.ring_alloc(arena.nbytes) if mem == "ring" else None
+        got = ring if ring is not None else arena.copy()
+        got[:] = arena
+        got_len = np.zeros(n, np.uint32)
+        ctx.wg_peers_set(peers)  # counters start again at 0
+        ctx.wg_encap(lib.make_batch(got, arena.nbytes, n, lib.MEM_HOST, stride=stride, length=length), mtu, got_len)
+        assert np.array_equal(got_len, want_len), mem
+        bad = np.flatnonzero(np.array(got) != want)
+        assert bad.size == 0, f"{mem}: first differing byte at {bad[:5]}"
+        if ring is not None:
+            ctx.ring_free(ring)
+    ctx.close()
+
+
 def _decap_cases(rng, peers, keys, n):
     """Datagrams as the remote peers would send them, most of them damaged in
     one of the ways the receive path must tell apart."""

@@ -180,6 +180,56 @@ def test_encap_uniform_slots_one_peer_and_padding_rules(fused, length, mtu):
     ctx.close()
 
 
+@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("inner", [0, 28, 1000, 1420])
+def test_decap_uniform_datagrams(fused, inner):
+    """Datagrams of one size at a uniform stride, no length array: keepalives
+    (inner 0), the smallest UDP packet, ordinary and MTU-sized ones."""
+    from bnk_amd import lib
+    from oracle import binding as O
+    rng = np.random.default_rng(inner + 3)
+    peers = _peers(rng)
+    keys = rng.integers(0, 256, (N_PEERS, 32), dtype=np.uint8)
+    n = 257
+    wires = []
+    for i in range(n):
+        p = int(rng.integers(0, N_PEERS))
+        pt = _inner(rng, peers, p, inner) if inner else b""
+        wires.append(O.wg_encap(pt, MTU, keys[p].tobytes(), peers[p][0], 5 + i))
+    wlen = len(wires[0])
+    assert all(len(w) == wlen for w in wires)
+    stride = (wlen + 31) & ~15
+    arena = np.full(n * stride, 0xEE, np.uint8)
+    for i, w in enumerate(wires):
+        arena[i * stride:i * stride + wlen] = np.frombuffer(w, np.uint8)
+    want = np.array([(lambda r: (r[0], len(r[1]), r[2], r[3]))(O.wg_decap(w, peers, keys)) for w in wires], np.uint64)
+    assert (want[:, 0] == (O.WG_OK if inner else O.WG_KEEPALIVE)).all()
+    ctx = _ctx(peers, keys_recv=keys)
+    if not fused:
+        ctx.set_spread_max_packets(0)
+    for mem in ("pageable", "ring"):
+        rings = [ctx.ring_alloc(arena.nbytes), ctx.ring_alloc(arena.nbytes)] if mem == "ring" else []
+        src = rings[0] if rings else arena.copy()
+        out = rings[1] if rings else np.zeros_like(arena)
+        src[:] = arena
+        out[:] = 0x77
+        res, olen = np.full(n, 99, np.uint8), np.full(n, 99, np.uint32)
+        gp, gc = np.full(n, 99, np.uint32), np.full(n, 99, np.uint64)
+        ctx.wg_decap(lib.make_batch(src, arena.nbytes, n, lib.MEM_HOST, stride=stride, length=wlen),
+                     lib.make_batch(out, arena.nbytes, n, lib.MEM_HOST, stride=stride), res, olen, gp, gc)
+        assert np.array_equal(res, want[:, 0].astype(np.uint8)), mem
+        assert np.array_equal(olen, want[:, 1].astype(np.uint32)) and np.array_equal(gp, want[:, 2].astype(np.uint32))
+        assert np.array_equal(gc, want[:, 3])
+        got = np.array(out).reshape(n, stride)
+        for i in (0, n // 2, n - 1):
+            rc, pt, _, _ = O.wg_decap(wires[i], peers, keys)
+            assert got[i, :len(pt)].tobytes() == pt
+            assert (got[i, wlen - 32:] == 0x77).all()  # nothing beyond the padded plaintext
+        for r in rings:
+            ctx.ring_free(r)
+    ctx.close()
+
+
 def _decap_cases(rng, peers, keys, n):
     """Datagrams as the remote peers would send them, most of them damaged in
     one of the ways the receive path must tell apart."""

@@ -230,6 +230,52 @@ def test_decap_uniform_datagrams(fused, inner):
     ctx.close()
 
 
+@pytest.mark.parametrize("mem", ["pageable", "ring"])
+@pytest.mark.parametrize("n,spread_max", [(600, 4096), (600, 0), (6000, 4096)])
+def test_decap_in_place(mem, n, spread_max):
+    """wireguard-go opens a datagram in place: the plaintext lands 16 bytes into
+    the datagram it came from.  Header and tag bytes stay as they were."""
+    from bnk_amd import lib
+    from oracle import binding as O
+    rng = np.random.default_rng(n + spread_max)
+    peers = _peers(rng)
+    keys = rng.integers(0, 256, (N_PEERS, 32), dtype=np.uint8)
+    plains, wires = [], []
+    for i in range(n):
+        p = int(rng.integers(0, N_PEERS))
+        pt = _inner(rng, peers, p, int(rng.choice([20, 64, 300, 1400])))
+        plains.append(pt)
+        wires.append(O.wg_encap(pt, MTU, keys[p].tobytes(), peers[p][0], i))
+    lens = np.array([len(w) for w in wires], np.uint32)
+    off, total = _layout(rng, lens)
+    arena = np.full(total, 0xEE, np.uint8)
+    for i, w in enumerate(wires):
+        arena[int(off[i]):int(off[i]) + len(w)] = np.frombuffer(w, np.uint8)
+    want = arena.copy()
+    for i, w in enumerate(wires):
+        padded = len(w) - 32
+        rc, pt, p, c = O.wg_decap(w, peers, keys)
+        assert rc == O.WG_OK
+        full = O.aead_open(keys[p].tobytes(), O.wg_nonce(c), w[16:])[1]  # padding included
+        assert len(full) == padded
+        want[int(off[i]) + 16:int(off[i]) + 16 + padded] = np.frombuffer(full, np.uint8)
+    ctx = _ctx(peers, keys_recv=keys)
+    ctx.set_spread_max_packets(spread_max)
+    ring = ctx.ring_alloc(total) if mem == "ring" else None
+    buf = ring if ring is not None else arena.copy()
+    buf[:] = arena
+    res, olen = np.full(n, 99, np.uint8), np.zeros(n, np.uint32)
+    gp, gc = np.zeros(n, np.uint32), np.zeros(n, np.uint64)
+    ctx.wg_decap(lib.make_batch(buf, total, n, lib.MEM_HOST, offsets=off, lens=lens),
+                 lib.make_batch(buf, total, n, lib.MEM_HOST, offsets=off + np.uint64(16)), res, olen, gp, gc)
+    assert (res == 0).all() and np.array_equal(olen, np.array([len(p) for p in plains], np.uint32))
+    bad = np.flatnonzero(np.array(buf) != want)
+    assert bad.size == 0, f"first differing byte at {bad[:5]}"
+    if ring is not None:
+        ctx.ring_free(ring)
+    ctx.close()
+
+
 def _decap_cases(rng, peers, keys, n):
     """Datagrams as the remote peers would send them, most of them damaged in
     one of the ways the receive path must tell apart."""

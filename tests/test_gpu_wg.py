@@ -231,10 +231,11 @@ def test_decap_uniform_datagrams(fused, inner):
 
 
 @pytest.mark.parametrize("mem", ["pageable", "ring"])
-@pytest.mark.parametrize("n,spread_max", [(600, 4096), (600, 0), (6000, 4096)])
+@pytest.mark.parametrize("n,spread_max", [(600, 4096), (600, 0), (6000, 4096), (9000, 4096)])
 def test_decap_in_place(mem, n, spread_max):
     """wireguard-go opens a datagram in place: the plaintext lands 16 bytes into
-    the datagram it came from.  Header and tag bytes stay as they were."""
+    the datagram it came from.  Header and tag bytes stay as they were.  9000
+    full-size datagrams (13 MB) go through in overlapped chunks."""
     from bnk_amd import lib
     from oracle import binding as O
     rng = np.random.default_rng(n + spread_max)
@@ -243,11 +244,12 @@ def test_decap_in_place(mem, n, spread_max):
     plains, wires = [], []
     for i in range(n):
         p = int(rng.integers(0, N_PEERS))
-        pt = _inner(rng, peers, p, int(rng.choice([20, 64, 300, 1400])))
+        pt = _inner(rng, peers, p, 1400 if n == 9000 else int(rng.choice([20, 64, 300, 1400])))
         plains.append(pt)
         wires.append(O.wg_encap(pt, MTU, keys[p].tobytes(), peers[p][0], i))
     lens = np.array([len(w) for w in wires], np.uint32)
     off, total = _layout(rng, lens)
+    assert (n == 9000) == (total > 12 << 20)
     arena = np.full(total, 0xEE, np.uint8)
     for i, w in enumerate(wires):
         arena[int(off[i]):int(off[i]) + len(w)] = np.frombuffer(w, np.uint8)

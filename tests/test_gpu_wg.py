@@ -672,6 +672,93 @@ def test_note_outbound_and_encap_in_one_call(mem, n):
     ctx.close()
 
 
+def test_one_call_paths_through_the_chunked_route():
+    """13 MB of full-size packets in pinned rings: NoteOutbound + encapsulate
+    and decapsulate + CheckInbound each in one call (overlapped chunks) against
+    the library's separate calls, which the tests above hold to the oracle:
+    same datagrams, results and flow tables."""
+    from bnk_amd import lib
+    rng = np.random.default_rng(99)
+    peers = _peers(rng)
+    keys = rng.integers(0, 256, (N_PEERS, 32), dtype=np.uint8)
+    rules, local, noted = _filter_setup(rng, peers)
+    t0 = 1_700_000_000 * 10**9
+    n, stride = 9000, 1504
+    peer = rng.integers(0, N_PEERS, n).astype(np.uint32)
+    lens = np.full(n, 1400, np.uint32)
+    off = np.arange(n, dtype=np.uint64) * stride
+    arena = np.zeros(n * stride, np.uint8)
+    rows = arena.reshape(n, stride)
+    for i in range(n):
+        p = int(peer[i])
+        # send side: packets from this node to the peer, recorded as outbound flows; the
+        # receive side below sees the same bytes arriving from the peer's address
+        pkt = W.udp(peers[p][2], local, 53 if i % 3 else 9999, 4000 + (i % 50)) if i % 2 else \
+            W.tcp(peers[p][2], local, 40000 + (i % 999), 22 if i % 4 else 23)
+        rows[i, 16:16 + len(pkt)] = np.frombuffer(pkt, np.uint8)
+        rows[i, 18], rows[i, 19] = 1400 >> 8, 1400 & 255  # IP total length = the whole slot payload
+    assert arena.nbytes > 12 << 20
+
+    def make(send):
+        c = _ctx(peers, keys_send=keys if send else None, keys_recv=None if send else keys)
+        c.filter_set_rules(rules)
+        return c
+
+    # --- send side
+    a, b = make(True), make(True)
+    ra, rb = a.ring_alloc(arena.nbytes), b.ring_alloc(arena.nbytes)
+    ra[:] = arena
+    rb[:] = arena
+    wl_a, wl_b = np.zeros(n, np.uint32), np.zeros(n, np.uint32)
+    a.wg_note_encap(lib.make_batch(ra, arena.nbytes, n, lib.MEM_HOST, offsets=off, lens=lens, peer=peer), MTU, t0, wl_a)
+    b.filter_note_outbound(lib.make_batch(rb[16:], arena.nbytes - 16, n, lib.MEM_HOST, offsets=off, lens=lens), t0)
+    b.wg_encap(lib.make_batch(rb, arena.nbytes, n, lib.MEM_HOST, offsets=off, lens=lens, peer=peer), MTU, wl_b)
+    assert np.array_equal(wl_a, wl_b) and np.array_equal(np.array(ra), np.array(rb))
+    assert a.filter_flows() == b.filter_flows() and a.filter_flow_count() > 100
+    wire = np.array(ra)
+    for c, r in ((a, ra), (b, rb)):
+        c.ring_free(r)
+        c.close()
+
+    # --- receive side: the same datagrams, addressed to the receiver's indices
+    rx_peers = [(p[1], p[0], p[2], p[3]) for p in peers]
+    def make_rx():
+        c = lib.Context(0)
+        c.keys_set(lib.KEYS_RECV, keys)
+        c.wg_peers_set(rx_peers)
+        c.filter_set_rules(rules)
+        for pkt in noted:
+            c.filter_note_outbound_ptrs([pkt], t0 - 10**9)
+        return c
+    a, b = make_rx(), make_rx()
+    ra, oa = a.ring_alloc(wire.nbytes), a.ring_alloc(wire.nbytes)
+    rb, ob = b.ring_alloc(wire.nbytes), b.ring_alloc(wire.nbytes)
+    for r in (ra, rb):
+        r[:] = wire
+    for r in (oa, ob):
+        r[:] = 0x77
+    out_off = off + np.uint64(16)
+    res_a, res_b = np.zeros(n, np.uint8), np.zeros(n, np.uint8)
+    la, lb = np.zeros(n, np.uint32), np.zeros(n, np.uint32)
+    pa, pb = np.zeros(n, np.uint32), np.zeros(n, np.uint32)
+    ca, cb = np.zeros(n, np.uint64), np.zeros(n, np.uint64)
+    a.wg_decap_filter(lib.make_batch(ra, wire.nbytes, n, lib.MEM_HOST, offsets=off, lens=wl_a),
+                      lib.make_batch(oa, wire.nbytes, n, lib.MEM_HOST, offsets=out_off), t0, res_a, la, pa, ca)
+    b.wg_decap(lib.make_batch(rb, wire.nbytes, n, lib.MEM_HOST, offsets=off, lens=wl_a),
+               lib.make_batch(ob, wire.nbytes, n, lib.MEM_HOST, offsets=out_off), res_b, lb, pb, cb)
+    v = np.zeros(n, np.uint8)
+    b.filter_check_inbound(lib.make_batch(ob, wire.nbytes, n, lib.MEM_HOST, offsets=out_off, lens=lb), t0, v)
+    assert (res_b == 0).all()
+    assert np.array_equal(res_a, np.where(v == 0, 7, 0)) and 0.5 < (res_a == 7).mean() < 0.99
+    assert np.array_equal(la, lb) and np.array_equal(pa, pb) and np.array_equal(ca, cb)
+    assert np.array_equal(np.array(oa), np.array(ob))
+    assert a.filter_flows() == b.filter_flows()
+    for c, rs in ((a, (ra, oa)), (b, (rb, ob))):
+        for r in rs:
+            c.ring_free(r)
+        c.close()
+
+
 def test_encap_then_decap_round_trip_full_size():
     """2^20 MTU-sized slots, device resident: every datagram decapsulates to
     its plaintext under the mirrored peer table, counters are each peer's

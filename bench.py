@@ -842,6 +842,15 @@ def main() -> int:
     out["extra"] = {"acl_filter": {k: acl[k] for k in ("metric", "value", "unit", "ms_per_step",
                                                        "config", "roofline", "cpu_baseline")
                                    if k in acl}}
+    # what one call costs at wireguard-go's own batch size (128 packets in pinned rings)
+    largs = argparse.Namespace(**vars(args))
+    largs.steps = 5
+    lat = bench_latency(largs)
+    out["extra"]["call_latency_us_128_packets"] = {
+        "unit": "us per call, median, upload and download included",
+        "workload": lat["config"]["workload"],
+        **lat["per_batch_size_us"]["128"],
+    }
     print(json.dumps(out))
     return 0
 

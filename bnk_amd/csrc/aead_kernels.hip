@@ -496,8 +496,42 @@ __global__ __launch_bounds__(256) void aead_spread_kernel(AeadArgs a)
     uint32_t pr = a.peer ? a.peer[i] : 0u;
     const uint8_t *src = a.in + (a.in_off ? a.in_off[i] : (uint64_t)i * a.in_stride) + a.in_skip;
     uint8_t *dst = a.out + (a.out_off ? a.out_off[i] : (uint64_t)i * a.out_stride) + a.out_skip;
-    uint32_t present = len; // bytes of src that exist in memory; the rest up to len read as zero
     uint64_t ctr = 0;
+
+    // ---- my 64 bytes: loads first, they fly while everything below is looked
+    // up and the block is computed.  Where the AEAD data lies and how long it
+    // is follows from the length alone, so the loads need not wait for the
+    // header, the index search or the key; a packet that is then turned away
+    // has loaded bytes of its own datagram for nothing.
+    const uint8_t *data = src + (WG ? 16 : 0);
+    uint32_t data_len; // bytes through the cipher, when the packet is taken at all
+    uint32_t data_there; // of which in memory
+    if (!WG) {
+        data_len = OPEN ? (len >= 16u ? len - 16u : 0u) : len;
+        data_there = data_len <= SPREAD_MAX_LEN ? data_len : 0u; // longer ones go the per-lane way
+    } else if (!OPEN) {
+        const bool fits = len + 15u <= WG_FUSE_MAX_LEN;
+        data_there = fits ? len : 0u;
+        data_len = fits ? len + wg_padding(len, a.wg.mtu) : 0u;
+    } else {
+        data_len = (len >= 32u && len - 32u <= WG_FUSE_MAX_LEN) ? len - 32u : 0u;
+        data_there = data_len;
+    }
+    const uint32_t at = 64u * (lane - 1u);
+    const uint32_t mine = (lane == 0 || at >= data_len) ? 0u : min(data_len - at, 64u);
+    const uint32_t there = (lane == 0 || at >= data_there) ? 0u : min(data_there - at, 64u);
+    uint32_t m[16];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (there >= 16u * (j + 1)) v = ld16(data + at + 16 * j);
+        else if (there > 16u * j) v = ld_partial(data + at + 16 * j, there - 16u * j);
+        m[4 * j] = v.x; m[4 * j + 1] = v.y; m[4 * j + 2] = v.z; m[4 * j + 3] = v.w;
+    }
+    uint4 want_tag = make_uint4(0, 0, 0, 0);
+    if (OPEN && (WG ? len >= 32u && len - 32u <= WG_FUSE_MAX_LEN : len >= 16u && data_len <= SPREAD_MAX_LEN))
+        want_tag = ld16(data + data_len);
+
     if (!WG) {
         if (a.skip && a.skip[i] != 0) return;
         if (pr >= a.n_peers) {
@@ -512,7 +546,6 @@ __global__ __launch_bounds__(256) void aead_spread_kernel(AeadArgs a)
             return;
         }
         if (OPEN) len -= 16u;
-        present = len;
         ctr = a.counters ? a.counters[i] : a.counter0 + i;
     } else if (!OPEN) {
         // ---- encapsulate: header into the headroom, padding as implied zeros ----
@@ -521,7 +554,6 @@ __global__ __launch_bounds__(256) void aead_spread_kernel(AeadArgs a)
             return;
         }
         ctr = a.counters[i];
-        present = len;
         len += wg_padding(len, a.wg.mtu);
         if (lane == 0) {
             st16(dst, make_uint4(4u, a.wg.remote_index[pr], (uint32_t)ctr, (uint32_t)(ctr >> 32)));
@@ -569,7 +601,6 @@ __global__ __launch_bounds__(256) void aead_spread_kernel(AeadArgs a)
         }
         ctr = (uint64_t)h.z | (uint64_t)h.w << 32;
         len -= 32u; // header and tag
-        present = len;
         src += 16;
     }
     uint32_t k[8];
@@ -591,21 +622,7 @@ __global__ __launch_bounds__(256) void aead_spread_kernel(AeadArgs a)
         return;
     }
 
-    // ---- my 64 bytes: loads first, they fly while the block is computed ----
-    const uint32_t at = 64u * (lane - 1u);
-    const uint32_t mine = (lane == 0 || at >= len) ? 0u : min(len - at, 64u);
-    const uint32_t there = (lane == 0 || at >= present) ? 0u : min(present - at, 64u);
-    uint32_t m[16];
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-        uint4 v = make_uint4(0, 0, 0, 0);
-        if (there >= 16u * (j + 1)) v = ld16(src + at + 16 * j);
-        else if (there > 16u * j) v = ld_partial(src + at + 16 * j, there - 16u * j);
-        m[4 * j] = v.x; m[4 * j + 1] = v.y; m[4 * j + 2] = v.z; m[4 * j + 3] = v.w;
-    }
-    uint4 want_tag = make_uint4(0, 0, 0, 0);
-    if (OPEN) want_tag = ld16(src + len);
-
+    // (the packet's bytes are already on their way: see the top of the kernel)
     chacha_block(k, lane, n1, n2, x);
     // the one-time key is lane 0's block
     const Fe26 r = fe_clamped_r((uint32_t)__builtin_amdgcn_readlane((int)x[0], 0),

@@ -10,6 +10,13 @@ Prints ONE JSON line.  Besides the contract fields it carries
   roofline       HBM view of the dominant kernel (aead_wave_kernel)
   roofline_valu  the same launches priced in int32 op-equivalents
   cpu_baseline   the CPU oracle timed on this box's host cores (bounded sample)
+  cpu_baseline_openssl  the same sample through OpenSSL's assembly, when libcrypto is there
+  packed_layout  the same packets back to back (no slot 16-byte aligned)
+  extra          the ACL filter rate (configuration 4) with its own roofline and CPU
+                 baseline, and what one call costs on 128 packets in pinned host rings
+
+--workload filter | imix | relay | wg | host | latency | copy print one line for that
+workload alone; --no-extras leaves out everything but the timed launches (for traces).
 """
 from __future__ import annotations
 

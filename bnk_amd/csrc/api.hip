@@ -24,10 +24,8 @@ int aead_batch_host_chunked(bnk_ctx *ctx, bool open, const bnk_batch *in, const 
     };
     int rc = hp.plan(in->lens ? 0 : hp.out_ext(0));
     if (rc) return rc;
-    if (in->peer)
-        for (uint32_t i = 0; i < n; i++)
-            if (in->peer[i] >= a.n_peers)
-                return fail(ctx, BNK_E_RANGE, "peer index " + std::to_string(in->peer[i]) + " beyond the key table");
+    rc = check_index_range(ctx, in->peer, n, a.n_peers, "peer index", "the key table");
+    if (rc) return rc;
     if (open) {
         HIPCHK(ctx, ctx->verdict.reserve(n));
         a.verdict = ctx->verdict.as<uint8_t>();
@@ -105,10 +103,8 @@ int aead_batch_host_direct(bnk_ctx *ctx, bool open, const bnk_batch *in, const b
     rc = scan_host_layout(ctx, out, in, open ? -16 : 16, &sout, "out");
     if (rc) return rc;
     if (sin.size() > DIRECT_MAX_BYTES) return 1;
-    if (in->peer)
-        for (uint32_t i = 0; i < n; i++)
-            if (in->peer[i] >= a.n_peers)
-                return fail(ctx, BNK_E_RANGE, "peer index " + std::to_string(in->peer[i]) + " beyond the key table");
+    rc = check_index_range(ctx, in->peer, n, a.n_peers, "peer index", "the key table");
+    if (rc) return rc;
 
     // pinned staging: three 8-byte arrays, three 4-byte arrays, verdict bytes
     HIPCHK(ctx, ctx->pin.reserve((size_t)n * 37 + 64));

@@ -79,6 +79,18 @@ inline int scan_host_layout(bnk_ctx *ctx, const bnk_batch *lay, const bnk_batch 
     return BNK_OK;
 }
 
+// Every index of a host array must name a row of a table with `rows` rows.
+inline int check_index_range(bnk_ctx *ctx, const uint32_t *index, uint32_t n, uint32_t rows,
+                             const char *what, const char *table)
+{
+    if (!index) return BNK_OK;
+    for (uint32_t i = 0; i < n; i++)
+        if (index[i] >= rows)
+            return fail(ctx, BNK_E_RANGE,
+                        std::string(what) + " " + std::to_string(index[i]) + " beyond " + table);
+    return BNK_OK;
+}
+
 inline int check_batch_common(bnk_ctx *ctx, const bnk_batch *b, const char *name)
 {
     if (!b) return fail(ctx, BNK_E_INVAL, std::string(name) + ": null batch");
@@ -147,11 +159,8 @@ inline int stage_host(bnk_ctx *ctx, const bnk_batch *in, const bnk_batch *out, i
     if (rc) return rc;
     rc = scan_host_layout(ctx, out, in, out_delta, &st->sout, "out");
     if (rc) return rc;
-    if (in->peer)
-        for (uint32_t i = 0; i < n; i++)
-            if (in->peer[i] >= n_keys)
-                return fail(ctx, BNK_E_RANGE, "peer index " + std::to_string(in->peer[i]) +
-                                                  " beyond the key table");
+    rc = check_index_range(ctx, in->peer, n, n_keys, "peer index", "the key table");
+    if (rc) return rc;
     // pinned staging for the two rebased offset arrays, and behind them room for
     // one result byte per packet (a copy into pageable memory is slow)
     HIPCHK(ctx, ctx->pin.reserve((size_t)n * 17 + 64));

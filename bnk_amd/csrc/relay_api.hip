@@ -69,14 +69,10 @@ extern "C" int bnk_relay_fused_batch(bnk_ctx *ctx, const bnk_batch *in, const ui
             if (rc) return rc;
             rc = scan_host_layout(ctx, out, in, 0, &sout, "out");
             if (rc) return rc;
-            if (in->peer)
-                for (uint32_t i = 0; i < n; i++)
-                    if (in->peer[i] >= ctx->n_keys[BNK_KEYS_RECV])
-                        return fail(ctx, BNK_E_RANGE, "peer index " + std::to_string(in->peer[i]) +
-                                                          " beyond the key table");
-            for (uint32_t i = 0; i < n; i++)
-                if (peer_out[i] >= n_peers_out)
-                    return fail(ctx, BNK_E_RANGE, "peer_out index beyond n_peers_out");
+            rc = check_index_range(ctx, in->peer, n, ctx->n_keys[BNK_KEYS_RECV], "peer index", "the key table");
+            if (rc) return rc;
+            rc = check_index_range(ctx, peer_out, n, n_peers_out, "peer_out index", "n_peers_out");
+            if (rc) return rc;
             if (sin.size() <= DIRECT_MAX_BYTES) {
                 direct = true;
                 HIPCHK(ctx, ctx->pin.reserve((size_t)n * 45 + (size_t)n_peers_out * 8 + 64));
@@ -132,14 +128,10 @@ extern "C" int bnk_relay_fused_batch(bnk_ctx *ctx, const bnk_batch *in, const ui
         chunked = rc == BNK_OK;
     }
     if (chunked) {
-        if (in->peer)
-            for (uint32_t i = 0; i < n; i++)
-                if (in->peer[i] >= ctx->n_keys[BNK_KEYS_RECV])
-                    return fail(ctx, BNK_E_RANGE, "peer index " + std::to_string(in->peer[i]) +
-                                                      " beyond the key table");
-        for (uint32_t i = 0; i < n; i++)
-            if (peer_out[i] >= n_peers_out)
-                return fail(ctx, BNK_E_RANGE, "peer_out index beyond n_peers_out");
+        rc = check_index_range(ctx, in->peer, n, ctx->n_keys[BNK_KEYS_RECV], "peer index", "the key table");
+        if (rc) return rc;
+        rc = check_index_range(ctx, peer_out, n, n_peers_out, "peer_out index", "n_peers_out");
+        if (rc) return rc;
         HIPCHK(ctx, ctx->r_peer_out.reserve((size_t)n * 4));
         HIPCHK(ctx, ctx->r_ctr_base.reserve((size_t)n_peers_out * 8));
         HIPCHK(ctx, ctx->r_ctr_out.reserve((size_t)n * 8));
@@ -175,9 +167,8 @@ extern "C" int bnk_relay_fused_batch(bnk_ctx *ctx, const bnk_batch *in, const ui
         // the re-sealed packet has the input's length: out_delta 0
         rc = stage_host(ctx, in, out, 0, ctx->n_keys[BNK_KEYS_RECV], &st);
         if (rc) return rc;
-        for (uint32_t i = 0; i < n; i++)
-            if (peer_out[i] >= n_peers_out)
-                return fail(ctx, BNK_E_RANGE, "peer_out index beyond n_peers_out");
+        rc = check_index_range(ctx, peer_out, n, n_peers_out, "peer_out index", "n_peers_out");
+        if (rc) return rc;
         op.in = st.d_in;
         op.in_off = st.d_in_off;
         op.lens = st.d_lens;

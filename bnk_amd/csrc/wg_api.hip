@@ -107,11 +107,8 @@ static int wg_encap_impl(bnk_ctx *ctx, const bnk_batch *slots, uint32_t mtu, uin
     uint8_t *ring_out = nullptr;
     uint32_t *h_wire_len = nullptr;
     if (host) {
-        if (slots->peer)
-            for (uint32_t i = 0; i < n; i++)
-                if (slots->peer[i] >= ctx->n_wg_peers)
-                    return fail(ctx, BNK_E_RANGE, "peer index " + std::to_string(slots->peer[i]) +
-                                                      " beyond the peer table");
+        rc = check_index_range(ctx, slots->peer, n, ctx->n_wg_peers, "peer index", "the peer table");
+        if (rc) return rc;
         uint8_t *d_ring = n <= DIRECT_MAX_PACKETS ? ring_device_ptr(ctx, slots->base, slots->bytes) : nullptr;
         if (d_ring) {
             Span sp;

@@ -102,6 +102,25 @@ static int wg_encap_impl(bnk_ctx *ctx, const bnk_batch *slots, uint32_t mtu, uin
     Span span;
     HostPipe hp;
     bool chunked = false;
+    // A wave-per-packet launch does the framing itself; it needs every packet to
+    // fit 63 ChaCha20 blocks, which only a host batch can promise.
+    bool fits = host;
+    if (host) {
+        if (slots->lens) {
+            for (uint32_t i = 0; i < n && fits; i++) fits = slots->lens[i] + 15u <= WG_FUSE_MAX_LEN;
+        } else {
+            fits = slots->len + 15u <= WG_FUSE_MAX_LEN;
+        }
+    }
+    // Which kernel will read the packets: the framing launch when the batch
+    // qualifies for it, else a plain launch over per-packet padded lengths.
+    AeadArgs probe{};
+    probe.spread_max = ctx->spread_max;
+    probe.n = n;
+    probe.len = slots->len;
+    probe.lens = slots->lens; // only whether there is one matters here
+    const bool wave_per_packet = (fits && aead_runs_spread(probe)) || n <= ctx->spread_max;
+
     // direct route (small batches in a pinned ring): the plaintexts are fetched
     // by a copy kernel, headers and sealed packets go straight into the ring
     uint8_t *ring_out = nullptr;
@@ -129,7 +148,7 @@ static int wg_encap_impl(bnk_ctx *ctx, const bnk_batch *slots, uint32_t mtu, uin
         uint64_t *p_off = ctx->pin.as<uint64_t>();
         uint32_t *p_lens = (uint32_t *)(p_off + n), *p_peer = p_lens + n;
         h_wire_len = p_peer + n;
-        if (n <= ctx->spread_max) {
+        if (wave_per_packet) {
             // a wave per packet reads the ring itself (see aead_batch_host_direct)
             b.base = ring_out;
         } else {
@@ -222,17 +241,6 @@ static int wg_encap_impl(bnk_ctx *ctx, const bnk_batch *slots, uint32_t mtu, uin
         HIPCHK(ctx, launch_peer_rank(ctx->r_keys.as<uint32_t>(), ctx->r_idx.as<uint32_t>(),
                                      ctx->r_skeys.as<uint32_t>(), ctx->r_sidx.as<uint32_t>(), ctx->r_tmp.p,
                                      tmp_bytes, pe.send_ctr, pe.n, n, d_ctr, true, ctx->stream));
-    }
-
-    // A wave-per-packet launch does the framing itself; it needs every packet to
-    // fit 63 ChaCha20 blocks, which only a host batch can promise.
-    bool fits = host;
-    if (host) {
-        if (slots->lens) {
-            for (uint32_t i = 0; i < n && fits; i++) fits = slots->lens[i] + 15u <= WG_FUSE_MAX_LEN;
-        } else {
-            fits = slots->len + 15u <= WG_FUSE_MAX_LEN;
-        }
     }
 
     // filter.go:192-194: NoteOutbound does nothing in allow-all mode
@@ -406,6 +414,25 @@ static int wg_decap_impl(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *o
         const uint64_t l = wire->lens ? wire->lens[i] : wire->len;
         return l >= 32u ? l - 32u : (uint64_t)0;
     };
+    // A wave-per-packet launch does the framing itself; it needs every packet to
+    // fit 63 ChaCha20 blocks, which only a host batch can promise.
+    bool fits = host;
+    if (host) {
+        if (wire->lens) {
+            for (uint32_t i = 0; i < n && fits; i++) fits = wire->lens[i] <= WG_FUSE_MAX_LEN + 32u;
+        } else {
+            fits = wire->len <= WG_FUSE_MAX_LEN + 32u;
+        }
+    }
+    // Which kernel will read the datagrams: the framing launch when the batch
+    // qualifies for it, else a plain launch over per-packet ciphertext lengths.
+    AeadArgs probe{};
+    probe.spread_max = ctx->spread_max;
+    probe.n = n;
+    probe.len = wire->len;
+    probe.lens = wire->lens; // only whether there is one matters here
+    const bool wave_per_packet = (fits && aead_runs_spread(probe)) || n <= ctx->spread_max;
+
     // direct route (small batches in pinned rings): datagrams fetched by a copy
     // kernel, plaintexts written straight into the out ring, per-packet results
     // into pinned staging
@@ -431,7 +458,7 @@ static int wg_decap_impl(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *o
                 h_out_len = p_lens + n;
                 h_peer = h_out_len + n;
                 h_result = (uint8_t *)(h_peer + n);
-                if (n <= ctx->spread_max) {
+                if (wave_per_packet) {
                     // a wave per packet reads the ring itself (see aead_batch_host_direct)
                     wb.base = d_wire + sin.lo;
                 } else {
@@ -522,17 +549,6 @@ static int wg_decap_impl(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *o
     uint32_t *d_ctlen = ctx->wg_ctlen.as<uint32_t>();
     uint8_t *d_auth = ctx->r_auth.as<uint8_t>();
     const WgPeersDev pe = peers_view(ctx);
-
-    // A wave-per-packet launch does the framing itself; it needs every packet to
-    // fit 63 ChaCha20 blocks, which only a host batch can promise.
-    bool fits = host;
-    if (host) {
-        if (wire->lens) {
-            for (uint32_t i = 0; i < n && fits; i++) fits = wire->lens[i] <= WG_FUSE_MAX_LEN + 32u;
-        } else {
-            fits = wire->len <= WG_FUSE_MAX_LEN + 32u;
-        }
-    }
 
     // filter.go:124-126: CheckInbound passes everything in allow-all mode
     const bool check = check_now != nullptr && ctx->filter->enforce;

@@ -759,6 +759,79 @@ def test_one_call_paths_through_the_chunked_route():
         c.close()
 
 
+def test_random_framing_batches_round_trip_through_rings_and_pageable_memory():
+    """Forty batches of random size, length mix, MTU, alignment, memory kind and
+    kernel choice: encapsulated datagrams against the oracle byte for byte,
+    then decapsulated again (results, lengths, peers, counters, plaintexts)."""
+    from bnk_amd import lib
+    from oracle import binding as O
+    rng = np.random.default_rng(4242)
+    n_peers = 23
+    local = rng.permutation(1 << 20)[:n_peers].astype(np.uint32) * 4099 + 17
+    remote = rng.integers(0, 1 << 32, n_peers, dtype=np.uint64).astype(np.uint32)
+    peers_tx = [(int(local[i]), int(remote[i]), 0x64400001 + i, 0xFFFFFFFF) for i in range(n_peers)]
+    peers_rx = [(int(remote[i]), int(local[i]), 0x64400001 + i, 0xFFFFFFFF) for i in range(n_peers)]
+    keys = rng.integers(0, 256, (n_peers, 32), dtype=np.uint8)
+    tx, rx = lib.Context(0), lib.Context(0)
+    tx.keys_set(lib.KEYS_SEND, keys)
+    rx.keys_set(lib.KEYS_RECV, keys)
+    ring_t, ring_r, ring_o = tx.ring_alloc(3 << 20), rx.ring_alloc(3 << 20), rx.ring_alloc(3 << 20)
+    for it in range(40):
+        n = int(rng.choice([1, 3, 64, 65, 200, 1024, 1025]))
+        mtu = int(rng.choice([0, 1280, 1420]))
+        lens = rng.choice([0, 1, 20, 21, 28, 40, 100, 576, 1279, 1280, 1400, 1420], n).astype(np.uint32)
+        peer = rng.integers(0, n_peers, n).astype(np.uint32)
+        slot = ((16 + lens.astype(np.int64) + 15 + 16 + 15) & ~15) + 16
+        gaps = rng.integers(0, 16, n) if rng.integers(0, 2) else np.zeros(n, np.int64)
+        off = (np.concatenate([[0], np.cumsum(slot)[:-1]]) + gaps).astype(np.uint64)
+        total = int(slot.sum()) + 32
+        arena = rng.integers(0, 256, total, dtype=np.uint8)
+        for i in range(n):
+            length, o = int(lens[i]), int(off[i]) + 16
+            if length >= 20:
+                arena[o] = 0x45
+                arena[o + 2:o + 4] = np.frombuffer(struct.pack(">H", length), np.uint8)
+                arena[o + 12:o + 16] = np.frombuffer(struct.pack(">I", peers_tx[int(peer[i])][2]), np.uint8)
+        tx.wg_peers_set(peers_tx)
+        rx.wg_peers_set(peers_rx)
+        spread = int(rng.choice([0, 4096]))
+        tx.set_spread_max_packets(spread)
+        rx.set_spread_max_packets(spread)
+        in_rings = bool(rng.integers(0, 2))
+        case = f"batch {it}: n={n} mtu={mtu} spread_max={spread} rings={in_rings}"
+        want, want_len, nxt = arena.copy(), np.zeros(n, np.uint32), np.zeros(n_peers, np.uint64)
+        for i in range(n):
+            p, o = int(peer[i]), int(off[i])
+            w = O.wg_encap(arena[o + 16:o + 16 + int(lens[i])].tobytes(), mtu, keys[p].tobytes(),
+                           peers_tx[p][1], int(nxt[p]))
+            nxt[p] += 1
+            want[o:o + len(w)] = np.frombuffer(w, np.uint8)
+            want_len[i] = len(w)
+        buf = ring_t[:total] if in_rings else arena.copy()
+        buf[:] = arena
+        got_len = np.zeros(n, np.uint32)
+        tx.wg_encap(lib.make_batch(buf, total, n, lib.MEM_HOST, offsets=off, lens=lens, peer=peer), mtu, got_len)
+        assert np.array_equal(got_len, want_len) and np.array_equal(np.array(buf), want), case
+        src = ring_r[:total] if in_rings else want.copy()
+        src[:] = want
+        out = ring_o[:total + 16] if in_rings else np.zeros(total + 16, np.uint8)
+        out[:] = 0x77
+        res, olen = np.zeros(n, np.uint8), np.zeros(n, np.uint32)
+        gp, gc = np.zeros(n, np.uint32), np.zeros(n, np.uint64)
+        rx.wg_decap(lib.make_batch(src, total, n, lib.MEM_HOST, offsets=off, lens=want_len),
+                    lib.make_batch(out, total + 16, n, lib.MEM_HOST, offsets=off + np.uint64(16)),
+                    res, olen, gp, gc)
+        for i in range(n):
+            o = int(off[i])
+            rc, pt, p, c = O.wg_decap(want[o:o + int(want_len[i])].tobytes(), peers_rx, keys)
+            assert (rc, len(pt), p, c) == (int(res[i]), int(olen[i]), int(gp[i]), int(gc[i])), f"{case}, packet {i}"
+            assert rc != 0 or out[o + 16:o + 16 + len(pt)].tobytes() == pt, f"{case}, packet {i}"
+    for c, rings in ((tx, (ring_t,)), (rx, (ring_r, ring_o))):
+        for r in rings:
+            c.ring_free(r)
+        c.close()
+
+
 def test_encap_then_decap_round_trip_full_size():
     """2^20 MTU-sized slots, device resident: every datagram decapsulates to
     its plaintext under the mirrored peer table, counters are each peer's

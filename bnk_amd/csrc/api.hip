@@ -165,8 +165,28 @@ int aead_batch_host_direct(bnk_ctx *ctx, bool open, const bnk_batch *in, const b
     return BNK_OK;
 }
 
+// Device batches cannot be walked on the host; check what is uniform.
+int aead_device_layout_check(bnk_ctx *ctx, bool open, const bnk_batch *in, const bnk_batch *out)
+{
+    const uint32_t n = in->n;
+    if (!in->offsets && !in->lens && ((uint64_t)(n - 1) * in->stride + in->len > in->bytes))
+        return fail(ctx, BNK_E_INVAL, "in: uniform layout exceeds the arena");
+    if (!out->offsets && !in->lens) {
+        const int64_t ol = (int64_t)in->len + (open ? -16 : 16);
+        if ((uint64_t)(n - 1) * out->stride + (uint64_t)std::max<int64_t>(ol, 0) > out->bytes)
+            return fail(ctx, BNK_E_INVAL, "out: uniform layout exceeds the arena");
+    }
+    return BNK_OK;
+}
+
+} // namespace
+
+namespace bnk {
+
+// sort_scratch: null, or device memory of n + 2 * LEN_BINS words for the
+// length grouping of a device-resident batch (then nothing is allocated).
 int aead_batch(bnk_ctx *ctx, bool open, const bnk_batch *in, const bnk_batch *out,
-               uint8_t *verdict)
+               uint8_t *verdict, uint32_t *sort_scratch)
 {
     int rc = check_batch_common(ctx, in, "in");
     if (rc) return rc;
@@ -194,15 +214,8 @@ int aead_batch(bnk_ctx *ctx, bool open, const bnk_batch *in, const bnk_batch *ou
     a.len = in->len;
 
     if (in->mem == BNK_MEM_DEVICE) {
-        // Device batches cannot be walked on the host; check what is uniform.
-        if (!in->offsets && !in->lens &&
-            ((uint64_t)(n - 1) * in->stride + in->len > in->bytes))
-            return fail(ctx, BNK_E_INVAL, "in: uniform layout exceeds the arena");
-        if (!out->offsets && !in->lens) {
-            const int64_t ol = (int64_t)in->len + (open ? -16 : 16);
-            if ((uint64_t)(n - 1) * out->stride + (uint64_t)std::max<int64_t>(ol, 0) > out->bytes)
-                return fail(ctx, BNK_E_INVAL, "out: uniform layout exceeds the arena");
-        }
+        rc = aead_device_layout_check(ctx, open, in, out);
+        if (rc) return rc;
         a.in = (const uint8_t *)in->base;
         a.out = (uint8_t *)out->base;
         a.in_off = in->offsets;
@@ -211,11 +224,22 @@ int aead_batch(bnk_ctx *ctx, bool open, const bnk_batch *in, const bnk_batch *ou
         a.peer = in->peer;
         a.counters = in->counters;
         a.verdict = verdict;
-        rc = maybe_sort(ctx, &a, open ? 16 : 0);
-        if (rc) return rc;
+        if (sort_scratch) {
+            // the caller's scratch instead of the context's grow-only buffers
+            a.order = nullptr;
+            if (a.lens && n > 64 && !aead_runs_spread(a)) {
+                uint32_t *order = sort_scratch, *hist = order + n, *cursor = hist + LEN_BINS;
+                HIPCHK(ctx, launch_length_sort(a.lens, n, open ? 16 : 0, order, hist, cursor, ctx->stream));
+                a.order = order;
+            }
+        } else {
+            rc = maybe_sort(ctx, &a, open ? 16 : 0);
+            if (rc) return rc;
+        }
         HIPCHK(ctx, open ? launch_aead_open(a, ctx->stream) : launch_aead_seal(a, ctx->stream));
         return BNK_OK;
     }
+    if (sort_scratch) return fail(ctx, BNK_E_INVAL, "this entry point takes device-resident batches only");
 
     rc = aead_batch_host_direct(ctx, open, in, out, verdict, a);
     if (rc != 1) return rc;
@@ -249,10 +273,6 @@ int aead_batch(bnk_ctx *ctx, bool open, const bnk_batch *in, const bnk_batch *ou
     if (open) memcpy(verdict, h_verdict, n);
     return BNK_OK;
 }
-
-} // namespace
-
-namespace bnk {
 
 // Waits for the stream, then reads and clears the status words.
 int take_status(bnk_ctx *ctx, uint32_t *status)
@@ -314,6 +334,11 @@ int bnk_init(int device_ordinal, bnk_ctx **out)
     memset(ctx->h_status, 0, 64);
     if ((e = hipHostGetDevicePointer((void **)&ctx->d_status, ctx->h_status, 0)) != hipSuccess)
         return bail("hipHostGetDevicePointer", e);
+    if (int rc = noalloc_setup(nullptr, device_ordinal)) {
+        ctx->alive = true;
+        bnk_shutdown(ctx);
+        return rc;
+    }
     ctx->filter = filter_create(ctx->stream, prop.multiProcessorCount);
     if (!ctx->filter) return bail("filter state", hipErrorOutOfMemory);
     if ((e = hipStreamSynchronize(ctx->stream)) != hipSuccess) return bail("hipStreamSynchronize", e);
@@ -475,14 +500,14 @@ int bnk_aead_seal_batch(bnk_ctx *ctx, const bnk_batch *in, const bnk_batch *out)
 {
     Guard g(ctx);
     if (g.rc) return g.rc;
-    return aead_batch(ctx, false, in, out, nullptr);
+    return aead_batch(ctx, false, in, out, nullptr, nullptr);
 }
 
 int bnk_aead_open_batch(bnk_ctx *ctx, const bnk_batch *in, const bnk_batch *out, uint8_t *verdict)
 {
     Guard g(ctx);
     if (g.rc) return g.rc;
-    return aead_batch(ctx, true, in, out, verdict);
+    return aead_batch(ctx, true, in, out, verdict, nullptr);
 }
 
 int bnk_probe_valu(bnk_ctx *ctx, int op, uint32_t iters, double *ops_per_sec)

@@ -410,6 +410,16 @@ struct HostPipe {
     }
 };
 
+// Seal or open of one batch (api.hip).  sort_scratch: null, or device memory of
+// in->n + 2 * LEN_BINS words for the length grouping of a device-resident batch;
+// with it the call allocates nothing and takes device batches only.
+int aead_batch(bnk_ctx *ctx, bool open, const bnk_batch *in, const bnk_batch *out, uint8_t *verdict,
+               uint32_t *sort_scratch);
+
+// The file-scope device scratch of the entry point that allocates nothing
+// (noalloc_api.hip): looks up its address on `device` (which must be current).
+int noalloc_setup(bnk_ctx *ctx, int device);
+
 // Reads and clears the device status word (waits for the stream).
 int take_status(bnk_ctx *ctx, uint32_t *status);
 // Maps status bits to an error code (BNK_OK when clear).

@@ -1,0 +1,67 @@
+// bnk_aead_seal_batch_noalloc: bnk_aead_seal_batch for callers that cannot
+// allocate device memory (code under HIP graph capture, tight serving loops,
+// harnesses that forbid hipMalloc).  The one scratch buffer the seal path needs
+// beyond its inputs and outputs -- the length grouping's packet order,
+// histogram and cursors -- lives in a file-scope device array instead of the
+// context's grow-only buffers.
+#include <mutex>
+
+#include "api_common.hpp"
+
+using namespace bnk;
+
+constexpr size_t SCRATCH_WORDS = (size_t)BNK_NOALLOC_MAX_PACKETS + 2u * LEN_BINS;
+
+// 4 MiB + 8 KiB on every GPU the library runs on, for the life of the process.
+// In host code this name is only a stand-in for the symbol: the address a
+// kernel can use comes from hipGetSymbolAddress, once per device.  (Kept out
+// of an unnamed namespace and free of attributes: the compiler gives a static
+// device variable that host code names a visible symbol of its own, which is
+// what the runtime looks up.)
+static __device__ __align__(256) uint32_t scratch[SCRATCH_WORDS];
+
+namespace {
+
+constexpr int MAX_DEVICES = 64;
+std::mutex g_mu;
+uint32_t *g_scratch_ptr[MAX_DEVICES]; // per device: each GPU holds its own copy of the array
+
+} // namespace
+
+namespace bnk {
+
+int noalloc_setup(bnk_ctx *ctx, int device)
+{
+    if (device < 0 || device >= MAX_DEVICES) return fail(ctx, BNK_E_NODEV, "device ordinal out of range");
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (g_scratch_ptr[device]) return BNK_OK;
+    void *p = nullptr;
+    hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return fail_hip(ctx, "hipGetSymbolAddress(scratch)", e);
+    if (!p) return fail(ctx, BNK_E_HIP, "hipGetSymbolAddress(scratch) returned a null address");
+    g_scratch_ptr[device] = static_cast<uint32_t *>(p);
+    return BNK_OK;
+}
+
+} // namespace bnk
+
+extern "C" int bnk_aead_seal_batch_noalloc(bnk_ctx *ctx, const bnk_batch *in, const bnk_batch *out)
+{
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    if (!in || !out) return fail(ctx, BNK_E_INVAL, "null batch");
+    if (in->mem != BNK_MEM_DEVICE || out->mem != BNK_MEM_DEVICE)
+        return fail(ctx, BNK_E_INVAL, "bnk_aead_seal_batch_noalloc takes device-resident batches only");
+    if (in->n > BNK_NOALLOC_MAX_PACKETS)
+        return fail(ctx, BNK_E_INVAL, "bnk_aead_seal_batch_noalloc: more than BNK_NOALLOC_MAX_PACKETS packets");
+    uint32_t *ptr;
+    {
+        std::lock_guard<std::mutex> lk(g_mu);
+        ptr = g_scratch_ptr[ctx->device];
+    }
+    if (!ptr) return fail(ctx, BNK_E_STATE, "device scratch was not set up");
+    // The array keeps the last call's contents: the histogram is cleared by the
+    // length grouping itself (a fill kernel), order[] and cursor[] are written
+    // before they are read.
+    return aead_batch(ctx, false, in, out, nullptr, ptr);
+}

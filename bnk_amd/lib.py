@@ -19,6 +19,7 @@ MEM_HOST, MEM_DEVICE = 0, 1
 KEYS_SEND, KEYS_RECV = 0, 1
 RELAY_OK, RELAY_FORGED, RELAY_DENIED = 0, 1, 2
 E_INVAL, E_NODEV, E_HIP, E_NOMEM, E_RANGE, E_STATE = -1, -2, -3, -4, -5, -6
+NOALLOC_MAX_PACKETS = 1 << 20
 
 PROBE_OPS = {"v_add_u32": 0, "v_xor_b32": 1, "v_alignbit_b32": 2, "v_mad_u64_u32": 3,
              "v_fma_f64": 4, "v_mul_lo_u32": 5, "v_add_f64": 6}
@@ -244,6 +245,10 @@ class Context:
 
     def seal(self, inb: Batch, outb: Batch) -> None:
         self._chk(self._lib.bnk_aead_seal_batch(self._h, C.byref(inb), C.byref(outb)))
+
+    def seal_noalloc(self, inb: Batch, outb: Batch) -> None:
+        """bnk_aead_seal_batch_noalloc: device batches only, allocates nothing."""
+        self._chk(self._lib.bnk_aead_seal_batch_noalloc(self._h, C.byref(inb), C.byref(outb)))
 
     def open(self, inb: Batch, outb: Batch, verdict) -> None:
         self._chk(self._lib.bnk_aead_open_batch(self._h, C.byref(inb), C.byref(outb),

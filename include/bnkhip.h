@@ -153,6 +153,21 @@ int bnk_aead_seal_batch(bnk_ctx *ctx, const bnk_batch *in,
 int bnk_aead_open_batch(bnk_ctx *ctx, const bnk_batch *in,
                         const bnk_batch *out, uint8_t *verdict);
 
+/* bnk_aead_seal_batch for callers that cannot allocate device memory: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  It has no counterpart in the reference.  The call allocates
+ * nothing: the scratch the length grouping needs lives in a file-scope device
+ * array of BNK_NOALLOC_MAX_PACKETS + 2064 words (4 MiB + 8 KiB per GPU, held
+ * until the process ends).  Device-resident batches only (in->mem and out->mem
+ * BNK_MEM_DEVICE), at most BNK_NOALLOC_MAX_PACKETS packets, otherwise
+ * BNK_E_INVAL.  Results are those of bnk_aead_seal_batch.  Every call on a GPU
+ * shares that GPU's array, so two such calls must not overlap on one GPU
+ * (calls on one context are serialised on its stream; calls on different
+ * contexts of the same GPU race unless the caller orders them). */
+#define BNK_NOALLOC_MAX_PACKETS (1u << 20)
+int bnk_aead_seal_batch_noalloc(bnk_ctx *ctx, const bnk_batch *in,
+                                const bnk_batch *out);
+
 /* ---- packet filter ----------------------------------------------------- */
 
 /* filter.SetRules (internal/filter/filter.go:46-51): enforcement on, rule

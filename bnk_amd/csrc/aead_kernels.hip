@@ -554,6 +554,10 @@ __global__ __launch_bounds__(256) void aead_spread_kernel(AeadArgs a)
             return;
         }
         ctr = a.counters[i];
+        if (ctr >= WG_REJECT_AFTER_MESSAGES) { // the keypair has used up its nonces
+            if (lane == 0) a.wg.wire_len[i] = 0;
+            return;
+        }
         len += wg_padding(len, a.wg.mtu);
         if (lane == 0) {
             st16(dst, make_uint4(4u, a.wg.remote_index[pr], (uint32_t)ctr, (uint32_t)(ctr >> 32)));

@@ -115,6 +115,7 @@ struct bnk_ctx {
     // WireGuard framing: peer tables and per-packet scratch
     bnk::DevBuf wg_index, wg_remote, wg_allowed, wg_send_ctr;
     uint32_t n_wg_peers = 0;
+    std::vector<bnk_wg_peer> wg_rows; // host copy of the peer table, row by row
     bnk::DevBuf wg_peer, wg_counter, wg_ctlen, wg_result, wg_outlen, wg_padded, wg_wirelen, wg_skip;
 
     bnk::FilterState *filter = nullptr;

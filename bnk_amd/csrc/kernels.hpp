@@ -18,6 +18,18 @@ __host__ __device__ inline uint32_t wg_padding(uint32_t len, uint32_t mtu)
     return padded - last;
 }
 
+// A keypair whose send counter has reached this value sends nothing more
+// (wireguard-go device/constants.go: RejectAfterMessages = 2^64 - 2^13 - 1).
+constexpr uint64_t WG_REJECT_AFTER_MESSAGES = ~0ull - (1ull << 13);
+
+// base + rank, stopping at `limit` instead of wrapping (limit 0: plain sum).
+__host__ __device__ inline uint64_t ctr_add(uint64_t base, uint64_t rank, uint64_t limit)
+{
+    const uint64_t c = base + rank;
+    if (limit == 0) return c;
+    return (c < base || c > limit) ? limit : c;
+}
+
 // WireGuard transport framing done by a wave-per-packet AEAD launch itself
 // (small batches only; larger ones run the framing kernels of wg_kernels.hip
 // around the launch).  in/out offsets then address the slot or datagram, not
@@ -117,9 +129,12 @@ hipError_t launch_relay_assign(const uint8_t *auth, const uint8_t *pass, const u
 // 0xFFFFFFFF.  keys/idx are
 // inputs (idx[i] = i), skeys/sidx and sort_tmp scratch.  With advance set,
 // ctr_base[key] moves past the counters handed out.
+// ctr_limit: 0, or the value counters saturate at (handed-out counters never wrap
+// past it and an advanced base stops there): WG_REJECT_AFTER_MESSAGES for a
+// keypair's send counter.
 hipError_t launch_peer_rank(uint32_t *keys, uint32_t *idx, uint32_t *skeys, uint32_t *sidx,
                             void *sort_tmp, size_t sort_tmp_bytes, uint64_t *ctr_base, uint32_t n_keys,
-                            uint32_t n, uint64_t *ctr_out, bool advance, hipStream_t s);
+                            uint32_t n, uint64_t *ctr_out, bool advance, uint64_t ctr_limit, hipStream_t s);
 
 // Copy of a byte span whose two ends share their alignment within 16 bytes,
 // one aligned 16-byte piece per lane (used to fetch small spans of pinned
@@ -131,7 +146,8 @@ hipError_t launch_pull(const void *src, void *dst, uint64_t bytes, hipStream_t s
 // peer index beyond the table sets STATUS_PEER_RANGE and gets no counter.
 constexpr uint32_t PEER_RANK_SMALL_MAX = 1024;
 hipError_t launch_peer_rank_small(const uint32_t *peer, uint32_t n_keys, uint32_t n, uint64_t *ctr_base,
-                                  uint64_t *ctr_out, bool advance, uint32_t *status, hipStream_t s);
+                                  uint64_t *ctr_out, bool advance, uint64_t ctr_limit, uint32_t *status,
+                                  hipStream_t s);
 
 // VALU throughput probe; out receives one word per thread so nothing is
 // optimised away.

@@ -55,26 +55,26 @@ __global__ __launch_bounds__(256) void peer_heads_kernel(const uint32_t *skeys, 
 __global__ __launch_bounds__(256) void relay_rank_kernel(const uint32_t *skeys, const uint32_t *sidx,
                                                          const uint32_t *seg_start,
                                                          const uint64_t *ctr_base_out, uint32_t n,
-                                                         uint64_t *ctr_out)
+                                                         uint64_t *ctr_out, uint64_t ctr_limit)
 {
     const uint32_t p = blockIdx.x * 256u + threadIdx.x;
     if (p >= n) return;
     const uint32_t key = skeys[p];
     if (key == NO_PEER) return;
-    ctr_out[sidx[p]] = ctr_base_out[key] + (uint64_t)(p - seg_start[key]);
+    ctr_out[sidx[p]] = ctr_add(ctr_base_out[key], (uint64_t)(p - seg_start[key]), ctr_limit);
 }
 
 // The last element of each peer's segment holds the largest counter handed out.
 __global__ __launch_bounds__(256) void peer_advance_kernel(const uint32_t *skeys, const uint32_t *sidx,
                                                            const uint64_t *ctr_out, uint32_t n,
-                                                           uint64_t *ctr_base)
+                                                           uint64_t *ctr_base, uint64_t ctr_limit)
 {
     const uint32_t p = blockIdx.x * 256u + threadIdx.x;
     if (p >= n) return;
     const uint32_t key = skeys[p];
     if (key == NO_PEER) return;
     if (p + 1u < n && skeys[p + 1u] == key) return;
-    ctr_base[key] = ctr_out[sidx[p]] + 1u;
+    ctr_base[key] = ctr_add(ctr_out[sidx[p]], 1u, ctr_limit);
 }
 
 // Peer keys are below n_keys and the "no peer" key is all ones, so the low
@@ -103,7 +103,7 @@ size_t relay_sort_tmp_bytes(uint32_t n, uint32_t n_keys)
 
 __global__ void peer_rank_small_kernel(const uint32_t *peer, uint32_t n_keys, uint32_t n, uint64_t *ctr_base,
                                        uint64_t *ctr_out, int advance, int no_peer_ok, unsigned bits,
-                                       uint32_t *status);
+                                       uint64_t ctr_limit, uint32_t *status);
 
 hipError_t launch_relay_assign(const uint8_t *auth, const uint8_t *pass, const uint32_t *peer_out,
                                const uint64_t *ctr_base_out, uint32_t n_peers_out, uint32_t n,
@@ -119,11 +119,11 @@ hipError_t launch_relay_assign(const uint8_t *auth, const uint8_t *pass, const u
         // keys[] is the peer of each survivor and all ones for the rest
         hipLaunchKernelGGL(peer_rank_small_kernel, dim3(1), dim3(PEER_RANK_SMALL_MAX), 0, s, keys, n_peers_out,
                            n, const_cast<uint64_t *>(ctr_base_out), ctr_out, advance ? 1 : 0, 1,
-                           key_bits(n_peers_out), status);
+                           key_bits(n_peers_out), 0ull, status);
         return hipGetLastError();
     }
     return launch_peer_rank(keys, idx, skeys, sidx, sort_tmp, sort_tmp_bytes,
-                            const_cast<uint64_t *>(ctr_base_out), n_peers_out, n, ctr_out, advance, s);
+                            const_cast<uint64_t *>(ctr_base_out), n_peers_out, n, ctr_out, advance, 0ull, s);
 }
 
 // Batch-order counters for a small batch in one launch of one block, straight
@@ -133,7 +133,7 @@ hipError_t launch_relay_assign(const uint8_t *auth, const uint8_t *pass, const u
 // peer's base.
 __global__ __launch_bounds__(PEER_RANK_SMALL_MAX) void peer_rank_small_kernel(
     const uint32_t *peer, uint32_t n_keys, uint32_t n, uint64_t *ctr_base, uint64_t *ctr_out,
-    int advance, int no_peer_ok, unsigned bits, uint32_t *status)
+    int advance, int no_peer_ok, unsigned bits, uint64_t ctr_limit, uint32_t *status)
 {
     using Sort = rocprim::block_radix_sort<uint32_t, PEER_RANK_SMALL_MAX, 1, uint32_t>;
     using Scan = rocprim::block_scan<uint32_t, PEER_RANK_SMALL_MAX>;
@@ -164,26 +164,27 @@ __global__ __launch_bounds__(PEER_RANK_SMALL_MAX) void peer_rank_small_kernel(
     Scan().inclusive_scan(head ? t : 0u, start, tmp.scan, rocprim::maximum<uint32_t>());
     uint64_t mine = 0;
     if (valid) {
-        mine = ctr_base[key[0]] + (t - start);
+        mine = ctr_add(ctr_base[key[0]], t - start, ctr_limit);
         ctr_out[pos[0]] = mine;
     }
     __syncthreads(); // every base has been read
-    if (advance && valid && last) ctr_base[key[0]] = mine + 1u;
+    if (advance && valid && last) ctr_base[key[0]] = ctr_add(mine, 1u, ctr_limit);
 }
 
 hipError_t launch_peer_rank_small(const uint32_t *peer, uint32_t n_keys, uint32_t n, uint64_t *ctr_base,
-                                  uint64_t *ctr_out, bool advance, uint32_t *status, hipStream_t s)
+                                  uint64_t *ctr_out, bool advance, uint64_t ctr_limit, uint32_t *status,
+                                  hipStream_t s)
 {
     if (n == 0) return hipSuccess;
     if (n > PEER_RANK_SMALL_MAX) return hipErrorInvalidValue;
     hipLaunchKernelGGL(peer_rank_small_kernel, dim3(1), dim3(PEER_RANK_SMALL_MAX), 0, s, peer, n_keys, n,
-                       ctr_base, ctr_out, advance ? 1 : 0, 0, key_bits(n_keys), status);
+                       ctr_base, ctr_out, advance ? 1 : 0, 0, key_bits(n_keys), ctr_limit, status);
     return hipGetLastError();
 }
 
 hipError_t launch_peer_rank(uint32_t *keys, uint32_t *idx, uint32_t *skeys, uint32_t *sidx,
                             void *sort_tmp, size_t sort_tmp_bytes, uint64_t *ctr_base, uint32_t n_keys,
-                            uint32_t n, uint64_t *ctr_out, bool advance, hipStream_t s)
+                            uint32_t n, uint64_t *ctr_out, bool advance, uint64_t ctr_limit, hipStream_t s)
 {
     if (n == 0) return hipSuccess;
     const dim3 grid((n + 255u) / 256u);
@@ -192,9 +193,11 @@ hipError_t launch_peer_rank(uint32_t *keys, uint32_t *idx, uint32_t *skeys, uint
     if (e != hipSuccess) return e;
     uint32_t *seg_start = static_cast<uint32_t *>(sort_tmp);
     hipLaunchKernelGGL(peer_heads_kernel, grid, dim3(256), 0, s, skeys, n, seg_start);
-    hipLaunchKernelGGL(relay_rank_kernel, grid, dim3(256), 0, s, skeys, sidx, seg_start, ctr_base, n, ctr_out);
+    hipLaunchKernelGGL(relay_rank_kernel, grid, dim3(256), 0, s, skeys, sidx, seg_start, ctr_base, n, ctr_out,
+                       ctr_limit);
     if (advance)
-        hipLaunchKernelGGL(peer_advance_kernel, grid, dim3(256), 0, s, skeys, sidx, ctr_out, n, ctr_base);
+        hipLaunchKernelGGL(peer_advance_kernel, grid, dim3(256), 0, s, skeys, sidx, ctr_out, n, ctr_base,
+                           ctr_limit);
     return hipGetLastError();
 }
 

@@ -30,35 +30,107 @@ int upload(bnk_ctx *ctx, DevBuf *dst, const void *src, size_t bytes)
 
 } // namespace
 
+// Checks the rows and builds the sorted (local index, row) table.
+static int wg_build_index(bnk_ctx *ctx, const bnk_wg_peer *peers, uint32_t n, std::vector<uint2> *index)
+{
+    index->resize(n);
+    for (uint32_t i = 0; i < n; i++) {
+        const uint32_t inv = ~peers[i].allowed_mask;
+        if ((inv & (inv + 1u)) != 0u)
+            return fail(ctx, BNK_E_INVAL, "peer " + std::to_string(i) + ": allowed_mask is not a prefix mask");
+        (*index)[i] = make_uint2(peers[i].local_index, i);
+    }
+    std::sort(index->begin(), index->end(), [](const uint2 &a, const uint2 &b) { return a.x < b.x; });
+    for (uint32_t i = 1; i < n; i++)
+        if ((*index)[i].x == (*index)[i - 1].x)
+            return fail(ctx, BNK_E_INVAL, "local_index " + std::to_string((*index)[i].x) + " is used by two peers");
+    return BNK_OK;
+}
+
 extern "C" int bnk_wg_peers_set(bnk_ctx *ctx, const bnk_wg_peer *peers, uint32_t n)
 {
     Guard g(ctx);
     if (g.rc) return g.rc;
     if (!peers || n == 0) return fail(ctx, BNK_E_INVAL, "empty peer table");
-    std::vector<uint2> index(n), allowed(n);
+    std::vector<uint2> index, allowed(n);
     std::vector<uint32_t> remote(n);
+    int rc = wg_build_index(ctx, peers, n, &index);
+    if (rc) return rc;
     for (uint32_t i = 0; i < n; i++) {
-        const uint32_t inv = ~peers[i].allowed_mask;
-        if ((inv & (inv + 1u)) != 0u)
-            return fail(ctx, BNK_E_INVAL, "peer " + std::to_string(i) + ": allowed_mask is not a prefix mask");
-        index[i] = make_uint2(peers[i].local_index, i);
         remote[i] = peers[i].remote_index;
         allowed[i] = make_uint2(peers[i].allowed_net, peers[i].allowed_mask);
     }
-    std::sort(index.begin(), index.end(), [](const uint2 &a, const uint2 &b) { return a.x < b.x; });
-    for (uint32_t i = 1; i < n; i++)
-        if (index[i].x == index[i - 1].x)
-            return fail(ctx, BNK_E_INVAL, "local_index " + std::to_string(index[i].x) + " is used by two peers");
     // in-flight batches may still read the old tables
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
-    std::vector<uint64_t> zeros(n, 0);
-    int rc = upload(ctx, &ctx->wg_index, index.data(), (size_t)n * 8);
+    // A row whose index pair is unchanged is the same keypair (a handshake
+    // hands out fresh indices on both sides): it keeps its send counter, or its
+    // next packet would reuse a nonce under an unchanged key.  Any other row is
+    // a fresh keypair and starts at 0.
+    const uint32_t n_old = ctx->n_wg_peers;
+    std::vector<uint64_t> ctr(std::max(n, n_old), 0);
+    if (n_old)
+        HIPCHK(ctx, hipMemcpy(ctr.data(), ctx->wg_send_ctr.p, (size_t)n_old * 8, hipMemcpyDeviceToHost));
+    for (uint32_t i = 0; i < n; i++) {
+        const bool same = i < n_old && ctx->wg_rows[i].local_index == peers[i].local_index &&
+                          ctx->wg_rows[i].remote_index == peers[i].remote_index;
+        if (!same) ctr[i] = 0;
+    }
+    rc = upload(ctx, &ctx->wg_index, index.data(), (size_t)n * 8);
     if (!rc) rc = upload(ctx, &ctx->wg_remote, remote.data(), (size_t)n * 4);
     if (!rc) rc = upload(ctx, &ctx->wg_allowed, allowed.data(), (size_t)n * 8);
-    if (!rc) rc = upload(ctx, &ctx->wg_send_ctr, zeros.data(), (size_t)n * 8);
-    if (rc) return rc;
+    if (!rc) rc = upload(ctx, &ctx->wg_send_ctr, ctr.data(), (size_t)n * 8);
+    if (rc) {
+        ctx->n_wg_peers = 0; // a half-installed table is no table
+        ctx->wg_rows.clear();
+        return rc;
+    }
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream)); // the vectors above go away
+    ctx->wg_rows.assign(peers, peers + n);
     ctx->n_wg_peers = n;
+    return BNK_OK;
+}
+
+extern "C" int bnk_wg_peer_set(bnk_ctx *ctx, uint32_t row, const bnk_wg_peer *peer, const uint8_t *key_send32,
+                               const uint8_t *key_recv32)
+{
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    if (!peer) return fail(ctx, BNK_E_INVAL, "null peer");
+    if (row >= ctx->n_wg_peers) return fail(ctx, BNK_E_RANGE, "row beyond the peer table");
+    if ((key_send32 && row >= ctx->n_keys[BNK_KEYS_SEND]) || (key_recv32 && row >= ctx->n_keys[BNK_KEYS_RECV]))
+        return fail(ctx, BNK_E_RANGE, "row beyond the key table");
+    std::vector<bnk_wg_peer> rows = ctx->wg_rows;
+    rows[row] = *peer;
+    std::vector<uint2> index;
+    int rc = wg_build_index(ctx, rows.data(), (uint32_t)rows.size(), &index);
+    if (rc) return rc;
+    // in-flight batches may still read the old row
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    const uint2 allowed = make_uint2(peer->allowed_net, peer->allowed_mask);
+    const uint64_t zero = 0;
+    hipStream_t s = ctx->stream;
+    HIPCHK(ctx, hipMemcpyAsync(ctx->wg_index.p, index.data(), index.size() * 8, hipMemcpyHostToDevice, s));
+    HIPCHK(ctx, hipMemcpyAsync(ctx->wg_remote.as<uint32_t>() + row, &peer->remote_index, 4, hipMemcpyHostToDevice, s));
+    HIPCHK(ctx, hipMemcpyAsync(ctx->wg_allowed.as<uint2>() + row, &allowed, 8, hipMemcpyHostToDevice, s));
+    // this row's keypair is new: its nonces start over; every other row goes on
+    HIPCHK(ctx, hipMemcpyAsync(ctx->wg_send_ctr.as<uint64_t>() + row, &zero, 8, hipMemcpyHostToDevice, s));
+    if (key_send32)
+        HIPCHK(ctx, hipMemcpyAsync(ctx->d_keys[BNK_KEYS_SEND] + 8u * row, key_send32, 32, hipMemcpyHostToDevice, s));
+    if (key_recv32)
+        HIPCHK(ctx, hipMemcpyAsync(ctx->d_keys[BNK_KEYS_RECV] + 8u * row, key_recv32, 32, hipMemcpyHostToDevice, s));
+    HIPCHK(ctx, hipStreamSynchronize(s));
+    ctx->wg_rows.swap(rows);
+    return BNK_OK;
+}
+
+extern "C" int bnk_wg_send_counter_set(bnk_ctx *ctx, uint32_t row, uint64_t next)
+{
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    if (row >= ctx->n_wg_peers) return fail(ctx, BNK_E_RANGE, "row beyond the peer table");
+    if (next > WG_REJECT_AFTER_MESSAGES) next = WG_REJECT_AFTER_MESSAGES;
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    HIPCHK(ctx, hipMemcpy(ctx->wg_send_ctr.as<uint64_t>() + row, &next, 8, hipMemcpyHostToDevice));
     return BNK_OK;
 }
 
@@ -234,13 +306,15 @@ static int wg_encap_impl(bnk_ctx *ctx, const bnk_batch *slots, uint32_t mtu, uin
     // counters in batch order per peer, advancing the peers' send counters:
     // needs the peer array only, so it runs ahead of the packet bytes
     if (n <= PEER_RANK_SMALL_MAX) {
-        HIPCHK(ctx, launch_peer_rank_small(d_peer, pe.n, n, pe.send_ctr, d_ctr, true, ctx->d_status, ctx->stream));
+        HIPCHK(ctx, launch_peer_rank_small(d_peer, pe.n, n, pe.send_ctr, d_ctr, true, WG_REJECT_AFTER_MESSAGES,
+                                           ctx->d_status, ctx->stream));
     } else {
         HIPCHK(ctx, launch_wg_keys(d_peer, pe.n, n, ctx->r_keys.as<uint32_t>(), ctx->r_idx.as<uint32_t>(),
                                    ctx->d_status, ctx->stream));
         HIPCHK(ctx, launch_peer_rank(ctx->r_keys.as<uint32_t>(), ctx->r_idx.as<uint32_t>(),
                                      ctx->r_skeys.as<uint32_t>(), ctx->r_sidx.as<uint32_t>(), ctx->r_tmp.p,
-                                     tmp_bytes, pe.send_ctr, pe.n, n, d_ctr, true, ctx->stream));
+                                     tmp_bytes, pe.send_ctr, pe.n, n, d_ctr, true, WG_REJECT_AFTER_MESSAGES,
+                                     ctx->stream));
     }
 
     // filter.go:192-194: NoteOutbound does nothing in allow-all mode

@@ -153,7 +153,10 @@ __global__ __launch_bounds__(256) void wg_encap_prep_kernel(WgBatch b, uint8_t *
     const uint32_t i = b.first + t;
     const uint32_t pr = peer ? peer[i] : 0u;
     const uint32_t len = b.lens ? b.lens[i] : b.len;
-    if (pr >= pe.n) {
+    // a peer beyond the table, or a keypair that has used up its nonces
+    // (wireguard-go device/send.go: nothing is sent at RejectAfterMessages)
+    const uint64_t c = pr < pe.n ? counter[i] : 0;
+    if (pr >= pe.n || c >= WG_REJECT_AFTER_MESSAGES) {
         skip[i] = 1;
         padded_len[i] = 0;
         wire_len[i] = 0;
@@ -162,7 +165,6 @@ __global__ __launch_bounds__(256) void wg_encap_prep_kernel(WgBatch b, uint8_t *
     const uint64_t at = b.off ? b.off[i] : (uint64_t)i * b.stride;
     uint8_t *w = const_cast<uint8_t *>(b.base) + at;
     const uint32_t pad = wg_padding(len, mtu);
-    const uint64_t c = counter[i];
     const u32x4 hdr = {4u, pe.remote_index[pr], (uint32_t)c, (uint32_t)(c >> 32)};
     *reinterpret_cast<u32x4_unaligned *>(hdr_base + at) = hdr;
     for (uint32_t k = 0; k < pad; k++) w[16u + len + k] = 0;

@@ -20,6 +20,7 @@ KEYS_SEND, KEYS_RECV = 0, 1
 RELAY_OK, RELAY_FORGED, RELAY_DENIED = 0, 1, 2
 E_INVAL, E_NODEV, E_HIP, E_NOMEM, E_RANGE, E_STATE = -1, -2, -3, -4, -5, -6
 NOALLOC_MAX_PACKETS = 1 << 20
+WG_REJECT_AFTER_MESSAGES = (1 << 64) - (1 << 13) - 1
 
 PROBE_OPS = {"v_add_u32": 0, "v_xor_b32": 1, "v_alignbit_b32": 2, "v_mad_u64_u32": 3,
              "v_fma_f64": 4, "v_mul_lo_u32": 5, "v_add_f64": 6}
@@ -334,6 +335,18 @@ class Context:
         arr = np.ascontiguousarray(np.array(peers, dtype=np.uint32).reshape(-1, 4))
         self._chk(self._lib.bnk_wg_peers_set(self._h, C.c_void_p(arr.ctypes.data),
                                              C.c_uint32(arr.shape[0])))
+
+    def wg_peer_set(self, row: int, peer, key_send=None, key_recv=None) -> None:
+        """One peer's new keypair: replaces row `row` (peer table and both key
+        tables) and restarts only that row's send counter."""
+        arr = np.ascontiguousarray(np.array(peer, dtype=np.uint32).reshape(4))
+        ks = None if key_send is None else np.ascontiguousarray(key_send, dtype=np.uint8).reshape(32)
+        kr = None if key_recv is None else np.ascontiguousarray(key_recv, dtype=np.uint8).reshape(32)
+        self._chk(self._lib.bnk_wg_peer_set(self._h, C.c_uint32(row), C.c_void_p(arr.ctypes.data),
+                                            C.c_void_p(_ptr(ks)), C.c_void_p(_ptr(kr))))
+
+    def wg_send_counter_set(self, row: int, value: int) -> None:
+        self._chk(self._lib.bnk_wg_send_counter_set(self._h, C.c_uint32(row), C.c_uint64(value)))
 
     def wg_send_counters(self, n: int) -> np.ndarray:
         out = np.zeros(max(n, 1), np.uint64)

@@ -256,9 +256,23 @@ typedef struct bnk_wg_peer {
     uint32_t allowed_mask;
 } bnk_wg_peer;
 
-/* Installs the peer table; peer i uses row i of both key tables.  Resets
- * every peer's send counter to 0 (a fresh keypair starts there). */
+/* Installs the whole peer table; peer i uses row i of both key tables.  A row
+ * whose local_index and remote_index are both unchanged from the table before
+ * is the same keypair and keeps its send counter (a handshake hands out fresh
+ * indices, so an unchanged pair means an unchanged key, and restarting its
+ * counter would reuse nonces); every other row starts at 0.  Use it for a
+ * netmap push (peers added or removed); after one peer's handshake use
+ * bnk_wg_peer_set. */
 int bnk_wg_peers_set(bnk_ctx *ctx, const bnk_wg_peer *peers, uint32_t n);
+/* One peer's new keypair, where wireguard-go installs it after that peer's
+ * Noise handshake: replaces row `row` of the peer table and of both key tables
+ * (a null key pointer leaves that key as it is) and restarts that row's send
+ * counter at 0.  No other row changes: WireGuard peers rekey independently. */
+int bnk_wg_peer_set(bnk_ctx *ctx, uint32_t row, const bnk_wg_peer *peer,
+                    const uint8_t *key_send32, const uint8_t *key_recv32);
+/* Sets one row's next send counter (values above RejectAfterMessages are
+ * stored as RejectAfterMessages): for restoring state into a fresh context. */
+int bnk_wg_send_counter_set(bnk_ctx *ctx, uint32_t row, uint64_t next);
 /* Copies the next send counter of peers [0, n) to a host array. */
 int bnk_wg_send_counters(bnk_ctx *ctx, uint64_t *out, uint32_t n);
 /* Outgoing: slot i starts at slots' offset i with 16 bytes of headroom,
@@ -267,8 +281,11 @@ int bnk_wg_send_counters(bnk_ctx *ctx, uint64_t *out, uint32_t n);
  * mtu; mtu 0 = no cap), gives each packet its peer's next counter in batch
  * order, writes the header into the headroom and seals in place.
  * wire_len[i] = 16 + lens[i] + padding + 16, the datagram to send from the
- * slot's start.  slots->counters and counter0 are ignored.  wire_len lives
- * where slots->mem says. */
+ * slot's start.  A keypair stops sending when its counter reaches
+ * RejectAfterMessages = 2^64 - 2^13 - 1 (wireguard-go device/send.go): such a
+ * packet is left as it was, gets wire_len[i] = 0 and uses no counter, and the
+ * peer needs a new handshake (bnk_wg_peer_set).  slots->counters and counter0
+ * are ignored.  wire_len lives where slots->mem says. */
 int bnk_wg_encap_batch(bnk_ctx *ctx, const bnk_batch *slots, uint32_t mtu,
                        uint32_t *wire_len);
 /* Incoming: wire->lens[i] bytes at wire's offset i are one datagram.

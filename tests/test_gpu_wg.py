@@ -170,7 +170,7 @@ def test_encap_uniform_slots_one_peer_and_padding_rules(fused, length, mtu):
         got = ring if ring is not None else arena.copy()
         got[:] = arena
         got_len = np.zeros(n, np.uint32)
-        ctx.wg_peers_set(peers)  # counters start again at 0
+        ctx.wg_send_counter_set(0, 0)  # the same keypair from the start again (test only: reuses nonces)
         ctx.wg_encap(lib.make_batch(got, arena.nbytes, n, lib.MEM_HOST, stride=stride, length=length), mtu, got_len)
         assert np.array_equal(got_len, want_len), mem
         bad = np.flatnonzero(np.array(got) != want)
@@ -776,6 +776,9 @@ def test_random_framing_batches_round_trip_through_rings_and_pageable_memory():
     tx.keys_set(lib.KEYS_SEND, keys)
     rx.keys_set(lib.KEYS_RECV, keys)
     ring_t, ring_r, ring_o = tx.ring_alloc(3 << 20), rx.ring_alloc(3 << 20), rx.ring_alloc(3 << 20)
+    tx.wg_peers_set(peers_tx)
+    rx.wg_peers_set(peers_rx)
+    nxt = np.zeros(n_peers, np.uint64)  # the peers' send counters run on from batch to batch
     for it in range(40):
         n = int(rng.choice([1, 3, 64, 65, 200, 1024, 1025]))
         mtu = int(rng.choice([0, 1280, 1420]))
@@ -792,14 +795,14 @@ def test_random_framing_batches_round_trip_through_rings_and_pageable_memory():
                 arena[o] = 0x45
                 arena[o + 2:o + 4] = np.frombuffer(struct.pack(">H", length), np.uint8)
                 arena[o + 12:o + 16] = np.frombuffer(struct.pack(">I", peers_tx[int(peer[i])][2]), np.uint8)
-        tx.wg_peers_set(peers_tx)
-        rx.wg_peers_set(peers_rx)
+        if it % 8 == 7:
+            tx.wg_peers_set(peers_tx)  # the same table again: counters must not move
         spread = int(rng.choice([0, 4096]))
         tx.set_spread_max_packets(spread)
         rx.set_spread_max_packets(spread)
         in_rings = bool(rng.integers(0, 2))
         case = f"batch {it}: n={n} mtu={mtu} spread_max={spread} rings={in_rings}"
-        want, want_len, nxt = arena.copy(), np.zeros(n, np.uint32), np.zeros(n_peers, np.uint64)
+        want, want_len = arena.copy(), np.zeros(n, np.uint32)
         for i in range(n):
             p, o = int(peer[i]), int(off[i])
             w = O.wg_encap(arena[o + 16:o + 16 + int(lens[i])].tobytes(), mtu, keys[p].tobytes(),
@@ -988,6 +991,138 @@ def test_large_host_rings_take_the_chunked_route():
     rx.ring_free(out)
     tx.close()
     rx.close()
+
+
+def _encap_host(ctx, arena, off, lens, peer, mtu=MTU):
+    from bnk_amd import lib
+    got = arena.copy()
+    wl = np.zeros(len(lens), np.uint32)
+    ctx.wg_encap(lib.make_batch(got, got.nbytes, len(lens), lib.MEM_HOST, offsets=off, lens=lens, peer=peer),
+                 mtu, wl)
+    return got, wl
+
+
+@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("n", [400, 3000])
+def test_rekey_of_one_peer_leaves_the_other_counters_alone(fused, n):
+    """WireGuard peers rekey independently: installing peer A's new keypair
+    (bnk_wg_peer_set, or bnk_wg_peers_set with A's row changed) restarts A's
+    counter only; every other peer's next packet continues its sequence, so no
+    (key, nonce) pair is ever used twice."""
+    from oracle import binding as O
+    rng = np.random.default_rng(77)
+    peers = _peers(rng)
+    keys = rng.integers(0, 256, (N_PEERS, 32), dtype=np.uint8)
+    lens = rng.integers(20, 600, n).astype(np.uint32)
+    peer = rng.integers(0, N_PEERS, n).astype(np.uint32)
+    off, total = _layout(rng, 16 + lens.astype(np.int64) + 31)
+    arena = np.full(total, 0xEE, np.uint8)
+    plains = []
+    for i in range(n):
+        pt = _inner(rng, peers, int(peer[i]), int(lens[i]))
+        plains.append(pt)
+        arena[int(off[i]) + 16:int(off[i]) + 16 + len(pt)] = np.frombuffer(pt, np.uint8)
+    ctx = _ctx(peers, keys_send=keys, keys_recv=keys)
+    if not fused:
+        ctx.set_spread_max_packets(0)
+    next_ctr = np.zeros(N_PEERS, np.uint64)
+
+    def check_batch():
+        want = arena.copy()
+        for i in range(n):
+            p = int(peer[i])
+            w = O.wg_encap(plains[i], MTU, keys[p].tobytes(), peers[p][1], int(next_ctr[p]))
+            next_ctr[p] += 1
+            want[int(off[i]):int(off[i]) + len(w)] = np.frombuffer(w, np.uint8)
+        got, _ = _encap_host(ctx, arena, off, lens, peer)
+        assert np.array_equal(got, want)
+        assert np.array_equal(ctx.wg_send_counters(N_PEERS), next_ctr)
+
+    check_batch()
+    assert next_ctr.min() > 0
+    # peer 5 completes a handshake: new indices, new keys, counter back to 0
+    a = 5
+    peers[a] = (peers[a][0] ^ 0x5A5A0000, peers[a][1] ^ 0x00A5A500, peers[a][2], peers[a][3])
+    keys[a] = rng.integers(0, 256, 32, dtype=np.uint8)
+    ctx.wg_peer_set(a, peers[a], key_send=keys[a], key_recv=keys[a])
+    next_ctr[a] = 0
+    assert np.array_equal(ctx.wg_send_counters(N_PEERS), next_ctr)
+    check_batch()
+    # a netmap push re-installs the whole table: rows with unchanged indices go
+    # on counting, the row with fresh indices (peer 9 rekeyed) starts over, and
+    # a row added at the end starts at 0
+    b = 9
+    peers[b] = (peers[b][0] + 1, peers[b][1] + 1, peers[b][2], peers[b][3])
+    grown = peers + [(0x7F000001, 0x12345678, 0x64410001, 0xFFFFFFFF)]
+    keys = np.concatenate([keys, rng.integers(0, 256, (1, 32), dtype=np.uint8)])
+    from bnk_amd import lib
+    ctx.keys_set(lib.KEYS_SEND, keys)
+    ctx.wg_peers_set(grown)
+    next_ctr[b] = 0
+    got = ctx.wg_send_counters(N_PEERS + 1)
+    assert np.array_equal(got[:N_PEERS], next_ctr) and got[N_PEERS] == 0
+    ctx.wg_peers_set(peers)  # and shrinking keeps the rest
+    check_batch()
+    # a duplicate local index is refused and changes nothing
+    with pytest.raises(lib.BnkError) as ei:
+        ctx.wg_peer_set(3, (peers[4][0], 1, 2, 0xFFFFFFFF))
+    assert ei.value.code == lib.E_INVAL
+    with pytest.raises(lib.BnkError) as ei:
+        ctx.wg_peer_set(N_PEERS, peers[0])
+    assert ei.value.code == lib.E_RANGE
+    check_batch()
+    ctx.close()
+
+
+@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("n", [64, 2500])
+def test_keypair_stops_sending_at_reject_after_messages(fused, n):
+    """wireguard-go sends nothing under a keypair whose nonce counter has
+    reached RejectAfterMessages = 2^64 - 2^13 - 1 (device/send.go): such packets
+    come back with wire_len 0, untouched, and the counter stays at the limit."""
+    from bnk_amd import lib
+    from oracle import binding as O
+    rng = np.random.default_rng(78)
+    peers = _peers(rng)
+    keys = rng.integers(0, 256, (N_PEERS, 32), dtype=np.uint8)
+    lens = np.full(n, 100, np.uint32)
+    peer = (np.arange(n) % 2).astype(np.uint32)  # peers 0 and 1 alternate
+    off, total = _layout(rng, 16 + lens.astype(np.int64) + 31)
+    arena = np.full(total, 0xEE, np.uint8)
+    plains = []
+    for i in range(n):
+        pt = _inner(rng, peers, int(peer[i]), 100)
+        plains.append(pt)
+        arena[int(off[i]) + 16:int(off[i]) + 116] = np.frombuffer(pt, np.uint8)
+    ctx = _ctx(peers, keys_send=keys)
+    if not fused:
+        ctx.set_spread_max_packets(0)
+    limit = lib.WG_REJECT_AFTER_MESSAGES
+    ctx.wg_send_counter_set(0, limit - 3)
+    ctx.wg_send_counter_set(1, (1 << 40) + 7)
+    nxt = {0: limit - 3, 1: (1 << 40) + 7}
+    want = arena.copy()
+    want_len = np.zeros(n, np.uint32)
+    for i in range(n):
+        p = int(peer[i])
+        if nxt[p] >= limit:
+            continue
+        w = O.wg_encap(plains[i], MTU, keys[p].tobytes(), peers[p][1], nxt[p])
+        nxt[p] += 1
+        want[int(off[i]):int(off[i]) + len(w)] = np.frombuffer(w, np.uint8)
+        want_len[i] = len(w)
+    got, got_len = _encap_host(ctx, arena, off, lens, peer)
+    assert np.array_equal(got_len, want_len) and int((want_len[::2] > 0).sum()) == 3
+    assert np.array_equal(got, want)
+    ctr = ctx.wg_send_counters(2)
+    assert int(ctr[0]) == limit and int(ctr[1]) == (1 << 40) + 7 + n // 2
+    # nothing more goes out for peer 0 until it has a new keypair
+    got, got_len = _encap_host(ctx, arena, off, lens, peer)
+    assert not got_len[::2].any() and got_len[1::2].all()
+    ctx.wg_peer_set(0, (peers[0][0] + 2, peers[0][1], peers[0][2], peers[0][3]), key_send=keys[0])
+    got, got_len = _encap_host(ctx, arena, off, lens, peer)
+    assert got_len.all() and int(ctx.wg_send_counters(1)[0]) == n // 2
+    ctx.close()
 
 
 def test_wg_argument_errors():

@@ -436,18 +436,24 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const bool skipped = a.skip != nullptr && skip_ld != 0;
     const bool bad_peer = pr >= a.n_peers;
     const bool too_short = OPEN && len < 16u;
-    const bool have = in_batch && !skipped && !bad_peer && !too_short;
+    const uint64_t in_at = (a.in_off ? in_off_ld : (uint64_t)i * a.in_stride) + a.in_skip;
+    const uint64_t out_at = (a.out_off ? out_off_ld : (uint64_t)i * a.out_stride) + a.out_skip;
+    // seal reads len and writes len + 16, open reads len (tag included) and writes len - 16
+    const bool outside = beyond_arena(in_at, len, a.in_limit) ||
+                         beyond_arena(out_at, OPEN ? (too_short ? 0u : len - 16u) : len + 16u, a.out_limit);
+    const bool have = in_batch && !skipped && !bad_peer && !too_short && !outside;
     // the key table has at least one row
     const uint4 *kp = reinterpret_cast<const uint4 *>(a.keys + 8u * (bad_peer ? 0u : pr));
     const uint4 k0 = kp[0], k1 = kp[1];
-    if (in_batch && !skipped && (bad_peer || too_short)) {
+    if (in_batch && !skipped && (bad_peer || too_short || outside)) {
         if (bad_peer) status_raise(a.status, STATUS_PEER_RANGE);
+        else if (outside) status_raise(a.status, STATUS_BOUNDS);
         if (OPEN) a.verdict[i] = 0;
     }
     if (OPEN) len -= 16u;
     len = have ? len : 0u;
-    const uint8_t *src = a.in + (a.in_off ? in_off_ld : (uint64_t)i * a.in_stride) + a.in_skip;
-    uint8_t *dst = a.out + (a.out_off ? out_off_ld : (uint64_t)i * a.out_stride) + a.out_skip;
+    const uint8_t *src = a.in + in_at;
+    uint8_t *dst = a.out + out_at;
     src = have ? src : nullptr;
     dst = have ? dst : nullptr;
     const uint32_t k[8] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
@@ -497,6 +503,19 @@ __global__ __launch_bounds__(256) void aead_spread_kernel(AeadArgs a)
     const uint8_t *src = a.in + (a.in_off ? a.in_off[i] : (uint64_t)i * a.in_stride) + a.in_skip;
     uint8_t *dst = a.out + (a.out_off ? a.out_off[i] : (uint64_t)i * a.out_stride) + a.out_skip;
     uint64_t ctr = 0;
+    if (!WG) {
+        // (framing launches only run on layouts the host has checked)
+        const uint64_t in_at = (uint64_t)(src - a.in), out_at = (uint64_t)(dst - a.out);
+        const bool short_ct = OPEN && len < 16u;
+        if (beyond_arena(in_at, len, a.in_limit) ||
+            beyond_arena(out_at, OPEN ? (short_ct ? 0u : len - 16u) : len + 16u, a.out_limit)) {
+            if (lane == 0 && !(a.skip && a.skip[i] != 0)) {
+                status_raise(a.status, STATUS_BOUNDS);
+                if (OPEN) a.verdict[i] = 0;
+            }
+            return;
+        }
+    }
 
     // ---- my 64 bytes: loads first, they fly while everything below is looked
     // up and the block is computed.  Where the AEAD data lies and how long it

@@ -169,6 +169,7 @@ int aead_batch_host_direct(bnk_ctx *ctx, bool open, const bnk_batch *in, const b
 int aead_device_layout_check(bnk_ctx *ctx, bool open, const bnk_batch *in, const bnk_batch *out)
 {
     const uint32_t n = in->n;
+    if (in->bytes == 0 || out->bytes == 0) return fail(ctx, BNK_E_INVAL, "arena size 0");
     if (!in->offsets && !in->lens && ((uint64_t)(n - 1) * in->stride + in->len > in->bytes))
         return fail(ctx, BNK_E_INVAL, "in: uniform layout exceeds the arena");
     if (!out->offsets && !in->lens) {
@@ -224,6 +225,11 @@ int aead_batch(bnk_ctx *ctx, bool open, const bnk_batch *in, const bnk_batch *ou
         a.peer = in->peer;
         a.counters = in->counters;
         a.verdict = verdict;
+        // offsets and lengths in device memory cannot be checked here: the lanes do it
+        if (in->offsets || in->lens) {
+            a.in_limit = in->bytes;
+            a.out_limit = out->bytes;
+        }
         if (sort_scratch) {
             // the caller's scratch instead of the context's grow-only buffers
             a.order = nullptr;
@@ -279,16 +285,20 @@ int take_status(bnk_ctx *ctx, uint32_t *status)
 {
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
     volatile uint32_t *h = ctx->h_status;
-    *status = (h[STATUS_PEER_RANGE] ? STATUS_PEER_RANGE : 0u) | (h[STATUS_FLOWS_FULL] ? STATUS_FLOWS_FULL : 0u);
+    *status = (h[STATUS_PEER_RANGE] ? STATUS_PEER_RANGE : 0u) | (h[STATUS_FLOWS_FULL] ? STATUS_FLOWS_FULL : 0u) |
+              (h[STATUS_BOUNDS] ? STATUS_BOUNDS : 0u);
     if (*status) {
         h[STATUS_PEER_RANGE] = 0;
         h[STATUS_FLOWS_FULL] = 0;
+        h[STATUS_BOUNDS] = 0;
     }
     return BNK_OK;
 }
 
 int status_to_rc(bnk_ctx *ctx, uint32_t status)
 {
+    if (status & STATUS_BOUNDS)
+        return fail(ctx, BNK_E_INVAL, "a packet of a device-resident batch reaches beyond its arena (it was skipped)");
     if (status & STATUS_PEER_RANGE) return fail(ctx, BNK_E_RANGE, "peer index beyond the key table");
     if (status & STATUS_FLOWS_FULL) return fail(ctx, BNK_E_NOMEM, "flow table overflow");
     return BNK_OK;
@@ -300,6 +310,7 @@ extern "C" {
 
 int bnk_init(int device_ordinal, bnk_ctx **out)
 {
+    BNK_API_TRY
     if (!out) return fail(nullptr, BNK_E_INVAL, "null out pointer");
     *out = nullptr;
     int count = 0;
@@ -345,10 +356,12 @@ int bnk_init(int device_ordinal, bnk_ctx **out)
     ctx->alive = true;
     *out = ctx;
     return BNK_OK;
+    BNK_API_CATCH(nullptr)
 }
 
 void bnk_shutdown(bnk_ctx *ctx)
 {
+    try {
     if (!ctx) return;
     {
         std::lock_guard<std::mutex> lk(ctx->mu);
@@ -366,6 +379,8 @@ void bnk_shutdown(bnk_ctx *ctx)
                           &ctx->wg_outlen, &ctx->wg_padded, &ctx->wg_wirelen, &ctx->wg_skip})
             b->release();
         ctx->pin.release();
+        for (const bnk_ctx::Ring &r : ctx->rings) (void)hipHostFree(reinterpret_cast<void *>(r.host));
+        ctx->rings.clear();
         for (int w = 0; w < 2; w++)
             if (ctx->d_keys[w]) (void)hipFree(ctx->d_keys[w]);
         if (ctx->h_status) (void)hipHostFree(ctx->h_status);
@@ -379,26 +394,54 @@ void bnk_shutdown(bnk_ctx *ctx)
         if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
     }
     delete ctx;
+    } catch (...) {
+    }
 }
 
-const char *bnk_last_error(bnk_ctx *ctx) { return ctx ? ctx->err.c_str() : g_init_err.c_str(); }
+const char *bnk_last_error(bnk_ctx *ctx)
+{
+    // a copy of the caller's own: another thread may fail on the same context
+    // while this one reads
+    static thread_local std::string copy;
+    try {
+        if (ctx) {
+            std::lock_guard<std::mutex> lk(ctx->err_mu);
+            copy = ctx->err;
+        } else {
+            copy = g_init_err;
+        }
+    } catch (...) {
+        return "out of host memory";
+    }
+    return copy.c_str();
+}
 
 int bnk_ring_alloc(bnk_ctx *ctx, size_t bytes, void **host_pinned)
 {
+    BNK_API_TRY
     Guard g(ctx);
     if (g.rc) return g.rc;
     if (!host_pinned || bytes == 0) return fail(ctx, BNK_E_INVAL, "bad ring request");
     HIPCHK(ctx, hipHostMalloc(host_pinned, bytes, hipHostMallocDefault));
     void *dev = nullptr;
-    if (hipHostGetDevicePointer(&dev, *host_pinned, 0) == hipSuccess && dev)
+    if (hipHostGetDevicePointer(&dev, *host_pinned, 0) != hipSuccess) {
+        dev = nullptr; // the ring still works through the copying routes
+        (void)hipGetLastError();
+    }
+    try {
         ctx->rings.push_back({(uintptr_t)*host_pinned, (uint8_t *)dev, bytes});
-    else
-        (void)hipGetLastError(); // the ring still works through the copying routes
+    } catch (...) {
+        (void)hipHostFree(*host_pinned);
+        *host_pinned = nullptr;
+        throw;
+    }
     return BNK_OK;
+    BNK_API_CATCH(ctx)
 }
 
 int bnk_ring_free(bnk_ctx *ctx, void *host_pinned)
 {
+    BNK_API_TRY
     Guard g(ctx);
     if (g.rc) return g.rc;
     if (!host_pinned) return BNK_OK;
@@ -410,37 +453,45 @@ int bnk_ring_free(bnk_ctx *ctx, void *host_pinned)
         }
     HIPCHK(ctx, hipHostFree(host_pinned));
     return BNK_OK;
+    BNK_API_CATCH(ctx)
 }
 
 int bnk_set_spread_max_packets(bnk_ctx *ctx, uint32_t max_packets)
 {
+    BNK_API_TRY
     Guard g(ctx);
     if (g.rc) return g.rc;
     ctx->spread_max = max_packets;
     return BNK_OK;
+    BNK_API_CATCH(ctx)
 }
 
 int bnk_dev_alloc(bnk_ctx *ctx, size_t bytes, void **dev)
 {
+    BNK_API_TRY
     Guard g(ctx);
     if (g.rc) return g.rc;
     if (!dev || bytes == 0) return fail(ctx, BNK_E_INVAL, "bad device allocation request");
     HIPCHK(ctx, hipMalloc(dev, bytes));
     return BNK_OK;
+    BNK_API_CATCH(ctx)
 }
 
 int bnk_dev_free(bnk_ctx *ctx, void *dev)
 {
+    BNK_API_TRY
     Guard g(ctx);
     if (g.rc) return g.rc;
     if (!dev) return BNK_OK;
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
     HIPCHK(ctx, hipFree(dev));
     return BNK_OK;
+    BNK_API_CATCH(ctx)
 }
 
 int bnk_copy_to_device(bnk_ctx *ctx, void *dev, const void *host, size_t bytes)
 {
+    BNK_API_TRY
     Guard g(ctx);
     if (g.rc) return g.rc;
     if (bytes == 0) return BNK_OK;
@@ -448,10 +499,12 @@ int bnk_copy_to_device(bnk_ctx *ctx, void *dev, const void *host, size_t bytes)
     HIPCHK(ctx, hipMemcpyAsync(dev, host, bytes, hipMemcpyHostToDevice, ctx->stream));
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
     return BNK_OK;
+    BNK_API_CATCH(ctx)
 }
 
 int bnk_copy_to_host(bnk_ctx *ctx, void *host, const void *dev, size_t bytes)
 {
+    BNK_API_TRY
     Guard g(ctx);
     if (g.rc) return g.rc;
     if (bytes == 0) return BNK_OK;
@@ -459,22 +512,26 @@ int bnk_copy_to_host(bnk_ctx *ctx, void *host, const void *dev, size_t bytes)
     HIPCHK(ctx, hipMemcpyAsync(host, dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
     return BNK_OK;
+    BNK_API_CATCH(ctx)
 }
 
 int bnk_sync(bnk_ctx *ctx)
 {
+    BNK_API_TRY
     Guard g(ctx);
     if (g.rc) return g.rc;
     uint32_t status = 0;
     int rc = take_status(ctx, &status);
     if (rc) return rc;
     return status_to_rc(ctx, status);
+    BNK_API_CATCH(ctx)
 }
 
 void *bnk_stream(bnk_ctx *ctx) { return ctx ? (void *)ctx->stream : nullptr; }
 
 int bnk_keys_set(bnk_ctx *ctx, int which, const uint8_t *keys32, uint32_t n_peers)
 {
+    BNK_API_TRY
     Guard g(ctx);
     if (g.rc) return g.rc;
     if (which != BNK_KEYS_SEND && which != BNK_KEYS_RECV)
@@ -494,24 +551,30 @@ int bnk_keys_set(bnk_ctx *ctx, int which, const uint8_t *keys32, uint32_t n_peer
     ctx->d_keys[which] = nk;
     ctx->n_keys[which] = n_peers;
     return BNK_OK;
+    BNK_API_CATCH(ctx)
 }
 
 int bnk_aead_seal_batch(bnk_ctx *ctx, const bnk_batch *in, const bnk_batch *out)
 {
+    BNK_API_TRY
     Guard g(ctx);
     if (g.rc) return g.rc;
     return aead_batch(ctx, false, in, out, nullptr, nullptr);
+    BNK_API_CATCH(ctx)
 }
 
 int bnk_aead_open_batch(bnk_ctx *ctx, const bnk_batch *in, const bnk_batch *out, uint8_t *verdict)
 {
+    BNK_API_TRY
     Guard g(ctx);
     if (g.rc) return g.rc;
     return aead_batch(ctx, true, in, out, verdict, nullptr);
+    BNK_API_CATCH(ctx)
 }
 
 int bnk_probe_valu(bnk_ctx *ctx, int op, uint32_t iters, double *ops_per_sec)
 {
+    BNK_API_TRY
     Guard g(ctx);
     if (g.rc) return g.rc;
     if (!ops_per_sec || iters == 0 || op < 0 || op >= PROBE_OPS) return fail(ctx, BNK_E_INVAL, "bad probe request");
@@ -530,10 +593,12 @@ int bnk_probe_valu(bnk_ctx *ctx, int op, uint32_t iters, double *ops_per_sec)
     const double ops = (double)blocks * PROBE_THREADS * (double)iters * PROBE_CHAINS * PROBE_UNROLL;
     *ops_per_sec = ops / ((double)ms * 1e-3);
     return BNK_OK;
+    BNK_API_CATCH(ctx)
 }
 
 int bnk_probe_copy(bnk_ctx *ctx, size_t bytes, uint32_t iters, double *bytes_per_sec)
 {
+    BNK_API_TRY
     Guard g(ctx);
     if (g.rc) return g.rc;
     if (!bytes_per_sec || iters == 0 || bytes < 4096 || (bytes & 15))
@@ -564,6 +629,7 @@ int bnk_probe_copy(bnk_ctx *ctx, size_t bytes, uint32_t iters, double *bytes_per
     // bytes read plus bytes written
     *bytes_per_sec = 2.0 * (double)bytes * iters / ((double)ms * 1e-3);
     return BNK_OK;
+    BNK_API_CATCH(ctx)
 }
 
 } // extern "C"

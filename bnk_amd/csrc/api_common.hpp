@@ -15,12 +15,37 @@ namespace bnk {
 
 inline thread_local std::string g_init_err;
 
+// The error text has a lock of its own: bnk_last_error may be called by a
+// thread that does not hold the context lock.
 inline int fail(bnk_ctx *ctx, int code, const std::string &what)
 {
-    if (ctx) ctx->err = what;
-    else g_init_err = what;
+    if (ctx) {
+        std::lock_guard<std::mutex> lk(ctx->err_mu);
+        ctx->err = what;
+    } else {
+        g_init_err = what;
+    }
     return code;
 }
+
+// For the exception barrier: must not throw itself.
+inline int fail_caught(bnk_ctx *ctx, int code, const char *what) noexcept
+{
+    try {
+        return fail(ctx, code, what);
+    } catch (...) {
+        return code;
+    }
+}
+
+// Nothing may unwind into a C (cgo) caller: every extern "C" body sits between
+// these two.  The context lock (a Guard inside the body) is released by the
+// unwinding before the handler runs.
+#define BNK_API_TRY try {
+#define BNK_API_CATCH(ctx)                                                                   \
+    }                                                                                        \
+    catch (const std::bad_alloc &) { return bnk::fail_caught((ctx), BNK_E_NOMEM, "out of host memory"); } \
+    catch (...) { return bnk::fail_caught((ctx), BNK_E_HIP, "unexpected C++ exception inside the library"); }
 
 inline int fail_hip(bnk_ctx *ctx, const char *what, hipError_t e)
 {
@@ -113,7 +138,7 @@ inline uint8_t *ring_device_ptr(const bnk_ctx *ctx, const void *p, uint64_t byte
 {
     const uintptr_t a = (uintptr_t)p;
     for (const bnk_ctx::Ring &r : ctx->rings)
-        if (a >= r.host && bytes <= r.bytes && a - r.host <= r.bytes - bytes) return r.dev + (a - r.host);
+        if (r.dev && a >= r.host && bytes <= r.bytes && a - r.host <= r.bytes - bytes) return r.dev + (a - r.host);
     return nullptr;
 }
 

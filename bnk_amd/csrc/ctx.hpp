@@ -85,6 +85,7 @@ struct FilterState; // filter_host.hpp
 
 struct bnk_ctx {
     std::mutex mu;
+    std::mutex err_mu; // guards err alone
     int device = -1;
     hipStream_t stream = nullptr;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;

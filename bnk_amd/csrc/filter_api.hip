@@ -1,4 +1,6 @@
 // C ABI entry points of the packet filter (see include/bnkhip.h).
+#include <stdio.h>
+
 #include "api_common.hpp"
 #include "filter_host.hpp"
 #include "netmap_json.hpp"
@@ -222,6 +224,7 @@ void base_args(bnk_ctx *ctx, uint32_t n, int64_t now_ns, FilterArgs *a)
 
 int check_device_layout(bnk_ctx *ctx, const bnk_batch *b)
 {
+    if (b->n && b->bytes == 0) return fail(ctx, BNK_E_INVAL, "pkts: arena size 0");
     if (!b->offsets && !b->lens && b->n &&
         (uint64_t)(b->n - 1) * b->stride + b->len > b->bytes)
         return fail(ctx, BNK_E_INVAL, "pkts: uniform layout exceeds the arena");
@@ -258,6 +261,7 @@ int filter_batch(bnk_ctx *ctx, bool check, const bnk_batch *pkts, int64_t now_ns
         a.stride = pkts->stride;
         a.len = pkts->len;
         a.verdict = verdict;
+        if (pkts->offsets || pkts->lens) a.limit = pkts->bytes; // the lanes check what the host cannot read
         HIPCHK(ctx, check ? launch_filter_check(a, f->max_blocks, ctx->stream)
                           : launch_filter_note(a, f->max_blocks, f->claimed_upper > 4096, ctx->stream));
         return BNK_OK;
@@ -307,6 +311,7 @@ extern "C" {
 
 int bnk_filter_set_rules(bnk_ctx *ctx, const bnk_rule *rules, uint32_t n)
 {
+    BNK_API_TRY
     Guard g(ctx);
     if (g.rc) return g.rc;
     if (n && !rules) return fail(ctx, BNK_E_INVAL, "null rule array");
@@ -318,11 +323,13 @@ int bnk_filter_set_rules(bnk_ctx *ctx, const bnk_rule *rules, uint32_t n)
     HIPCHK(ctx, upload_rule_index(ctx->filter, h, ctx->stream));
     ctx->filter->enforce = true;
     return BNK_OK;
+    BNK_API_CATCH(ctx)
 }
 
 int bnk_rules_from_netmap_json(const char *json, size_t len, bnk_rule *out, uint32_t cap,
                                uint32_t *n_tuples, int *filter_enabled, char *err, size_t err_cap)
 {
+    BNK_API_TRY
     if (err && err_cap) err[0] = '\0';
     if (!json || !n_tuples || !filter_enabled || (cap && !out)) return BNK_E_INVAL;
     NetmapFilter nf;
@@ -339,10 +346,20 @@ int bnk_rules_from_netmap_json(const char *json, size_t len, bnk_rule *out, uint
     const size_t k = std::min<size_t>(cap, nf.tuples.size());
     if (k) memcpy(out, nf.tuples.data(), k * sizeof(bnk_rule));
     return BNK_OK;
+    }
+    catch (const std::bad_alloc &) {
+        if (err && err_cap) snprintf(err, err_cap, "out of host memory");
+        return BNK_E_NOMEM;
+    }
+    catch (...) {
+        if (err && err_cap) snprintf(err, err_cap, "unexpected C++ exception inside the library");
+        return BNK_E_HIP;
+    }
 }
 
 int bnk_filter_apply_netmap_json(bnk_ctx *ctx, const char *json, size_t len)
 {
+    BNK_API_TRY
     if (!ctx) return fail(nullptr, BNK_E_INVAL, "null context");
     if (!json) return fail(ctx, BNK_E_INVAL, "null document");
     NetmapFilter nf;
@@ -354,10 +371,12 @@ int bnk_filter_apply_netmap_json(bnk_ctx *ctx, const char *json, size_t len)
     // engine.go:279-283
     if (nf.filter_enabled) return bnk_filter_set_rules(ctx, nf.tuples.data(), (uint32_t)nf.tuples.size());
     return bnk_filter_set_allow_all(ctx);
+    BNK_API_CATCH(ctx)
 }
 
 int bnk_filter_set_allow_all(bnk_ctx *ctx)
 {
+    BNK_API_TRY
     Guard g(ctx);
     if (g.rc) return g.rc;
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
@@ -367,41 +386,51 @@ int bnk_filter_set_allow_all(bnk_ctx *ctx)
     HIPCHK(ctx, upload_rule_index(ctx->filter, h, ctx->stream));
     ctx->filter->enforce = false;
     return BNK_OK;
+    BNK_API_CATCH(ctx)
 }
 
 int bnk_filter_note_outbound_batch(bnk_ctx *ctx, const bnk_batch *pkts, int64_t now_ns)
 {
+    BNK_API_TRY
     Guard g(ctx);
     if (g.rc) return g.rc;
     return filter_batch(ctx, false, pkts, now_ns, nullptr);
+    BNK_API_CATCH(ctx)
 }
 
 int bnk_filter_check_inbound_batch(bnk_ctx *ctx, const bnk_batch *pkts, int64_t now_ns,
                                    uint8_t *verdict)
 {
+    BNK_API_TRY
     Guard g(ctx);
     if (g.rc) return g.rc;
     return filter_batch(ctx, true, pkts, now_ns, verdict);
+    BNK_API_CATCH(ctx)
 }
 
 int bnk_filter_note_outbound_ptrs(bnk_ctx *ctx, const uint8_t *const *pkts, const uint32_t *lens,
                                   uint32_t n, int64_t now_ns)
 {
+    BNK_API_TRY
     Guard g(ctx);
     if (g.rc) return g.rc;
     return filter_ptrs(ctx, false, pkts, lens, n, now_ns, nullptr);
+    BNK_API_CATCH(ctx)
 }
 
 int bnk_filter_check_inbound_ptrs(bnk_ctx *ctx, const uint8_t *const *pkts, const uint32_t *lens,
                                   uint32_t n, int64_t now_ns, uint8_t *verdict)
 {
+    BNK_API_TRY
     Guard g(ctx);
     if (g.rc) return g.rc;
     return filter_ptrs(ctx, true, pkts, lens, n, now_ns, verdict);
+    BNK_API_CATCH(ctx)
 }
 
 int bnk_filter_flow_count(bnk_ctx *ctx, uint32_t *count)
 {
+    BNK_API_TRY
     Guard g(ctx);
     if (g.rc) return g.rc;
     if (!count) return fail(ctx, BNK_E_INVAL, "null count");
@@ -411,11 +440,13 @@ int bnk_filter_flow_count(bnk_ctx *ctx, uint32_t *count)
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
     *count = c[FLOW_LIVE];
     return BNK_OK;
+    BNK_API_CATCH(ctx)
 }
 
 int bnk_filter_flow_dump(bnk_ctx *ctx, uint64_t *key, uint8_t *proto, int64_t *expiry_ns,
                          uint32_t cap, uint32_t *count)
 {
+    BNK_API_TRY
     Guard g(ctx);
     if (g.rc) return g.rc;
     if (!count || (cap && (!key || !proto || !expiry_ns))) return fail(ctx, BNK_E_INVAL, "null output");
@@ -439,6 +470,7 @@ int bnk_filter_flow_dump(bnk_ctx *ctx, uint64_t *key, uint8_t *proto, int64_t *e
     }
     *count = k;
     return BNK_OK;
+    BNK_API_CATCH(ctx)
 }
 
 } // extern "C"

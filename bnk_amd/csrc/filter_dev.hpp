@@ -70,6 +70,9 @@ struct FilterArgs {
     uint32_t *status;
     int64_t now;
     uint32_t n, stride, len;
+    uint64_t limit;       // arena size for device-resident batches with per-packet arrays: a
+                          // packet reaching beyond it is not read, fails the parse and
+                          // raises STATUS_BOUNDS.  0: the host has checked the layout
     uint32_t trim;        // bytes at the end of each packet that are not payload
     uint32_t small_in_lds; // set by the launcher: presence questions go to the folded bitmap in LDS
     RuleIndexDev rules;

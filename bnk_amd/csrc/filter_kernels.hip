@@ -281,9 +281,14 @@ __global__ __launch_bounds__(FILTER_THREADS, 8) void filter_check_kernel(FilterA
         bool valid = i < a.n && !(a.gate && a.gate[i] == 0);
         Parsed h{};
         if (valid) {
-            const uint8_t *p = a.pkts + (a.off ? a.off[i] : (uint64_t)i * a.stride);
+            const uint64_t at = a.off ? a.off[i] : (uint64_t)i * a.stride;
             const uint32_t len = a.lens ? a.lens[i] : a.len;
-            valid = parse_packet(p, len - (len >= a.trim ? a.trim : len), h);
+            if (beyond_arena(at, len, a.limit)) {
+                status_raise(a.status, STATUS_BOUNDS);
+                valid = false;
+            } else {
+                valid = parse_packet(a.pkts + at, len - (len >= a.trim ? a.trim : len), h);
+            }
         }
         uint32_t key = 0, iv = 0;
         bool maybe = false;
@@ -351,8 +356,13 @@ __global__ __launch_bounds__(256) void filter_note_kernel(FilterArgs a)
 {
     const uint32_t stride = gridDim.x * 256u;
     for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < a.n; i += stride) {
-        const uint8_t *p = a.pkts + (a.off ? a.off[i] : (uint64_t)i * a.stride);
+        const uint64_t at = a.off ? a.off[i] : (uint64_t)i * a.stride;
         const uint32_t len = a.lens ? a.lens[i] : a.len;
+        if (beyond_arena(at, len, a.limit)) {
+            status_raise(a.status, STATUS_BOUNDS);
+            continue;
+        }
+        const uint8_t *p = a.pkts + at;
         Parsed h;
         if (!parse_packet(p, len, h)) continue;
         // remote = dst, remotePort = dstPort, localPort = srcPort

@@ -72,6 +72,10 @@ struct AeadArgs {
     uint32_t n_peers;
     uint32_t trim;             // seal only: lens[i] - trim is the plaintext length
     uint32_t in_skip, out_skip; // bytes between a packet's offset and its AEAD data
+    uint64_t in_limit, out_limit; // arena sizes for batches whose per-packet arrays the host cannot
+                               // read (device resident): a packet reaching beyond them is left
+                               // alone, gets verdict 0 and raises STATUS_BOUNDS.  0: the host
+                               // has checked the layout
     uint32_t first;            // the launch covers packets first .. first+n-1; order[] is relative to first
     uint32_t spread_max;       // launches of at most this many packets run one wave per packet
     WgFuse wg;                 // only with aead_runs_spread(); mode 0: plain AEAD
@@ -86,8 +90,14 @@ constexpr uint32_t SPREAD_MAX_PACKETS = 4096;
 // plain store of 1 (the same store from every lane that has the news, so no
 // atomic is needed), and read by the host after it has waited for the stream,
 // with no copy.
-enum : uint32_t { STATUS_PEER_RANGE = 1u, STATUS_FLOWS_FULL = 2u };
-constexpr uint32_t STATUS_WORDS = 4; // word [bit value] holds that condition
+enum : uint32_t { STATUS_PEER_RANGE = 1u, STATUS_FLOWS_FULL = 2u, STATUS_BOUNDS = 4u };
+constexpr uint32_t STATUS_WORDS = 8; // word [bit value] holds that condition
+
+// True when [off, off + len) does not fit an arena of `limit` bytes (limit 0: not checked).
+__host__ __device__ inline bool beyond_arena(uint64_t off, uint64_t len, uint64_t limit)
+{
+    return limit != 0 && (off > limit || len > limit - off);
+}
 #if defined(__HIPCC__)
 __device__ inline void status_raise(uint32_t *status, uint32_t condition)
 {

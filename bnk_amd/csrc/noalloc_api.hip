@@ -47,6 +47,7 @@ int noalloc_setup(bnk_ctx *ctx, int device)
 
 extern "C" int bnk_aead_seal_batch_noalloc(bnk_ctx *ctx, const bnk_batch *in, const bnk_batch *out)
 {
+    BNK_API_TRY
     Guard g(ctx);
     if (g.rc) return g.rc;
     if (!in || !out) return fail(ctx, BNK_E_INVAL, "null batch");
@@ -64,4 +65,5 @@ extern "C" int bnk_aead_seal_batch_noalloc(bnk_ctx *ctx, const bnk_batch *in, co
     // length grouping itself (a fill kernel), order[] and cursor[] are written
     // before they are read.
     return aead_batch(ctx, false, in, out, nullptr, ptr);
+    BNK_API_CATCH(ctx)
 }

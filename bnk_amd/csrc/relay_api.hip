@@ -18,6 +18,7 @@ extern "C" int bnk_relay_fused_batch(bnk_ctx *ctx, const bnk_batch *in, const ui
                                      int64_t now_ns, const bnk_batch *out, uint8_t *verdict,
                                      uint64_t *ctr_out)
 {
+    BNK_API_TRY
     Guard g(ctx);
     if (g.rc) return g.rc;
     int rc = check_batch_common(ctx, in, "in");
@@ -52,6 +53,7 @@ extern "C" int bnk_relay_fused_batch(bnk_ctx *ctx, const bnk_batch *in, const ui
     uint8_t *d_verdict = nullptr;
     uint64_t *d_ctr_out = nullptr;
     uint64_t plain_bytes = 0;
+    uint64_t seal_out_limit = 0;
     Staged st;
     // direct route (small batches in pinned rings): the datagrams are fetched by
     // a copy kernel, the re-sealed ones written straight into the out ring, the
@@ -202,6 +204,12 @@ extern "C" int bnk_relay_fused_batch(bnk_ctx *ctx, const bnk_batch *in, const ui
         d_out = (uint8_t *)out->base;
         d_out_off = out->offsets;
         plain_bytes = in->bytes;
+        if (in->bytes == 0 || out->bytes == 0) return fail(ctx, BNK_E_INVAL, "arena size 0");
+        if (in->offsets || in->lens || out->offsets) {
+            // what the host cannot read the lanes check; the plaintext scratch mirrors the input arena
+            op.in_limit = op.out_limit = in->bytes;
+            seal_out_limit = out->bytes;
+        }
         d_peer_out = peer_out;
         d_ctr_base = ctr_base_out;
         d_verdict = verdict;
@@ -289,6 +297,8 @@ extern "C" int bnk_relay_fused_batch(bnk_ctx *ctx, const bnk_batch *in, const ui
         se.trim = 16;
         se.peer = d_peer_out;
         se.counters = d_ctr_out;
+        se.in_limit = op.in_limit;
+        se.out_limit = seal_out_limit;
         se.skip = d_verdict; // BNK_RELAY_OK is 0
         se.order = o.order;
         HIPCHK(ctx, launch_aead_seal(se, ctx->stream));
@@ -329,4 +339,5 @@ extern "C" int bnk_relay_fused_batch(bnk_ctx *ctx, const bnk_batch *in, const ui
     rc = take_status(ctx, &status);
     if (rc) return rc;
     return status_to_rc(ctx, status);
+    BNK_API_CATCH(ctx)
 }

@@ -49,6 +49,7 @@ static int wg_build_index(bnk_ctx *ctx, const bnk_wg_peer *peers, uint32_t n, st
 
 extern "C" int bnk_wg_peers_set(bnk_ctx *ctx, const bnk_wg_peer *peers, uint32_t n)
 {
+    BNK_API_TRY
     Guard g(ctx);
     if (g.rc) return g.rc;
     if (!peers || n == 0) return fail(ctx, BNK_E_INVAL, "empty peer table");
@@ -88,11 +89,13 @@ extern "C" int bnk_wg_peers_set(bnk_ctx *ctx, const bnk_wg_peer *peers, uint32_t
     ctx->wg_rows.assign(peers, peers + n);
     ctx->n_wg_peers = n;
     return BNK_OK;
+    BNK_API_CATCH(ctx)
 }
 
 extern "C" int bnk_wg_peer_set(bnk_ctx *ctx, uint32_t row, const bnk_wg_peer *peer, const uint8_t *key_send32,
                                const uint8_t *key_recv32)
 {
+    BNK_API_TRY
     Guard g(ctx);
     if (g.rc) return g.rc;
     if (!peer) return fail(ctx, BNK_E_INVAL, "null peer");
@@ -121,10 +124,12 @@ extern "C" int bnk_wg_peer_set(bnk_ctx *ctx, uint32_t row, const bnk_wg_peer *pe
     HIPCHK(ctx, hipStreamSynchronize(s));
     ctx->wg_rows.swap(rows);
     return BNK_OK;
+    BNK_API_CATCH(ctx)
 }
 
 extern "C" int bnk_wg_send_counter_set(bnk_ctx *ctx, uint32_t row, uint64_t next)
 {
+    BNK_API_TRY
     Guard g(ctx);
     if (g.rc) return g.rc;
     if (row >= ctx->n_wg_peers) return fail(ctx, BNK_E_RANGE, "row beyond the peer table");
@@ -132,10 +137,12 @@ extern "C" int bnk_wg_send_counter_set(bnk_ctx *ctx, uint32_t row, uint64_t next
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
     HIPCHK(ctx, hipMemcpy(ctx->wg_send_ctr.as<uint64_t>() + row, &next, 8, hipMemcpyHostToDevice));
     return BNK_OK;
+    BNK_API_CATCH(ctx)
 }
 
 extern "C" int bnk_wg_send_counters(bnk_ctx *ctx, uint64_t *out, uint32_t n)
 {
+    BNK_API_TRY
     Guard g(ctx);
     if (g.rc) return g.rc;
     if (!out) return fail(ctx, BNK_E_INVAL, "null out pointer");
@@ -144,6 +151,7 @@ extern "C" int bnk_wg_send_counters(bnk_ctx *ctx, uint64_t *out, uint32_t n)
     HIPCHK(ctx, hipMemcpyAsync(out, ctx->wg_send_ctr.p, (size_t)n * 8, hipMemcpyDeviceToHost, ctx->stream));
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
     return BNK_OK;
+    BNK_API_CATCH(ctx)
 }
 
 // bnk_wg_encap_batch, with NoteOutbound at *note_now on the plaintexts first
@@ -280,9 +288,11 @@ static int wg_encap_impl(bnk_ctx *ctx, const bnk_batch *slots, uint32_t mtu, uin
         if (!slots->offsets && !slots->lens &&
             (uint64_t)(n - 1) * slots->stride + slot_ext(0) > slots->bytes)
             return fail(ctx, BNK_E_INVAL, "slots: uniform layout exceeds the arena");
+        if (slots->bytes == 0) return fail(ctx, BNK_E_INVAL, "slots: arena size 0");
         b.base = (const uint8_t *)slots->base;
         b.off = slots->offsets;
         b.lens = slots->lens;
+        if (slots->offsets || slots->lens) b.limit = slots->bytes; // the lanes check what the host cannot read
         d_peer = slots->peer;
         d_wire_len = wire_len;
     }
@@ -371,7 +381,8 @@ static int wg_encap_impl(bnk_ctx *ctx, const bnk_batch *slots, uint32_t mtu, uin
                 return BNK_OK;
             }
         }
-        HIPCHK(ctx, launch_wg_encap_prep(c, sealed, pe, d_peer, d_ctr, mtu, d_padded, d_wire_len, d_skip, ctx->stream));
+        HIPCHK(ctx, launch_wg_encap_prep(c, sealed, pe, d_peer, d_ctr, mtu, d_padded, d_wire_len, d_skip, ctx->d_status,
+                                         ctx->stream));
         AeadArgs se{};
         se.spread_max = ctx->spread_max;
         se.keys = ctx->d_keys[BNK_KEYS_SEND];
@@ -436,17 +447,21 @@ static int wg_encap_impl(bnk_ctx *ctx, const bnk_batch *slots, uint32_t mtu, uin
 
 extern "C" int bnk_wg_encap_batch(bnk_ctx *ctx, const bnk_batch *slots, uint32_t mtu, uint32_t *wire_len)
 {
+    BNK_API_TRY
     Guard g(ctx);
     if (g.rc) return g.rc;
     return wg_encap_impl(ctx, slots, mtu, wire_len, nullptr);
+    BNK_API_CATCH(ctx)
 }
 
 extern "C" int bnk_wg_note_encap_batch(bnk_ctx *ctx, const bnk_batch *slots, uint32_t mtu, int64_t now_ns,
                                        uint32_t *wire_len)
 {
+    BNK_API_TRY
     Guard g(ctx);
     if (g.rc) return g.rc;
     return wg_encap_impl(ctx, slots, mtu, wire_len, &now_ns);
+    BNK_API_CATCH(ctx)
 }
 
 // bnk_wg_decap_batch, with CheckInbound at *check_now on the delivered
@@ -603,11 +618,18 @@ static int wg_decap_impl(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *o
         if (!out->offsets && !wire->lens &&
             (uint64_t)(n - 1) * out->stride + (wire->len >= 32u ? wire->len - 32u : 0u) > out->bytes)
             return fail(ctx, BNK_E_INVAL, "out: uniform layout exceeds the arena");
+        if (wire->bytes == 0 || out->bytes == 0) return fail(ctx, BNK_E_INVAL, "arena size 0");
         wb.base = (const uint8_t *)wire->base;
         wb.off = wire->offsets;
         wb.lens = wire->lens;
         ob.base = (const uint8_t *)out->base;
         ob.off = out->offsets;
+        if (wire->offsets || wire->lens || out->offsets) {
+            // the lanes check what the host cannot read: the datagram where it is
+            // parsed, the plaintext where it is written
+            wb.limit = wire->bytes;
+            ob.limit = out->bytes;
+        }
         d_result = result;
         d_out_len = out_len;
         d_peer = peer;
@@ -684,7 +706,7 @@ static int wg_decap_impl(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *o
                 return filter_range(lo, hi);
             }
         }
-        HIPCHK(ctx, launch_wg_parse(cw, pe, d_peer, d_counter, d_ctlen, d_result, ctx->stream));
+        HIPCHK(ctx, launch_wg_parse(cw, pe, d_peer, d_counter, d_ctlen, d_result, ctx->d_status, ctx->stream));
         AeadArgs op{};
         op.spread_max = ctx->spread_max;
         op.keys = ctx->d_keys[BNK_KEYS_RECV];
@@ -703,6 +725,7 @@ static int wg_decap_impl(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *o
         op.peer = d_peer;
         op.counters = d_counter;
         op.verdict = d_auth;
+        op.out_limit = ob.limit; // (the datagram's own bounds were checked by the parse)
         op.skip = d_result; // BNK_WG_OK is 0: header failures are not opened
         if (wire->lens && op.n > 64 && !aead_runs_spread(op)) {
             HIPCHK(ctx, launch_length_sort(d_ctlen + lo, op.n, 16, ctx->order.as<uint32_t>() + lo,
@@ -754,16 +777,20 @@ static int wg_decap_impl(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *o
 extern "C" int bnk_wg_decap_batch(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *out,
                                   uint8_t *result, uint32_t *out_len, uint32_t *peer, uint64_t *counter)
 {
+    BNK_API_TRY
     Guard g(ctx);
     if (g.rc) return g.rc;
     return wg_decap_impl(ctx, wire, out, result, out_len, peer, counter, nullptr);
+    BNK_API_CATCH(ctx)
 }
 
 extern "C" int bnk_wg_decap_filter_batch(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *out,
                                          int64_t now_ns, uint8_t *result, uint32_t *out_len,
                                          uint32_t *peer, uint64_t *counter)
 {
+    BNK_API_TRY
     Guard g(ctx);
     if (g.rc) return g.rc;
     return wg_decap_impl(ctx, wire, out, result, out_len, peer, counter, &now_ns);
+    BNK_API_CATCH(ctx)
 }

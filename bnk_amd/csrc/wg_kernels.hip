@@ -32,7 +32,7 @@ constexpr uint32_t WG_LDS_PEERS_MAX = 8192; // 64 KiB of (index, peer) pairs
 // would otherwise each go out to L2); the header comes in with one load.
 __global__ __launch_bounds__(256) void wg_parse_kernel(WgBatch b, WgPeersDev pe, uint32_t *peer,
                                                        uint64_t *counter, uint32_t *ct_len,
-                                                       uint8_t *result)
+                                                       uint8_t *result, uint32_t *status)
 {
     extern __shared__ uint2 ltab[];
     const bool in_lds = pe.n <= WG_LDS_PEERS_MAX;
@@ -44,11 +44,17 @@ __global__ __launch_bounds__(256) void wg_parse_kernel(WgBatch b, WgPeersDev pe,
     const uint32_t t = blockIdx.x * 256u + threadIdx.x;
     if (t >= b.n) return;
     const uint32_t i = b.first + t;
-    const uint8_t *w = b.base + (b.off ? b.off[i] : (uint64_t)i * b.stride);
+    const uint64_t at = b.off ? b.off[i] : (uint64_t)i * b.stride;
+    const uint8_t *w = b.base + at;
     const uint32_t len = b.lens ? b.lens[i] : b.len;
     peer[i] = 0xFFFFFFFFu;
     counter[i] = 0;
     ct_len[i] = 0;
+    if (beyond_arena(at, len, b.limit)) {
+        status_raise(status, STATUS_BOUNDS);
+        result[i] = BNK_WG_BAD_HEADER;
+        return;
+    }
     if (len < 32u) {
         result[i] = BNK_WG_BAD_HEADER;
         return;
@@ -146,7 +152,7 @@ __global__ __launch_bounds__(256) void wg_keys_kernel(const uint32_t *peer, uint
 __global__ __launch_bounds__(256) void wg_encap_prep_kernel(WgBatch b, uint8_t *hdr_base, WgPeersDev pe, const uint32_t *peer,
                                                             const uint64_t *counter, uint32_t mtu,
                                                             uint32_t *padded_len, uint32_t *wire_len,
-                                                            uint8_t *skip)
+                                                            uint8_t *skip, uint32_t *status)
 {
     const uint32_t t = blockIdx.x * 256u + threadIdx.x;
     if (t >= b.n) return;
@@ -156,15 +162,17 @@ __global__ __launch_bounds__(256) void wg_encap_prep_kernel(WgBatch b, uint8_t *
     // a peer beyond the table, or a keypair that has used up its nonces
     // (wireguard-go device/send.go: nothing is sent at RejectAfterMessages)
     const uint64_t c = pr < pe.n ? counter[i] : 0;
-    if (pr >= pe.n || c >= WG_REJECT_AFTER_MESSAGES) {
+    const uint64_t at = b.off ? b.off[i] : (uint64_t)i * b.stride;
+    const uint32_t pad = wg_padding(len, mtu);
+    const bool outside = beyond_arena(at, 16ull + len + pad + 16ull, b.limit);
+    if (outside) status_raise(status, STATUS_BOUNDS);
+    if (pr >= pe.n || c >= WG_REJECT_AFTER_MESSAGES || outside) {
         skip[i] = 1;
         padded_len[i] = 0;
         wire_len[i] = 0;
         return;
     }
-    const uint64_t at = b.off ? b.off[i] : (uint64_t)i * b.stride;
     uint8_t *w = const_cast<uint8_t *>(b.base) + at;
-    const uint32_t pad = wg_padding(len, mtu);
     const u32x4 hdr = {4u, pe.remote_index[pr], (uint32_t)c, (uint32_t)(c >> 32)};
     *reinterpret_cast<u32x4_unaligned *>(hdr_base + at) = hdr;
     for (uint32_t k = 0; k < pad; k++) w[16u + len + k] = 0;
@@ -190,7 +198,7 @@ hipError_t launch_wg_mark_filtered(uint8_t *result, const uint8_t *pass, uint32_
 }
 
 hipError_t launch_wg_parse(const WgBatch &b, const WgPeersDev &pe, uint32_t *peer, uint64_t *counter,
-                           uint32_t *ct_len, uint8_t *result, hipStream_t s)
+                           uint32_t *ct_len, uint8_t *result, uint32_t *status, hipStream_t s)
 {
     if (b.n == 0) return hipSuccess;
     const uint32_t lds = pe.n <= WG_LDS_PEERS_MAX ? pe.n * 8u : 0u;
@@ -200,7 +208,7 @@ hipError_t launch_wg_parse(const WgBatch &b, const WgPeersDev &pe, uint32_t *pee
                                            (int)(WG_LDS_PEERS_MAX * 8u));
         if (e != hipSuccess) return e;
     }
-    hipLaunchKernelGGL(wg_parse_kernel, grid_of(b.n), dim3(256), lds, s, b, pe, peer, counter, ct_len, result);
+    hipLaunchKernelGGL(wg_parse_kernel, grid_of(b.n), dim3(256), lds, s, b, pe, peer, counter, ct_len, result, status);
     return hipGetLastError();
 }
 
@@ -224,11 +232,11 @@ hipError_t launch_wg_keys(const uint32_t *peer, uint32_t n_peers, uint32_t n, ui
 
 hipError_t launch_wg_encap_prep(const WgBatch &b, uint8_t *hdr_base, const WgPeersDev &pe, const uint32_t *peer,
                                 const uint64_t *counter, uint32_t mtu, uint32_t *padded_len,
-                                uint32_t *wire_len, uint8_t *skip, hipStream_t s)
+                                uint32_t *wire_len, uint8_t *skip, uint32_t *status, hipStream_t s)
 {
     if (b.n == 0) return hipSuccess;
     hipLaunchKernelGGL(wg_encap_prep_kernel, grid_of(b.n), dim3(256), 0, s, b, hdr_base, pe, peer, counter, mtu,
-                       padded_len, wire_len, skip);
+                       padded_len, wire_len, skip, status);
     return hipGetLastError();
 }
 

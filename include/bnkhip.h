@@ -65,7 +65,15 @@ enum { BNK_KEYS_SEND = 0, BNK_KEYS_RECV = 1 };
  */
 typedef struct bnk_batch {
     void *base;              /* arena */
-    uint64_t bytes;          /* arena size; every packet must lie inside it */
+    uint64_t bytes;          /* arena size; every packet must lie inside it.
+                                Host batches are checked before anything runs
+                                (BNK_E_INVAL).  Device batches whose offsets or
+                                lengths are device arrays are checked by the
+                                kernels: a packet reaching beyond the arena is
+                                neither read nor written (verdict 0, wire_len
+                                0, BNK_WG_BAD_HEADER, BNK_RELAY_FORGED), the
+                                rest of the batch runs, and the next bnk_sync
+                                returns BNK_E_INVAL */
     uint32_t n;              /* packets */
     uint32_t mem;            /* BNK_MEM_HOST or BNK_MEM_DEVICE: applies to base
                                 and to every array below */

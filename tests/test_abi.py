@@ -87,3 +87,31 @@ def test_rule_flattening_matches_reference_semantics():
         (W.ip("1.2.3.4"), 0xFFFFFFFF, 0, 0, 1),
         (0, 0, 7, 8, 17),
     ]
+
+
+def test_allocation_failure_inside_the_library_is_an_error_code_not_an_unwind():
+    """Nothing may throw across the C boundary: with the address space capped,
+    parsing a netmap document that needs more memory than is left must come
+    back as BNK_E_NOMEM (the std::bad_alloc is caught at the boundary), not
+    abort the process.  Runs in a child process because of the cap."""
+    import subprocess
+    import sys
+    code = r'''
+import ctypes as C, resource, sys
+sys.path.insert(0, %r)
+from bnk_amd import lib
+so = lib.load()
+rule = b'{"srcs":["100.64.0.7/32","100.64.9.0/24"],"proto":"tcp","ports":[{"first":22,"last":22},{"first":80,"last":90}]},'
+doc = b'{"filter_enabled":true,"filter":[' + rule * 1000000
+doc = doc[:-1] + b']}'
+vm = [int(l.split()[1]) * 1024 for l in open("/proc/self/status") if l.startswith("VmSize")][0]
+resource.setrlimit(resource.RLIMIT_AS, (vm + (48 << 20), vm + (48 << 20)))
+n = C.c_uint32(); en = C.c_int(); err = C.create_string_buffer(256)
+arr = (lib.Rule * 16)()
+rc = so.bnk_rules_from_netmap_json(doc, C.c_size_t(len(doc)), arr, C.c_uint32(16), C.byref(n),
+                                   C.byref(en), err, C.c_size_t(256))
+print("rc", rc, err.value.decode())
+''' % ROOT
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr[-400:]
+    assert r.stdout.strip() == "rc -4 out of host memory"

@@ -8,6 +8,8 @@
 // one-time key; data uses blocks 1..; the MAC covers the zero-padded
 // ciphertext and one length block.
 #include "aead_lane.hpp"
+#include <stdlib.h>
+
 #include <algorithm>
 
 #include "../../include/bnkhip.h"
@@ -69,6 +71,19 @@ BNK_DEV void st_partial(uint8_t *p, uint4 v, uint32_t m)
 #pragma unroll
     for (int i = 0; i < 15; i++)
         if ((uint32_t)i < m) st8(p + i, (uint8_t)(w[i >> 2] >> (8 * (i & 3))));
+}
+
+// The same for a 16-byte aligned p: dwords, then a halfword, then a byte.
+BNK_DEV void st_partial_aligned(uint8_t *p, uint4 v, uint32_t m)
+{
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    const uint32_t nd = m >> 2;
+#pragma unroll
+    for (int q = 0; q < 3; q++)
+        if ((uint32_t)q < nd) *reinterpret_cast<BNK_GLOBAL uint32_t *>((uintptr_t)(p + 4 * q)) = w[q];
+    const uint32_t last = nd == 0 ? w[0] : nd == 1 ? w[1] : nd == 2 ? w[2] : w[3];
+    if (m & 2u) *reinterpret_cast<BNK_GLOBAL uint16_t *>((uintptr_t)(p + 4u * nd)) = (uint16_t)last;
+    if (m & 1u) st8(p + 4u * nd + (m & 2u), (uint8_t)(last >> (8u * (m & 2u))));
 }
 
 // Keeps the low m (0..16) bytes of a 16-byte little-endian value.
@@ -144,6 +159,22 @@ BNK_DEV void crypt_tail(Poly32 &mac, const uint32_t (&x)[16], int j, const uint8
     if (OPEN) mac.block(v.x, v.y, v.z, v.w);
     else mac.block(o.x, o.y, o.z, o.w);
     st_partial(d, o, m);
+}
+
+// The same when the cell holding those bytes has come into LDS with the rest of
+// its line (bytes beyond the packet are whatever memory held: masked off) and
+// the destination is 16-byte aligned.
+template <bool OPEN>
+BNK_DEV void crypt_tail_lds(Poly32 &mac, const uint32_t (&x)[16], int j, const uint8_t *cell, uint8_t *d,
+                            uint32_t m)
+{
+    const uint4 raw = *reinterpret_cast<const uint4 *>(cell);
+    const uint4 v = keep_bytes(raw, m);
+    const uint4 o = keep_bytes(make_uint4(v.x ^ x[4 * j], v.y ^ x[4 * j + 1], v.z ^ x[4 * j + 2],
+                                          v.w ^ x[4 * j + 3]), m);
+    if (OPEN) mac.block(v.x, v.y, v.z, v.w);
+    else mac.block(o.x, o.y, o.z, o.w);
+    st_partial_aligned(d, o, m);
 }
 
 template <bool OPEN>
@@ -226,20 +257,23 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
     // byte.  Stream position K lives in line K / 8 and in ring cell K % 16.
     const uint32_t skew = (uint32_t)(uintptr_t)src & 127u;
     const uint32_t c0 = skew >> 4;
-    const uint32_t ncell = len >> 4; // whole cells; a shorter tail is handled by its owner
+    const uint32_t ncell = len >> 4; // whole cells; the last 1-15 bytes are written by their owner,
+                                     // but their cell comes in with the others
     const uint32_t steps = (len + 127u) >> 7;
     const uint32_t sub = lane & 7u;
     // the eight (packet, cell-of-line) positions this lane moves per line
     const uint8_t *csrc[8];
     uint8_t *cdst[8];
-    uint32_t cfirst[8], cend[8];
+    uint32_t cfirst[8], cend[8], cend_ld[8];
 #pragma unroll
     for (int q = 0; q < 8; q++) {
         const int owner = 8 * q + (int)(lane >> 3);
         csrc[q] = reinterpret_cast<const uint8_t *>(shfl64((uint64_t)(uintptr_t)(src - skew), owner)) + 16u * sub;
         cdst[q] = reinterpret_cast<uint8_t *>(shfl64((uint64_t)(uintptr_t)(dst - skew), owner)) + 16u * sub;
         cfirst[q] = (uint32_t)__shfl((int)c0, owner, 64);
-        cend[q] = cfirst[q] + (uint32_t)__shfl((int)ncell, owner, 64);
+        const uint32_t olen = (uint32_t)__shfl((int)len, owner, 64);
+        cend[q] = cfirst[q] + (olen >> 4);
+        cend_ld[q] = cfirst[q] + ((olen + 15u) >> 4);
     }
     uint32_t maxsteps = steps;
 #pragma unroll
@@ -269,14 +303,15 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
           pre5 = pre0, pre6 = pre0, pre7 = pre0;
     uint8_t *mycell = tile + (lane >> 3) * RING_ROW;
 #define BNK_INSIDE(q, m) (8u * (m) + sub >= cfirst[q] && 8u * (m) + sub < cend[q])
+#define BNK_INSIDE_LD(q, m) (8u * (m) + sub >= cfirst[q] && 8u * (m) + sub < cend_ld[q])
 #define BNK_SLOT(q, m) reinterpret_cast<uint4 *>(mycell + 8u * q * RING_ROW + (((8u * (m) + sub) & 15u) << 4))
     // Boundary lines: a load under a branch makes the wave wait for it before the
     // branch closes, eight times per line; loading unconditionally from a harmless
     // address instead keeps all eight in flight (cells outside the packet are
     // fetched from `safe` and never leave their register).
-#define BNK_ISSUE(q, m) pre##q = ld16a(BNK_INSIDE(q, m) ? csrc[q] + 128u * (m) : safe)
+#define BNK_ISSUE(q, m) pre##q = ld16a(BNK_INSIDE_LD(q, m) ? csrc[q] + 128u * (m) : safe)
 #define BNK_ISSUE_ALL(q, m) pre##q = ld16a(csrc[q] + 128u * (m))
-#define BNK_COMMIT(q, m) if (BNK_INSIDE(q, m)) *BNK_SLOT(q, m) = pre##q
+#define BNK_COMMIT(q, m) if (BNK_INSIDE_LD(q, m)) *BNK_SLOT(q, m) = pre##q
 #define BNK_COMMIT_ALL(q, m) *BNK_SLOT(q, m) = pre##q
 #define BNK_STORE(q, m)                                                                     \
     do {                                                                                    \
@@ -332,7 +367,8 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
                             const uint32_t kc = 4u * b + j;
                             if (kc < ncell) crypt_cell<OPEN>(mac, x, j, row + (((c0 + kc) & 15u) << 4));
                             else if (kc == ncell && (len & 15u))
-                                crypt_tail<OPEN>(mac, x, j, src + 16u * kc, dst + 16u * kc, len & 15u);
+                                crypt_tail_lds<OPEN>(mac, x, j, row + (((c0 + kc) & 15u) << 4), dst + 16u * kc,
+                                                     len & 15u);
                         }
                     }
                 }
@@ -343,6 +379,7 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
         wave_sync();
     }
 #undef BNK_INSIDE
+#undef BNK_INSIDE_LD
 #undef BNK_SLOT
 #undef BNK_ISSUE
 #undef BNK_ISSUE_ALL
@@ -793,9 +830,10 @@ BNK_DEV uint32_t len_bin(uint32_t len, uint32_t tag_bytes)
 // Adds one to bins[b] for every participating lane and returns what the
 // lane's own atomicAdd would have returned, with one LDS atomic per distinct
 // bin of the wave instead of one per lane: traffic is a handful of sizes, so
-// most lanes of a wave hit the same bin and would serialise on it.  After
-// eight rounds the remaining lanes (a wave with many distinct sizes) go one
-// by one.
+// most lanes of a wave hit the same bin and would serialise on it.  The
+// leader's values travel through scalar registers (v_readlane), not through
+// LDS.  After eight rounds the remaining lanes (a wave with many distinct
+// sizes) go one by one.
 BNK_DEV uint32_t wave_bin_add(uint32_t *bins, uint32_t b, bool active)
 {
     const uint32_t lane = threadIdx.x & 63u;
@@ -805,12 +843,12 @@ BNK_DEV uint32_t wave_bin_add(uint32_t *bins, uint32_t b, bool active)
         const unsigned long long left = __ballot(todo);
         if (left == 0ull) return result;
         const int leader = __ffsll((long long)left) - 1;
-        const uint32_t lb = (uint32_t)__shfl((int)b, leader, 64);
+        const uint32_t lb = (uint32_t)__builtin_amdgcn_readlane((int)b, leader);
         const bool mine = todo && b == lb;
         const unsigned long long same = __ballot(mine);
         uint32_t old = 0;
         if ((int)lane == leader) old = atomicAdd(&bins[lb], (uint32_t)__popcll(same));
-        old = (uint32_t)__shfl((int)old, leader, 64);
+        old = (uint32_t)__builtin_amdgcn_readlane((int)old, leader);
         if (mine) {
             result = old + (uint32_t)__popcll(same & ((1ull << lane) - 1ull));
             todo = false;
@@ -820,49 +858,63 @@ BNK_DEV uint32_t wave_bin_add(uint32_t *bins, uint32_t b, bool active)
     return result;
 }
 
-__global__ __launch_bounds__(256) void len_hist_kernel(const uint32_t *lens, uint32_t n,
-                                                       uint32_t tag_bytes, uint32_t *hist)
+// A block of GROUP_THREADS threads takes GROUP_CHUNK consecutive packets, four
+// per thread, loaded together so that their latencies overlap.
+constexpr uint32_t GROUP_THREADS = 1024;
+constexpr uint32_t GROUP_PER_THREAD = 4;
+constexpr uint32_t GROUP_CHUNK = GROUP_THREADS * GROUP_PER_THREAD;
+
+__global__ __launch_bounds__(GROUP_THREADS) void len_hist_kernel(const uint32_t *lens, uint32_t n,
+                                                                 uint32_t tag_bytes, uint32_t *hist)
 {
     __shared__ uint32_t lh[LEN_BINS];
-    for (uint32_t b = threadIdx.x; b < LEN_BINS; b += 256) lh[b] = 0;
-    __syncthreads();
-    const uint32_t stride = gridDim.x * 256u;
-    // whole waves stay in the loop together (the helper uses wave-wide votes)
-    for (uint32_t i0 = blockIdx.x * 256u; i0 < n; i0 += stride) {
-        const uint32_t i = i0 + threadIdx.x;
-        const bool in = i < n;
-        (void)wave_bin_add(lh, in ? len_bin(lens[i], tag_bytes) : 0u, in);
+    for (uint32_t b = threadIdx.x; b < LEN_BINS; b += GROUP_THREADS) lh[b] = 0;
+    const uint32_t base = blockIdx.x * GROUP_CHUNK + threadIdx.x;
+    uint32_t len[GROUP_PER_THREAD];
+#pragma unroll
+    for (uint32_t j = 0; j < GROUP_PER_THREAD; j++) {
+        const uint32_t i = base + j * GROUP_THREADS;
+        len[j] = i < n ? lens[i] : 0u;
     }
     __syncthreads();
-    for (uint32_t b = threadIdx.x; b < LEN_BINS; b += 256)
+    // whole waves call the helper together (it uses wave-wide votes)
+#pragma unroll
+    for (uint32_t j = 0; j < GROUP_PER_THREAD; j++)
+        (void)wave_bin_add(lh, len_bin(len[j], tag_bytes), base + j * GROUP_THREADS < n);
+    __syncthreads();
+    for (uint32_t b = threadIdx.x; b < LEN_BINS; b += GROUP_THREADS)
         if (lh[b]) atomicAdd(&hist[b], lh[b]);
 }
 
-// Exclusive scan of hist into cursor (one block).
-__global__ __launch_bounds__(256) void len_scan_kernel(const uint32_t *hist, uint32_t *cursor)
+// Exclusive scan of hist into cursor (one block of LEN_SCAN_THREADS), leaving
+// hist all zeros for the next grouping (so no separate clearing launch).
+constexpr uint32_t LEN_SCAN_THREADS = 1024;
+__global__ __launch_bounds__(LEN_SCAN_THREADS) void len_scan_kernel(uint32_t *hist, uint32_t *cursor)
 {
-    __shared__ uint32_t part[256];
-    constexpr uint32_t PER = (LEN_BINS + 255) / 256;
+    __shared__ uint32_t wave_sum[LEN_SCAN_THREADS / 64];
+    constexpr uint32_t PER = (LEN_BINS + LEN_SCAN_THREADS - 1) / LEN_SCAN_THREADS;
+    const uint32_t lane = threadIdx.x & 63u, wv = threadIdx.x >> 6;
     uint32_t loc[PER];
     uint32_t sum = 0;
 #pragma unroll
     for (uint32_t q = 0; q < PER; q++) {
         const uint32_t b = threadIdx.x * PER + q;
         loc[q] = b < LEN_BINS ? hist[b] : 0u;
+        if (b < LEN_BINS) hist[b] = 0u;
         sum += loc[q];
     }
-    part[threadIdx.x] = sum;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        uint32_t run = 0;
-        for (int t = 0; t < 256; t++) {
-            const uint32_t v = part[t];
-            part[t] = run;
-            run += v;
-        }
+    // inclusive scan within the wave, then across the waves
+    uint32_t inc = sum;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const uint32_t o = (uint32_t)__shfl_up((int)inc, off, 64);
+        if ((int)lane >= off) inc += o;
     }
+    if (lane == 63u) wave_sum[wv] = inc;
     __syncthreads();
-    uint32_t run = part[threadIdx.x];
+    uint32_t before = 0;
+    for (uint32_t w = 0; w < wv; w++) before += wave_sum[w];
+    uint32_t run = before + inc - sum;
 #pragma unroll
     for (uint32_t q = 0; q < PER; q++) {
         const uint32_t b = threadIdx.x * PER + q;
@@ -871,34 +923,36 @@ __global__ __launch_bounds__(256) void len_scan_kernel(const uint32_t *hist, uin
     }
 }
 
-__global__ __launch_bounds__(256) void len_scatter_kernel(const uint32_t *lens, uint32_t n,
-                                                          uint32_t tag_bytes, uint32_t *cursor,
-                                                          uint32_t *order)
+__global__ __launch_bounds__(GROUP_THREADS) void len_scatter_kernel(const uint32_t *lens, uint32_t n,
+                                                                    uint32_t tag_bytes, uint32_t *cursor,
+                                                                    uint32_t *order)
 {
     __shared__ uint32_t cnt[LEN_BINS];
     __shared__ uint32_t base[LEN_BINS];
-    for (uint32_t b = threadIdx.x; b < LEN_BINS; b += 256) cnt[b] = 0;
-    __syncthreads();
-    const uint32_t stride = gridDim.x * 256u;
-    // every block walks its strided share twice: count, reserve, place
-    for (uint32_t i0 = blockIdx.x * 256u; i0 < n; i0 += stride) {
-        const uint32_t i = i0 + threadIdx.x;
-        const bool in = i < n;
-        (void)wave_bin_add(cnt, in ? len_bin(lens[i], tag_bytes) : 0u, in);
+    for (uint32_t b = threadIdx.x; b < LEN_BINS; b += GROUP_THREADS) cnt[b] = 0;
+    const uint32_t first = blockIdx.x * GROUP_CHUNK + threadIdx.x;
+    uint32_t bin[GROUP_PER_THREAD], at[GROUP_PER_THREAD];
+#pragma unroll
+    for (uint32_t j = 0; j < GROUP_PER_THREAD; j++) {
+        const uint32_t i = first + j * GROUP_THREADS;
+        bin[j] = len_bin(i < n ? lens[i] : 0u, tag_bytes);
     }
     __syncthreads();
-    for (uint32_t b = threadIdx.x; b < LEN_BINS; b += 256) {
+    // a packet's place within its block's share of the bin, then one
+    // reservation per bin for the whole block
+#pragma unroll
+    for (uint32_t j = 0; j < GROUP_PER_THREAD; j++)
+        at[j] = wave_bin_add(cnt, bin[j], first + j * GROUP_THREADS < n);
+    __syncthreads();
+    for (uint32_t b = threadIdx.x; b < LEN_BINS; b += GROUP_THREADS) {
         const uint32_t c = cnt[b];
-        base[b] = c ? atomicAdd(&cursor[b], c) : 0u;
-        cnt[b] = 0;
+        if (c) base[b] = atomicAdd(&cursor[b], c);
     }
     __syncthreads();
-    for (uint32_t i0 = blockIdx.x * 256u; i0 < n; i0 += stride) {
-        const uint32_t i = i0 + threadIdx.x;
-        const bool in = i < n;
-        const uint32_t b = in ? len_bin(lens[i], tag_bytes) : 0u;
-        const uint32_t at = wave_bin_add(cnt, b, in);
-        if (in) order[base[b] + at] = i;
+#pragma unroll
+    for (uint32_t j = 0; j < GROUP_PER_THREAD; j++) {
+        const uint32_t i = first + j * GROUP_THREADS;
+        if (i < n) order[base[bin[j]] + at[j]] = i;
     }
 }
 
@@ -949,13 +1003,12 @@ hipError_t launch_length_sort(const uint32_t *lens, uint32_t n, uint32_t tag_byt
                               hipStream_t s)
 {
     if (n == 0) return hipSuccess;
-    hipLaunchKernelGGL(fill_u32_kernel, dim3((LEN_BINS + 255u) / 256u), dim3(256), 0, s, hist,
-                       LEN_BINS, 0u);
-    uint32_t blocks = (n + 255u) / 256u;
-    if (blocks > 1024u) blocks = 1024u;
-    hipLaunchKernelGGL(len_hist_kernel, dim3(blocks), dim3(256), 0, s, lens, n, tag_bytes, hist);
-    hipLaunchKernelGGL(len_scan_kernel, dim3(1), dim3(256), 0, s, hist, cursor);
-    hipLaunchKernelGGL(len_scatter_kernel, dim3(blocks), dim3(256), 0, s, lens, n, tag_bytes,
+    // hist is all zeros on entry: its owner clears it once when it is allocated
+    // and every grouping leaves it cleared (len_scan_kernel)
+    const uint32_t blocks = (n + GROUP_CHUNK - 1u) / GROUP_CHUNK;
+    hipLaunchKernelGGL(len_hist_kernel, dim3(blocks), dim3(GROUP_THREADS), 0, s, lens, n, tag_bytes, hist);
+    hipLaunchKernelGGL(len_scan_kernel, dim3(1), dim3(LEN_SCAN_THREADS), 0, s, hist, cursor);
+    hipLaunchKernelGGL(len_scatter_kernel, dim3(blocks), dim3(GROUP_THREADS), 0, s, lens, n, tag_bytes,
                        cursor, order);
     return hipGetLastError();
 }

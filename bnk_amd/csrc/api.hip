@@ -184,8 +184,10 @@ int aead_device_layout_check(bnk_ctx *ctx, bool open, const bnk_batch *in, const
 
 namespace bnk {
 
-// sort_scratch: null, or device memory of n + 2 * LEN_BINS words for the
-// length grouping of a device-resident batch (then nothing is allocated).
+// sort_scratch: null, or device memory of 2 * LEN_BINS + n words for the
+// length grouping of a device-resident batch (then nothing is allocated); its
+// first LEN_BINS words must be zeros on the first call and are zeros again
+// after every call.
 int aead_batch(bnk_ctx *ctx, bool open, const bnk_batch *in, const bnk_batch *out,
                uint8_t *verdict, uint32_t *sort_scratch)
 {
@@ -234,7 +236,8 @@ int aead_batch(bnk_ctx *ctx, bool open, const bnk_batch *in, const bnk_batch *ou
             // the caller's scratch instead of the context's grow-only buffers
             a.order = nullptr;
             if (a.lens && n > 64 && !aead_runs_spread(a)) {
-                uint32_t *order = sort_scratch, *hist = order + n, *cursor = hist + LEN_BINS;
+                // the histogram keeps its place from call to call: it is left all zeros by each grouping
+                uint32_t *hist = sort_scratch, *cursor = hist + LEN_BINS, *order = cursor + LEN_BINS;
                 HIPCHK(ctx, launch_length_sort(a.lens, n, open ? 16 : 0, order, hist, cursor, ctx->stream));
                 a.order = order;
             }
@@ -345,6 +348,11 @@ int bnk_init(int device_ordinal, bnk_ctx **out)
     memset(ctx->h_status, 0, 64);
     if ((e = hipHostGetDevicePointer((void **)&ctx->d_status, ctx->h_status, 0)) != hipSuccess)
         return bail("hipHostGetDevicePointer", e);
+    // the length grouping's histogram starts out cleared and every grouping
+    // leaves it cleared
+    if ((e = ctx->hist.reserve(LEN_BINS * 4)) != hipSuccess) return bail("hipMalloc", e);
+    if ((e = ctx->cursor.reserve(LEN_BINS * 4)) != hipSuccess) return bail("hipMalloc", e);
+    if ((e = hipMemsetAsync(ctx->hist.p, 0, LEN_BINS * 4, ctx->stream)) != hipSuccess) return bail("hipMemsetAsync", e);
     if (int rc = noalloc_setup(nullptr, device_ordinal)) {
         ctx->alive = true;
         bnk_shutdown(ctx);

@@ -61,9 +61,9 @@ extern "C" int bnk_aead_seal_batch_noalloc(bnk_ctx *ctx, const bnk_batch *in, co
         ptr = g_scratch_ptr[ctx->device];
     }
     if (!ptr) return fail(ctx, BNK_E_STATE, "device scratch was not set up");
-    // The array keeps the last call's contents: the histogram is cleared by the
-    // length grouping itself (a fill kernel), order[] and cursor[] are written
-    // before they are read.
+    // The array keeps the last call's contents: the histogram starts as zeros
+    // (static storage) and every length grouping clears it again before it ends
+    // (a kernel, no memset), order[] and cursor[] are written before they are read.
     return aead_batch(ctx, false, in, out, nullptr, ptr);
     BNK_API_CATCH(ctx)
 }

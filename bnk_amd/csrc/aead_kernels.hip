@@ -135,6 +135,16 @@ BNK_DEV void wave_sync()
 constexpr uint32_t LDS_ROW = 80;    // generic: 64 data bytes + 16 pad
 constexpr uint32_t RING_ROW = 272;  // line path: 2 x 128-byte lines + 16 pad
 constexpr uint32_t WAVES_PER_BLOCK = 4;
+// Short path: a wave whose packets all have at most SHORT_BLOCKS data blocks
+// (128 plaintext bytes: at most eight cells, in at most two lines) brings each
+// packet in whole, computes it in one go and writes it back, with rows that
+// hold the packet's cells from its first one.  Straight-line code, every load
+// of the wave in flight at once: 2^20 x 60 bytes seal in 101 us against 113 us
+// through the ring.  (Running such waves three to a SIMD on smaller rows was
+// tried too: the 168 registers that allows cost the long packets 15 % and the
+// short ones gained nothing.)
+constexpr uint32_t SHORT_BLOCKS = 2;
+constexpr uint32_t SHORT_ROW = 144;          // 8 cells + 16 pad
 
 template <bool OPEN>
 BNK_DEV void crypt_cell(Poly32 &mac, const uint32_t (&x)[16], int j, uint8_t *cell)
@@ -393,6 +403,87 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
 #undef BNK_COMMIT_LINE
 }
 
+// Short path (see SHORT_BLOCKS): cell j of a packet lives at row + 16 j.  Same
+// cooperative movement as body_lines: eight adjacent lanes per aligned
+// 128-byte line, only cells of the packet read into LDS or written back.
+template <bool OPEN>
+BNK_DEV void body_short(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_t *dst, uint32_t len,
+                        const uint8_t *safe, const uint32_t (&k)[8], uint32_t n1, uint32_t n2,
+                        Poly32 &mac, uint32_t (&x)[16])
+{
+    const uint32_t skew = (uint32_t)(uintptr_t)src & 127u;
+    const uint32_t c0 = skew >> 4;
+    const uint32_t ncell = len >> 4;           // whole cells, stored cooperatively
+    const uint32_t sub = lane & 7u;
+    // does any packet of the wave reach into a second line?
+    const bool two = __ballot(c0 + ((len + 15u) >> 4) > 8u) != 0ull;
+    uint8_t *rows = tile + (lane >> 3) * SHORT_ROW;
+    uint4 pre[2][8];
+    uint32_t jcell[8], nst[8], nld[8]; // my cell's index in the owner's packet for line 0; its cell counts
+    const uint8_t *csrc[8];
+    uint8_t *cdst[8];
+#pragma unroll
+    for (int q = 0; q < 8; q++) {
+        const int owner = 8 * q + (int)(lane >> 3);
+        csrc[q] = reinterpret_cast<const uint8_t *>(shfl64((uint64_t)(uintptr_t)(src - skew), owner)) + 16u * sub;
+        cdst[q] = reinterpret_cast<uint8_t *>(shfl64((uint64_t)(uintptr_t)(dst - skew), owner)) + 16u * sub;
+        const uint32_t olen = (uint32_t)__shfl((int)len, owner, 64);
+        jcell[q] = sub - (uint32_t)__shfl((int)c0, owner, 64); // wraps below zero for cells before the packet
+        nst[q] = olen >> 4;
+        nld[q] = (olen + 15u) >> 4;
+    }
+    // unconditional loads, from a harmless address when the cell is not the
+    // packet's (a load under a branch is waited for where the branch closes)
+#pragma unroll
+    for (int q = 0; q < 8; q++) pre[0][q] = ld16a(jcell[q] < nld[q] ? csrc[q] : safe);
+    if (two) {
+#pragma unroll
+        for (int q = 0; q < 8; q++) pre[1][q] = ld16a(jcell[q] + 8u < nld[q] ? csrc[q] + 128u : safe);
+    }
+    // keystream block 0 (the Poly1305 key) while the loads fly
+    chacha_block(k, 0, n1, n2, x);
+    mac.init(x);
+#pragma unroll
+    for (int q = 0; q < 8; q++)
+        if (jcell[q] < nld[q]) *reinterpret_cast<uint4 *>(rows + 8u * q * SHORT_ROW + (jcell[q] << 4)) = pre[0][q];
+    if (two) {
+#pragma unroll
+        for (int q = 0; q < 8; q++)
+            if (jcell[q] + 8u < nld[q])
+                *reinterpret_cast<uint4 *>(rows + 8u * q * SHORT_ROW + ((jcell[q] + 8u) << 4)) = pre[1][q];
+    }
+    wave_sync();
+    uint8_t *row = tile + lane * SHORT_ROW;
+#pragma unroll 1
+    for (uint32_t b = 0; b < SHORT_BLOCKS; b++) {
+        if (64u * b < len) {
+            chacha_block(k, b + 1, n1, n2, x);
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const uint32_t kc = 4u * b + j;
+                if (kc < ncell) crypt_cell<OPEN>(mac, x, j, row + (kc << 4));
+                else if (kc == ncell && (len & 15u))
+                    crypt_tail_lds<OPEN>(mac, x, j, row + (kc << 4), dst + 16u * kc, len & 15u);
+            }
+        }
+    }
+    wave_sync();
+#pragma unroll
+    for (int q = 0; q < 8; q++) {
+        // read first, unconditionally (from cell 0 when mine is not the packet's)
+        const uint4 v = *reinterpret_cast<const uint4 *>(rows + 8u * q * SHORT_ROW + ((jcell[q] < 8u ? jcell[q] : 0u) << 4));
+        if (jcell[q] < nst[q]) st16a(cdst[q], v);
+    }
+    if (two) {
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+            const uint32_t j1 = jcell[q] + 8u;
+            const uint4 v = *reinterpret_cast<const uint4 *>(rows + 8u * q * SHORT_ROW + ((j1 < 8u ? j1 : 0u) << 4));
+            if (j1 < nst[q]) st16a(cdst[q] + 128u, v);
+        }
+    }
+}
+
 // Tag and verdict of each lane's packet once its bytes have gone through the
 // MAC, and the zero-fill of rejected plaintexts.
 template <bool OPEN>
@@ -442,10 +533,11 @@ template <bool OPEN>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void aead_wave_kernel(AeadArgs a)
 {
     __shared__ __attribute__((aligned(16))) uint8_t tile_all[WAVES_PER_BLOCK][64 * RING_ROW];
-    static_assert(RING_ROW >= LDS_ROW, "the generic path reuses the tile");
+    static_assert(RING_ROW >= LDS_ROW && RING_ROW >= SHORT_ROW, "the other paths reuse the tile");
     const uint32_t lane = threadIdx.x & 63u;
     uint8_t *tile = tile_all[threadIdx.x >> 6];
     const uint32_t t = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t t_end = a.n;
 
     // ---- this lane's packet ----
     // Straight-line code: every load below is issued whether or not the lane
@@ -457,7 +549,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // wash elsewhere.
     const uint32_t *safe32 = a.keys;
     const uint64_t *safe64 = reinterpret_cast<const uint64_t *>(a.keys);
-    const bool in_batch = t < a.n;
+    const bool in_batch = t < t_end;
     const uint32_t tt = in_batch ? t : 0u;
     const uint32_t ord = *(a.order ? a.order + tt : safe32);
     const uint32_t i = a.first + (a.order ? ord : tt);
@@ -502,8 +594,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
     const bool lane_lines = (((uintptr_t)src | (uintptr_t)dst) & 15u) == 0 &&
                             (((uintptr_t)src ^ (uintptr_t)dst) & 127u) == 0;
-    if (__ballot(!lane_lines) == 0ull) body_lines<OPEN>(tile, lane, src, dst, len, reinterpret_cast<const uint8_t *>(a.keys), k, n1, n2, mac, x);
-    else body_generic<OPEN>(tile, lane, src, dst, len, reinterpret_cast<const uint8_t *>(a.keys), k, n1, n2, mac, x);
+    const uint8_t *safe = reinterpret_cast<const uint8_t *>(a.keys);
+    if (__ballot(!lane_lines) != 0ull) body_generic<OPEN>(tile, lane, src, dst, len, safe, k, n1, n2, mac, x);
+    else if (__ballot(len > 64u * SHORT_BLOCKS) == 0ull) body_short<OPEN>(tile, lane, src, dst, len, safe, k, n1, n2, mac, x);
+    else body_lines<OPEN>(tile, lane, src, dst, len, safe, k, n1, n2, mac, x);
 
     lane_finish<OPEN>(a, lane, have, i, len, src, dst, mac);
 }
@@ -787,6 +881,13 @@ bool aead_runs_spread(const AeadArgs &a)
     return a.n <= std::min<uint64_t>(4ull * a.spread_max, by_len);
 }
 
+template <bool OPEN>
+static hipError_t launch_wave(const AeadArgs &a, hipStream_t s)
+{
+    hipLaunchKernelGGL(aead_wave_kernel<OPEN>, dim3((a.n + 255u) / 256u), dim3(256), 0, s, a);
+    return hipGetLastError();
+}
+
 hipError_t launch_aead_seal(const AeadArgs &a, hipStream_t s)
 {
     if (a.n == 0) return hipSuccess;
@@ -797,7 +898,7 @@ hipError_t launch_aead_seal(const AeadArgs &a, hipStream_t s)
     } else if (aead_runs_spread(a))
         hipLaunchKernelGGL((aead_spread_kernel<false, false>), waves, dim3(256), 0, s, a);
     else
-        hipLaunchKernelGGL(aead_wave_kernel<false>, dim3((a.n + 255u) / 256u), dim3(256), 0, s, a);
+        return launch_wave<false>(a, s);
     return hipGetLastError();
 }
 
@@ -811,7 +912,7 @@ hipError_t launch_aead_open(const AeadArgs &a, hipStream_t s)
     } else if (aead_runs_spread(a))
         hipLaunchKernelGGL((aead_spread_kernel<true, false>), waves, dim3(256), 0, s, a);
     else
-        hipLaunchKernelGGL(aead_wave_kernel<true>, dim3((a.n + 255u) / 256u), dim3(256), 0, s, a);
+        return launch_wave<true>(a, s);
     return hipGetLastError();
 }
 

@@ -44,7 +44,7 @@ int aead_batch_host_chunked(bnk_ctx *ctx, bool open, const bnk_batch *in, const 
         a.lens = ctx->lens.as<uint32_t>();
         HIPCHK(ctx, ctx->order.reserve((size_t)n * 4));
         HIPCHK(ctx, ctx->hist.reserve(LEN_BINS * 4));
-        HIPCHK(ctx, ctx->cursor.reserve(LEN_BINS * 4));
+        HIPCHK(ctx, ctx->cursor.reserve(LEN_CURSOR_WORDS * 4));
     }
     if (in->peer) {
         HIPCHK(ctx, up(&ctx->peer, in->peer, (size_t)n * 4));
@@ -184,7 +184,7 @@ int aead_device_layout_check(bnk_ctx *ctx, bool open, const bnk_batch *in, const
 
 namespace bnk {
 
-// sort_scratch: null, or device memory of 2 * LEN_BINS + n words for the
+// sort_scratch: null, or device memory of LEN_BINS + LEN_CURSOR_WORDS + n words for the
 // length grouping of a device-resident batch (then nothing is allocated); its
 // first LEN_BINS words must be zeros on the first call and are zeros again
 // after every call.
@@ -237,7 +237,7 @@ int aead_batch(bnk_ctx *ctx, bool open, const bnk_batch *in, const bnk_batch *ou
             a.order = nullptr;
             if (a.lens && n > 64 && !aead_runs_spread(a)) {
                 // the histogram keeps its place from call to call: it is left all zeros by each grouping
-                uint32_t *hist = sort_scratch, *cursor = hist + LEN_BINS, *order = cursor + LEN_BINS;
+                uint32_t *hist = sort_scratch, *cursor = hist + LEN_BINS, *order = cursor + LEN_CURSOR_WORDS;
                 HIPCHK(ctx, launch_length_sort(a.lens, n, open ? 16 : 0, order, hist, cursor, ctx->stream));
                 a.order = order;
             }
@@ -351,7 +351,7 @@ int bnk_init(int device_ordinal, bnk_ctx **out)
     // the length grouping's histogram starts out cleared and every grouping
     // leaves it cleared
     if ((e = ctx->hist.reserve(LEN_BINS * 4)) != hipSuccess) return bail("hipMalloc", e);
-    if ((e = ctx->cursor.reserve(LEN_BINS * 4)) != hipSuccess) return bail("hipMalloc", e);
+    if ((e = ctx->cursor.reserve(LEN_CURSOR_WORDS * 4)) != hipSuccess) return bail("hipMalloc", e);
     if ((e = hipMemsetAsync(ctx->hist.p, 0, LEN_BINS * 4, ctx->stream)) != hipSuccess) return bail("hipMemsetAsync", e);
     if (int rc = noalloc_setup(nullptr, device_ordinal)) {
         ctx->alive = true;

@@ -248,7 +248,7 @@ inline int maybe_sort(bnk_ctx *ctx, AeadArgs *a, uint32_t tag_bytes)
     if (!a->lens || a->n <= 64 || aead_runs_spread(*a)) return BNK_OK;
     HIPCHK(ctx, ctx->order.reserve((size_t)a->n * 4));
     HIPCHK(ctx, ctx->hist.reserve(LEN_BINS * 4));
-    HIPCHK(ctx, ctx->cursor.reserve(LEN_BINS * 4));
+    HIPCHK(ctx, ctx->cursor.reserve(LEN_CURSOR_WORDS * 4));
     HIPCHK(ctx, launch_length_sort(a->lens, a->n, tag_bytes, ctx->order.as<uint32_t>(),
                                    ctx->hist.as<uint32_t>(), ctx->cursor.as<uint32_t>(),
                                    ctx->stream));
@@ -436,7 +436,7 @@ struct HostPipe {
 };
 
 // Seal or open of one batch (api.hip).  sort_scratch: null, or device memory of
-// in->n + 2 * LEN_BINS words for the length grouping of a device-resident batch;
+// LEN_BINS + LEN_CURSOR_WORDS + in->n words for the length grouping of a device-resident batch;
 // with it the call allocates nothing and takes device batches only.
 int aead_batch(bnk_ctx *ctx, bool open, const bnk_batch *in, const bnk_batch *out, uint8_t *verdict,
                uint32_t *sort_scratch);

@@ -113,9 +113,10 @@ hipError_t launch_aead_open(const AeadArgs &a, hipStream_t s);
 
 // order[] = packet indices grouped by ChaCha20 block count, longest first, so
 // the lanes of a wave run the same number of rounds.  hist and cursor are
-// device scratch of LEN_BINS words each; hist must be all zeros on entry and
+// device scratch of LEN_BINS and LEN_CURSOR_WORDS words; hist must be all zeros on entry and
 // is all zeros again when the grouping has run.
 constexpr uint32_t LEN_BINS = 1032;
+constexpr uint32_t LEN_CURSOR_WORDS = LEN_BINS;
 hipError_t launch_length_sort(const uint32_t *lens, uint32_t n, uint32_t tag_bytes,
                               uint32_t *order, uint32_t *hist, uint32_t *cursor,
                               hipStream_t s);

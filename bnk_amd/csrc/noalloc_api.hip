@@ -10,7 +10,7 @@
 
 using namespace bnk;
 
-constexpr size_t SCRATCH_WORDS = (size_t)BNK_NOALLOC_MAX_PACKETS + 2u * LEN_BINS;
+constexpr size_t SCRATCH_WORDS = (size_t)BNK_NOALLOC_MAX_PACKETS + LEN_BINS + LEN_CURSOR_WORDS;
 
 // 4 MiB + 8 KiB on every GPU the library runs on, for the life of the process.
 // In host code this name is only a stand-in for the symbol: the address a

@@ -226,7 +226,7 @@ extern "C" int bnk_relay_fused_batch(bnk_ctx *ctx, const bnk_batch *in, const ui
     if (in->lens) {
         HIPCHK(ctx, ctx->order.reserve((size_t)n * 4));
         HIPCHK(ctx, ctx->hist.reserve(LEN_BINS * 4));
-        HIPCHK(ctx, ctx->cursor.reserve(LEN_BINS * 4));
+        HIPCHK(ctx, ctx->cursor.reserve(LEN_CURSOR_WORDS * 4));
     }
     FilterState *f = ctx->filter;
     uint8_t *d_pass = ctx->r_pass.as<uint8_t>();

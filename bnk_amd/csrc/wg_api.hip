@@ -306,7 +306,7 @@ static int wg_encap_impl(bnk_ctx *ctx, const bnk_batch *slots, uint32_t mtu, uin
     if (slots->lens) {
         HIPCHK(ctx, ctx->order.reserve((size_t)n * 4));
         HIPCHK(ctx, ctx->hist.reserve(LEN_BINS * 4));
-        HIPCHK(ctx, ctx->cursor.reserve(LEN_BINS * 4));
+        HIPCHK(ctx, ctx->cursor.reserve(LEN_CURSOR_WORDS * 4));
     }
     const WgPeersDev pe = peers_view(ctx);
     uint64_t *d_ctr = ctx->r_ctr_out.as<uint64_t>();
@@ -640,7 +640,7 @@ static int wg_decap_impl(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *o
     if (wire->lens) {
         HIPCHK(ctx, ctx->order.reserve((size_t)n * 4));
         HIPCHK(ctx, ctx->hist.reserve(LEN_BINS * 4));
-        HIPCHK(ctx, ctx->cursor.reserve(LEN_BINS * 4));
+        HIPCHK(ctx, ctx->cursor.reserve(LEN_CURSOR_WORDS * 4));
     }
     uint32_t *d_ctlen = ctx->wg_ctlen.as<uint32_t>();
     uint8_t *d_auth = ctx->r_auth.as<uint8_t>();

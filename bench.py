@@ -7,8 +7,9 @@ at a 1440-byte stride), inputs resident in HBM before the timed region.  The
 value is plaintext Gbit/s through the seal+open pair on one MI355X.
 
 Prints ONE JSON line.  Besides the contract fields it carries
-  roofline       HBM view of the dominant kernel (aead_wave_kernel)
-  roofline_valu  the same launches priced in int32 op-equivalents
+  roofline       the binding one: int32 VALU instructions issued by the dominant kernel
+                 (aead_wave_kernel) against the lane-op peak, with the survey's op model beside it
+  roofline_hbm   the same launches as algorithmic bytes against the HBM peak
   cpu_baseline   the CPU oracle timed on this box's host cores (bounded sample)
   cpu_baseline_openssl  the same sample through OpenSSL's assembly, when libcrypto is there
   packed_layout  the same packets back to back (no slot 16-byte aligned)
@@ -34,6 +35,11 @@ L = 1420
 STRIDE = 1440
 HBM_PEAK_GBS = 8000.0
 VALU_PEAK_TOPS = 39.3  # 256 CU x 64 lanes x 2.4 GHz, one int32 op per lane per clock
+# Counter readings for one launch of aead_wave_kernel over 2^20 packets x 1420 B (mean of
+# seal and open), taken with rocprofv3 --pmc and kept in profiles/aead_wave_kernel_cfg2.md;
+# they change only when the kernel does.
+VALU_LANE_INSTR_PER_PACKET = 31276   # SQ_INSTS_VALU x 64 / 2^20
+TRAFFIC_BYTES_PER_LAUNCH = 3.187e9   # FETCH_SIZE + WRITE_SIZE, scaled by copy_kernel
 
 
 def ops_chacha(length: int) -> int:
@@ -589,11 +595,9 @@ def bench_latency(args) -> dict:
 def bench_copy(args) -> dict:
     """Plain device-to-device copy of 1 GiB: the measured HBM ceiling and the
     known-size launch the FETCH_SIZE / WRITE_SIZE counters are scaled by."""
-    from bnk_amd import lib
-    ctx = lib.Context(0)
+    from bnk_amd import probe
     nbytes = 1 << 30
-    rate = ctx.probe_copy(nbytes, max(args.steps, 1))
-    ctx.close()
+    rate = probe.copy(nbytes, max(args.steps, 1))
     return {"metric": "hbm_copy_gb_per_s", "value": round(rate / 1e9, 1), "unit": "GB/s",
             "n_gpus": 1, "steps": args.steps, "warmup": 1, "higher_is_better": True,
             "config": {"workload": "copy_kernel: %d bytes read + %d bytes written per launch"
@@ -697,9 +701,13 @@ def main() -> int:
     ops = n * ops_aead(L)
     achieved_tops = ops / (kern_ms * 1e-3) / 1e12
 
+    from bnk_amd import probe
     probes = {}
     for name in ("v_add_u32", "v_xor_b32", "v_alignbit_b32", "v_mad_u64_u32"):
-        probes[name] = round(ctx.probe_valu(name, 2000) / 1e12, 2)
+        probes[name] = round(probe.valu(name, 2000) / 1e12, 2)
+    lane_instr = n * VALU_LANE_INSTR_PER_PACKET
+    achieved_lane_tops = lane_instr / (kern_ms * 1e-3) / 1e12
+    counters_apply = n == 1 << 20
 
     out = {
         "metric": "aead_seal_open_gbit_per_s_1420B",
@@ -722,21 +730,38 @@ def main() -> int:
         "seal_ms": round(seal_ms, 4),
         "open_ms": round(open_ms, 4),
         "mpkt_per_s_pair": round(n / (ms_per_step * 1e-3) / 1e6, 1),
+        # The kernel is bound by VALU issue, not by memory: the binding roofline is
+        # instructions actually issued (one int32 lane-op per lane per clock).
         "roofline": {
+            "bound": "valu_int32", "kernel": "aead_wave_kernel",
+            "achieved": round(achieved_lane_tops, 2), "peak": VALU_PEAK_TOPS,
+            "unit": "T int32 lane-op/s (VALU instructions issued x 64 lanes)",
+            "frac": round(achieved_lane_tops / VALU_PEAK_TOPS, 4),
+            "instructions_per_packet": VALU_LANE_INSTR_PER_PACKET,
+            "instructions_source": "SQ_INSTS_VALU per launch x 64 / packets, rocprofv3 --pmc, mean of the "
+                                   "seal and the open launch (profiles/aead_wave_kernel_cfg2.md); "
+                                   "not re-measured in this run",
+            "avg_launch_ms": round(kern_ms, 4),
+            "traffic": TRAFFIC_BYTES_PER_LAUNCH if counters_apply else None,
+            "traffic_source": "profiles/aead_wave_kernel_cfg2.md (FETCH_SIZE and WRITE_SIZE under "
+                              "rocprofv3 --pmc, scaled by copy_kernel; not re-measured in this run)",
+            # the survey's op model beside it: it prices a 64-bit multiply-add at 4 and
+            # assumes 25 of them per Poly1305 block (radix 2^26), the kernel issues 20
+            # (radix 2^32), so this ratio is not bounded by 1 and is no roofline fraction
+            "op_equivalent_model": {
+                "ops_per_packet": ops_aead(L), "achieved": round(achieved_tops, 2),
+                "unit": "Top/s (int32 op-equivalents)",
+                "ratio_to_peak": round(achieved_tops / VALU_PEAK_TOPS, 4),
+            },
+            "measured_ceilings_tops": probes,
+        },
+        "roofline_hbm": {
             "bound": "hbm", "kernel": "aead_wave_kernel",
             "achieved": round(achieved_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": round(achieved_gbs / HBM_PEAK_GBS, 4),
-            # FETCH_SIZE x2 + WRITE_SIZE under rocprofv3 --pmc, mean of the seal and the open
-            # launch (profiles/aead_wave_kernel_cfg2.md); not re-measured by this run
-            "traffic": 3.214e9 if n == 1 << 20 else None,
+            "traffic": TRAFFIC_BYTES_PER_LAUNCH if counters_apply else None,
+            "traffic_source": "profiles/aead_wave_kernel_cfg2.md (not re-measured in this run)",
             "bytes_per_launch": alg_bytes, "avg_launch_ms": round(kern_ms, 4),
-        },
-        "roofline_valu": {
-            "bound": "valu_int32", "achieved": round(achieved_tops, 2),
-            "peak": VALU_PEAK_TOPS, "unit": "Top/s (int32 op-equivalents)",
-            "frac": round(achieved_tops / VALU_PEAK_TOPS, 4),
-            "ops_per_packet": ops_aead(L),
-            "measured_ceilings_tops": probes,
         },
     }
 

@@ -580,64 +580,4 @@ int bnk_aead_open_batch(bnk_ctx *ctx, const bnk_batch *in, const bnk_batch *out,
     BNK_API_CATCH(ctx)
 }
 
-int bnk_probe_valu(bnk_ctx *ctx, int op, uint32_t iters, double *ops_per_sec)
-{
-    BNK_API_TRY
-    Guard g(ctx);
-    if (g.rc) return g.rc;
-    if (!ops_per_sec || iters == 0 || op < 0 || op >= PROBE_OPS) return fail(ctx, BNK_E_INVAL, "bad probe request");
-    hipDeviceProp_t prop;
-    HIPCHK(ctx, hipGetDeviceProperties(&prop, ctx->device));
-    // 8 workgroups of 4 waves per CU: every SIMD holds 8 waves
-    const uint32_t blocks = (uint32_t)prop.multiProcessorCount * 8u;
-    HIPCHK(ctx, ctx->misc.reserve((size_t)blocks * PROBE_THREADS * 4));
-    HIPCHK(ctx, launch_probe(op, 4, blocks, ctx->misc.as<uint32_t>(), ctx->stream)); // warm-up
-    HIPCHK(ctx, hipEventRecord(ctx->ev0, ctx->stream));
-    HIPCHK(ctx, launch_probe(op, iters, blocks, ctx->misc.as<uint32_t>(), ctx->stream));
-    HIPCHK(ctx, hipEventRecord(ctx->ev1, ctx->stream));
-    HIPCHK(ctx, hipEventSynchronize(ctx->ev1));
-    float ms = 0;
-    HIPCHK(ctx, hipEventElapsedTime(&ms, ctx->ev0, ctx->ev1));
-    const double ops = (double)blocks * PROBE_THREADS * (double)iters * PROBE_CHAINS * PROBE_UNROLL;
-    *ops_per_sec = ops / ((double)ms * 1e-3);
-    return BNK_OK;
-    BNK_API_CATCH(ctx)
-}
-
-int bnk_probe_copy(bnk_ctx *ctx, size_t bytes, uint32_t iters, double *bytes_per_sec)
-{
-    BNK_API_TRY
-    Guard g(ctx);
-    if (g.rc) return g.rc;
-    if (!bytes_per_sec || iters == 0 || bytes < 4096 || (bytes & 15))
-        return fail(ctx, BNK_E_INVAL, "bad copy probe request");
-    hipDeviceProp_t prop;
-    HIPCHK(ctx, hipGetDeviceProperties(&prop, ctx->device));
-    const uint32_t blocks = (uint32_t)prop.multiProcessorCount * 16u;
-    void *src = nullptr, *dst = nullptr;
-    HIPCHK(ctx, hipMalloc(&src, bytes));
-    hipError_t e = hipMalloc(&dst, bytes);
-    if (e != hipSuccess) {
-        (void)hipFree(src);
-        return fail_hip(ctx, "hipMalloc", e);
-    }
-    float ms = 0;
-    e = launch_fill_u32((uint32_t *)src, (uint32_t)std::min<size_t>(bytes / 4, 1u << 30), 0x5a5a5a5au,
-                        ctx->stream);
-    if (e == hipSuccess) e = launch_copy(src, dst, bytes, blocks, ctx->stream); // warm-up
-    if (e == hipSuccess) e = hipEventRecord(ctx->ev0, ctx->stream);
-    for (uint32_t i = 0; i < iters && e == hipSuccess; i++)
-        e = launch_copy(src, dst, bytes, blocks, ctx->stream);
-    if (e == hipSuccess) e = hipEventRecord(ctx->ev1, ctx->stream);
-    if (e == hipSuccess) e = hipEventSynchronize(ctx->ev1);
-    if (e == hipSuccess) e = hipEventElapsedTime(&ms, ctx->ev0, ctx->ev1);
-    (void)hipFree(src);
-    (void)hipFree(dst);
-    if (e != hipSuccess) return fail_hip(ctx, "copy probe", e);
-    // bytes read plus bytes written
-    *bytes_per_sec = 2.0 * (double)bytes * iters / ((double)ms * 1e-3);
-    return BNK_OK;
-    BNK_API_CATCH(ctx)
-}
-
 } // extern "C"

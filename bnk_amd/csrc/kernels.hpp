@@ -161,14 +161,4 @@ hipError_t launch_peer_rank_small(const uint32_t *peer, uint32_t n_keys, uint32_
                                   uint64_t *ctr_out, bool advance, uint64_t ctr_limit, uint32_t *status,
                                   hipStream_t s);
 
-// VALU throughput probe; out receives one word per thread so nothing is
-// optimised away.
-hipError_t launch_probe(int op, uint32_t iters, uint32_t blocks, uint32_t *out,
-                        hipStream_t s);
-hipError_t launch_copy(const void *src, void *dst, size_t bytes, uint32_t blocks, hipStream_t s);
-constexpr int PROBE_OPS = 24;
-constexpr uint32_t PROBE_THREADS = 256;
-constexpr uint32_t PROBE_CHAINS = 8;   // independent dependency chains per lane
-constexpr uint32_t PROBE_UNROLL = 16;  // instructions per chain per iteration
-
 } // namespace bnk

@@ -22,9 +22,6 @@ E_INVAL, E_NODEV, E_HIP, E_NOMEM, E_RANGE, E_STATE = -1, -2, -3, -4, -5, -6
 NOALLOC_MAX_PACKETS = 1 << 20
 WG_REJECT_AFTER_MESSAGES = (1 << 64) - (1 << 13) - 1
 
-PROBE_OPS = {"v_add_u32": 0, "v_xor_b32": 1, "v_alignbit_b32": 2, "v_mad_u64_u32": 3,
-             "v_fma_f64": 4, "v_mul_lo_u32": 5, "v_add_f64": 6}
-
 
 class BnkError(RuntimeError):
     def __init__(self, code: int, text: str):
@@ -372,20 +369,6 @@ class Context:
     def wg_note_encap(self, slots: Batch, mtu: int, now_ns: int, wire_len) -> None:
         self._chk(self._lib.bnk_wg_note_encap_batch(self._h, C.byref(slots), C.c_uint32(mtu),
                                                     C.c_int64(now_ns), C.c_void_p(_ptr(wire_len))))
-
-    # ---- measurement ----
-    def probe_valu(self, op: str | int, iters: int = 2000) -> float:
-        code = PROBE_OPS[op] if isinstance(op, str) else op
-        r = C.c_double()
-        self._chk(self._lib.bnk_probe_valu(self._h, C.c_int(code), C.c_uint32(iters), C.byref(r)))
-        return float(r.value)
-
-
-    def probe_copy(self, nbytes: int, iters: int) -> float:
-        r = C.c_double()
-        self._chk(self._lib.bnk_probe_copy(self._h, C.c_size_t(nbytes), C.c_uint32(iters),
-                                           C.byref(r)))
-        return float(r.value)
 
 
 class HostFilter:

@@ -1,9 +1,20 @@
-// Dependency-free VALU instruction streams: the measured per-op ceilings the
-// AEAD roofline fractions are quoted against.  Every lane runs PROBE_CHAINS
-// independent chains so no instruction waits on the previous one.
-#include "kernels.hpp"
+// libbnkprobe.so: measurement probes for the benchmark, kept apart from the
+// product library.  Dependency-free VALU instruction streams (the measured
+// per-instruction ceilings the AEAD roofline is read against; every lane runs
+// PROBE_CHAINS independent chains so no instruction waits on the previous one)
+// and a plain streaming copy (the measured HBM ceiling, and the known-size
+// launch that memory-traffic counters are scaled against).
+#include <hip/hip_runtime.h>
+#include <stdint.h>
 
-namespace bnk {
+#include "bnkprobe.h"
+
+namespace {
+
+constexpr int PROBE_OPS = 24;
+constexpr uint32_t PROBE_THREADS = 256;
+constexpr uint32_t PROBE_CHAINS = 8;   // independent dependency chains per lane
+constexpr uint32_t PROBE_UNROLL = 16;  // instructions per chain per iteration
 
 template <int OP>
 __global__ __launch_bounds__(256) void probe_kernel(uint32_t iters, uint32_t *out)
@@ -74,7 +85,7 @@ __global__ __launch_bounds__(256) void copy_kernel(const uint4 *src, uint4 *dst,
     for (size_t i = (size_t)blockIdx.x * 256u + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
 }
 
-hipError_t launch_copy(const void *src, void *dst, size_t bytes, uint32_t blocks, hipStream_t s)
+static hipError_t launch_copy(const void *src, void *dst, size_t bytes, uint32_t blocks, hipStream_t s)
 {
     hipLaunchKernelGGL(copy_kernel, dim3(blocks), dim3(256), 0, s, (const uint4 *)src, (uint4 *)dst,
                        bytes / 16);
@@ -92,9 +103,85 @@ static hipError_t probe_dispatch(int op, uint32_t iters, uint32_t blocks, uint32
     return hipErrorInvalidValue;
 }
 
-hipError_t launch_probe(int op, uint32_t iters, uint32_t blocks, uint32_t *out, hipStream_t s)
+static hipError_t launch_probe(int op, uint32_t iters, uint32_t blocks, uint32_t *out, hipStream_t s)
 {
     return probe_dispatch<0>(op, iters, blocks, out, s);
 }
 
-} // namespace bnk
+} // namespace
+
+#define PROBE_CHK(expr)                       \
+    do {                                      \
+        if ((expr) != hipSuccess) goto fail;  \
+    } while (0)
+
+extern "C" int bnkp_valu(int device, int op, uint32_t iters, double *ops_per_sec)
+{
+    if (!ops_per_sec || iters == 0 || op < 0 || op >= PROBE_OPS) return -1;
+    hipDeviceProp_t prop;
+    hipStream_t s = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    uint32_t *out = nullptr;
+    float ms = 0;
+    int rc = -3;
+    uint32_t blocks = 0;
+    PROBE_CHK(hipSetDevice(device));
+    PROBE_CHK(hipGetDeviceProperties(&prop, device));
+    // 8 workgroups of 4 waves per CU: every SIMD holds 8 waves
+    blocks = (uint32_t)prop.multiProcessorCount * 8u;
+    PROBE_CHK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    PROBE_CHK(hipEventCreate(&e0));
+    PROBE_CHK(hipEventCreate(&e1));
+    PROBE_CHK(hipMalloc((void **)&out, (size_t)blocks * PROBE_THREADS * 4));
+    PROBE_CHK(launch_probe(op, 4, blocks, out, s)); // warm-up
+    PROBE_CHK(hipEventRecord(e0, s));
+    PROBE_CHK(launch_probe(op, iters, blocks, out, s));
+    PROBE_CHK(hipEventRecord(e1, s));
+    PROBE_CHK(hipEventSynchronize(e1));
+    PROBE_CHK(hipEventElapsedTime(&ms, e0, e1));
+    *ops_per_sec = (double)blocks * PROBE_THREADS * (double)iters * PROBE_CHAINS * PROBE_UNROLL / ((double)ms * 1e-3);
+    rc = 0;
+fail:
+    if (out) (void)hipFree(out);
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    if (s) (void)hipStreamDestroy(s);
+    return rc;
+}
+
+extern "C" int bnkp_copy(int device, size_t bytes, uint32_t iters, double *bytes_per_sec)
+{
+    if (!bytes_per_sec || iters == 0 || bytes < 4096 || (bytes & 15)) return -1;
+    hipDeviceProp_t prop;
+    hipStream_t s = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    void *src = nullptr, *dst = nullptr;
+    float ms = 0;
+    int rc = -3;
+    uint32_t blocks = 0;
+    PROBE_CHK(hipSetDevice(device));
+    PROBE_CHK(hipGetDeviceProperties(&prop, device));
+    blocks = (uint32_t)prop.multiProcessorCount * 16u;
+    PROBE_CHK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    PROBE_CHK(hipEventCreate(&e0));
+    PROBE_CHK(hipEventCreate(&e1));
+    PROBE_CHK(hipMalloc(&src, bytes));
+    PROBE_CHK(hipMalloc(&dst, bytes));
+    PROBE_CHK(hipMemsetAsync(src, 0x5a, bytes, s));
+    PROBE_CHK(launch_copy(src, dst, bytes, blocks, s)); // warm-up
+    PROBE_CHK(hipEventRecord(e0, s));
+    for (uint32_t i = 0; i < iters; i++) PROBE_CHK(launch_copy(src, dst, bytes, blocks, s));
+    PROBE_CHK(hipEventRecord(e1, s));
+    PROBE_CHK(hipEventSynchronize(e1));
+    PROBE_CHK(hipEventElapsedTime(&ms, e0, e1));
+    // bytes read plus bytes written
+    *bytes_per_sec = 2.0 * (double)bytes * iters / ((double)ms * 1e-3);
+    rc = 0;
+fail:
+    if (src) (void)hipFree(src);
+    if (dst) (void)hipFree(dst);
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    if (s) (void)hipStreamDestroy(s);
+    return rc;
+}

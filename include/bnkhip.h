@@ -346,21 +346,6 @@ int bnk_relay_fused_batch(bnk_ctx *ctx, const bnk_batch *in,
                           int64_t now_ns, const bnk_batch *out,
                           uint8_t *verdict, uint64_t *ctr_out);
 
-/* ---- measurement ------------------------------------------------------- */
-
-/* Runs a dependency-free VALU instruction stream and reports lane-ops per
- * second: the measured int32 ceiling the AEAD roofline is quoted against.
- * op: 0 v_add_u32, 1 v_xor_b32, 2 v_alignbit_b32, 3 v_mad_u64_u32,
- * 4 v_fma_f64, 5 v_mul_lo_u32, 6 v_add_f64, 7.. further instruction kinds
- * (see probe_kernels.hip). */
-int bnk_probe_valu(bnk_ctx *ctx, int op, uint32_t iters, double *ops_per_sec);
-
-/* Streams `bytes` (a multiple of 16) from one device buffer to another `iters`
- * times and reports bytes read plus bytes written per second: the measured HBM
- * ceiling, and the known-size launch (copy_kernel) that memory-traffic counters
- * are scaled against. */
-int bnk_probe_copy(bnk_ctx *ctx, size_t bytes, uint32_t iters, double *bytes_per_sec);
-
 #ifdef __cplusplus
 }
 #endif

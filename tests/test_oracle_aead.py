@@ -241,3 +241,27 @@ def test_openssl_batch_baseline_agrees_with_the_oracle():
     for i in (0, 1, b.n - 1):
         o, l = int(b.off[i]), int(b.lens[i])
         assert np.array_equal(opened[o:o + l], b.plain[o:o + l])
+
+
+@pytest.mark.parametrize("cfg", ["cfg2", "cfg3"])
+def test_oracle_matches_the_openssl_digests_at_full_size(cfg):
+    """The oracle's sealed bytes for configurations 2 and 3 at 2^20 packets,
+    hashed in packet order, against the digests OpenSSL produced for the same
+    seeded inputs (tests/golden/make_aead_digests.py)."""
+    import hashlib
+    import json
+    import os
+    g = json.load(open(os.path.join(os.path.dirname(__file__), "golden",
+                                    "aead_cfg2_cfg3_digests.json")))
+    n = g["packets"]
+    b = W.aead_uniform(2, n, 1420, 1440) if cfg == "cfg2" else W.aead_imix(3, n, n_peers=256)
+    out = np.zeros_like(b.plain)
+    O.seal_batch(np.ascontiguousarray(b.keys), b.peer, b.counters, b.plain, b.off, b.lens, out, b.off, 8)
+    h = hashlib.sha256()
+    if cfg == "cfg2":
+        h.update(np.ascontiguousarray(out.reshape(n, 1440)[:, :1436]).data)
+    else:
+        mv = memoryview(out)
+        for o, L in zip(b.off.tolist(), b.lens.tolist()):
+            h.update(mv[o:o + L + 16])
+    assert h.hexdigest() == g[cfg]["sha256_sealed"]

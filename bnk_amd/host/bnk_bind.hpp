@@ -10,8 +10,11 @@
 //       internal/magicsock/bind.go:296-377
 //   disco.IsDisco, disco.Magic
 //       internal/disco/disco.go:20, 177-179
-// Not mirrored: the relay path (receiveRelay, relaySend) and the path manager,
-// which carry no batch of packets.  Linux only (recvmmsg / sendmmsg).
+//   Bind.receiveRelay / Send's relay fallback / SetRelaySender / SetPeerRelay /
+//   DeliverRelay / RelayStats / ClearPeerAddr
+//       internal/magicsock/bind.go:108-139, 313-320, 431-473, 489-493
+// Not mirrored: the path manager, which carries no batch of packets.  Linux
+// only (recvmmsg / sendmmsg).
 #pragma once
 
 #ifndef _GNU_SOURCE
@@ -27,6 +30,9 @@
 #include <unistd.h>
 
 #include <array>
+#include <atomic>
+#include <condition_variable>
+#include <deque>
 #include <functional>
 #include <map>
 #include <mutex>
@@ -176,10 +182,13 @@ public:
 
     void Close()
     {
-        std::lock_guard<std::mutex> lk(mu_);
-        if (fd_ >= 0) close(fd_);
-        fd_ = -1;
-        port_ = 0;
+        {
+            std::lock_guard<std::mutex> lk(mu_);
+            if (fd_ >= 0) close(fd_);
+            fd_ = -1;
+            port_ = 0;
+        }
+        relay_cv_.notify_all(); // a receiver waiting on the relay queue sees the bind closed
     }
 
     int BatchSize() const { return kIdealBatchSize; }
@@ -198,6 +207,79 @@ public:
         if (it != peers_.end()) by_addr_.erase(it->second.addr);
         peers_[key] = Peer{addr, peer_index};
         by_addr_[addr] = key;
+    }
+    // Bind.ClearPeerAddr: forgets the direct address; Send falls back to the
+    // relay.  (The reverse map keeps the address, as in the reference.)
+    void ClearPeerAddr(const NodeKey &key)
+    {
+        std::lock_guard<std::mutex> lk(mu_);
+        peers_.erase(key);
+    }
+    // Bind.SetRelaySender: the transport for peers with no direct path.  The
+    // function reports failure by throwing; Send passes that on.
+    void SetRelaySender(std::function<void(uint32_t dst, const uint8_t *pkt, uint32_t len)> send)
+    {
+        std::lock_guard<std::mutex> lk(mu_);
+        relay_send_ = std::move(send);
+    }
+    // Bind.SetPeerRelay: the peer's relay ID, and the dense index the GPU
+    // tables use for it (ReceiveRelay reports that index).
+    void SetPeerRelay(const NodeKey &key, uint32_t id, uint32_t peer_index = 0)
+    {
+        std::lock_guard<std::mutex> lk(mu_);
+        auto it = relay_ids_.find(key);
+        if (it != relay_ids_.end()) by_relay_id_.erase(it->second.id);
+        relay_ids_[key] = RelayPeer{id, peer_index};
+        by_relay_id_[id] = key;
+    }
+    // Bind.DeliverRelay: one WireGuard packet that arrived through the relay
+    // from the peer registered under src.  Unknown IDs are dropped, and so is
+    // the packet when 64 are already waiting (UDP semantics).
+    void DeliverRelay(uint32_t src, const uint8_t *pkt, uint32_t len)
+    {
+        {
+            std::lock_guard<std::mutex> lk(mu_);
+            auto it = by_relay_id_.find(src);
+            if (it == by_relay_id_.end()) return;
+            if (relay_q_.size() >= kRelayQueue) return;
+            relay_q_.push_back(RelayPacket{it->second, relay_ids_[it->second].index,
+                                           std::vector<uint8_t>(pkt, pkt + len)});
+        }
+        relay_rx_.fetch_add(1);
+        relay_cv_.notify_one();
+    }
+    // Bind.RelayStats
+    void RelayStats(uint64_t *tx, uint64_t *rx) const
+    {
+        *tx = relay_tx_.load();
+        *rx = relay_rx_.load();
+    }
+    // Bind.receiveRelay into ring slots [0, max): waits for the first queued
+    // packet (or timeout_ms; < 0 waits until the bind closes), then drains what
+    // else has queued up to max.  Same outputs as Receive.
+    uint32_t ReceiveRelay(const Ring &ring, uint32_t max, uint32_t *sizes, uint32_t *peer,
+                          NodeKey *keys = nullptr, int timeout_ms = -1)
+    {
+        std::unique_lock<std::mutex> lk(mu_);
+        if (fd_ < 0) throw ErrClosed();
+        if (max > ring.slots()) max = ring.slots();
+        if (max == 0) return 0;
+        const auto ready = [this] { return fd_ < 0 || !relay_q_.empty(); };
+        if (timeout_ms < 0) relay_cv_.wait(lk, ready);
+        else if (!relay_cv_.wait_for(lk, std::chrono::milliseconds(timeout_ms), ready)) return 0;
+        if (fd_ < 0) throw ErrClosed();
+        uint32_t n = 0;
+        while (n < max && !relay_q_.empty()) {
+            RelayPacket &rp = relay_q_.front();
+            const uint32_t len = (uint32_t)std::min<size_t>(rp.pkt.size(), ring.room()); // copy() truncates
+            memcpy(ring.slot(n), rp.pkt.data(), len);
+            sizes[n] = len;
+            peer[n] = rp.index;
+            if (keys) keys[n] = rp.key;
+            relay_q_.pop_front();
+            n++;
+        }
+        return n;
     }
     void RemovePeer(const NodeKey &key)
     {
@@ -281,23 +363,43 @@ public:
         }
     }
 
-    // Bind.Send for the direct path: datagram i is lens[i] bytes at
-    // ring.base + offsets[i]; all go to the peer's current address in
-    // sendmmsg chunks of at most BatchSize().  Safe to call from several
-    // threads.
+    // Bind.Send: datagram i is lens[i] bytes at ring.base + offsets[i].  With
+    // a direct address known all go there in sendmmsg chunks of at most
+    // BatchSize(); else, when the peer has a relay ID and a relay sender is
+    // set, one by one through the relay (the first failure stops the batch);
+    // else ErrNoPath.  Safe to call from several threads.
     void Send(const uint8_t *base, const uint64_t *offsets, const uint32_t *lens, uint32_t n,
               const NodeKey &to)
     {
         int fd;
         AddrPort addr;
+        bool direct = false, has_relay = false;
+        uint32_t relay_id = 0;
+        std::function<void(uint32_t, const uint8_t *, uint32_t)> relay_send;
         {
             std::lock_guard<std::mutex> lk(mu_);
             fd = fd_;
             auto it = peers_.find(to);
-            if (fd >= 0 && it == peers_.end()) throw ErrNoPath();
-            if (it != peers_.end()) addr = it->second.addr;
+            if (it != peers_.end()) {
+                addr = it->second.addr;
+                direct = true;
+            }
+            auto rt = relay_ids_.find(to);
+            if (rt != relay_ids_.end()) {
+                relay_id = rt->second.id;
+                has_relay = true;
+            }
+            relay_send = relay_send_;
         }
         if (fd < 0) throw ErrClosed();
+        if (!direct) {
+            if (!(has_relay && relay_send)) throw ErrNoPath();
+            for (uint32_t i = 0; i < n; i++) {
+                relay_send(relay_id, base + offsets[i], lens[i]);
+                relay_tx_.fetch_add(1);
+            }
+            return;
+        }
         sockaddr_in6 sa = ToSockaddr(addr);
         mmsghdr msgs[kIdealBatchSize];
         iovec iov[kIdealBatchSize];
@@ -364,10 +466,26 @@ private:
         return true;
     }
 
+    struct RelayPeer {
+        uint32_t id = 0, index = 0;
+    };
+    struct RelayPacket {
+        NodeKey key;
+        uint32_t index;
+        std::vector<uint8_t> pkt;
+    };
+    static constexpr size_t kRelayQueue = 64; // the reference's channel capacity
+
     std::mutex mu_;
     int fd_ = -1;
     uint16_t port_ = 0;
     std::map<NodeKey, Peer> peers_;
+    std::map<NodeKey, RelayPeer> relay_ids_;
+    std::map<uint32_t, NodeKey> by_relay_id_;
+    std::function<void(uint32_t, const uint8_t *, uint32_t)> relay_send_;
+    std::deque<RelayPacket> relay_q_;
+    std::condition_variable relay_cv_;
+    std::atomic<uint64_t> relay_tx_{0}, relay_rx_{0};
     std::map<AddrPort, NodeKey> by_addr_;
     std::function<void(const AddrPort &, std::vector<uint8_t>)> on_disco_;
     std::function<void(std::vector<uint8_t>)> on_stun_;

@@ -9,6 +9,7 @@
 
 #include <set>
 #include <string>
+#include <thread>
 
 #include "../../bnk_amd/host/bnk_bind.hpp"
 
@@ -207,6 +208,99 @@ static void removed_and_moved_peers()
     EXPECT(B.Receive(ar.ring, 8, sizes, peer, nullptr, 200) == 0, "a removed peer's packets are dropped");
 }
 
+// internal/magicsock/relay_path_test.go:15-127, clear_addr_test.go:8-46
+static void relay_fallback_and_relay_receive()
+{
+    const NodeKey keyA = key_of(21), keyB = key_of(22);
+    RingBind A, B;
+    A.Open(0);
+    const uint16_t portB = B.Open(0);
+    Arena ar(8, 256, 16);
+    std::vector<std::pair<uint32_t, std::string>> relayed;
+    A.SetRelaySender([&](uint32_t dst, const uint8_t *p, uint32_t len) {
+        relayed.emplace_back(dst, std::string((const char *)p, len));
+    });
+    A.SetPeerRelay(keyB, 2, 7);
+    // TestSendPrefersRelayWhenNoDirectPath
+    const std::string pay = "payload", second = "second";
+    std::vector<uint8_t> buf(pay.begin(), pay.end());
+    buf.insert(buf.end(), second.begin(), second.end());
+    const uint64_t offs[2] = {0, pay.size()};
+    const uint32_t lens[2] = {(uint32_t)pay.size(), (uint32_t)second.size()};
+    A.Send(buf.data(), offs, lens, 2, keyB);
+    EXPECT(relayed.size() == 2 && relayed[0].first == 2 && relayed[0].second == "payload" &&
+               relayed[1].second == "second", "no direct path: every packet goes through the relay sender");
+    uint64_t tx = 0, rx = 0;
+    A.RelayStats(&tx, &rx);
+    EXPECT(tx == 2 && rx == 0, "relay tx counts packets");
+    A.SetPeerRelay(keyA, 1);
+    A.DeliverRelay(1, (const uint8_t *)"inbound", 7);
+    A.RelayStats(&tx, &rx);
+    EXPECT(rx == 1, "relay rx counts delivered packets");
+    // TestDirectPathStillWinsOverRelay + TestClearPeerAddrFallsBackToRelay
+    relayed.clear();
+    A.SetPeerAddr(keyB, 7, AddrPort::Loopback(portB));
+    B.SetPeerAddr(keyA, 3, AddrPort::Loopback(A.LocalPort()));
+    A.Send(buf.data(), offs, lens, 1, keyB);
+    uint32_t sizes[8], peer[8];
+    NodeKey keys[8];
+    uint32_t k = B.Receive(ar.ring, 8, sizes, peer, keys, 2000);
+    EXPECT(k == 1 && std::string((const char *)ar.ring.slot(0), sizes[0]) == "payload" && relayed.empty(),
+           "a known direct path wins over the relay");
+    A.ClearPeerAddr(keyB);
+    A.Send(buf.data(), offs + 1, lens + 1, 1, keyB);
+    EXPECT(relayed.size() == 1 && relayed[0].second == "second", "after ClearPeerAddr Send uses the relay");
+    // a failing relay sender stops the batch and surfaces
+    int calls = 0;
+    A.SetRelaySender([&](uint32_t, const uint8_t *, uint32_t) {
+        calls++;
+        throw BindError("relay down");
+    });
+    bool threw = false;
+    try {
+        A.Send(buf.data(), offs, lens, 2, keyB);
+    } catch (const BindError &) {
+        threw = true;
+    }
+    EXPECT(threw && calls == 1, "the first relay failure stops the batch");
+    // no relay ID, no address: ErrNoPath as before
+    threw = false;
+    try {
+        A.Send(buf.data(), offs, lens, 1, key_of(99));
+    } catch (const ErrNoPath &) {
+        threw = true;
+    }
+    EXPECT(threw, "no path at all");
+    // TestDeliverRelaySurfacesIdentityEndpoint + TestDeliverRelayFromUnknownIDIsDropped
+    B.SetPeerRelay(keyA, 1, 3);
+    B.DeliverRelay(99, (const uint8_t *)"stranger", 8);
+    B.DeliverRelay(1, (const uint8_t *)"known", 5);
+    B.DeliverRelay(1, (const uint8_t *)"again", 5);
+    k = B.ReceiveRelay(ar.ring, 8, sizes, peer, keys, 1000);
+    EXPECT(k == 2 && std::string((const char *)ar.ring.slot(0), sizes[0]) == "known" &&
+               std::string((const char *)ar.ring.slot(1), sizes[1]) == "again" && peer[0] == 3 && keys[0] == keyA,
+           "relay packets surface in order, tagged with the registered identity");
+    EXPECT(B.ReceiveRelay(ar.ring, 8, sizes, peer, keys, 50) == 0, "nothing queued: the wait times out");
+    // the queue holds 64; the rest are dropped
+    for (int i = 0; i < 80; i++) B.DeliverRelay(1, (const uint8_t *)"x", 1);
+    uint32_t total = 0;
+    while ((k = B.ReceiveRelay(ar.ring, 8, sizes, peer, keys, 20)) != 0) total += k;
+    EXPECT(total == 64, "the relay queue drops beyond 64 waiting packets");
+    // a closed bind ends a waiting relay receiver
+    std::thread closer([&] {
+        usleep(50 * 1000);
+        B.Close();
+    });
+    threw = false;
+    try {
+        (void)B.ReceiveRelay(ar.ring, 8, sizes, peer, keys, -1);
+    } catch (const ErrClosed &) {
+        threw = true;
+    }
+    closer.join();
+    EXPECT(threw, "ReceiveRelay on a closed bind");
+}
+
 int main()
 {
     batch_size_is_ideal();
@@ -214,6 +308,7 @@ int main()
     receive_peels_disco_and_stun_and_drops_strangers();
     send_without_known_path_fails_and_closed_bind_errors();
     removed_and_moved_peers();
+    relay_fallback_and_relay_receive();
     if (failures) {
         printf("%d failure(s)\n", failures);
         return 1;

@@ -292,7 +292,10 @@ def bench_relay(args) -> dict:
 def bench_wg(args) -> dict:
     """Transport framing around the AEAD: encapsulate (header, padding, per-peer
     counters, seal in place) and decapsulate (header checks, index lookup, open,
-    IPv4 trim, allowed-IP check) 2^20 MTU-sized packets across 1024 peers."""
+    anti-replay windows, IPv4 trim, allowed-IP check) 2^20 MTU-sized packets
+    across 1024 peers.  One step = encapsulate an arena in place, decapsulate
+    it into a second arena; the next step sends what was just received, so
+    every step carries fresh counters through the windows."""
     import numpy as np
     import torch
     from bnk_amd import lib, workloads as W
@@ -300,75 +303,69 @@ def bench_wg(args) -> dict:
     n, n_peers, plen, mtu, stride = 1 << 20, 1024, 1420, 1420, 1456
     wire_len = 16 + plen + 16
     keys = W.rand_bytes(W.stream_seed(2, 40), n_peers * 32).reshape(n_peers, 32)
-    idx_a = (np.arange(n_peers, dtype=np.uint32) * 7919 + 3).astype(np.uint32)
-    idx_b = (np.arange(n_peers, dtype=np.uint32) * 104729 + 11).astype(np.uint32)
+    # both ends in one context: each peer's two indices are the same number
+    idx = (np.arange(n_peers, dtype=np.uint32) * 7919 + 3).astype(np.uint32)
     addr = (0x64400000 + np.arange(n_peers, dtype=np.uint32)).astype(np.uint32)
     full = np.full(n_peers, 0xFFFFFFFF, np.uint32)
     peer = W.rand_below(W.stream_seed(2, 41), n, n_peers).astype(np.uint32)
     d_peer = torch.from_numpy(peer.astype(np.int32)).to(dev)
 
-    def slots():
-        a = W.rand_bytes_torch(W.stream_seed(2, 42), n * stride, dev).view(n, stride)
-        a[:, 16] = 0x45
-        a[:, 18] = plen >> 8
-        a[:, 19] = plen & 0xFF
-        src = torch.from_numpy(addr.astype(np.int64)).to(dev)[d_peer.long()]
-        for k in range(4):
-            a[:, 28 + k] = ((src >> (24 - 8 * k)) & 0xFF).to(torch.uint8)
-        return a
-
-    wire = slots()       # encapsulated once; the receive side reads it every step
-    scratch = slots()    # encapsulated in place again every step
-    out = torch.zeros(n * stride + 16, dtype=torch.uint8, device=dev)
+    a = torch.zeros(n * stride + 16, dtype=torch.uint8, device=dev)
+    b = torch.zeros(n * stride + 16, dtype=torch.uint8, device=dev)
+    slots = a[:n * stride].view(n, stride)
+    slots.copy_(W.rand_bytes_torch(W.stream_seed(2, 42), n * stride, dev).view(n, stride))
+    slots[:, 16] = 0x45
+    slots[:, 18] = plen >> 8
+    slots[:, 19] = plen & 0xFF
+    src = torch.from_numpy(addr.astype(np.int64)).to(dev)[d_peer.long()]
+    for k in range(4):
+        slots[:, 28 + k] = ((src >> (24 - 8 * k)) & 0xFF).to(torch.uint8)
+    first_plain = slots[:, 16:16 + plen].clone()
     d_wl = torch.zeros(n, dtype=torch.int32, device=dev)
     d_res = torch.zeros(n, dtype=torch.uint8, device=dev)
     d_olen = torch.zeros(n, dtype=torch.int32, device=dev)
     d_gp = torch.zeros(n, dtype=torch.int32, device=dev)
     d_gc = torch.zeros(n, dtype=torch.int64, device=dev)
     torch.cuda.synchronize()
-    tx, rx = lib.Context(0), lib.Context(0)
-    tx.keys_set(lib.KEYS_SEND, keys)
-    tx.wg_peers_set(np.stack([idx_a, idx_b, addr, full], 1))
-    rx.keys_set(lib.KEYS_RECV, keys)
-    rx.wg_peers_set(np.stack([idx_b, idx_a, addr, full], 1))
+    ctx = lib.Context(0)
+    ctx.keys_set(lib.KEYS_SEND, keys)
+    ctx.keys_set(lib.KEYS_RECV, keys)
+    ctx.wg_peers_set(np.stack([idx, idx, addr, full], 1))
     nbytes = n * stride
-    tx.wg_encap(lib.make_batch(wire, nbytes, n, lib.MEM_DEVICE, stride=stride, length=plen, peer=d_peer),
-                mtu, d_wl)
-    tx.sync()
-    assert bool((d_wl == wire_len).all())
-    b_enc = lib.make_batch(scratch, nbytes, n, lib.MEM_DEVICE, stride=stride, length=plen, peer=d_peer)
-    b_wire = lib.make_batch(wire, nbytes, n, lib.MEM_DEVICE, stride=stride, length=wire_len)
-    b_out = lib.make_batch(out[16:], nbytes, n, lib.MEM_DEVICE, stride=stride)
+    arenas = (a, b)
 
-    def step():
-        tx.wg_encap(b_enc, mtu, d_wl)
-        if args.serial:
-            tx.sync()
-        rx.wg_decap(b_wire, b_out, d_res, d_olen, d_gp, d_gc)
-        if args.serial:
-            rx.sync()
+    def step(k):
+        cur, nxt = arenas[k & 1], arenas[1 - (k & 1)]
+        ctx.wg_encap(lib.make_batch(cur, nbytes, n, lib.MEM_DEVICE, stride=stride, length=plen, peer=d_peer),
+                     mtu, d_wl)
+        # the plaintext lands 16 bytes into the other arena's slots: headroom for the next header
+        ctx.wg_decap(lib.make_batch(cur, nbytes, n, lib.MEM_DEVICE, stride=stride, length=wire_len),
+                     lib.make_batch(nxt[16:], nbytes, n, lib.MEM_DEVICE, stride=stride), d_res, d_olen, d_gp, d_gc)
 
-    for _ in range(args.warmup):
-        step()
-    tx.sync()
-    rx.sync()
+    for k in range(args.warmup):
+        step(k)
+    ctx.sync()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    tx.sync()
-    rx.sync()
+    for k in range(args.warmup, args.warmup + args.steps):
+        step(k)
+    ctx.sync()
     ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    last = arenas[(args.warmup + args.steps) & 1][:n * stride].view(n, stride)[:, 16:16 + plen]
     assert bool((d_res == 0).all()) and bool((d_olen == plen).all()) and bool((d_gp == d_peer).all())
+    assert bool((d_wl == wire_len).all()) and torch.equal(last, first_plain), "the packets did not survive the trips"
+    want_ctr = W.per_peer_sequence(peer, n_peers) + np.bincount(peer, minlength=n_peers)[peer].astype(np.uint64) * \
+        np.uint64(args.warmup + args.steps - 1)
+    assert np.array_equal(d_gc.cpu().numpy().astype(np.uint64), want_ctr), "counters do not follow the send order"
     ops = n * ops_aead(plen)
-    tx.close()
-    rx.close()
+    ctx.close()
     return {
         "metric": "wg_encap_decap_gbit_per_s", "value": round(n * plen * 8 / (ms * 1e-3) / 1e9, 1),
         "unit": "Gbit/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "u32", "data": "synthetic",
-        "config": {"workload": "transport framing: encapsulate in place + decapsulate %d packets x %d B "
-                               "(wire %d B, slot stride %d), %d peers, device resident"
+        "config": {"workload": "transport framing: encapsulate in place + decapsulate (anti-replay windows "
+                               "included) %d packets x %d B (wire %d B, slot stride %d), %d peers, device "
+                               "resident; every step sends what the step before received"
                                % (n, plen, wire_len, stride, n_peers), "packets": n},
         "mpkt_per_s_pair": round(n / (ms * 1e-3) / 1e6, 1),
         "roofline_valu": {"achieved": round(2 * ops / (ms * 1e-3) / 1e12, 2), "peak": VALU_PEAK_TOPS,
@@ -613,9 +610,6 @@ def main() -> int:
     ap.add_argument("--workload", default="aead", choices=["aead", "filter", "imix", "relay", "wg", "host", "latency", "copy"],
                     help="aead (default, the headline line, with the ACL filter rate as an extra); "
                          "filter / imix / relay / wg / host / latency / copy print one line for that workload alone")
-    ap.add_argument("--serial", action="store_true",
-                    help="wg: wait for the send side before starting the receive side, so a kernel "
-                         "trace shows undisturbed durations (the two sides use separate streams)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true",
                     help="aead: leave out the packed-layout leg and the ACL filter extra, so that a "

@@ -384,9 +384,11 @@ void bnk_shutdown(bnk_ctx *ctx)
                           &ctx->r_peer_out, &ctx->r_ctr_base, &ctx->r_ctr_out, &ctx->r_verdict,
                           &ctx->wg_index, &ctx->wg_remote, &ctx->wg_allowed, &ctx->wg_send_ctr,
                           &ctx->wg_peer, &ctx->wg_counter, &ctx->wg_ctlen, &ctx->wg_result,
-                          &ctx->wg_outlen, &ctx->wg_padded, &ctx->wg_wirelen, &ctx->wg_skip})
+                          &ctx->wg_outlen, &ctx->wg_padded, &ctx->wg_wirelen, &ctx->wg_skip, &ctx->wg_sctr,
+                          &ctx->wg_sval, &ctx->wg_pmax, &ctx->wg_lastb, &ctx->wg_rtable, &ctx->wg_rflags})
             b->release();
         ctx->pin.release();
+        if (ctx->wg_replay) (void)hipFree(ctx->wg_replay);
         for (const bnk_ctx::Ring &r : ctx->rings) (void)hipHostFree(reinterpret_cast<void *>(r.host));
         ctx->rings.clear();
         for (int w = 0; w < 2; w++)

@@ -117,6 +117,11 @@ struct bnk_ctx {
     bnk::DevBuf wg_index, wg_remote, wg_allowed, wg_send_ctr;
     uint32_t n_wg_peers = 0;
     std::vector<bnk_wg_peer> wg_rows; // host copy of the peer table, row by row
+    // anti-replay windows, one per row, and the scratch of a replay pass
+    uint64_t *wg_replay = nullptr;
+    uint32_t wg_replay_rows = 0;
+    bool wg_replay_on = true;
+    bnk::DevBuf wg_sctr, wg_sval, wg_pmax, wg_lastb, wg_rtable, wg_rflags;
     bnk::DevBuf wg_peer, wg_counter, wg_ctlen, wg_result, wg_outlen, wg_padded, wg_wirelen, wg_skip;
 
     bnk::FilterState *filter = nullptr;

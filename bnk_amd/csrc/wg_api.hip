@@ -30,6 +30,33 @@ int upload(bnk_ctx *ctx, DevBuf *dst, const void *src, size_t bytes)
 
 } // namespace
 
+// The anti-replay windows follow the peer table: n rows, those flagged in
+// `fresh` (n bytes, host) start empty, the others keep what they hold.
+static int wg_replay_rows(bnk_ctx *ctx, uint32_t n, const std::vector<uint8_t> &fresh)
+{
+    if (n > ctx->wg_replay_rows) {
+        uint64_t *grown = nullptr;
+        const size_t row = (size_t)WG_REPLAY_WORDS * 8;
+        HIPCHK(ctx, hipMalloc((void **)&grown, (size_t)n * row));
+        hipError_t e = hipMemsetAsync(grown, 0, (size_t)n * row, ctx->stream);
+        if (e == hipSuccess && ctx->wg_replay_rows)
+            e = hipMemcpyAsync(grown, ctx->wg_replay, (size_t)ctx->wg_replay_rows * row, hipMemcpyDeviceToDevice,
+                               ctx->stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+        if (e != hipSuccess) {
+            (void)hipFree(grown);
+            return fail_hip(ctx, "replay windows", e);
+        }
+        if (ctx->wg_replay) (void)hipFree(ctx->wg_replay);
+        ctx->wg_replay = grown;
+        ctx->wg_replay_rows = n;
+    }
+    int rc = upload(ctx, &ctx->wg_rflags, fresh.data(), n);
+    if (rc) return rc;
+    HIPCHK(ctx, launch_wg_replay_reset(ctx->wg_replay, ctx->wg_rflags.as<uint8_t>(), n, ctx->stream));
+    return BNK_OK;
+}
+
 // Checks the rows and builds the sorted (local index, row) table.
 static int wg_build_index(bnk_ctx *ctx, const bnk_wg_peer *peers, uint32_t n, std::vector<uint2> *index)
 {
@@ -69,17 +96,20 @@ extern "C" int bnk_wg_peers_set(bnk_ctx *ctx, const bnk_wg_peer *peers, uint32_t
     // a fresh keypair and starts at 0.
     const uint32_t n_old = ctx->n_wg_peers;
     std::vector<uint64_t> ctr(std::max(n, n_old), 0);
+    std::vector<uint8_t> fresh(n, 1);
     if (n_old)
         HIPCHK(ctx, hipMemcpy(ctr.data(), ctx->wg_send_ctr.p, (size_t)n_old * 8, hipMemcpyDeviceToHost));
     for (uint32_t i = 0; i < n; i++) {
         const bool same = i < n_old && ctx->wg_rows[i].local_index == peers[i].local_index &&
                           ctx->wg_rows[i].remote_index == peers[i].remote_index;
         if (!same) ctr[i] = 0;
+        fresh[i] = same ? 0 : 1; // the anti-replay window belongs to the keypair as well
     }
     rc = upload(ctx, &ctx->wg_index, index.data(), (size_t)n * 8);
     if (!rc) rc = upload(ctx, &ctx->wg_remote, remote.data(), (size_t)n * 4);
     if (!rc) rc = upload(ctx, &ctx->wg_allowed, allowed.data(), (size_t)n * 8);
     if (!rc) rc = upload(ctx, &ctx->wg_send_ctr, ctr.data(), (size_t)n * 8);
+    if (!rc) rc = wg_replay_rows(ctx, n, fresh);
     if (rc) {
         ctx->n_wg_peers = 0; // a half-installed table is no table
         ctx->wg_rows.clear();
@@ -115,8 +145,10 @@ extern "C" int bnk_wg_peer_set(bnk_ctx *ctx, uint32_t row, const bnk_wg_peer *pe
     HIPCHK(ctx, hipMemcpyAsync(ctx->wg_index.p, index.data(), index.size() * 8, hipMemcpyHostToDevice, s));
     HIPCHK(ctx, hipMemcpyAsync(ctx->wg_remote.as<uint32_t>() + row, &peer->remote_index, 4, hipMemcpyHostToDevice, s));
     HIPCHK(ctx, hipMemcpyAsync(ctx->wg_allowed.as<uint2>() + row, &allowed, 8, hipMemcpyHostToDevice, s));
-    // this row's keypair is new: its nonces start over; every other row goes on
+    // this row's keypair is new: its nonces and its anti-replay window start
+    // over; every other row goes on
     HIPCHK(ctx, hipMemcpyAsync(ctx->wg_send_ctr.as<uint64_t>() + row, &zero, 8, hipMemcpyHostToDevice, s));
+    HIPCHK(ctx, hipMemsetAsync(ctx->wg_replay + (size_t)row * WG_REPLAY_WORDS, 0, (size_t)WG_REPLAY_WORDS * 8, s));
     if (key_send32)
         HIPCHK(ctx, hipMemcpyAsync(ctx->d_keys[BNK_KEYS_SEND] + 8u * row, key_send32, 32, hipMemcpyHostToDevice, s));
     if (key_recv32)
@@ -136,6 +168,16 @@ extern "C" int bnk_wg_send_counter_set(bnk_ctx *ctx, uint32_t row, uint64_t next
     if (next > WG_REJECT_AFTER_MESSAGES) next = WG_REJECT_AFTER_MESSAGES;
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
     HIPCHK(ctx, hipMemcpy(ctx->wg_send_ctr.as<uint64_t>() + row, &next, 8, hipMemcpyHostToDevice));
+    return BNK_OK;
+    BNK_API_CATCH(ctx)
+}
+
+extern "C" int bnk_wg_set_replay(bnk_ctx *ctx, int on)
+{
+    BNK_API_TRY
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    ctx->wg_replay_on = on != 0;
     return BNK_OK;
     BNK_API_CATCH(ctx)
 }
@@ -650,6 +692,43 @@ static int wg_decap_impl(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *o
     const bool check = check_now != nullptr && ctx->filter->enforce;
     if (check) HIPCHK(ctx, ctx->r_pass.reserve(n));
 
+    // the anti-replay windows, walked per chunk in batch order
+    const bool replay = ctx->wg_replay_on;
+    WgReplayDev rpd{ctx->wg_replay, pe.n};
+    WgReplayScratch rsc{};
+    if (replay && n > WG_REPLAY_SMALL_MAX) {
+        const uint32_t biggest = chunked ? hp.per : n;
+        for (DevBuf *buf : {&ctx->r_keys, &ctx->r_idx, &ctx->r_skeys, &ctx->r_sidx})
+            HIPCHK(ctx, buf->reserve((size_t)biggest * 4));
+        for (DevBuf *buf : {&ctx->wg_sctr, &ctx->wg_sval, &ctx->wg_pmax}) HIPCHK(ctx, buf->reserve((size_t)biggest * 8));
+        HIPCHK(ctx, ctx->wg_lastb.reserve((size_t)biggest + 64));
+        rsc.table_slots = wg_replay_table_slots(biggest);
+        HIPCHK(ctx, ctx->wg_rtable.reserve((size_t)rsc.table_slots * 4));
+        rsc.tmp_bytes = wg_replay_tmp_bytes(biggest, pe.n);
+        HIPCHK(ctx, ctx->r_tmp.reserve(rsc.tmp_bytes + 16));
+        rsc.keys = ctx->r_keys.as<uint32_t>();
+        rsc.idx = ctx->r_idx.as<uint32_t>();
+        rsc.skeys = ctx->r_skeys.as<uint32_t>();
+        rsc.sidx = ctx->r_sidx.as<uint32_t>();
+        rsc.sctr = ctx->wg_sctr.as<uint64_t>();
+        rsc.sval = ctx->wg_sval.as<uint64_t>();
+        rsc.pmax = ctx->wg_pmax.as<uint64_t>();
+        rsc.cls = ctx->wg_lastb.as<uint8_t>() + 64;
+        rsc.flags = ctx->wg_lastb.as<uint32_t>();
+        rsc.table = ctx->wg_rtable.as<uint32_t>();
+        rsc.tmp = ctx->r_tmp.p;
+    }
+    // wireguard-go's sequential receiver validates the counter of every
+    // authentic packet before it looks inside: ahead of the inbound filter
+    auto replay_range = [&](uint32_t lo, uint32_t hi) -> int {
+        if (!replay) return BNK_OK;
+        WgReplayScratch c = rsc;
+        c.table_slots = hi - lo > WG_REPLAY_SMALL_MAX ? wg_replay_table_slots(hi - lo) : 0;
+        HIPCHK(ctx, launch_wg_replay(d_result + lo, d_out_len + lo, d_peer + lo, d_counter + lo, hi - lo, rpd, c,
+                                     ctx->stream));
+        return BNK_OK;
+    };
+
     // CheckInbound of what packets [lo, hi) delivered: a packet that was not
     // delivered has length 0 here, which the filter refuses without a side effect
     auto filter_range = [&](uint32_t lo, uint32_t hi) -> int {
@@ -703,6 +782,7 @@ static int wg_decap_impl(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *o
                 op.wg.peer_out = d_peer;
                 op.wg.counter_out = d_counter;
                 HIPCHK(ctx, launch_aead_open(op, ctx->stream));
+                if (int rr = replay_range(lo, hi)) return rr;
                 return filter_range(lo, hi);
             }
         }
@@ -734,6 +814,7 @@ static int wg_decap_impl(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *o
         }
         HIPCHK(ctx, launch_aead_open(op, ctx->stream));
         HIPCHK(ctx, launch_wg_finish(co, 0, pe, d_peer, d_ctlen, d_auth, d_result, d_out_len, ctx->stream));
+        if (int rr = replay_range(lo, hi)) return rr;
         return filter_range(lo, hi);
     };
 

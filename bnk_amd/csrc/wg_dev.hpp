@@ -35,6 +35,40 @@ hipError_t launch_wg_encap_prep(const WgBatch &b, uint8_t *hdr_base, const WgPee
                                 const uint64_t *counter, uint32_t mtu, uint32_t *padded_len,
                                 uint32_t *wire_len, uint8_t *skip, uint32_t *status, hipStream_t s);
 
+// Anti-replay windows (wg_replay.hip): per peer WG_REPLAY_WORDS 64-bit words,
+// `last` then a ring of WG_REPLAY_BLOCKS blocks of 64 counters (RFC 6479 as
+// wireguard-go's replay.Filter: window (128 - 1) * 64 = 8128).
+constexpr uint32_t WG_REPLAY_BLOCKS = 128;
+constexpr uint32_t WG_REPLAY_WORDS = 1 + WG_REPLAY_BLOCKS;
+constexpr uint32_t WG_REPLAY_SMALL_MAX = 1024; // at most this many packets: one launch of one block
+
+struct WgReplayDev {
+    uint64_t *state; // [n_peers][WG_REPLAY_WORDS]
+    uint32_t n_peers;
+};
+
+// Device scratch of one replay pass over n packets (beyond WG_REPLAY_SMALL_MAX).
+struct WgReplayScratch {
+    uint32_t *keys, *idx, *skeys, *sidx;   // n words each
+    uint64_t *sctr, *sval, *pmax;          // n each
+    uint8_t *cls;                          // n
+    uint32_t *flags;                       // one word
+    uint32_t *table;                       // table_slots words, a power of two >= 2 n
+    uint32_t table_slots;
+    void *tmp;                             // wg_replay_tmp_bytes(n, n_peers)
+    size_t tmp_bytes;
+};
+size_t wg_replay_tmp_bytes(uint32_t n, uint32_t n_peers);
+uint32_t wg_replay_table_slots(uint32_t n);
+// Runs every packet whose result so far says "authentic" (anything but
+// BAD_HEADER, UNKNOWN_INDEX, AUTH_FAIL) through its peer's window, in batch
+// order per peer; a packet the window turns away gets BNK_WG_REPLAY and
+// out_len 0.  The arrays are indexed from the first packet of the pass.
+hipError_t launch_wg_replay(uint8_t *result, uint32_t *out_len, const uint32_t *peer, const uint64_t *counter,
+                            uint32_t n, const WgReplayDev &rp, const WgReplayScratch &sc, hipStream_t s);
+// Clears the windows of the rows whose flag is set.
+hipError_t launch_wg_replay_reset(uint64_t *state, const uint8_t *flags, uint32_t n_peers, hipStream_t s);
+
 // result[i] = BNK_WG_FILTERED where it was BNK_WG_OK and pass[i] == 0.
 hipError_t launch_wg_mark_filtered(uint8_t *result, const uint8_t *pass, uint32_t n, hipStream_t s);
 

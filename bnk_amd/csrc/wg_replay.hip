@@ -1,0 +1,446 @@
+// Anti-replay window of the WireGuard receive path (RFC 6479 as wireguard-go's
+// replay.Filter keeps it: a ring of 128 64-bit blocks, window 8128 counters),
+// one window per peer, device resident, applied to a whole batch at once with
+// the result the sequential receiver would reach packet by packet.
+//
+// wireguard-go validates the counter of every authentic packet, in arrival
+// order per peer, before it looks at the plaintext (device/receive.go,
+// RoutineSequentialReceiver; the reference only instantiates that device,
+// internal/dataplane/engine.go:51).  Sequentially the filter does, per packet:
+// reject counter >= limit; if counter > last, clear the blocks passed over and
+// move last; else reject when last - counter > window; then test-and-set the
+// counter's bit.  For a batch this unrolls without walking it in order:
+//
+//   last before packet j  = max(last before the batch, counters of earlier
+//                           packets of the same peer)   -- a running maximum,
+//                           whether those packets were accepted or not, because
+//                           a packet that does not move last is not above it;
+//   packet j reaches the bit test iff counter < limit and it is not more than
+//                           the window behind that last;
+//   its bit is already set iff the counter was seen before: in the window the
+//                           batch started with, or by an earlier packet of the
+//                           batch with the same counter (which reached the bit
+//                           test too, the window having only moved forward
+//                           since).  Inside the window a bit is never stale:
+//                           a slot is cleared the moment last enters or passes
+//                           its block.
+//
+// So: a stable sort of (peer, position) brings each peer's packets together in
+// batch order, a segmented running maximum gives every packet its `last`, a
+// hash table keyed by (peer, counter) finds the first of equal counters (only
+// packets at or below an earlier counter can be repeats, so a batch whose
+// counters rise within every peer never touches the table), and the windows
+// are brought up to date afterwards (clear what last passed over, then set the
+// bits of everything that reached the bit test and still lies in the final
+// window).
+#include <string.h>
+
+#include <algorithm>
+
+#include <rocprim/rocprim.hpp>
+
+#include "../../include/bnkhip.h"
+#include "kernels.hpp"
+#include "wg_dev.hpp"
+
+namespace bnk {
+
+namespace {
+
+constexpr uint32_t NO_PEER = 0xFFFFFFFFu;
+constexpr uint32_t HASH_EMPTY = 0xFFFFFFFFu;
+constexpr uint64_t WINDOW = (WG_REPLAY_BLOCKS - 1u) * 64u; // 8128
+
+__device__ __forceinline__ bool replay_subject(uint8_t result)
+{
+    // everything that was authentic: the tag verified
+    return result != BNK_WG_BAD_HEADER && result != BNK_WG_UNKNOWN_INDEX && result != BNK_WG_AUTH_FAIL;
+}
+
+__device__ __forceinline__ uint64_t mix(uint64_t x)
+{
+    x ^= x >> 33;
+    x *= 0xff51afd7ed558ccdULL;
+    x ^= x >> 33;
+    x *= 0xc4ceb9fe1a85ec53ULL;
+    x ^= x >> 33;
+    return x;
+}
+
+// Does the packet reach the filter's bit test, given `last` just before it?
+__device__ __forceinline__ bool reaches_bit_test(uint64_t c, uint64_t last)
+{
+    return c < WG_REJECT_AFTER_MESSAGES && (c > last || last - c <= WINDOW);
+}
+
+// Was counter c (at or below last0, inside the window) seen before the batch?
+__device__ __forceinline__ bool seen_before(const uint64_t *st, uint64_t c)
+{
+    return (st[1u + ((c >> 6) & (WG_REPLAY_BLOCKS - 1u))] >> (c & 63u)) & 1ull;
+}
+
+// Brings one peer's window to `new_last`: clears the blocks passed over.
+__device__ __forceinline__ void advance_window(uint64_t *st, uint64_t new_last)
+{
+    const uint64_t last0 = st[0];
+    if (new_last <= last0) return;
+    const uint64_t cur = last0 >> 6;
+    uint64_t diff = (new_last >> 6) - cur;
+    if (diff > WG_REPLAY_BLOCKS) diff = WG_REPLAY_BLOCKS;
+    for (uint64_t b = cur + 1; b <= cur + diff; b++) st[1u + (b & (WG_REPLAY_BLOCKS - 1u))] = 0;
+    st[0] = new_last;
+}
+
+// ---- large batches ---------------------------------------------------------
+
+__global__ __launch_bounds__(256) void replay_keys_kernel(const uint8_t *result, const uint32_t *peer,
+                                                          uint32_t n_peers, uint32_t n, uint32_t *keys,
+                                                          uint32_t *idx)
+{
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i >= n) return;
+    const uint32_t p = peer[i];
+    keys[i] = (replay_subject(result[i]) && p < n_peers) ? p : NO_PEER;
+    idx[i] = i;
+}
+
+// Counters in sorted order; a counter the filter turns away outright counts as
+// 0 for the running maximum (it never moves last).
+__global__ __launch_bounds__(256) void replay_gather_kernel(const uint32_t *skeys, const uint32_t *sidx,
+                                                            const uint64_t *counter, uint32_t n,
+                                                            uint64_t *sctr, uint64_t *sval)
+{
+    const uint32_t p = blockIdx.x * 256u + threadIdx.x;
+    if (p >= n) return;
+    const uint64_t c = skeys[p] != NO_PEER ? counter[sidx[p]] : 0;
+    sctr[p] = c;
+    sval[p] = c < WG_REJECT_AFTER_MESSAGES ? c : 0;
+}
+
+// What the window decides about a packet without looking at other packets'
+// counters: turned away outright, ahead of everything before it (fresh for
+// certain), or inside the window at or below an earlier counter ("late": fresh
+// unless that counter was seen before).
+enum : uint8_t { RP_NONE = 0, RP_AHEAD = 1, RP_LATE = 2 };
+
+__device__ __forceinline__ uint32_t table_home(uint32_t key, uint64_t c, uint32_t mask)
+{
+    return (uint32_t)mix(c ^ ((uint64_t)key << 40) ^ key) & mask;
+}
+
+// Classifies every packet; turns away what never reaches the bit test; enters
+// the late ones into the table (slot = earliest sorted position carrying that
+// peer and counter) and raises flags[0] when there are any.
+__global__ __launch_bounds__(256) void replay_classify_kernel(const uint32_t *skeys, const uint32_t *sidx,
+                                                              const uint64_t *sctr, const uint64_t *pmax,
+                                                              const uint64_t *state, uint32_t n, uint8_t *cls,
+                                                              uint32_t *table, uint32_t mask, uint32_t *flags,
+                                                              uint8_t *result, uint32_t *out_len)
+{
+    const uint32_t p = blockIdx.x * 256u + threadIdx.x;
+    if (p >= n) return;
+    const uint32_t key = skeys[p];
+    uint8_t k = RP_NONE;
+    if (key != NO_PEER) {
+        const uint64_t c = sctr[p];
+        const uint64_t last0 = state[(size_t)key * WG_REPLAY_WORDS];
+        const uint64_t last = last0 > pmax[p] ? last0 : pmax[p];
+        if (reaches_bit_test(c, last)) k = c > last ? RP_AHEAD : RP_LATE;
+        if (k == RP_NONE) {
+            const uint32_t i = sidx[p];
+            result[i] = BNK_WG_REPLAY;
+            out_len[i] = 0;
+        } else if (k == RP_LATE) {
+            flags[0] = 1u; // the same value from every lane that has the news
+            uint32_t h = table_home(key, c, mask);
+            for (;;) {
+                const uint32_t old = atomicCAS(&table[h], HASH_EMPTY, p);
+                if (old == HASH_EMPTY) break;
+                if (skeys[old] == key && sctr[old] == c) {
+                    atomicMin(&table[h], p);
+                    break;
+                }
+                h = (h + 1u) & mask; // the table has at least twice as many slots as packets
+            }
+        }
+    }
+    cls[p] = k;
+}
+
+// A late packet may repeat a packet that was ahead when it came: those look
+// their counter up and take the slot over when they are the earlier one.
+// Nothing to do in a batch without late packets.
+__global__ __launch_bounds__(256) void replay_claim_kernel(const uint32_t *skeys, const uint64_t *sctr,
+                                                           const uint8_t *cls, uint32_t n, uint32_t *table,
+                                                           uint32_t mask, const uint32_t *flags)
+{
+    if (flags[0] == 0u) return;
+    const uint32_t p = blockIdx.x * 256u + threadIdx.x;
+    if (p >= n || cls[p] != RP_AHEAD) return;
+    const uint32_t key = skeys[p];
+    const uint64_t c = sctr[p];
+    uint32_t h = table_home(key, c, mask);
+    for (;;) {
+        const uint32_t at = table[h];
+        if (at == HASH_EMPTY) return; // no late packet carries my counter
+        if (skeys[at] == key && sctr[at] == c) {
+            atomicMin(&table[h], p);
+            return;
+        }
+        h = (h + 1u) & mask;
+    }
+}
+
+// A late packet is fresh when its counter was not seen before the batch and no
+// earlier packet of the batch carried it.
+__global__ __launch_bounds__(256) void replay_late_kernel(const uint32_t *skeys, const uint32_t *sidx,
+                                                          const uint64_t *sctr, const uint8_t *cls,
+                                                          const uint64_t *state, uint32_t n,
+                                                          const uint32_t *table, uint32_t mask,
+                                                          const uint32_t *flags, uint8_t *result,
+                                                          uint32_t *out_len)
+{
+    if (flags[0] == 0u) return;
+    const uint32_t p = blockIdx.x * 256u + threadIdx.x;
+    if (p >= n || cls[p] != RP_LATE) return;
+    const uint32_t key = skeys[p];
+    const uint64_t c = sctr[p];
+    const uint64_t *st = state + (size_t)key * WG_REPLAY_WORDS;
+    bool fresh = !(c <= st[0] && seen_before(st, c));
+    if (fresh) {
+        uint32_t h = table_home(key, c, mask);
+        for (;;) {
+            const uint32_t at = table[h];
+            if (at == HASH_EMPTY) break; // cannot happen: it was entered
+            if (skeys[at] == key && sctr[at] == c) {
+                fresh = at == p;
+                break;
+            }
+            h = (h + 1u) & mask;
+        }
+    }
+    if (!fresh) {
+        const uint32_t i = sidx[p];
+        result[i] = BNK_WG_REPLAY;
+        out_len[i] = 0;
+    }
+}
+
+// The last packet of each peer's run knows where that peer's `last` ends up.
+__global__ __launch_bounds__(256) void replay_advance_kernel(const uint32_t *skeys, const uint64_t *sctr,
+                                                             const uint64_t *pmax, uint64_t *state,
+                                                             uint32_t n)
+{
+    const uint32_t p = blockIdx.x * 256u + threadIdx.x;
+    if (p >= n) return;
+    const uint32_t key = skeys[p];
+    if (key == NO_PEER) return;
+    if (p + 1u < n && skeys[p + 1u] == key) return;
+    const uint64_t c = sctr[p];
+    uint64_t last = pmax[p];
+    if (c < WG_REJECT_AFTER_MESSAGES && c > last) last = c;
+    advance_window(state + (size_t)key * WG_REPLAY_WORDS, last);
+}
+
+// Sets the bit of every packet that reached the bit test and still lies in the
+// window its peer ends the batch with.  Neighbours in sorted order mostly
+// share their peer and their block of 64 counters: a lane whose left neighbour
+// differs gathers the bits of the lanes behind it that agree with it and
+// issues one atomic for all of them.
+__global__ __launch_bounds__(256) void replay_mark_kernel(const uint32_t *skeys, const uint64_t *sctr,
+                                                          const uint8_t *cls, uint64_t *state, uint32_t n)
+{
+    const uint32_t p = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t lane = threadIdx.x & 63u;
+    uint32_t key = NO_PEER;
+    uint64_t block = ~0ull, bit = 0;
+    if (p < n && cls[p] != RP_NONE) {
+        key = skeys[p];
+        const uint64_t c = sctr[p];
+        const uint64_t final_last = state[(size_t)key * WG_REPLAY_WORDS];
+        if ((final_last >> 6) - (c >> 6) < WG_REPLAY_BLOCKS) { // else its slot now belongs to a later block
+            block = c >> 6;
+            bit = 1ull << (c & 63u);
+        } else {
+            key = NO_PEER;
+        }
+    }
+    // runs of equal (peer, block) among neighbouring lanes
+    const uint32_t pkey = (uint32_t)__shfl_up((int)key, 1, 64);
+    const uint32_t pblo = (uint32_t)__shfl_up((int)(uint32_t)block, 1, 64);
+    const uint32_t pbhi = (uint32_t)__shfl_up((int)(uint32_t)(block >> 32), 1, 64);
+    const bool head = lane == 0 || pkey != key || pblo != (uint32_t)block || pbhi != (uint32_t)(block >> 32);
+    const unsigned long long heads = __ballot(head);
+    // my run ends before the next head after me
+    const unsigned long long after = lane == 63u ? 0ull : heads & ~((2ull << lane) - 1ull);
+    const uint32_t end = after ? (uint32_t)__ffsll((long long)after) - 1u : 64u;
+    uint64_t acc = bit;
+    // suffix OR within the run: six doubling steps cover 64 lanes
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const uint32_t lo = (uint32_t)__shfl_down((int)(uint32_t)acc, off, 64);
+        const uint32_t hi = (uint32_t)__shfl_down((int)(uint32_t)(acc >> 32), off, 64);
+        if (lane + (uint32_t)off < end) acc |= (uint64_t)hi << 32 | lo;
+    }
+    if (head && key != NO_PEER && acc != 0)
+        atomicOr(reinterpret_cast<unsigned long long *>(
+                     &state[(size_t)key * WG_REPLAY_WORDS + 1u + (block & (WG_REPLAY_BLOCKS - 1u))]),
+                 (unsigned long long)acc);
+}
+
+unsigned key_bits(uint32_t n_keys)
+{
+    unsigned bits = 1;
+    while (bits < 32 && (n_keys >> bits) != 0) bits++;
+    return bits;
+}
+
+using SortConfig = rocprim::radix_sort_config<rocprim::default_config, rocprim::default_config,
+                                              rocprim::default_config, 32768>;
+
+// ---- small batches: one block, everything in LDS ----------------------------
+
+constexpr uint32_t SMALL = WG_REPLAY_SMALL_MAX;
+
+__global__ __launch_bounds__(SMALL) void replay_small_kernel(uint8_t *result, uint32_t *out_len,
+                                                             const uint32_t *peer, const uint64_t *counter,
+                                                             uint32_t n_peers, uint32_t n, uint64_t *state,
+                                                             unsigned bits)
+{
+    using Sort = rocprim::block_radix_sort<uint32_t, SMALL, 1, uint32_t>;
+    using Scan = rocprim::block_scan<uint32_t, SMALL>;
+    __shared__ union {
+        typename Sort::storage_type sort;
+        typename Scan::storage_type scan;
+    } tmp;
+    __shared__ uint32_t sk[SMALL + 1];
+    __shared__ uint64_t sc[SMALL];
+    const uint32_t t = threadIdx.x;
+    uint32_t key[1] = {NO_PEER}, pos[1] = {t};
+    if (t < n) {
+        const uint32_t p = peer[t];
+        if (replay_subject(result[t]) && p < n_peers) key[0] = p;
+    }
+    // stable: a peer's packets stay in batch order
+    Sort().sort(key, pos, tmp.sort, 0, bits);
+    const bool valid = key[0] != NO_PEER;
+    const uint64_t c = valid ? counter[pos[0]] : 0;
+    sk[t] = key[0];
+    sc[t] = c;
+    if (t == 0) sk[SMALL] = NO_PEER;
+    __syncthreads();
+    const bool head = t == 0 || sk[t - 1] != key[0];
+    uint32_t start = 0;
+    Scan().inclusive_scan(head ? t : 0u, start, tmp.scan, rocprim::maximum<uint32_t>());
+    uint64_t *st = valid ? state + (size_t)key[0] * WG_REPLAY_WORDS : nullptr;
+    const uint64_t last0 = valid ? st[0] : 0;
+    // the packets of my peer ahead of me: their running maximum, and whether
+    // one of them carried my counter
+    uint64_t last = last0;
+    bool dup = false;
+    if (valid) {
+        for (uint32_t u = start; u < t; u++) {
+            const uint64_t cu = sc[u];
+            if (cu < WG_REJECT_AFTER_MESSAGES && cu > last) last = cu;
+            dup |= cu == c;
+        }
+    }
+    const bool reached = valid && reaches_bit_test(c, last);
+    bool fresh = reached && !dup;
+    if (fresh && c <= last0 && seen_before(st, c)) fresh = false;
+    if (valid && !fresh) {
+        result[pos[0]] = BNK_WG_REPLAY;
+        out_len[pos[0]] = 0;
+    }
+    __syncthreads(); // every window has been read as the batch found it
+    const bool tail = valid && sk[t + 1] != key[0];
+    if (tail) {
+        uint64_t nl = last;
+        if (c < WG_REJECT_AFTER_MESSAGES && c > nl) nl = c;
+        advance_window(st, nl);
+    }
+    __threadfence();
+    __syncthreads(); // the cleared blocks are in place before bits go in
+    if (reached) {
+        const uint64_t final_last = *reinterpret_cast<volatile uint64_t *>(st);
+        if ((final_last >> 6) - (c >> 6) < WG_REPLAY_BLOCKS)
+            atomicOr(reinterpret_cast<unsigned long long *>(&st[1u + ((c >> 6) & (WG_REPLAY_BLOCKS - 1u))]),
+                     1ull << (c & 63u));
+    }
+}
+
+__global__ __launch_bounds__(256) void replay_reset_kernel(uint64_t *state, const uint8_t *flags, uint32_t n_peers)
+{
+    const uint32_t total = n_peers * WG_REPLAY_WORDS;
+    const uint32_t stride = gridDim.x * 256u;
+    for (uint32_t w = blockIdx.x * 256u + threadIdx.x; w < total; w += stride)
+        if (flags[w / WG_REPLAY_WORDS]) state[w] = 0;
+}
+
+} // namespace
+
+hipError_t launch_wg_replay_reset(uint64_t *state, const uint8_t *flags, uint32_t n_peers, hipStream_t s)
+{
+    if (n_peers == 0) return hipSuccess;
+    const uint32_t blocks = std::min<uint32_t>((n_peers * WG_REPLAY_WORDS + 255u) / 256u, 2048u);
+    hipLaunchKernelGGL(replay_reset_kernel, dim3(blocks), dim3(256), 0, s, state, flags, n_peers);
+    return hipGetLastError();
+}
+
+size_t wg_replay_tmp_bytes(uint32_t n, uint32_t n_peers)
+{
+    size_t a = 0, b = 0;
+    (void)rocprim::radix_sort_pairs<SortConfig>(nullptr, a, (const uint32_t *)nullptr, (uint32_t *)nullptr,
+                                                (const uint32_t *)nullptr, (uint32_t *)nullptr, (size_t)n, 0,
+                                                key_bits(n_peers));
+    (void)rocprim::exclusive_scan_by_key(nullptr, b, (const uint32_t *)nullptr, (const uint64_t *)nullptr,
+                                         (uint64_t *)nullptr, (uint64_t)0, (size_t)n,
+                                         rocprim::maximum<uint64_t>(), rocprim::equal_to<uint32_t>());
+    return std::max(a, b);
+}
+
+uint32_t wg_replay_table_slots(uint32_t n)
+{
+    uint32_t s = 1024;
+    while (s < 2u * n && s < (1u << 31)) s <<= 1;
+    return s;
+}
+
+hipError_t launch_wg_replay(uint8_t *result, uint32_t *out_len, const uint32_t *peer, const uint64_t *counter,
+                            uint32_t n, const WgReplayDev &rp, const WgReplayScratch &sc, hipStream_t s)
+{
+    if (n == 0) return hipSuccess;
+    if (n <= SMALL) {
+        hipLaunchKernelGGL(replay_small_kernel, dim3(1), dim3(SMALL), 0, s, result, out_len, peer, counter,
+                           rp.n_peers, n, rp.state, key_bits(rp.n_peers));
+        return hipGetLastError();
+    }
+    const dim3 grid((n + 255u) / 256u);
+    hipLaunchKernelGGL(replay_keys_kernel, grid, dim3(256), 0, s, result, peer, rp.n_peers, n, sc.keys, sc.idx);
+    size_t bytes = sc.tmp_bytes;
+    hipError_t e = rocprim::radix_sort_pairs<SortConfig>(sc.tmp, bytes, sc.keys, sc.skeys, sc.idx, sc.sidx,
+                                                         (size_t)n, 0, key_bits(rp.n_peers), s);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(replay_gather_kernel, grid, dim3(256), 0, s, sc.skeys, sc.sidx, counter, n, sc.sctr,
+                       sc.sval);
+    bytes = sc.tmp_bytes;
+    e = rocprim::exclusive_scan_by_key(sc.tmp, bytes, sc.skeys, sc.sval, sc.pmax, (uint64_t)0, (size_t)n,
+                                       rocprim::maximum<uint64_t>(), rocprim::equal_to<uint32_t>(), s);
+    if (e != hipSuccess) return e;
+    e = launch_fill_u32(sc.table, sc.table_slots, HASH_EMPTY, s);
+    if (e != hipSuccess) return e;
+    e = launch_fill_u32(sc.flags, 1, 0u, s);
+    if (e != hipSuccess) return e;
+    const uint32_t mask = sc.table_slots - 1u;
+    hipLaunchKernelGGL(replay_classify_kernel, grid, dim3(256), 0, s, sc.skeys, sc.sidx, sc.sctr, sc.pmax,
+                       rp.state, n, sc.cls, sc.table, mask, sc.flags, result, out_len);
+    hipLaunchKernelGGL(replay_claim_kernel, grid, dim3(256), 0, s, sc.skeys, sc.sctr, sc.cls, n, sc.table, mask,
+                       sc.flags);
+    hipLaunchKernelGGL(replay_late_kernel, grid, dim3(256), 0, s, sc.skeys, sc.sidx, sc.sctr, sc.cls, rp.state, n,
+                       sc.table, mask, sc.flags, result, out_len);
+    hipLaunchKernelGGL(replay_advance_kernel, grid, dim3(256), 0, s, sc.skeys, sc.sctr, sc.pmax, rp.state, n);
+    hipLaunchKernelGGL(replay_mark_kernel, grid, dim3(256), 0, s, sc.skeys, sc.sctr, sc.cls, rp.state, n);
+    return hipGetLastError();
+}
+
+} // namespace bnk

@@ -40,6 +40,7 @@ class Batch(C.Structure):
 WG_OK, WG_KEEPALIVE, WG_BAD_HEADER, WG_UNKNOWN_INDEX, WG_AUTH_FAIL, WG_BAD_IP, \
     WG_NOT_ALLOWED = range(7)
 WG_FILTERED = 7
+WG_REPLAY = 8
 
 
 class Rule(C.Structure):
@@ -344,6 +345,10 @@ class Context:
 
     def wg_send_counter_set(self, row: int, value: int) -> None:
         self._chk(self._lib.bnk_wg_send_counter_set(self._h, C.c_uint32(row), C.c_uint64(value)))
+
+    def wg_set_replay(self, on: bool) -> None:
+        """Anti-replay windows on (default) or off for the decapsulating calls."""
+        self._chk(self._lib.bnk_wg_set_replay(self._h, C.c_int(1 if on else 0)))
 
     def wg_send_counters(self, n: int) -> np.ndarray:
         out = np.zeros(max(n, 1), np.uint64)

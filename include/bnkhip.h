@@ -241,9 +241,7 @@ int bnk_filter_flow_dump(bnk_ctx *ctx, uint64_t *key, uint8_t *proto,
  * configures with one /32 allowed IP per peer (engine.go:292-299); that
  * package is not in the reference tree, so these entry points follow the
  * WireGuard protocol paper (section 5.4.6) and wireguard-go's documented
- * behaviour (device/send.go, device/receive.go).  The anti-replay window
- * (RFC 6479) is order dependent and stays on the host, fed with the peer and
- * counter this call reports. */
+ * behaviour (device/send.go, device/receive.go, replay/replay.go). */
 
 enum {
     BNK_WG_OK = 0,            /* data packet, delivered */
@@ -253,8 +251,11 @@ enum {
     BNK_WG_AUTH_FAIL = 4,     /* tag mismatch */
     BNK_WG_BAD_IP = 5,        /* not IPv4/IPv6 or length fields beyond the plaintext */
     BNK_WG_NOT_ALLOWED = 6,   /* inner source outside the peer's allowed IP */
-    BNK_WG_FILTERED = 7       /* bnk_wg_decap_filter_batch only: delivered by
+    BNK_WG_FILTERED = 7,      /* bnk_wg_decap_filter_batch only: delivered by
                                  WireGuard, dropped by the inbound filter */
+    BNK_WG_REPLAY = 8         /* authentic, but its counter was seen before, lies
+                                 more than 8128 behind the peer's newest, or is
+                                 at or beyond RejectAfterMessages */
 };
 
 typedef struct bnk_wg_peer {
@@ -300,21 +301,34 @@ int bnk_wg_encap_batch(bnk_ctx *ctx, const bnk_batch *slots, uint32_t mtu,
  * result[i] is BNK_WG_*; for BNK_WG_OK the inner packet, trimmed to its IP
  * total length, is out_len[i] bytes at out's offset i.  For every result but
  * BAD_HEADER/UNKNOWN_INDEX peer[i] and counter[i] name the sender and the
- * nonce counter (feed them to the replay window when result is OK or
- * KEEPALIVE); otherwise peer[i] = 0xFFFFFFFF.  A failed open leaves zeros in
- * `out`, like the AEAD entry points.  wire->peer/counters are ignored.
+ * nonce counter; otherwise peer[i] = 0xFFFFFFFF.  A failed open leaves zeros in
+ * `out`, like the AEAD entry points.
+ * Every authentic packet (any result but BAD_HEADER, UNKNOWN_INDEX, AUTH_FAIL)
+ * goes through its peer's anti-replay window (RFC 6479, 8128 counters, kept on
+ * the device per row of the peer table) in batch order, before the keepalive,
+ * IP and allowed-IP checks count, as wireguard-go's sequential receiver does:
+ * a packet the window turns away reports BNK_WG_REPLAY (out_len 0, plaintext
+ * left in `out`), and an authentic packet with a bad or disallowed inner
+ * header still moves the window.  bnk_wg_set_replay(ctx, 0) leaves the windows
+ * out (for a caller that keeps its own).  wire->peer/counters are ignored.
  * result, out_len, peer and counter live where wire->mem says. */
 int bnk_wg_decap_batch(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *out,
                        uint8_t *result, uint32_t *out_len, uint32_t *peer,
                        uint64_t *counter);
+
+/* Anti-replay windows on (default) or off for bnk_wg_decap_batch and
+ * bnk_wg_decap_filter_batch.  Off: no packet reports BNK_WG_REPLAY and the
+ * windows stand still; the caller then feeds peer[i]/counter[i] of every
+ * authentic packet to a window of its own. */
+int bnk_wg_set_replay(bnk_ctx *ctx, int on);
 
 /* The receive path of a tunnel in one call: bnk_wg_decap_batch, then
  * CheckInbound (internal/filter/filter.go:121-147) with one now_ns on every
  * packet that came out BNK_WG_OK, as filteredTUN.Write (filter.go:171-186)
  * does with what wireguard-go hands it.  A packet the filter denies reports
  * BNK_WG_FILTERED; everything else about it (plaintext in its slot, out_len,
- * peer, counter) is as for BNK_WG_OK, because wireguard-go runs the replay
- * window before the write that filters: feed its counter to the window too.
+ * peer, counter) is as for BNK_WG_OK, and its counter has moved the replay
+ * window, because wireguard-go runs the window before the write that filters.
  * In allow-all mode nothing is filtered.  Same arguments as
  * bnk_wg_decap_batch otherwise. */
 int bnk_wg_decap_filter_batch(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *out,

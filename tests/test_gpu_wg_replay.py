@@ -1,0 +1,213 @@
+"""The anti-replay windows of bnk_wg_decap_batch (RFC 6479 as wireguard-go's
+replay.Filter, one per peer, on the device, a whole batch at a time) against
+the sequential filter of the oracle (bnko_replay_validate) fed packet by
+packet in batch order, with wireguard-go's ordering: every authentic packet
+goes through its peer's window before its inner header counts.  The window
+itself is pinned on the CPU (tests/cpp/replay_test.cpp, tests/test_oracle_wg.py);
+like the rest of the framing it is spec-derived, not a reference artefact."""
+import struct
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+P = 6
+LIMIT = (1 << 64) - (1 << 13) - 1
+WINDOW = 8128
+
+
+def _peers():
+    tx = [(1000 + 13 * i, 7000 + 17 * i, 0x64400001 + i, 0xFFFFFFFF) for i in range(P)]
+    rx = [(p[1], p[0], p[2], p[3]) for p in tx]
+    return tx, rx
+
+
+def _inner(rng, src, length, kind):
+    if kind == "keepalive":
+        return b""
+    pkt = bytearray(rng.integers(0, 256, length, dtype=np.uint8).tobytes())
+    pkt[0] = 0x45 if kind != "badip" else 0x15
+    pkt[2:4] = struct.pack(">H", length)
+    pkt[12:16] = struct.pack(">I", src if kind != "notallowed" else src ^ 0x00010000)
+    return bytes(pkt)
+
+
+def _counters(rng, n, last):
+    """A walk around each peer's newest counter: forward steps, repeats,
+    reordering, the window's edges on both sides, far jumps."""
+    peer = rng.integers(0, P, n)
+    ctr = np.zeros(n, np.uint64)
+    last = list(last)
+    recent = [[] for _ in range(P)]
+    for i in range(n):
+        p = int(peer[i])
+        r = rng.random()
+        if r < 0.55:
+            c = last[p] + int(rng.integers(1, 4))
+        elif r < 0.70 and recent[p]:
+            c = recent[p][int(rng.integers(0, len(recent[p])))]          # an exact repeat
+        elif r < 0.80:
+            c = max(0, last[p] - int(rng.integers(0, 200)))              # a little late
+        elif r < 0.86:
+            c = max(0, last[p] - WINDOW + int(rng.integers(-2, 3)))      # the far edge of the window
+        elif r < 0.90:
+            c = last[p] + int(rng.integers(60, 70)) * int(rng.integers(1, 200))  # over one or many blocks
+        elif r < 0.93:
+            c = last[p] + WINDOW + int(rng.integers(-2, 3)) + 64         # just beyond a whole ring
+        elif r < 0.95:
+            c = 0
+        else:
+            c = last[p] + int(rng.integers(1, 3))
+        c = min(c, LIMIT + 3)
+        ctr[i] = c
+        if c < LIMIT:
+            last[p] = max(last[p], c)
+        recent[p] = (recent[p] + [c])[-50:]
+    return peer.astype(np.uint32), ctr, last
+
+
+def _batch(rng, tx, keys, n, last, near_limit=False):
+    from oracle import binding as O
+    peer, ctr, last = _counters(rng, n, last)
+    if near_limit:
+        ctr[:6] = np.array([LIMIT - 2, LIMIT - 1, LIMIT, LIMIT + 1, LIMIT - 1, LIMIT - 2], np.uint64)
+        peer[:6] = 0
+    kinds = rng.choice(["ok", "ok", "ok", "ok", "keepalive", "notallowed", "badip", "forged"], n)
+    wires, offs, pos = [], np.zeros(n, np.uint64), 0
+    for i in range(n):
+        p = int(peer[i])
+        inner = _inner(rng, tx[p][2], int(rng.choice([20, 28, 60, 200, 576])), kinds[i])
+        w = bytearray(O.wg_encap(inner, 1420, keys[p].tobytes(), tx[p][1], int(ctr[i])))
+        if kinds[i] == "forged":
+            w[-1] ^= 1
+        offs[i] = pos
+        wires.append(bytes(w))
+        pos += (len(w) + 15) & ~15
+    arena = np.zeros(pos + 16, np.uint8)
+    for i, w in enumerate(wires):
+        arena[int(offs[i]):int(offs[i]) + len(w)] = np.frombuffer(w, np.uint8)
+    lens = np.array([len(w) for w in wires], np.uint32)
+    return arena, offs, lens, wires, last
+
+
+def _expect(wires, rx, keys, filters):
+    """Oracle result per packet, then the sequential window per peer in batch order."""
+    from bnk_amd import lib
+    from oracle import binding as O
+    n = len(wires)
+    res, olen, peer, ctr = np.zeros(n, np.uint8), np.zeros(n, np.uint32), np.zeros(n, np.uint32), np.zeros(n, np.uint64)
+    for i, w in enumerate(wires):
+        rc, pt, p, c = O.wg_decap(w, rx, keys)
+        res[i], olen[i], peer[i], ctr[i] = rc, len(pt), p, c
+        if rc not in (lib.WG_BAD_HEADER, lib.WG_UNKNOWN_INDEX, lib.WG_AUTH_FAIL):
+            if not filters[p].validate(c):
+                res[i], olen[i] = lib.WG_REPLAY, 0
+    return res, olen, peer, ctr
+
+
+@pytest.mark.parametrize("mode", ["host_fused", "host_unfused", "device_large", "ring_fused"])
+def test_replay_windows_match_the_sequential_filter(mode):
+    import torch
+    from bnk_amd import lib
+    from oracle import binding as O
+    rng = np.random.default_rng(2024)
+    tx, rx = _peers()
+    keys = rng.integers(0, 256, (P, 32), dtype=np.uint8)
+    filters = [O.ReplayFilter() for _ in range(P)]
+    last = [0] * P
+    sizes = {"host_fused": [1, 64, 300, 1024, 700], "host_unfused": [300, 1024, 2000, 150],
+             "device_large": [5000, 1025, 9000, 3000], "ring_fused": [128, 900, 128]}[mode]
+    seen = set()
+    with lib.Context(0) as ctx:
+        ctx.keys_set(lib.KEYS_RECV, keys)
+        ctx.wg_peers_set(rx)
+        if mode == "host_unfused":
+            ctx.set_spread_max_packets(0)
+        for b, n in enumerate(sizes):
+            arena, offs, lens, wires, last = _batch(rng, tx, keys, n, last, near_limit=(b == 2))
+            want = _expect(wires, rx, keys, filters)
+            total = arena.nbytes
+            if mode == "device_large":
+                d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to("cuda:0")  # noqa: E731
+                d_arena, d_out = d(arena), torch.zeros(total, dtype=torch.uint8, device="cuda:0")
+                res = torch.zeros(n, dtype=torch.uint8, device="cuda:0")
+                olen = torch.zeros(n, dtype=torch.int32, device="cuda:0")
+                gp = torch.zeros(n, dtype=torch.int32, device="cuda:0")
+                gc = torch.zeros(n, dtype=torch.int64, device="cuda:0")
+                d_off, d_len = d(offs.astype(np.int64)), d(lens.astype(np.int32))
+                torch.cuda.synchronize()
+                ctx.wg_decap(lib.make_batch(d_arena, total, n, lib.MEM_DEVICE, offsets=d_off, lens=d_len),
+                             lib.make_batch(d_out, total, n, lib.MEM_DEVICE, offsets=d_off), res, olen, gp, gc)
+                ctx.sync()
+                got = (res.cpu().numpy(), olen.cpu().numpy().astype(np.uint32), gp.cpu().numpy().astype(np.uint32),
+                       gc.cpu().numpy().astype(np.uint64))
+            else:
+                rings = []
+                if mode == "ring_fused":
+                    rings = [ctx.ring_alloc(total), ctx.ring_alloc(total)]
+                    rings[0][:] = arena
+                src = rings[0] if rings else arena
+                out = rings[1] if rings else np.zeros(total, np.uint8)
+                res, olen = np.zeros(n, np.uint8), np.zeros(n, np.uint32)
+                gp, gc = np.zeros(n, np.uint32), np.zeros(n, np.uint64)
+                ctx.wg_decap(lib.make_batch(src, total, n, lib.MEM_HOST, offsets=offs, lens=lens),
+                             lib.make_batch(out, total, n, lib.MEM_HOST, offsets=offs), res, olen, gp, gc)
+                got = (res, olen, gp, gc)
+                for r in rings:
+                    ctx.ring_free(r)
+            bad = np.flatnonzero(got[0] != want[0])
+            assert bad.size == 0, f"batch {b}: result differs at {bad[:5]}: got {got[0][bad[:5]]} want {want[0][bad[:5]]}"
+            assert np.array_equal(got[1], want[1]) and np.array_equal(got[2], want[2]) and np.array_equal(got[3], want[3])
+            seen.update(np.unique(want[0]).tolist())
+    # the walk exercised every outcome, replays among them
+    assert {lib.WG_OK, lib.WG_KEEPALIVE, lib.WG_AUTH_FAIL, lib.WG_BAD_IP, lib.WG_NOT_ALLOWED, lib.WG_REPLAY} <= seen
+
+
+def test_a_rekeyed_peer_starts_with_an_empty_window_and_the_switch_turns_windows_off():
+    from bnk_amd import lib
+    from oracle import binding as O
+    rng = np.random.default_rng(7)
+    tx, rx = _peers()
+    keys = rng.integers(0, 256, (P, 32), dtype=np.uint8)
+
+    def decap(ctx, wires):
+        n = len(wires)
+        offs = np.arange(n, dtype=np.uint64) * 128
+        arena = np.zeros(n * 128, np.uint8)
+        for i, w in enumerate(wires):
+            arena[i * 128:i * 128 + len(w)] = np.frombuffer(w, np.uint8)
+        lens = np.array([len(w) for w in wires], np.uint32)
+        out = np.zeros_like(arena)
+        res, olen, gp, gc = np.zeros(n, np.uint8), np.zeros(n, np.uint32), np.zeros(n, np.uint32), np.zeros(n, np.uint64)
+        ctx.wg_decap(lib.make_batch(arena, arena.nbytes, n, lib.MEM_HOST, offsets=offs, lens=lens),
+                     lib.make_batch(out, out.nbytes, n, lib.MEM_HOST, offsets=offs), res, olen, gp, gc)
+        return res.tolist()
+
+    def dg(p, c, key=None, remote=None):
+        inner = _inner(rng, tx[p][2], 40, "ok")
+        return O.wg_encap(inner, 1420, (keys[p] if key is None else key).tobytes(), tx[p][1] if remote is None else remote, c)
+
+    with lib.Context(0) as ctx:
+        ctx.keys_set(lib.KEYS_RECV, keys)
+        ctx.wg_peers_set(rx)
+        assert decap(ctx, [dg(0, 5), dg(1, 5), dg(0, 5), dg(0, 4)]) == [lib.WG_OK, lib.WG_OK, lib.WG_REPLAY, lib.WG_OK]
+        assert decap(ctx, [dg(0, 5), dg(0, 4), dg(1, 5), dg(0, 6)]) == [lib.WG_REPLAY] * 3 + [lib.WG_OK]
+        # peer 0 rekeys: new indices, new key, and a window that has seen nothing;
+        # peer 1's window stands
+        new_key = rng.integers(0, 256, 32, dtype=np.uint8)
+        ctx.wg_peer_set(0, (rx[0][0] + 1, rx[0][1], rx[0][2], rx[0][3]), key_recv=new_key)
+        assert decap(ctx, [dg(0, 5, new_key, rx[0][0] + 1), dg(1, 5), dg(0, 5)]) == \
+            [lib.WG_OK, lib.WG_REPLAY, lib.WG_UNKNOWN_INDEX]
+        # the same table again keeps the windows; a changed row starts over
+        rows = [(rx[0][0] + 1, rx[0][1], rx[0][2], rx[0][3])] + rx[1:]
+        ctx.wg_peers_set(rows)
+        assert decap(ctx, [dg(0, 5, new_key, rx[0][0] + 1), dg(1, 5)]) == [lib.WG_REPLAY, lib.WG_REPLAY]
+        rows[1] = (rx[1][0] + 1, rx[1][1], rx[1][2], rx[1][3])
+        ctx.wg_peers_set(rows)
+        assert decap(ctx, [dg(1, 5, None, rx[1][0] + 1), dg(0, 5, new_key, rx[0][0] + 1)]) == [lib.WG_OK, lib.WG_REPLAY]
+        # windows off: nothing is turned away and nothing is recorded
+        ctx.wg_set_replay(False)
+        assert decap(ctx, [dg(2, 9), dg(2, 9)]) == [lib.WG_OK, lib.WG_OK]
+        ctx.wg_set_replay(True)
+        assert decap(ctx, [dg(2, 9), dg(2, 9)]) == [lib.WG_OK, lib.WG_REPLAY]

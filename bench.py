@@ -40,6 +40,8 @@ VALU_PEAK_TOPS = 39.3  # 256 CU x 64 lanes x 2.4 GHz, one int32 op per lane per 
 # they change only when the kernel does.
 VALU_LANE_INSTR_PER_PACKET = 31276   # SQ_INSTS_VALU x 64 / 2^20
 TRAFFIC_BYTES_PER_LAUNCH = 3.187e9   # FETCH_SIZE + WRITE_SIZE, scaled by copy_kernel
+# the same for filter_check_kernel over 2^22 headers (profiles/filter_check_kernel_cfg4.md)
+FILTER_TRAFFIC_BYTES_PER_LAUNCH = 191.6e6
 
 
 def ops_chacha(length: int) -> int:
@@ -64,9 +66,9 @@ def _events(torch, stream, k):
 
 
 def bench_filter(args) -> dict:
-    """Configuration 4: 2^22 IPv4 headers (32-byte records) against 4096 rules
-    and a flow table built from 65,536 noted outbound packets; one step = one
-    CheckInbound batch."""
+    """Configuration 4: 2^22 IPv4 headers (28-byte records back to back) against
+    4096 rules and a flow table built from 65,536 noted outbound packets; one
+    step = one CheckInbound batch."""
     import numpy as np
     import torch
     from bnk_amd import lib, workloads as W
@@ -79,10 +81,11 @@ def bench_filter(args) -> dict:
         ctx.filter_note_outbound(
             lib.make_batch(buf, buf.nbytes, rec.shape[0], lib.MEM_HOST, stride=32, length=28), now)
     dev = torch.device("cuda:0")
-    d_rec = torch.from_numpy(w.check).to(dev)
+    # the headers back to back: 20 bytes of IPv4 + 8 of L4, nothing between them
+    d_rec = torch.from_numpy(np.ascontiguousarray(w.check[:, :28])).to(dev)
     d_v = torch.zeros(n, dtype=torch.uint8, device=dev)
     torch.cuda.synchronize()
-    batch = lib.make_batch(d_rec, n * 32, n, lib.MEM_DEVICE, stride=32, length=28)
+    batch = lib.make_batch(d_rec, n * 28, n, lib.MEM_DEVICE, stride=28, length=28)
     for _ in range(args.warmup):
         ctx.filter_check_inbound(batch, w.now_ns, d_v)
     ctx.sync()
@@ -108,14 +111,15 @@ def bench_filter(args) -> dict:
         "unit": "Mpkt/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "u32", "data": "synthetic",
-        "config": {"workload": "cfg4: CheckInbound of %d IPv4 headers, 4096 rules, flow table from "
-                               "65536 noted packets, device resident" % n,
+        "config": {"workload": "cfg4: CheckInbound of %d IPv4 headers (28-byte records back to back), 4096 "
+                               "rules, flow table from 65536 noted packets, device resident" % n,
                    "packets": n, "rules": 4096, "allowed_fraction": round(allowed, 4)},
         "roofline": {"bound": "hbm", "kernel": "filter_check_kernel", "achieved": round(gbs, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
-                     # FETCH_SIZE x2 + WRITE_SIZE under rocprofv3 --pmc for this launch
-                     # (profiles/filter_check_kernel_cfg4.md); not re-measured by this run
-                     "traffic": 234.8e6 if n == 1 << 22 else None, "bytes_per_launch": alg_bytes,
+                     "traffic": FILTER_TRAFFIC_BYTES_PER_LAUNCH if n == 1 << 22 else None,
+                     "traffic_source": "profiles/filter_check_kernel_cfg4.md (FETCH_SIZE and WRITE_SIZE under "
+                                       "rocprofv3 --pmc, scaled by copy_kernel; not re-measured in this run)",
+                     "bytes_per_launch": alg_bytes,
                      "avg_launch_ms": round(kern_ms, 4)},
     }
     if not args.no_cpu_baseline:
@@ -138,6 +142,41 @@ def bench_filter(args) -> dict:
                       "of filter.go/acl.go (linear rule scan under one lock, as the reference), "
                       "1 thread" % sample,
             "gpu_output_matches": bool(np.array_equal(ov, v[:sample])),
+        }
+        # All cores: the reference serialises CheckInbound behind one mutex
+        # (filter.go:122), so more cores do not help it; this is what the same
+        # algorithm gives with one private filter (rules and flows) per core.
+        import threading
+        threads = min(16, os.cpu_count() or 1)
+        per = 1 << 15
+        filters = []
+        for _ in range(threads):
+            f = O.Filter()
+            f.set_rules(w.rules_ref)
+            for now, rec in w.note_batches:
+                m = rec.shape[0]
+                f.note_outbound_batch(np.ascontiguousarray(rec).reshape(-1),
+                                      np.arange(m, dtype=np.uint64) * 32, np.full(m, 28, np.uint32), now)
+            filters.append(f)
+        outs = [None] * threads
+
+        def work(t):
+            part = np.ascontiguousarray(w.check[t * per:(t + 1) * per]).reshape(-1)
+            outs[t] = filters[t].check_inbound_batch(part, np.arange(per, dtype=np.uint64) * 32,
+                                                     np.full(per, 28, np.uint32), w.now_ns)
+
+        ths = [threading.Thread(target=work, args=(t,)) for t in range(threads)]
+        tp = time.perf_counter()
+        for th in ths:
+            th.start()
+        for th in ths:
+            th.join()
+        dt = time.perf_counter() - tp
+        out["cpu_baseline_all_cores"] = {
+            "value": round(threads * per / dt / 1e6, 4), "unit": "Mpkt/s", "cores": threads, "kind": "port",
+            "sample": "%d threads x %d headers of the same workload, one private filter per thread (the "
+                      "reference's single mutex would serialise them)" % (threads, per),
+            "gpu_output_matches": bool(np.array_equal(np.concatenate(outs), v[:threads * per])),
         }
     ctx.close()
     return out
@@ -866,7 +905,8 @@ def main() -> int:
     ctx.close()
     acl = bench_filter(args)
     out["extra"] = {"acl_filter": {k: acl[k] for k in ("metric", "value", "unit", "ms_per_step",
-                                                       "config", "roofline", "cpu_baseline")
+                                                       "config", "roofline", "cpu_baseline",
+                                                       "cpu_baseline_all_cores")
                                    if k in acl}}
     # what one call costs at wireguard-go's own batch size (128 packets in pinned rings)
     largs = argparse.Namespace(**vars(args))

@@ -305,6 +305,10 @@ __global__ __launch_bounds__(FILTER_THREADS, 8) void filter_check_kernel(FilterA
             s = flow_slot(a.flows, h.src, h.sport, h.dport, h.proto);
             if (small) {
                 maybe = ((lsmall[s.sbit0 >> 5] >> (s.sbit0 & 31u)) & (lsmall[s.sbit1 >> 5] >> (s.sbit1 & 31u)) & 1u) != 0u;
+                // one in eleven keys that were never stored passes the small
+                // filter; the large one (a word from L2) turns nine in ten of
+                // those away before they cost a 128-byte line of the table
+                if (maybe) maybe = ((a.flows.present[s.bit >> 5] >> (s.bit & 31u)) & 1u) != 0u;
             } else {
                 maybe = ((a.flows.present[s.bit >> 5] >> (s.bit & 31u)) & 1u) != 0u;
             }

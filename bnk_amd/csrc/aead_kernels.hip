@@ -55,34 +55,37 @@ BNK_DEV void st16a(uint8_t *p, uint4 v)
 BNK_DEV uint8_t ld8(const uint8_t *p) { return *reinterpret_cast<const BNK_GLOBAL uint8_t *>((uintptr_t)p); }
 BNK_DEV void st8(uint8_t *p, uint8_t v) { *reinterpret_cast<BNK_GLOBAL uint8_t *>((uintptr_t)p) = v; }
 
-// m in 1..15 bytes at p, zero-extended to 16.
+typedef uint32_t __attribute__((aligned(1))) u32_unaligned;
+typedef uint16_t __attribute__((aligned(1))) u16_unaligned;
+
+// m in 1..15 bytes at p (any alignment), zero-extended to 16, without touching
+// a byte beyond them: whole words first, then a halfword, then a byte.
 BNK_DEV uint4 ld_partial(const uint8_t *p, uint32_t m)
 {
     uint32_t w[4] = {0, 0, 0, 0};
+    const uint32_t nd = m >> 2;
 #pragma unroll
-    for (int i = 0; i < 15; i++)
-        if ((uint32_t)i < m) w[i >> 2] |= (uint32_t)ld8(p + i) << (8 * (i & 3));
+    for (int q = 0; q < 3; q++)
+        if ((uint32_t)q < nd) w[q] = *reinterpret_cast<const BNK_GLOBAL u32_unaligned *>((uintptr_t)(p + 4 * q));
+    uint32_t last = 0;
+    if (m & 2u) last = *reinterpret_cast<const BNK_GLOBAL u16_unaligned *>((uintptr_t)(p + 4u * nd));
+    if (m & 1u) last |= (uint32_t)ld8(p + 4u * nd + (m & 2u)) << (8u * (m & 2u));
+    if (nd == 0) w[0] = last;
+    else if (nd == 1) w[1] = last;
+    else if (nd == 2) w[2] = last;
+    else w[3] = last;
     return make_uint4(w[0], w[1], w[2], w[3]);
 }
 
 BNK_DEV void st_partial(uint8_t *p, uint4 v, uint32_t m)
 {
     const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-    for (int i = 0; i < 15; i++)
-        if ((uint32_t)i < m) st8(p + i, (uint8_t)(w[i >> 2] >> (8 * (i & 3))));
-}
-
-// The same for a 16-byte aligned p: dwords, then a halfword, then a byte.
-BNK_DEV void st_partial_aligned(uint8_t *p, uint4 v, uint32_t m)
-{
-    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
     const uint32_t nd = m >> 2;
 #pragma unroll
     for (int q = 0; q < 3; q++)
-        if ((uint32_t)q < nd) *reinterpret_cast<BNK_GLOBAL uint32_t *>((uintptr_t)(p + 4 * q)) = w[q];
+        if ((uint32_t)q < nd) *reinterpret_cast<BNK_GLOBAL u32_unaligned *>((uintptr_t)(p + 4 * q)) = w[q];
     const uint32_t last = nd == 0 ? w[0] : nd == 1 ? w[1] : nd == 2 ? w[2] : w[3];
-    if (m & 2u) *reinterpret_cast<BNK_GLOBAL uint16_t *>((uintptr_t)(p + 4u * nd)) = (uint16_t)last;
+    if (m & 2u) *reinterpret_cast<BNK_GLOBAL u16_unaligned *>((uintptr_t)(p + 4u * nd)) = (uint16_t)last;
     if (m & 1u) st8(p + 4u * nd + (m & 2u), (uint8_t)(last >> (8u * (m & 2u))));
 }
 
@@ -184,7 +187,7 @@ BNK_DEV void crypt_tail_lds(Poly32 &mac, const uint32_t (&x)[16], int j, const u
                                           v.w ^ x[4 * j + 3]), m);
     if (OPEN) mac.block(v.x, v.y, v.z, v.w);
     else mac.block(o.x, o.y, o.z, o.w);
-    st_partial_aligned(d, o, m);
+    st_partial(d, o, m);
 }
 
 template <bool OPEN>
@@ -257,7 +260,13 @@ BNK_DEV void body_generic(uint8_t *tile, uint32_t lane, const uint8_t *src, uint
     }
 }
 
-template <bool OPEN>
+// ALIGNED: every packet of the wave 16-byte aligned, source and destination at
+// the same place within a 128-byte line: the stream of cells starts at the line
+// holding the packet's first byte and every access is a whole aligned cell.
+// Otherwise the stream starts at the packet itself (any alignment, source and
+// destination independent): the same pipeline over 128-byte pieces of the
+// packet, which then straddle two lines each.
+template <bool OPEN, bool ALIGNED>
 BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_t *dst, uint32_t len,
                         const uint8_t *safe, const uint32_t (&k)[8], uint32_t n1, uint32_t n2,
                         Poly32 &mac, uint32_t (&x)[16])
@@ -265,7 +274,7 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
     // Cells are 16 bytes; a packet's cell kc sits at stream position c0 + kc,
     // where the stream starts at the 128-byte line holding the packet's first
     // byte.  Stream position K lives in line K / 8 and in ring cell K % 16.
-    const uint32_t skew = (uint32_t)(uintptr_t)src & 127u;
+    const uint32_t skew = ALIGNED ? (uint32_t)(uintptr_t)src & 127u : 0u;
     const uint32_t c0 = skew >> 4;
     const uint32_t ncell = len >> 4; // whole cells; the last 1-15 bytes are written by their owner,
                                      // but their cell comes in with the others
@@ -283,7 +292,9 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
         cfirst[q] = (uint32_t)__shfl((int)c0, owner, 64);
         const uint32_t olen = (uint32_t)__shfl((int)len, owner, 64);
         cend[q] = cfirst[q] + (olen >> 4);
-        cend_ld[q] = cfirst[q] + ((olen + 15u) >> 4);
+        // (a cell that is not aligned may reach into the next page: only aligned ones
+        // are fetched beyond the packet's last byte)
+        cend_ld[q] = cfirst[q] + ((olen + (ALIGNED ? 15u : 0u)) >> 4);
     }
     uint32_t maxsteps = steps;
 #pragma unroll
@@ -319,16 +330,18 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
     // branch closes, eight times per line; loading unconditionally from a harmless
     // address instead keeps all eight in flight (cells outside the packet are
     // fetched from `safe` and never leave their register).
-#define BNK_ISSUE(q, m) pre##q = ld16a(BNK_INSIDE_LD(q, m) ? csrc[q] + 128u * (m) : safe)
-#define BNK_ISSUE_ALL(q, m) pre##q = ld16a(csrc[q] + 128u * (m))
+#define BNK_LD(p) (ALIGNED ? ld16a(p) : ld16(p))
+#define BNK_ST(p, v) do { if (ALIGNED) st16a(p, v); else st16(p, v); } while (0)
+#define BNK_ISSUE(q, m) pre##q = BNK_LD(BNK_INSIDE_LD(q, m) ? csrc[q] + 128u * (m) : safe)
+#define BNK_ISSUE_ALL(q, m) pre##q = BNK_LD(csrc[q] + 128u * (m))
 #define BNK_COMMIT(q, m) if (BNK_INSIDE_LD(q, m)) *BNK_SLOT(q, m) = pre##q
 #define BNK_COMMIT_ALL(q, m) *BNK_SLOT(q, m) = pre##q
 #define BNK_STORE(q, m)                                                                     \
     do {                                                                                    \
         const uint4 out_##q = *BNK_SLOT(q, m); /* read first, unconditionally: same reason */ \
-        if (BNK_INSIDE(q, m)) st16a(cdst[q] + 128u * (m), out_##q);                         \
+        if (BNK_INSIDE(q, m)) BNK_ST(cdst[q] + 128u * (m), out_##q);                         \
     } while (0)
-#define BNK_STORE_ALL(q, m) st16a(cdst[q] + 128u * (m), *BNK_SLOT(q, m))
+#define BNK_STORE_ALL(q, m) BNK_ST(cdst[q] + 128u * (m), *BNK_SLOT(q, m))
 #define BNK_EIGHT(OP, m)                                                                    \
     do {                                                                                    \
         OP(0, m); OP(1, m); OP(2, m); OP(3, m); OP(4, m); OP(5, m); OP(6, m); OP(7, m);     \
@@ -376,9 +389,13 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
                         for (int j = 0; j < 4; j++) {
                             const uint32_t kc = 4u * b + j;
                             if (kc < ncell) crypt_cell<OPEN>(mac, x, j, row + (((c0 + kc) & 15u) << 4));
-                            else if (kc == ncell && (len & 15u))
-                                crypt_tail_lds<OPEN>(mac, x, j, row + (((c0 + kc) & 15u) << 4), dst + 16u * kc,
-                                                     len & 15u);
+                            else if (kc == ncell && (len & 15u)) {
+                                if (ALIGNED)
+                                    crypt_tail_lds<OPEN>(mac, x, j, row + (((c0 + kc) & 15u) << 4), dst + 16u * kc,
+                                                         len & 15u);
+                                else
+                                    crypt_tail<OPEN>(mac, x, j, src + 16u * kc, dst + 16u * kc, len & 15u);
+                            }
                         }
                     }
                 }
@@ -389,6 +406,8 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
         wave_sync();
     }
 #undef BNK_INSIDE
+#undef BNK_LD
+#undef BNK_ST
 #undef BNK_INSIDE_LD
 #undef BNK_SLOT
 #undef BNK_ISSUE
@@ -595,9 +614,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const bool lane_lines = (((uintptr_t)src | (uintptr_t)dst) & 15u) == 0 &&
                             (((uintptr_t)src ^ (uintptr_t)dst) & 127u) == 0;
     const uint8_t *safe = reinterpret_cast<const uint8_t *>(a.keys);
-    if (__ballot(!lane_lines) != 0ull) body_generic<OPEN>(tile, lane, src, dst, len, safe, k, n1, n2, mac, x);
+    if (__ballot(!lane_lines) != 0ull) body_lines<OPEN, false>(tile, lane, src, dst, len, safe, k, n1, n2, mac, x);
     else if (__ballot(len > 64u * SHORT_BLOCKS) == 0ull) body_short<OPEN>(tile, lane, src, dst, len, safe, k, n1, n2, mac, x);
-    else body_lines<OPEN>(tile, lane, src, dst, len, safe, k, n1, n2, mac, x);
+    else body_lines<OPEN, true>(tile, lane, src, dst, len, safe, k, n1, n2, mac, x);
 
     lane_finish<OPEN>(a, lane, have, i, len, src, dst, mac);
 }

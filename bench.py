@@ -16,7 +16,7 @@ Prints ONE JSON line.  Besides the contract fields it carries
   extra          the ACL filter rate (configuration 4) with its own roofline and CPU
                  baseline, and what one call costs on 128 packets in pinned host rings
 
---workload filter | imix | relay | wg | host | latency | copy print one line for that
+--workload filter | imix | relay | wg | host | latency | copy | sizes print one line for that
 workload alone; --no-extras leaves out everything but the timed launches (for traces).
 """
 from __future__ import annotations
@@ -628,6 +628,64 @@ def bench_latency(args) -> dict:
     }
 
 
+def bench_sizes(args) -> dict:
+    """Seal and open of 2^20 packets of one common length, for each of a list
+    of lengths (--sizes, default the three IMIX sizes): how far short packets
+    are from the long ones.  Slots at the next multiple of 16 above length + 16."""
+    import torch
+    from bnk_amd import lib, workloads as W
+    n = 1 << 20
+    dev = torch.device("cuda:0")
+    ctx = lib.Context(0)
+    key = W.rand_bytes(W.stream_seed(2, 0), 32).reshape(1, 32)
+    ctx.keys_set(lib.KEYS_SEND, key)
+    ctx.keys_set(lib.KEYS_RECV, key)
+    stream = torch.cuda.ExternalStream(ctx.stream, device=dev)
+    per = {}
+    for length in [int(x) for x in args.sizes.split(",")]:
+        stride = (length + 16 + 15) // 16 * 16
+        plain = W.rand_bytes_torch(W.stream_seed(2, 50), n * stride, dev).clone()
+        sealed = torch.zeros_like(plain)
+        back = torch.zeros_like(plain)
+        v = torch.zeros(n, dtype=torch.uint8, device=dev)
+        torch.cuda.synchronize()
+        bi = lib.make_batch(plain, n * stride, n, lib.MEM_DEVICE, stride=stride, length=length)
+        bs = lib.make_batch(sealed, n * stride, n, lib.MEM_DEVICE, stride=stride)
+        bc = lib.make_batch(sealed, n * stride, n, lib.MEM_DEVICE, stride=stride, length=length + 16)
+        bb = lib.make_batch(back, n * stride, n, lib.MEM_DEVICE, stride=stride)
+        for _ in range(args.warmup):
+            ctx.seal(bi, bs)
+            ctx.open(bc, bb, v)
+        ctx.sync()
+        ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+        for k in range(args.steps):
+            ev[k][0].record(stream)
+            ctx.seal(bi, bs)
+            ev[k][1].record(stream)
+            ctx.open(bc, bb, v)
+            ev[k][2].record(stream)
+        ctx.sync()
+        torch.cuda.synchronize()
+        seal_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / args.steps
+        open_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / args.steps
+        assert bool(v.all()) and torch.equal(back.view(n, stride)[:, :length], plain.view(n, stride)[:, :length])
+        ops = n * ops_aead(length)
+        per[str(length)] = {
+            "seal_us": round(seal_ms * 1e3, 1), "open_us": round(open_ms * 1e3, 1),
+            "gbit_per_s_pair": round(n * length * 8 / ((seal_ms + open_ms) * 1e-3) / 1e9, 1),
+            "op_equivalent_ratio_to_peak": round(2 * ops / ((seal_ms + open_ms) * 1e-3) / 1e12 / VALU_PEAK_TOPS, 4),
+        }
+        del plain, sealed, back
+    ctx.close()
+    first = per[args.sizes.split(",")[0]]
+    return {"metric": "aead_seal_open_us_by_length", "value": first["seal_us"], "unit": "us per seal launch, first length",
+            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": False,
+            "dtype": "u32", "data": "synthetic",
+            "config": {"workload": "seal and open of %d packets of one common length, device resident, "
+                                   "HIP events around each launch" % n, "lengths": args.sizes},
+            "per_length": per}
+
+
 def bench_copy(args) -> dict:
     """Plain device-to-device copy of 1 GiB: the measured HBM ceiling and the
     known-size launch the FETCH_SIZE / WRITE_SIZE counters are scaled by."""
@@ -646,9 +704,10 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--packets", type=int, default=1 << 20)
-    ap.add_argument("--workload", default="aead", choices=["aead", "filter", "imix", "relay", "wg", "host", "latency", "copy"],
+    ap.add_argument("--workload", default="aead", choices=["aead", "filter", "imix", "relay", "wg", "host", "latency", "copy", "sizes"],
                     help="aead (default, the headline line, with the ACL filter rate as an extra); "
                          "filter / imix / relay / wg / host / latency / copy print one line for that workload alone")
+    ap.add_argument("--sizes", default="60,576,1420", help="sizes: packet lengths, comma separated")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true",
                     help="aead: leave out the packed-layout leg and the ACL filter extra, so that a "
@@ -670,7 +729,8 @@ def main() -> int:
         return 2
     if args.workload != "aead":
         out = {"filter": bench_filter, "imix": bench_imix, "relay": bench_relay,
-               "wg": bench_wg, "host": bench_host, "latency": bench_latency, "copy": bench_copy}[args.workload](args)
+               "wg": bench_wg, "host": bench_host, "latency": bench_latency, "copy": bench_copy,
+               "sizes": bench_sizes}[args.workload](args)
         print(json.dumps(out))
         return 0
     n = args.packets

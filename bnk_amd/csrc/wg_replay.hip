@@ -300,8 +300,21 @@ using SortConfig = rocprim::radix_sort_config<rocprim::default_config, rocprim::
 
 // ---- small batches: one block, everything in LDS ----------------------------
 
-constexpr uint32_t SMALL = WG_REPLAY_SMALL_MAX;
+// Segmented running maximum: the value restarts where the key changes.
+struct RunMax {
+    uint32_t k;
+    uint64_t v;
+};
+struct RunMaxOp {
+    __device__ RunMax operator()(const RunMax &a, const RunMax &b) const
+    {
+        return RunMax{b.k, (a.k == b.k && a.v > b.v) ? a.v : b.v};
+    }
+};
 
+// (SMALL threads: 256 for the batches wireguard-go itself hands over, 1024 up to
+// the limit of the one-block form)
+template <uint32_t SMALL>
 __global__ __launch_bounds__(SMALL) void replay_small_kernel(uint8_t *result, uint32_t *out_len,
                                                              const uint32_t *peer, const uint64_t *counter,
                                                              uint32_t n_peers, uint32_t n, uint64_t *state,
@@ -309,12 +322,15 @@ __global__ __launch_bounds__(SMALL) void replay_small_kernel(uint8_t *result, ui
 {
     using Sort = rocprim::block_radix_sort<uint32_t, SMALL, 1, uint32_t>;
     using Scan = rocprim::block_scan<uint32_t, SMALL>;
+    using ScanMax = rocprim::block_scan<RunMax, SMALL>;
     __shared__ union {
         typename Sort::storage_type sort;
         typename Scan::storage_type scan;
+        typename ScanMax::storage_type scan_max;
     } tmp;
     __shared__ uint32_t sk[SMALL + 1];
     __shared__ uint64_t sc[SMALL];
+    __shared__ uint64_t smax[SMALL];
     const uint32_t t = threadIdx.x;
     uint32_t key[1] = {NO_PEER}, pos[1] = {t};
     if (t < n) {
@@ -332,19 +348,21 @@ __global__ __launch_bounds__(SMALL) void replay_small_kernel(uint8_t *result, ui
     const bool head = t == 0 || sk[t - 1] != key[0];
     uint32_t start = 0;
     Scan().inclusive_scan(head ? t : 0u, start, tmp.scan, rocprim::maximum<uint32_t>());
+    __syncthreads();
+    // running maximum of the counters within each peer's run
+    RunMax mine{key[0], c < WG_REJECT_AFTER_MESSAGES ? c : 0}, upto;
+    ScanMax().inclusive_scan(mine, upto, tmp.scan_max, RunMaxOp());
+    smax[t] = upto.v;
+    __syncthreads();
     uint64_t *st = valid ? state + (size_t)key[0] * WG_REPLAY_WORDS : nullptr;
     const uint64_t last0 = valid ? st[0] : 0;
-    // the packets of my peer ahead of me: their running maximum, and whether
-    // one of them carried my counter
     uint64_t last = last0;
+    if (valid && !head && smax[t - 1] > last) last = smax[t - 1];
+    // only a packet at or below an earlier counter can repeat one: it looks
+    // through the packets of its peer ahead of it
     bool dup = false;
-    if (valid) {
-        for (uint32_t u = start; u < t; u++) {
-            const uint64_t cu = sc[u];
-            if (cu < WG_REJECT_AFTER_MESSAGES && cu > last) last = cu;
-            dup |= cu == c;
-        }
-    }
+    if (valid && c <= last)
+        for (uint32_t u = start; u < t; u++) dup |= sc[u] == c;
     const bool reached = valid && reaches_bit_test(c, last);
     bool fresh = reached && !dup;
     if (fresh && c <= last0 && seen_before(st, c)) fresh = false;
@@ -410,9 +428,14 @@ hipError_t launch_wg_replay(uint8_t *result, uint32_t *out_len, const uint32_t *
                             uint32_t n, const WgReplayDev &rp, const WgReplayScratch &sc, hipStream_t s)
 {
     if (n == 0) return hipSuccess;
-    if (n <= SMALL) {
-        hipLaunchKernelGGL(replay_small_kernel, dim3(1), dim3(SMALL), 0, s, result, out_len, peer, counter,
+    if (n <= 256u) {
+        hipLaunchKernelGGL(replay_small_kernel<256>, dim3(1), dim3(256), 0, s, result, out_len, peer, counter,
                            rp.n_peers, n, rp.state, key_bits(rp.n_peers));
+        return hipGetLastError();
+    }
+    if (n <= WG_REPLAY_SMALL_MAX) {
+        hipLaunchKernelGGL(replay_small_kernel<WG_REPLAY_SMALL_MAX>, dim3(1), dim3(WG_REPLAY_SMALL_MAX), 0, s,
+                           result, out_len, peer, counter, rp.n_peers, n, rp.state, key_bits(rp.n_peers));
         return hipGetLastError();
     }
     const dim3 grid((n + 255u) / 256u);

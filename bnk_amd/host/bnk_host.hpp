@@ -350,9 +350,11 @@ inline std::unique_ptr<tun::Device> WrapTUN(tun::Device *inner, PacketFilter *f)
 // so a counter is still acceptable while it trails the newest one by at most
 // (128 - 1) * 64 = 8128.  The reference gets this from
 // golang.zx2c4.com/wireguard/replay through device.NewDevice
-// (internal/dataplane/engine.go:51).  One filter per peer keypair; feed it
-// the (peer, counter) pairs bnk_wg_decap_batch reports for authentic packets,
-// in arrival order.
+// (internal/dataplane/engine.go:51).  bnk_wg_decap_batch keeps these windows
+// on the device by default; this sequential form is for a caller that has
+// switched them off there (bnk_wg_set_replay(ctx, 0)) and keeps them itself:
+// one filter per peer keypair, fed the (peer, counter) pairs the call reports
+// for authentic packets, in arrival order.
 class ReplayFilter {
 public:
     static constexpr uint64_t kBlocks = 128;

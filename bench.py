@@ -195,7 +195,7 @@ def bench_imix(args) -> dict:
     import torch
     from bnk_amd import lib, workloads as W
     n = 1 << 20
-    b = W.aead_imix(3, n, n_peers=256, payload=False)
+    b = W.aead_imix(3, n, n_peers=256, payload=False, align=args.slot_align)
     dev = torch.device("cuda:0")
     total = b.meta["total"]
     plain = W.imix_plain_torch(b, dev)
@@ -246,7 +246,8 @@ def bench_imix(args) -> dict:
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "u32", "data": "synthetic",
         "config": {"workload": "cfg3: seal+open of %d IMIX packets (60/576/1420 B 7:4:1), 256 peers, "
-                               "1%% forged tags on open, device resident" % n, "packets": n},
+                               "1%% forged tags on open, device resident, slots back to back at "
+                               "%d-byte alignment" % (n, args.slot_align), "packets": n},
         "mpkt_per_s_pair": round(n / (ms * 1e-3) / 1e6, 1),
         "rejected": int((vv == 0).sum()),
         "roofline_valu": {"achieved": round(2 * ops / (ms * 1e-3) / 1e12, 2), "peak": VALU_PEAK_TOPS,
@@ -262,7 +263,7 @@ def bench_relay(args) -> dict:
     import torch
     from bnk_amd import lib, workloads as W
     n = 1 << 22
-    w = W.relay_workload(n=n, payload=False)
+    w = W.relay_workload(n=n, payload=False, align=args.slot_align)
     b = w.batch
     dev = torch.device("cuda:0")
     total = b.meta["total"]
@@ -321,7 +322,8 @@ def bench_relay(args) -> dict:
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "u32", "data": "synthetic",
         "config": {"workload": "cfg5: open->filter->re-seal of %d IMIX packets, 4096 peers, 4096 rules, "
-                               "0.5%% forged, 5%% denied, device resident" % n, "packets": n},
+                               "0.5%% forged, 5%% denied, device resident, slots back to back at %d-byte "
+                               "alignment" % (n, args.slot_align), "packets": n},
         "gbit_per_s_plaintext": round(payload * 8 / (ms * 1e-3) / 1e9, 1),
         "verdicts": {"ok": int((v == 0).sum()), "forged": int((v == 1).sum()),
                      "denied": int((v == 2).sum())},
@@ -708,6 +710,10 @@ def main() -> int:
                     help="aead (default, the headline line, with the ACL filter rate as an extra); "
                          "filter / imix / relay / wg / host / latency / copy print one line for that workload alone")
     ap.add_argument("--sizes", default="60,576,1420", help="sizes: packet lengths, comma separated")
+    ap.add_argument("--slot-align", type=int, default=128, choices=[16, 32, 64, 128],
+                    help="imix, relay: packets lie back to back, each starting at a multiple of this "
+                         "(128: every packet in 128-byte lines of its own, as in a ring of buffers; "
+                         "16: packets share lines)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true",
                     help="aead: leave out the packed-layout leg and the ACL filter extra, so that a "

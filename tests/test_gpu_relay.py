@@ -96,7 +96,9 @@ def test_relay_full_size_device_resident_properties():
     from bnk_amd import lib
     from oracle import binding as O
     n = 1 << 22
-    w = W.relay_workload(n=n, payload=False)
+    # slots at 128-byte alignment, the layout bench.py times (the smaller cases above
+    # pack them at 16, where packets share lines)
+    w = W.relay_workload(n=n, payload=False, align=128)
     b = w.batch
     dev = torch.device("cuda:0")
     keys_in = np.ascontiguousarray(b.keys)

@@ -172,9 +172,11 @@ BNK_DEV void crypt_cell(Poly32 &mac, const uint32_t (&x)[16], int j, uint8_t *ce
 }
 
 // The final 1..15 bytes of a packet go straight from and to global memory.
+// `cell`: where the packet's cell of that number lives in the lane's LDS row;
+// the output is left there as well (zero-extended), for capture_head().
 template <bool OPEN>
 BNK_DEV void crypt_tail(Poly32 &mac, const uint32_t (&x)[16], int j, const uint8_t *s, uint8_t *d,
-                        uint32_t m)
+                        uint32_t m, uint8_t *cell)
 {
     const uint4 v = ld_partial(s, m);
     const uint4 o = keep_bytes(make_uint4(v.x ^ x[4 * j], v.y ^ x[4 * j + 1], v.z ^ x[4 * j + 2],
@@ -183,13 +185,14 @@ BNK_DEV void crypt_tail(Poly32 &mac, const uint32_t (&x)[16], int j, const uint8
     if (OPEN) mac.block(v.x, v.y, v.z, v.w);
     else mac.block(o.x, o.y, o.z, o.w);
     st_partial(d, o, m);
+    if (OPEN) *reinterpret_cast<uint4 *>(cell) = o;
 }
 
 // The same when the cell holding those bytes has come into LDS with the rest of
 // its line (bytes beyond the packet are whatever memory held: masked off) and
 // the destination is 16-byte aligned.
 template <bool OPEN>
-BNK_DEV void crypt_tail_lds(Poly32 &mac, const uint32_t (&x)[16], int j, const uint8_t *cell, uint8_t *d,
+BNK_DEV void crypt_tail_lds(Poly32 &mac, const uint32_t (&x)[16], int j, uint8_t *cell, uint8_t *d,
                             uint32_t m)
 {
     const uint4 raw = *reinterpret_cast<const uint4 *>(cell);
@@ -199,12 +202,30 @@ BNK_DEV void crypt_tail_lds(Poly32 &mac, const uint32_t (&x)[16], int j, const u
     if (OPEN) mac.block(v.x, v.y, v.z, v.w);
     else mac.block(o.x, o.y, o.z, o.w);
     st_partial(d, o, m);
+    if (OPEN) *reinterpret_cast<uint4 *>(cell) = o; // this cell never goes back to memory from here
+}
+
+// Open only: what a lane keeps of its plaintext's first bytes for the packet's
+// record in AeadArgs::heads, read from its LDS row once the first data block has
+// been through (cells c0 and c1 of the packet; bytes beyond a packet shorter
+// than that are whatever the row held).
+struct Head {
+    uint4 c0, c1;
+    bool on; // the launch writes records (the same for every lane)
+};
+
+BNK_DEV void capture_head(Head &h, const uint8_t *c0, const uint8_t *c1)
+{
+    if (h.on) {
+        h.c0 = *reinterpret_cast<const uint4 *>(c0);
+        h.c1 = *reinterpret_cast<const uint4 *>(c1);
+    }
 }
 
 template <bool OPEN>
 BNK_DEV void body_generic(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_t *dst,
                           uint32_t len, const uint8_t *safe, const uint32_t (&k)[8], uint32_t n1,
-                          uint32_t n2, Poly32 &mac, uint32_t (&x)[16])
+                          uint32_t n2, Poly32 &mac, uint32_t (&x)[16], Head &head)
 {
     const uint32_t nfull = len >> 6, rem = len & 63u;
     const uint32_t steps = nfull + (rem ? 1u : 0u);
@@ -253,9 +274,10 @@ BNK_DEV void body_generic(uint8_t *tile, uint32_t lane, const uint8_t *src, uint
                     if (rem >= 16u * (j + 1)) crypt_cell<OPEN>(mac, x, j, row + 16 * j);
                     else if (rem > 16u * j)
                         crypt_tail<OPEN>(mac, x, j, src + 64u * b + 16 * j, dst + 64u * b + 16 * j,
-                                         rem - 16u * j);
+                                         rem - 16u * j, row + 16 * j);
                 }
             }
+            if (OPEN && b == 0) capture_head(head, row, row + 16);
         }
         wave_sync();
         // LDS -> global
@@ -280,7 +302,7 @@ BNK_DEV void body_generic(uint8_t *tile, uint32_t lane, const uint8_t *src, uint
 template <bool OPEN, bool ALIGNED>
 BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_t *dst, uint32_t len,
                         const uint8_t *safe, const uint32_t (&k)[8], uint32_t n1, uint32_t n2,
-                        Poly32 &mac, uint32_t (&x)[16])
+                        Poly32 &mac, uint32_t (&x)[16], Head &head)
 {
     // Cells are 16 bytes; a packet's cell kc sits at stream position c0 + kc,
     // where the stream starts at the 128-byte line holding the packet's first
@@ -405,12 +427,14 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
                                     crypt_tail_lds<OPEN>(mac, x, j, row + (((c0 + kc) & 15u) << 4), dst + 16u * kc,
                                                          len & 15u);
                                 else
-                                    crypt_tail<OPEN>(mac, x, j, src + 16u * kc, dst + 16u * kc, len & 15u);
+                                    crypt_tail<OPEN>(mac, x, j, src + 16u * kc, dst + 16u * kc, len & 15u,
+                                                     row + (((c0 + kc) & 15u) << 4));
                             }
                         }
                     }
                 }
             }
+            if (OPEN && s == 0) capture_head(head, row + (c0 << 4), row + (((c0 + 1u) & 15u) << 4));
         }
         wave_sync();
         store_line(s);
@@ -439,7 +463,7 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
 template <bool OPEN>
 BNK_DEV void body_short(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_t *dst, uint32_t len,
                         const uint8_t *safe, const uint32_t (&k)[8], uint32_t n1, uint32_t n2,
-                        Poly32 &mac, uint32_t (&x)[16])
+                        Poly32 &mac, uint32_t (&x)[16], Head &head)
 {
     const uint32_t skew = (uint32_t)(uintptr_t)src & 127u;
     const uint32_t c0 = skew >> 4;
@@ -497,6 +521,7 @@ BNK_DEV void body_short(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
             }
         }
     }
+    if (OPEN) capture_head(head, row, row + 16);
     wave_sync();
 #pragma unroll
     for (int q = 0; q < 8; q++) {
@@ -518,7 +543,7 @@ BNK_DEV void body_short(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
 // MAC, and the zero-fill of rejected plaintexts.
 template <bool OPEN>
 BNK_DEV void lane_finish(const AeadArgs &a, uint32_t lane, bool have, uint32_t i, uint32_t len,
-                         const uint8_t *src, uint8_t *dst, Poly32 &mac)
+                         const uint8_t *src, uint8_t *dst, Poly32 &mac, const Head &head, uint8_t *record)
 {
     bool reject = false;
     if (have) {
@@ -536,6 +561,12 @@ BNK_DEV void lane_finish(const AeadArgs &a, uint32_t lane, bool have, uint32_t i
             reject = diff != 0;
             a.verdict[i] = reject ? 0 : 1;
         }
+    }
+    if (OPEN && head.on && record) {
+        // bytes 0-23 of the plaintext, its length, 1 if it is authentic: the lanes'
+        // records lie side by side
+        st16a(record, head.c0);
+        st16a(record + 16, make_uint4(head.c1.x, head.c1.y, len, have && !reject ? 1u : 0u));
     }
     if (OPEN) {
         unsigned long long rej = __ballot(reject);
@@ -625,11 +656,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const bool lane_lines = (((uintptr_t)src | (uintptr_t)dst) & 15u) == 0 &&
                             (((uintptr_t)src ^ (uintptr_t)dst) & 127u) == 0;
     const uint8_t *safe = reinterpret_cast<const uint8_t *>(a.keys);
-    if (__ballot(!lane_lines) != 0ull) body_lines<OPEN, false>(tile, lane, src, dst, len, safe, k, n1, n2, mac, x);
-    else if (__ballot(len > 64u * SHORT_BLOCKS) == 0ull) body_short<OPEN>(tile, lane, src, dst, len, safe, k, n1, n2, mac, x);
-    else body_lines<OPEN, true>(tile, lane, src, dst, len, safe, k, n1, n2, mac, x);
+    Head head;
+    head.on = OPEN && a.heads != nullptr;
+    head.c0 = head.c1 = make_uint4(0, 0, 0, 0);
+    if (__ballot(!lane_lines) != 0ull) body_lines<OPEN, false>(tile, lane, src, dst, len, safe, k, n1, n2, mac, x, head);
+    else if (__ballot(len > 64u * SHORT_BLOCKS) == 0ull) body_short<OPEN>(tile, lane, src, dst, len, safe, k, n1, n2, mac, x, head);
+    else body_lines<OPEN, true>(tile, lane, src, dst, len, safe, k, n1, n2, mac, x, head);
 
-    lane_finish<OPEN>(a, lane, have, i, len, src, dst, mac);
+    lane_finish<OPEN>(a, lane, have, i, len, src, dst, mac, head, in_batch && head.on ? a.heads + 32ull * t : nullptr);
 }
 
 // One wave = one packet, for batches too small to fill the chip with a packet
@@ -800,9 +834,11 @@ __global__ __launch_bounds__(256) void aead_spread_kernel(AeadArgs a)
     if (!WG && len > SPREAD_MAX_LEN) {
         const bool have = lane == 0;
         Poly32 mac;
+        Head no_head;
+        no_head.on = false;
         body_generic<OPEN>(tile_all[threadIdx.x >> 6], lane, have ? src : nullptr, have ? dst : nullptr,
-                           have ? len : 0u, reinterpret_cast<const uint8_t *>(a.keys), k, n1, n2, mac, x);
-        lane_finish<OPEN>(a, lane, have, i, len, have ? src : nullptr, have ? dst : nullptr, mac);
+                           have ? len : 0u, reinterpret_cast<const uint8_t *>(a.keys), k, n1, n2, mac, x, no_head);
+        lane_finish<OPEN>(a, lane, have, i, len, have ? src : nullptr, have ? dst : nullptr, mac, no_head, nullptr);
         return;
     }
 

@@ -385,7 +385,8 @@ void bnk_shutdown(bnk_ctx *ctx)
                           &ctx->wg_index, &ctx->wg_remote, &ctx->wg_allowed, &ctx->wg_send_ctr,
                           &ctx->wg_peer, &ctx->wg_counter, &ctx->wg_ctlen, &ctx->wg_result,
                           &ctx->wg_outlen, &ctx->wg_padded, &ctx->wg_wirelen, &ctx->wg_skip, &ctx->wg_sctr,
-                          &ctx->wg_sval, &ctx->wg_pmax, &ctx->wg_lastb, &ctx->wg_rtable, &ctx->wg_rflags})
+                          &ctx->wg_sval, &ctx->wg_pmax, &ctx->wg_lastb, &ctx->wg_rtable, &ctx->wg_rflags,
+                          &ctx->r_heads})
             b->release();
         ctx->pin.release();
         if (ctx->wg_replay) (void)hipFree(ctx->wg_replay);

@@ -111,6 +111,7 @@ struct bnk_ctx {
     uint32_t spread_max = bnk::SPREAD_MAX_PACKETS; // see AeadArgs::spread_max
     // fused relay: plaintext scratch, per-packet flags, sort buffers, staged arrays
     bnk::DevBuf r_plain, r_auth, r_pass, r_keys, r_idx, r_skeys, r_sidx, r_tmp;
+    bnk::DevBuf r_heads; // 32 bytes per packet: AeadArgs::heads of the relay's open
     bnk::DevBuf r_peer_out, r_ctr_base, r_ctr_out, r_verdict;
 
     // WireGuard framing: peer tables and per-packet scratch

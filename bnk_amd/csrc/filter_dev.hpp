@@ -66,6 +66,12 @@ struct FilterArgs {
     const uint64_t *off;  // or nullptr: i * stride
     const uint32_t *lens; // or nullptr: len
     const uint8_t *gate;  // or nullptr; gate[i] == 0 skips packet i (verdict 0)
+    const uint8_t *heads; // check only, or nullptr: the records AeadArgs::heads describes.  With
+                          // them the kernel goes through the records (record t is packet
+                          // order[t], or t), takes length and authenticity from them (lens
+                          // and gate are not read) and looks at the packet itself only for
+                          // an IP header with options
+    const uint32_t *order; // with heads, or nullptr
     uint8_t *verdict;     // check only
     uint32_t *status;
     int64_t now;

@@ -54,30 +54,30 @@ typedef u32x2 __attribute__((aligned(1))) u32x2_unaligned;
 // and, without IP options, the ports) in a second when the packet has them:
 // every load instruction here reads 64 different lines, so their number is
 // what the kernel pays for.
-BNK_DEV bool parse_packet(const uint8_t *p, uint32_t len, Parsed &o)
+// Where packet i lies in its arena, worked out only when somebody asks.
+struct PacketAt {
+    const uint8_t *pkts;
+    const uint64_t *off;
+    uint32_t stride, i;
+    BNK_DEV const uint8_t *get() const { return pkts + (off ? off[i] : (uint64_t)i * stride); }
+};
+
+// `p`: the packet's first 24 bytes (as many as it has); `full`: the packet
+// where it lies, looked at only for a header with options.
+BNK_DEV bool parse_words(const u32x4 a, uint32_t dst_w, uint32_t l4_w, bool wide, uint32_t len, Parsed &o,
+                         const PacketAt &full)
 {
-    if (len < 20u) return false;
-    const u32x4 a = *reinterpret_cast<const u32x4_unaligned *>(p);
     const uint32_t w0 = a.x;
     if (((w0 >> 4) & 0xFu) != 4u) return false;
     const uint32_t ihl = (w0 & 0xFu) * 4u;
     if (ihl < 20u || len < ihl) return false;
     o.proto = (a.z >> 8) & 0xFFu;
     o.src = __builtin_bswap32(a.w);
-    uint32_t dst_w, l4_w = 0;
-    const bool wide = len >= 24u;
-    if (wide) {
-        const u32x2 b = *reinterpret_cast<const u32x2_unaligned *>(p + 16);
-        dst_w = b.x;
-        l4_w = b.y;
-    } else {
-        dst_w = ld32u(p + 16);
-    }
     o.dst = __builtin_bswap32(dst_w);
     const uint32_t body = len - ihl;
     if (o.proto == 6u || o.proto == 17u) {
         if (body < 4u) return false;
-        const uint32_t w = __builtin_bswap32(wide && ihl == 20u ? l4_w : ld32u(p + ihl));
+        const uint32_t w = __builtin_bswap32(wide && ihl == 20u ? l4_w : ld32u(full.get() + ihl));
         o.sport = w >> 16;
         o.dport = w & 0xFFFFu;
         return true;
@@ -89,6 +89,22 @@ BNK_DEV bool parse_packet(const uint8_t *p, uint32_t len, Parsed &o)
         return true;
     }
     return false;
+}
+
+BNK_DEV bool parse_packet(const uint8_t *p, uint32_t len, Parsed &o, const PacketAt &full)
+{
+    if (len < 20u) return false;
+    const u32x4 a = *reinterpret_cast<const u32x4_unaligned *>(p);
+    uint32_t dst_w, l4_w = 0;
+    const bool wide = len >= 24u;
+    if (wide) {
+        const u32x2 b = *reinterpret_cast<const u32x2_unaligned *>(p + 16);
+        dst_w = b.x;
+        l4_w = b.y;
+    } else {
+        dst_w = ld32u(p + 16);
+    }
+    return parse_words(a, dst_w, l4_w, wide, len, o, full);
 }
 
 BNK_DEV uint32_t proto_class(uint32_t proto) { return proto == 1u ? 0u : proto == 6u ? 1u : 2u; }
@@ -277,17 +293,33 @@ __global__ __launch_bounds__(FILTER_THREADS, 8) void filter_check_kernel(FilterA
     const uint32_t lane = threadIdx.x & 63u;
     // whole waves stay in the loop together: the rule lookup is a joint effort
     for (uint32_t i0 = blockIdx.x * FILTER_THREADS + (threadIdx.x & ~63u); i0 < a.n; i0 += stride) {
-        const uint32_t i = i0 + lane;
-        bool valid = i < a.n && !(a.gate && a.gate[i] == 0);
+        // t: this lane's place in the sweep; i: the packet it answers for
+        const uint32_t t = i0 + lane;
+        uint32_t i = t;
+        bool valid;
         Parsed h{};
-        if (valid) {
-            const uint64_t at = a.off ? a.off[i] : (uint64_t)i * a.stride;
-            const uint32_t len = a.lens ? a.lens[i] : a.len;
-            if (beyond_arena(at, len, a.limit)) {
-                status_raise(a.status, STATUS_BOUNDS);
-                valid = false;
-            } else {
-                valid = parse_packet(a.pkts + at, len - (len >= a.trim ? a.trim : len), h);
+        if (a.heads) {
+            valid = t < a.n;
+            const uint32_t tt = valid ? t : 0u;
+            const u32x4 r0 = *reinterpret_cast<const u32x4 *>(a.heads + 32ull * tt);
+            const u32x4 r1 = *reinterpret_cast<const u32x4 *>(a.heads + 32ull * tt + 16);
+            if (a.order) i = a.order[tt];
+            // whoever wrote the records has checked the packets against the arena
+            const uint32_t plen = r1.z;
+            valid = valid && r1.w != 0u && plen >= 20u &&
+                    parse_words(r0, r1.x, r1.y, plen >= 24u, plen, h, PacketAt{a.pkts, a.off, a.stride, i});
+        } else {
+            valid = t < a.n && !(a.gate && a.gate[t] == 0);
+            if (valid) {
+                const uint32_t len = a.lens ? a.lens[t] : a.len;
+                const uint32_t plen = len - (len >= a.trim ? a.trim : len);
+                const uint64_t at = a.off ? a.off[t] : (uint64_t)t * a.stride;
+                if (beyond_arena(at, len, a.limit)) {
+                    status_raise(a.status, STATUS_BOUNDS);
+                    valid = false;
+                } else {
+                    valid = parse_packet(a.pkts + at, plen, h, PacketAt{a.pkts, a.off, a.stride, t});
+                }
             }
         }
         uint32_t key = 0, iv = 0;
@@ -350,7 +382,7 @@ __global__ __launch_bounds__(FILTER_THREADS, 8) void filter_check_kernel(FilterA
                 break;
             }
         }
-        if (i < a.n) a.verdict[i] = pass;
+        if (t < a.n) a.verdict[i] = pass;
     }
 }
 
@@ -368,7 +400,7 @@ __global__ __launch_bounds__(256) void filter_note_kernel(FilterArgs a)
         }
         const uint8_t *p = a.pkts + at;
         Parsed h;
-        if (!parse_packet(p, len, h)) continue;
+        if (!parse_packet(p, len, h, PacketAt{a.pkts, a.off, a.stride, i})) continue;
         // remote = dst, remotePort = dstPort, localPort = srcPort
         const FlowSlot s = flow_slot(a.flows, h.dst, h.dport, h.sport, h.proto);
         const unsigned long long expiry = (unsigned long long)(a.now + flow_ttl_ns(h.proto));

@@ -63,6 +63,10 @@ struct AeadArgs {
     const uint64_t *counters;  // or nullptr: counter0 + i
     const uint32_t *order;     // or nullptr: lane t handles packet t
     uint8_t *verdict;          // open only
+    uint8_t *heads;            // open by aead_wave_kernel only, or nullptr: one 32-byte record per
+                               // lane of the launch, in launch order (record t belongs to packet
+                               // first + order[t], or first + t without order[]): bytes 0-23 of the
+                               // plaintext, then its length and 1 if it is authentic (two words)
     const uint8_t *skip;       // or nullptr; skip[i] != 0 leaves packet i alone
     uint32_t *status;          // device status word, bit 0 = peer out of range
     uint64_t counter0;

@@ -216,6 +216,7 @@ extern "C" int bnk_relay_fused_batch(bnk_ctx *ctx, const bnk_batch *in, const ui
         d_ctr_out = ctr_out;
     }
     HIPCHK(ctx, ctx->r_plain.reserve(plain_bytes + 16));
+    HIPCHK(ctx, ctx->r_heads.reserve((size_t)n * 32));
     HIPCHK(ctx, ctx->r_auth.reserve(n));
     HIPCHK(ctx, ctx->r_pass.reserve(n));
     for (DevBuf *b : {&ctx->r_keys, &ctx->r_idx, &ctx->r_skeys, &ctx->r_sidx})
@@ -248,6 +249,10 @@ extern "C" int bnk_relay_fused_batch(bnk_ctx *ctx, const bnk_batch *in, const ui
                                            ctx->hist.as<uint32_t>(), ctx->cursor.as<uint32_t>(), ctx->stream));
             o.order = ctx->order.as<uint32_t>() + lo;
         }
+        // a lane-per-packet open leaves each plaintext's first 32 bytes in a record of
+        // its own for the filter, which then need not touch the arena again
+        const bool heads = f->enforce && !aead_runs_spread(o);
+        if (heads) o.heads = ctx->r_heads.as<uint8_t>() + 32ull * lo;
         HIPCHK(ctx, launch_aead_open(o, ctx->stream));
 
         // ---- 2. CheckInbound on the authentic plaintexts ----
@@ -262,6 +267,8 @@ extern "C" int bnk_relay_fused_batch(bnk_ctx *ctx, const bnk_batch *in, const ui
             fa.len = in->len;
             fa.trim = 16; // lens count the tag
             fa.gate = o.verdict + lo;
+            fa.heads = heads ? o.heads : nullptr;
+            fa.order = heads ? o.order : nullptr;
             fa.verdict = d_pass + lo;
             fa.status = ctx->d_status;
             fa.now = now_ns;

@@ -86,6 +86,70 @@ def test_relay_matches_oracle_host_path(mem, n):
     ctx.close()
 
 
+@pytest.mark.parametrize("n", [12000, 900])
+def test_relay_ip_options_and_ragged_headers(n):
+    """The filter inside the relay reads each plaintext's first bytes from a
+    compact record the open leaves behind (lane-per-packet launches), and goes
+    back to the packet itself only for an IP header with options.  Packets
+    with options (ports 4 to 40 bytes further in), packets cut short anywhere
+    inside their headers, and non-IP payloads: verdicts, counters and output
+    equal the oracle's."""
+    from bnk_amd import lib
+    from oracle import binding as O
+    w = W.relay_workload(n=n, n_peers=16, n_rules=128, forged_fraction=0.01)
+    b = w.batch
+    rng = np.random.default_rng(n)
+    plain = b.plain.copy()
+    lens = b.lens.copy()
+    off = b.off.astype(np.int64)
+    kind = rng.integers(0, 10, n)
+    for i in np.flatnonzero(kind == 0):                # options: ihl 6..15, ports moved
+        if lens[i] < 576:
+            continue
+        words = int(rng.integers(6, 16))
+        o = off[i]
+        l4 = plain[o + 20:o + 28].copy()
+        plain[o] = 0x40 | words
+        plain[o + 20:o + 4 * words] = rng.integers(0, 256, 4 * words - 20, dtype=np.uint8)
+        plain[o + 4 * words:o + 4 * words + 8] = l4
+    short = np.flatnonzero(kind == 1)                  # cut inside the headers (or to nothing)
+    lens[short] = rng.integers(0, 40, short.shape[0]).astype(lens.dtype)
+    for i in np.flatnonzero(kind == 2):                # not IPv4
+        plain[off[i]] = rng.integers(0, 256, dtype=np.uint8) | 0x20 if rng.integers(0, 2) else 0x60
+    keys_in = np.ascontiguousarray(b.keys)
+    keys_out = np.ascontiguousarray(w.keys_out)
+    sealed = np.zeros_like(plain)
+    O.seal_batch(keys_in, b.peer, b.counters, plain, b.off, lens, sealed, b.off, 4)
+    W.forge_tags(5, sealed, b.off, lens, w.forged_fraction)
+    ct_lens = (lens + 16).astype(np.uint32)
+    ora = O.Filter()
+    ora.set_rules(w.rules_ref)
+    ctx = lib.Context(0)
+    ctx.filter_set_rules(w.rules_ref)
+    ctx.keys_set(lib.KEYS_RECV, keys_in)
+    ctx.keys_set(lib.KEYS_SEND, keys_out)
+    _note(ctx, ora, w)
+    want_out = np.full_like(plain, 0x77)
+    want_v, want_c = ora.relay_fused_batch(keys_in, b.peer, b.counters, keys_out, w.peer_out,
+                                           w.ctr_base_out, sealed, b.off, ct_lens, want_out, b.off,
+                                           w.now_ns)
+    got_out = np.full_like(plain, 0x77)
+    got_v = np.full(b.n, 9, np.uint8)
+    got_c = np.full(b.n, 123, np.uint64)
+    ctx.relay_fused(
+        lib.make_batch(sealed, sealed.nbytes, b.n, lib.MEM_HOST, offsets=b.off, lens=ct_lens,
+                       peer=b.peer, counters=b.counters),
+        w.peer_out, w.ctr_base_out, len(w.ctr_base_out), w.now_ns,
+        lib.make_batch(got_out, got_out.nbytes, b.n, lib.MEM_HOST, offsets=b.off), got_v, got_c)
+    assert np.array_equal(got_v, want_v)
+    assert np.array_equal(got_c, want_c)
+    assert np.array_equal(got_out, want_out)
+    # the options case is really in there, on both sides of the verdict
+    opt = (kind == 0) & (lens >= 576)
+    assert (want_v[opt] == 0).any() and opt.sum() > n // 50
+    ctx.close()
+
+
 def test_relay_full_size_device_resident_properties():
     """Configuration 5 at full size (2^22 IMIX packets, 4096 peers, 4096
     rules): verdicts equal the construction, counters equal base + per-peer

@@ -171,38 +171,42 @@ BNK_DEV void crypt_cell(Poly32 &mac, const uint32_t (&x)[16], int j, uint8_t *ce
     *reinterpret_cast<uint4 *>(cell) = o;
 }
 
-// The final 1..15 bytes of a packet go straight from and to global memory.
-// `cell`: where the packet's cell of that number lives in the lane's LDS row;
-// the output is left there as well (zero-extended), for capture_head().
+// A cell at the end of a packet: m_in of its bytes are input (the rest count as
+// zeros: WireGuard's padding, which is not in memory) and m_out come out,
+// m_in <= m_out <= 16.  Without padding both are the packet's last 1..15 bytes.
+// This one goes straight from and to global memory; `cell` is where the
+// packet's cell of that number lives in the lane's LDS row, and the output is
+// left there as well (zero-extended), for capture_head().
 template <bool OPEN>
 BNK_DEV void crypt_tail(Poly32 &mac, const uint32_t (&x)[16], int j, const uint8_t *s, uint8_t *d,
-                        uint32_t m, uint8_t *cell)
+                        uint32_t m_in, uint32_t m_out, uint8_t *cell)
 {
-    const uint4 v = ld_partial(s, m);
+    const uint4 v = ld_partial(s, m_in);
     const uint4 o = keep_bytes(make_uint4(v.x ^ x[4 * j], v.y ^ x[4 * j + 1], v.z ^ x[4 * j + 2],
-                                          v.w ^ x[4 * j + 3]), m);
+                                          v.w ^ x[4 * j + 3]), m_out);
     // the MAC sees the ciphertext zero-padded to 16 bytes
     if (OPEN) mac.block(v.x, v.y, v.z, v.w);
     else mac.block(o.x, o.y, o.z, o.w);
-    st_partial(d, o, m);
+    st_partial(d, o, m_out);
     if (OPEN) *reinterpret_cast<uint4 *>(cell) = o;
 }
 
-// The same when the cell holding those bytes has come into LDS with the rest of
-// its line (bytes beyond the packet are whatever memory held: masked off) and
-// the destination is 16-byte aligned.
+// The same when the cell has come into LDS with the rest of its line (bytes
+// beyond the input are whatever memory held: masked off).  A whole cell of
+// output stays in LDS and leaves with its line; fewer bytes are written here,
+// to a 16-byte aligned destination.
 template <bool OPEN>
 BNK_DEV void crypt_tail_lds(Poly32 &mac, const uint32_t (&x)[16], int j, uint8_t *cell, uint8_t *d,
-                            uint32_t m)
+                            uint32_t m_in, uint32_t m_out)
 {
     const uint4 raw = *reinterpret_cast<const uint4 *>(cell);
-    const uint4 v = keep_bytes(raw, m);
+    const uint4 v = keep_bytes(raw, m_in);
     const uint4 o = keep_bytes(make_uint4(v.x ^ x[4 * j], v.y ^ x[4 * j + 1], v.z ^ x[4 * j + 2],
-                                          v.w ^ x[4 * j + 3]), m);
+                                          v.w ^ x[4 * j + 3]), m_out);
     if (OPEN) mac.block(v.x, v.y, v.z, v.w);
     else mac.block(o.x, o.y, o.z, o.w);
-    st_partial(d, o, m);
-    if (OPEN) *reinterpret_cast<uint4 *>(cell) = o; // this cell never goes back to memory from here
+    if (m_out < 16u) st_partial(d, o, m_out);
+    if (OPEN || m_out == 16u) *reinterpret_cast<uint4 *>(cell) = o;
 }
 
 // Open only: what a lane keeps of its plaintext's first bytes for the packet's
@@ -274,7 +278,7 @@ BNK_DEV void body_generic(uint8_t *tile, uint32_t lane, const uint8_t *src, uint
                     if (rem >= 16u * (j + 1)) crypt_cell<OPEN>(mac, x, j, row + 16 * j);
                     else if (rem > 16u * j)
                         crypt_tail<OPEN>(mac, x, j, src + 64u * b + 16 * j, dst + 64u * b + 16 * j,
-                                         rem - 16u * j, row + 16 * j);
+                                         rem - 16u * j, rem - 16u * j, row + 16 * j);
                 }
             }
             if (OPEN && b == 0) capture_head(head, row, row + 16);
@@ -301,9 +305,13 @@ BNK_DEV void body_generic(uint8_t *tile, uint32_t lane, const uint8_t *src, uint
 // packet, which then straddle two lines each.
 template <bool OPEN, bool ALIGNED>
 BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_t *dst, uint32_t len,
-                        const uint8_t *safe, const uint32_t (&k)[8], uint32_t n1, uint32_t n2,
+                        uint32_t len_in, const uint8_t *safe, const uint32_t (&k)[8], uint32_t n1, uint32_t n2,
                         Poly32 &mac, uint32_t (&x)[16], Head &head)
 {
+    // len_in <= len: the packet's bytes in memory; the up to 15 between the two
+    // are padding that counts as zeros (a sealing WireGuard launch; otherwise
+    // the two are equal)
+    const uint32_t ncell_in = len_in >> 4;
     // Cells are 16 bytes; a packet's cell kc sits at stream position c0 + kc,
     // where the stream starts at the 128-byte line holding the packet's first
     // byte.  Stream position K lives in line K / 8 and in ring cell K % 16.
@@ -403,7 +411,7 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
         if (s + 2 <= maxsteps) BNK_ISSUE_LINE(s + 2);
         wave_sync();
         if (s < steps) {
-            if (8u * s + 8u <= ncell) {
+            if (8u * s + 8u <= ncell_in) {
                 // all eight cells of this step are whole cells of the packet
 #pragma unroll 1
                 for (uint32_t h = 0; h < 2; h++) {
@@ -421,14 +429,16 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
 #pragma unroll
                         for (int j = 0; j < 4; j++) {
                             const uint32_t kc = 4u * b + j;
-                            if (kc < ncell) crypt_cell<OPEN>(mac, x, j, row + (((c0 + kc) & 15u) << 4));
-                            else if (kc == ncell && (len & 15u)) {
-                                if (ALIGNED)
-                                    crypt_tail_lds<OPEN>(mac, x, j, row + (((c0 + kc) & 15u) << 4), dst + 16u * kc,
-                                                         len & 15u);
+                            uint8_t *cell = row + (((c0 + kc) & 15u) << 4);
+                            if (kc < ncell_in) crypt_cell<OPEN>(mac, x, j, cell);
+                            else if (kc < ncell || (kc == ncell && (len & 15u))) {
+                                const uint32_t m_out = kc < ncell ? 16u : len & 15u;
+                                const uint32_t m_in = len_in > 16u * kc ? min(len_in - 16u * kc, m_out) : 0u;
+                                // (not aligned: only whole cells of the packet have come into LDS)
+                                if (ALIGNED || kc < ncell)
+                                    crypt_tail_lds<OPEN>(mac, x, j, cell, dst + 16u * kc, m_in, m_out);
                                 else
-                                    crypt_tail<OPEN>(mac, x, j, src + 16u * kc, dst + 16u * kc, len & 15u,
-                                                     row + (((c0 + kc) & 15u) << 4));
+                                    crypt_tail<OPEN>(mac, x, j, src + 16u * kc, dst + 16u * kc, m_in, m_out, cell);
                             }
                         }
                     }
@@ -462,9 +472,10 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
 // 128-byte line, only cells of the packet read into LDS or written back.
 template <bool OPEN>
 BNK_DEV void body_short(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_t *dst, uint32_t len,
-                        const uint8_t *safe, const uint32_t (&k)[8], uint32_t n1, uint32_t n2,
+                        uint32_t len_in, const uint8_t *safe, const uint32_t (&k)[8], uint32_t n1, uint32_t n2,
                         Poly32 &mac, uint32_t (&x)[16], Head &head)
 {
+    const uint32_t ncell_in = len_in >> 4; // see body_lines
     const uint32_t skew = (uint32_t)(uintptr_t)src & 127u;
     const uint32_t c0 = skew >> 4;
     const uint32_t ncell = len >> 4;           // whole cells, stored cooperatively
@@ -515,9 +526,12 @@ BNK_DEV void body_short(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 const uint32_t kc = 4u * b + j;
-                if (kc < ncell) crypt_cell<OPEN>(mac, x, j, row + (kc << 4));
-                else if (kc == ncell && (len & 15u))
-                    crypt_tail_lds<OPEN>(mac, x, j, row + (kc << 4), dst + 16u * kc, len & 15u);
+                if (kc < ncell_in) crypt_cell<OPEN>(mac, x, j, row + (kc << 4));
+                else if (kc < ncell || (kc == ncell && (len & 15u))) {
+                    const uint32_t m_out = kc < ncell ? 16u : len & 15u;
+                    const uint32_t m_in = len_in > 16u * kc ? min(len_in - 16u * kc, m_out) : 0u;
+                    crypt_tail_lds<OPEN>(mac, x, j, row + (kc << 4), dst + 16u * kc, m_in, m_out);
+                }
             }
         }
     }
@@ -622,6 +636,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const uint64_t ctr_ld = *(a.counters ? a.counters + i : safe64);
     uint32_t len = a.lens ? len_ld : a.len;
     if (!OPEN) len = len >= a.trim ? len - a.trim : 0u;
+    // Sealing with WireGuard's framing (a.wg.mode, with in_skip = out_skip = 16:
+    // a packet's offset is where its header goes): the bytes after the
+    // plaintext up to its padded length count as zeros without being in memory.
+    const bool encap = !OPEN && a.wg.mode == WG_FUSE_ENCAP;
+    const uint32_t len_plain = len;
+    if (encap) len += wg_padding(len, a.wg.mtu);
     const uint32_t pr = a.peer ? peer_ld : 0u;
     const bool skipped = a.skip != nullptr && skip_ld != 0;
     const bool bad_peer = pr >= a.n_peers;
@@ -631,7 +651,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // seal reads len and writes len + 16, open reads len (tag included) and writes len - 16
     const bool outside = beyond_arena(in_at, len, a.in_limit) ||
                          beyond_arena(out_at, OPEN ? (too_short ? 0u : len - 16u) : len + 16u, a.out_limit);
-    const bool have = in_batch && !skipped && !bad_peer && !too_short && !outside;
+    const uint64_t ctr = a.counters ? ctr_ld : a.counter0 + i;
+    // a keypair that has used up its nonces sends nothing more (wireguard-go device/send.go)
+    const bool spent = encap && ctr >= WG_REJECT_AFTER_MESSAGES;
+    const bool have = in_batch && !skipped && !bad_peer && !too_short && !outside && !spent;
     // the key table has at least one row
     const uint4 *kp = reinterpret_cast<const uint4 *>(a.keys + 8u * (bad_peer ? 0u : pr));
     const uint4 k0 = kp[0], k1 = kp[1];
@@ -642,12 +665,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
     if (OPEN) len -= 16u;
     len = have ? len : 0u;
+    const uint32_t len_in = encap ? min(len_plain, len) : len; // bytes of it in memory
     const uint8_t *src = a.in + in_at;
     uint8_t *dst = a.out + out_at;
+    if (encap && in_batch && !skipped) {
+        // the transport header: type 4, the receiver's index, the counter
+        if (have) st16(dst - 16, make_uint4(4u, a.wg.remote_index[pr], (uint32_t)ctr, (uint32_t)(ctr >> 32)));
+        a.wg.wire_len[i] = have ? 16u + len + 16u : 0u;
+    }
     src = have ? src : nullptr;
     dst = have ? dst : nullptr;
     const uint32_t k[8] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
-    const uint64_t ctr = a.counters ? ctr_ld : a.counter0 + i;
 
     const uint32_t n1 = (uint32_t)ctr, n2 = (uint32_t)(ctr >> 32);
     uint32_t x[16];
@@ -659,9 +687,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     Head head;
     head.on = OPEN && a.heads != nullptr;
     head.c0 = head.c1 = make_uint4(0, 0, 0, 0);
-    if (__ballot(!lane_lines) != 0ull) body_lines<OPEN, false>(tile, lane, src, dst, len, safe, k, n1, n2, mac, x, head);
-    else if (__ballot(len > 64u * SHORT_BLOCKS) == 0ull) body_short<OPEN>(tile, lane, src, dst, len, safe, k, n1, n2, mac, x, head);
-    else body_lines<OPEN, true>(tile, lane, src, dst, len, safe, k, n1, n2, mac, x, head);
+    if (__ballot(!lane_lines) != 0ull) body_lines<OPEN, false>(tile, lane, src, dst, len, len_in, safe, k, n1, n2, mac, x, head);
+    else if (__ballot(len > 64u * SHORT_BLOCKS) == 0ull) body_short<OPEN>(tile, lane, src, dst, len, len_in, safe, k, n1, n2, mac, x, head);
+    else body_lines<OPEN, true>(tile, lane, src, dst, len, len_in, safe, k, n1, n2, mac, x, head);
 
     lane_finish<OPEN>(a, lane, have, i, len, src, dst, mac, head, in_batch && head.on ? a.heads + 32ull * t : nullptr);
 }
@@ -958,8 +986,11 @@ hipError_t launch_aead_seal(const AeadArgs &a, hipStream_t s)
 {
     if (a.n == 0) return hipSuccess;
     const dim3 waves((a.n + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK);
+    // (the two framing launches differ in what a packet's offset means: see AeadArgs::wg)
     if (a.wg.mode != WG_FUSE_OFF) {
-        if (a.wg.mode != WG_FUSE_ENCAP || !aead_runs_spread(a)) return hipErrorInvalidValue;
+        if (a.wg.mode != WG_FUSE_ENCAP) return hipErrorInvalidValue;
+        if (!aead_runs_spread(a)) return a.in_skip == 16u && a.out_skip == 16u ? launch_wave<false>(a, s) : hipErrorInvalidValue;
+        if (a.in_skip != 0u) return hipErrorInvalidValue;
         hipLaunchKernelGGL((aead_spread_kernel<false, true>), waves, dim3(256), 0, s, a);
     } else if (aead_runs_spread(a))
         hipLaunchKernelGGL((aead_spread_kernel<false, false>), waves, dim3(256), 0, s, a);

@@ -122,6 +122,7 @@ struct bnk_ctx {
     uint64_t *wg_replay = nullptr;
     uint32_t wg_replay_rows = 0;
     bool wg_replay_on = true;
+    bool wg_unfused = false; // framing of lane-per-packet launches in kernels of its own
     bnk::DevBuf wg_sctr, wg_sval, wg_pmax, wg_lastb, wg_rtable, wg_rflags;
     bnk::DevBuf wg_peer, wg_counter, wg_ctlen, wg_result, wg_outlen, wg_padded, wg_wirelen, wg_skip;
 

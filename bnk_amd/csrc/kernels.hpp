@@ -30,11 +30,12 @@ __host__ __device__ inline uint64_t ctr_add(uint64_t base, uint64_t rank, uint64
     return (c < base || c > limit) ? limit : c;
 }
 
-// WireGuard transport framing done by a wave-per-packet AEAD launch itself
-// (small batches only; larger ones run the framing kernels of wg_kernels.hip
-// around the launch).  in/out offsets then address the slot or datagram, not
-// the AEAD data inside it, and every packet must be at most WG_FUSE_MAX_LEN
-// bytes long, padding included.
+// WireGuard transport framing done by the AEAD launch itself.  A wave-per-packet
+// launch (small batches): in/out offsets address the slot or datagram
+// (in_skip = out_skip = 0) and every packet must be at most WG_FUSE_MAX_LEN
+// bytes long, padding included.  A lane-per-packet launch: in_skip and
+// out_skip say where the AEAD data starts within the slot or datagram (16 past
+// the header), any length.
 struct WgFuse {
     uint32_t mode;               // WG_FUSE_*
     uint32_t n_peers;            // rows of the peer tables

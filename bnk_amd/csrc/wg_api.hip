@@ -182,6 +182,16 @@ extern "C" int bnk_wg_set_replay(bnk_ctx *ctx, int on)
     BNK_API_CATCH(ctx)
 }
 
+extern "C" int bnk_wg_set_fused(bnk_ctx *ctx, int on)
+{
+    BNK_API_TRY
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    ctx->wg_unfused = on == 0;
+    return BNK_OK;
+    BNK_API_CATCH(ctx)
+}
+
 extern "C" int bnk_wg_send_counters(bnk_ctx *ctx, uint64_t *out, uint32_t n)
 {
     BNK_API_TRY
@@ -423,8 +433,6 @@ static int wg_encap_impl(bnk_ctx *ctx, const bnk_batch *slots, uint32_t mtu, uin
                 return BNK_OK;
             }
         }
-        HIPCHK(ctx, launch_wg_encap_prep(c, sealed, pe, d_peer, d_ctr, mtu, d_padded, d_wire_len, d_skip, ctx->d_status,
-                                         ctx->stream));
         AeadArgs se{};
         se.spread_max = ctx->spread_max;
         se.keys = ctx->d_keys[BNK_KEYS_SEND];
@@ -440,9 +448,28 @@ static int wg_encap_impl(bnk_ctx *ctx, const bnk_batch *slots, uint32_t mtu, uin
         se.lens = d_padded;
         se.peer = d_peer;
         se.counters = d_ctr;
-        se.skip = d_skip;
-        if (slots->lens && se.n > 64 && !aead_runs_spread(se)) { // equal plaintext lengths pad to equal lengths
-            HIPCHK(ctx, launch_length_sort(d_padded + lo, se.n, 0, ctx->order.as<uint32_t>() + lo,
+        if (!ctx->wg_unfused && !aead_runs_spread(se)) {
+            // a lane per packet: header, padding (as implied zeros) and lengths are
+            // the launch's own work too
+            se.lens = b.lens;
+            se.len = slots->len;
+            // the slot from its first byte to the end of the tag, as the separate kernel checks it
+            se.in_limit = se.out_limit = b.limit;
+            se.wg.mode = WG_FUSE_ENCAP;
+            se.wg.n_peers = pe.n;
+            se.wg.mtu = mtu;
+            se.wg.remote_index = pe.remote_index;
+            se.wg.wire_len = d_wire_len;
+        } else {
+            // the framing in a kernel of its own, then a plain seal of the padded packets
+            se.skip = d_skip;
+            HIPCHK(ctx, launch_wg_encap_prep(c, sealed, pe, d_peer, d_ctr, mtu, d_padded, d_wire_len, d_skip,
+                                             ctx->d_status, ctx->stream));
+        }
+        // (padding never changes a packet's number of 64-byte blocks, so the plaintext
+        // lengths group the packets as the padded ones would)
+        if (slots->lens && se.n > 64 && !aead_runs_spread(se)) {
+            HIPCHK(ctx, launch_length_sort(se.lens + lo, se.n, 0, ctx->order.as<uint32_t>() + lo,
                                            ctx->hist.as<uint32_t>(), ctx->cursor.as<uint32_t>(), ctx->stream));
             se.order = ctx->order.as<uint32_t>() + lo;
         }

@@ -350,6 +350,10 @@ class Context:
         """Anti-replay windows on (default) or off for the decapsulating calls."""
         self._chk(self._lib.bnk_wg_set_replay(self._h, C.c_int(1 if on else 0)))
 
+    def wg_set_fused(self, on: bool) -> None:
+        """Framing of large batches inside the AEAD launch (default) or in kernels of its own."""
+        self._chk(self._lib.bnk_wg_set_fused(self._h, C.c_int(1 if on else 0)))
+
     def wg_send_counters(self, n: int) -> np.ndarray:
         out = np.zeros(max(n, 1), np.uint64)
         self._chk(self._lib.bnk_wg_send_counters(self._h, C.c_void_p(out.ctypes.data),

@@ -66,10 +66,21 @@ def _ctx(peers, keys_send=None, keys_recv=None):
     return ctx
 
 
+def _launch_shape(ctx, fused):
+    """"wave": small batches take a wave per packet with the framing inside the
+    AEAD launch (the default); "lane": every batch takes a lane per packet,
+    framing inside as well; "separate": a lane per packet between framing
+    kernels of their own."""
+    if fused != "wave":
+        ctx.set_spread_max_packets(0)
+    if fused == "separate":
+        ctx.wg_set_fused(False)
+
+
 @pytest.mark.parametrize("mem", ["host", "ring", "device"])
 @pytest.mark.parametrize("misalign", [False, True])
 @pytest.mark.parametrize("n", [3000, 700])
-@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("fused", ["wave", "lane", "separate"])
 def test_encap_matches_oracle(mem, misalign, n, fused):
     """"ring": the slots lie in a pinned ring of the context, which small
     batches seal in place without staging copies.  700 packets also take the
@@ -96,8 +107,7 @@ def test_encap_matches_oracle(mem, misalign, n, fused):
         plains.append(pt)
         arena[int(off[i]) + 16:int(off[i]) + 16 + len(pt)] = np.frombuffer(pt, np.uint8)
     ctx = _ctx(peers, keys_send=keys)
-    if not fused:
-        ctx.set_spread_max_packets(0)
+    _launch_shape(ctx, fused)
     next_ctr = np.zeros(N_PEERS, np.uint64)
     for round_ in range(2):  # the second batch continues the peers' counters
         want = arena.copy()
@@ -142,7 +152,7 @@ def test_encap_matches_oracle(mem, misalign, n, fused):
     ctx.close()
 
 
-@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("fused", ["wave", "lane", "separate"])
 @pytest.mark.parametrize("length,mtu", [(100, 1420), (1500, 1420), (1413, 1420), (37, 0), (0, 1420), (2839, 1420)])
 def test_encap_uniform_slots_one_peer_and_padding_rules(fused, length, mtu):
     """Uniform slots without length or peer arrays (everything goes to peer 0),
@@ -166,8 +176,7 @@ def test_encap_uniform_slots_one_peer_and_padding_rules(fused, length, mtu):
         want_len[i] = len(w)
     assert want_len[0] == 32 + length + O.wg_padding(length, mtu)
     ctx = _ctx(peers, keys_send=keys)
-    if not fused:
-        ctx.set_spread_max_packets(0)
+    _launch_shape(ctx, fused)
     for mem in ("pageable", "ring"):
         ring = ctx.ring_alloc(arena.nbytes) if mem == "ring" else None
         got = ring if ring is not None else arena.copy()
@@ -183,7 +192,7 @@ def test_encap_uniform_slots_one_peer_and_padding_rules(fused, length, mtu):
     ctx.close()
 
 
-@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("fused", ["wave", "lane", "separate"])
 @pytest.mark.parametrize("inner", [0, 28, 1000, 1420])
 def test_decap_uniform_datagrams(fused, inner):
     """Datagrams of one size at a uniform stride, no length array: keepalives
@@ -208,8 +217,7 @@ def test_decap_uniform_datagrams(fused, inner):
     want = np.array([(lambda r: (r[0], len(r[1]), r[2], r[3]))(O.wg_decap(w, peers, keys)) for w in wires], np.uint64)
     assert (want[:, 0] == (O.WG_OK if inner else O.WG_KEEPALIVE)).all()
     ctx = _ctx(peers, keys_recv=keys)
-    if not fused:
-        ctx.set_spread_max_packets(0)
+    _launch_shape(ctx, fused)
     for mem in ("pageable", "ring"):
         rings = [ctx.ring_alloc(arena.nbytes), ctx.ring_alloc(arena.nbytes)] if mem == "ring" else []
         src = rings[0] if rings else arena.copy()
@@ -329,7 +337,7 @@ def _decap_cases(rng, peers, keys, n):
 
 @pytest.mark.parametrize("mem", ["host", "ring", "device"])
 @pytest.mark.parametrize("aligned", [True, False])
-@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("fused", ["wave", "lane", "separate"])
 def test_decap_matches_oracle(mem, aligned, fused):
     import torch
     from bnk_amd import lib
@@ -364,8 +372,7 @@ def test_decap_matches_oracle(mem, aligned, fused):
             want_out[int(out_off[i]):int(out_off[i]) + plen] = np.frombuffer(body, np.uint8)
     assert len(set(want[:, 0].tolist())) == 7  # every result class occurs
     ctx = _ctx(peers, keys_recv=keys)
-    if not fused:
-        ctx.set_spread_max_packets(0)
+    _launch_shape(ctx, fused)
     if mem == "host":
         got_out = np.full(total + 16, 0x77, np.uint8)
         res = np.full(n, 99, np.uint8)
@@ -419,7 +426,7 @@ def test_decap_matches_oracle(mem, aligned, fused):
 
 
 @pytest.mark.parametrize("n_peers", [65, 4097, 70000])
-@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("fused", ["wave", "lane", "separate"])
 def test_receiver_index_lookup_in_large_peer_tables(n_peers, fused):
     """The sender is found by its receiver index in a sorted table: searched 64
     entries at a time by the lanes of a wave (small batches), or by binary
@@ -457,8 +464,7 @@ def test_receiver_index_lookup_in_large_peer_tables(n_peers, fused):
                     np.uint64)
     assert (want[:, 0] == O.WG_UNKNOWN_INDEX).sum() >= n // 5 - 1 and (want[:, 0] == 0).sum() >= n // 2
     ctx = _ctx(peers, keys_recv=keys)
-    if not fused:
-        ctx.set_spread_max_packets(0)
+    _launch_shape(ctx, fused)
     out = np.zeros(n * 128, np.uint8)
     res, olen = np.full(n, 99, np.uint8), np.full(n, 99, np.uint32)
     gp, gc = np.full(n, 99, np.uint32), np.full(n, 99, np.uint64)
@@ -483,7 +489,7 @@ def _filter_setup(rng, peers):
 
 
 @pytest.mark.parametrize("mem", ["host", "ring", "device"])
-@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("fused", ["wave", "lane", "separate"])
 def test_decap_with_the_inbound_filter_in_one_call(mem, fused):
     """bnk_wg_decap_filter_batch = decapsulate, then CheckInbound with one `now`
     on what was delivered: results (FILTERED for the denied), plaintexts,
@@ -546,8 +552,7 @@ def test_decap_with_the_inbound_filter_in_one_call(mem, fused):
 
     def fresh_ctx():
         ctx = _ctx(peers, keys_recv=keys)
-        if not fused:
-            ctx.set_spread_max_packets(0)
+        _launch_shape(ctx, fused)
         ctx.filter_set_rules(rules)
         for pkt in noted:
             ctx.filter_note_outbound_ptrs([pkt], t0 - 10**9)
@@ -1005,7 +1010,7 @@ def _encap_host(ctx, arena, off, lens, peer, mtu=MTU):
     return got, wl
 
 
-@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("fused", ["wave", "lane", "separate"])
 @pytest.mark.parametrize("n", [400, 3000])
 def test_rekey_of_one_peer_leaves_the_other_counters_alone(fused, n):
     """WireGuard peers rekey independently: installing peer A's new keypair
@@ -1026,8 +1031,7 @@ def test_rekey_of_one_peer_leaves_the_other_counters_alone(fused, n):
         plains.append(pt)
         arena[int(off[i]) + 16:int(off[i]) + 16 + len(pt)] = np.frombuffer(pt, np.uint8)
     ctx = _ctx(peers, keys_send=keys, keys_recv=keys)
-    if not fused:
-        ctx.set_spread_max_packets(0)
+    _launch_shape(ctx, fused)
     next_ctr = np.zeros(N_PEERS, np.uint64)
 
     def check_batch():
@@ -1077,7 +1081,7 @@ def test_rekey_of_one_peer_leaves_the_other_counters_alone(fused, n):
     ctx.close()
 
 
-@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("fused", ["wave", "lane", "separate"])
 @pytest.mark.parametrize("n", [64, 2500])
 def test_keypair_stops_sending_at_reject_after_messages(fused, n):
     """wireguard-go sends nothing under a keypair whose nonce counter has
@@ -1098,8 +1102,7 @@ def test_keypair_stops_sending_at_reject_after_messages(fused, n):
         plains.append(pt)
         arena[int(off[i]) + 16:int(off[i]) + 116] = np.frombuffer(pt, np.uint8)
     ctx = _ctx(peers, keys_send=keys)
-    if not fused:
-        ctx.set_spread_max_packets(0)
+    _launch_shape(ctx, fused)
     limit = lib.WG_REJECT_AFTER_MESSAGES
     ctx.wg_send_counter_set(0, limit - 3)
     ctx.wg_send_counter_set(1, (1 << 40) + 7)

@@ -383,19 +383,35 @@ def bench_wg(args) -> dict:
         ctx.wg_decap(lib.make_batch(cur, nbytes, n, lib.MEM_DEVICE, stride=stride, length=wire_len),
                      lib.make_batch(nxt[16:], nbytes, n, lib.MEM_DEVICE, stride=stride), d_res, d_olen, d_gp, d_gc)
 
-    for k in range(args.warmup):
-        step(k)
-    ctx.sync()
-    t0 = time.perf_counter()
-    for k in range(args.warmup, args.warmup + args.steps):
-        step(k)
-    ctx.sync()
-    ms = (time.perf_counter() - t0) * 1e3 / args.steps
-    last = arenas[(args.warmup + args.steps) & 1][:n * stride].view(n, stride)[:, 16:16 + plen]
+    done = 0
+
+    def timed(steps):
+        nonlocal done
+        ctx.sync()
+        t0 = time.perf_counter()
+        for k in range(done, done + steps):
+            step(k)
+        ctx.sync()
+        done += steps
+        return (time.perf_counter() - t0) * 1e3 / steps
+
+    timed(args.warmup)
+    ms = timed(args.steps)
+    # the same steps with the framing in kernels of its own, and without the windows
+    ctx.wg_set_fused(False)
+    timed(1)
+    ms_separate = timed(args.steps)
+    ctx.wg_set_fused(True)
+    timed(1)
+    ms_again = timed(args.steps)  # clocks drift over a run: the first figure once more
+    ctx.wg_set_replay(False)
+    timed(1)
+    ms_no_windows = timed(args.steps)
+    last = arenas[done & 1][:n * stride].view(n, stride)[:, 16:16 + plen]
     assert bool((d_res == 0).all()) and bool((d_olen == plen).all()) and bool((d_gp == d_peer).all())
     assert bool((d_wl == wire_len).all()) and torch.equal(last, first_plain), "the packets did not survive the trips"
     want_ctr = W.per_peer_sequence(peer, n_peers) + np.bincount(peer, minlength=n_peers)[peer].astype(np.uint64) * \
-        np.uint64(args.warmup + args.steps - 1)
+        np.uint64(done - 1)
     assert np.array_equal(d_gc.cpu().numpy().astype(np.uint64), want_ctr), "counters do not follow the send order"
     ops = n * ops_aead(plen)
     ctx.close()
@@ -409,6 +425,9 @@ def bench_wg(args) -> dict:
                                "resident; every step sends what the step before received"
                                % (n, plen, wire_len, stride, n_peers), "packets": n},
         "mpkt_per_s_pair": round(n / (ms * 1e-3) / 1e6, 1),
+        "same_run_ms_per_step": {"framing_in_kernels_of_its_own": round(ms_separate, 4),
+                                 "as_value_measured_again": round(ms_again, 4),
+                                 "anti_replay_windows_off": round(ms_no_windows, 4)},
         "roofline_valu": {"achieved": round(2 * ops / (ms * 1e-3) / 1e12, 2), "peak": VALU_PEAK_TOPS,
                           "unit": "Top/s (int32 op-equivalents)",
                           "frac": round(2 * ops / (ms * 1e-3) / 1e12 / VALU_PEAK_TOPS, 4)},

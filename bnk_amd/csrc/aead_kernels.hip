@@ -557,7 +557,8 @@ BNK_DEV void body_short(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
 // MAC, and the zero-fill of rejected plaintexts.
 template <bool OPEN>
 BNK_DEV void lane_finish(const AeadArgs &a, uint32_t lane, bool have, uint32_t i, uint32_t len,
-                         const uint8_t *src, uint8_t *dst, Poly32 &mac, const Head &head, uint8_t *record)
+                         const uint8_t *src, uint8_t *dst, Poly32 &mac, const Head &head, uint8_t *record,
+                         bool decap = false, uint32_t pr = 0)
 {
     bool reject = false;
     if (have) {
@@ -573,10 +574,33 @@ BNK_DEV void lane_finish(const AeadArgs &a, uint32_t lane, bool have, uint32_t i
             const uint32_t diff = (tg.x ^ tag[0]) | (tg.y ^ tag[1]) | (tg.z ^ tag[2]) |
                                   (tg.w ^ tag[3]);
             reject = diff != 0;
-            a.verdict[i] = reject ? 0 : 1;
+            if (a.verdict) a.verdict[i] = reject ? 0 : 1;
         }
     }
-    if (OPEN && head.on && record) {
+    if (OPEN && decap) {
+        // what WireGuard does with an opened datagram: keepalive, IP version, the
+        // trim to the IP header's total length, the sender's allowed prefix (the
+        // header's first 16 bytes were kept when they went through the cipher)
+        uint32_t res = BNK_WG_OK, out_len = 0;
+        const uint32_t version = (head.c0.x >> 4) & 0xFu;
+        if (!have || reject) res = BNK_WG_AUTH_FAIL; // (no packet here: it reached beyond the output arena)
+        else if (len == 0u) res = BNK_WG_KEEPALIVE;
+        else if (len < 16u) res = BNK_WG_BAD_IP; // too short for either header
+        else if (version == 4u) {
+            const uint32_t total = __builtin_bswap32(head.c0.x) & 0xFFFFu;
+            const uint2 al = a.wg.allowed[pr];
+            if (len < 20u || total > len || total < 20u) res = BNK_WG_BAD_IP;
+            else if ((__builtin_bswap32(head.c0.w) & al.y) != (al.x & al.y)) res = BNK_WG_NOT_ALLOWED;
+            else out_len = total;
+        } else if (version == 6u) {
+            // peers own IPv4 addresses only
+            const uint32_t total = (__builtin_bswap32(head.c0.y) >> 16) + 40u;
+            res = (len < 40u || total > len) ? BNK_WG_BAD_IP : BNK_WG_NOT_ALLOWED;
+        } else res = BNK_WG_BAD_IP;
+        a.wg.result[i] = (uint8_t)res;
+        a.wg.out_len[i] = out_len;
+    }
+    if (OPEN && record) {
         // bytes 0-23 of the plaintext, its length, 1 if it is authentic: the lanes'
         // records lie side by side
         st16a(record, head.c0);
@@ -636,14 +660,56 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const uint64_t ctr_ld = *(a.counters ? a.counters + i : safe64);
     uint32_t len = a.lens ? len_ld : a.len;
     if (!OPEN) len = len >= a.trim ? len - a.trim : 0u;
+    // Opening with WireGuard's framing (a.wg.mode, in_skip = 16: a packet's
+    // offset and length are its datagram's): the header names the sender and
+    // the counter.  A datagram that fails here is reported and not opened.
+    const bool decap = OPEN && a.wg.mode == WG_FUSE_DECAP;
+    uint32_t wg_peer = 0;
+    uint64_t wg_ctr = 0;
+    uint32_t wg_res = BNK_WG_OK;
+    if (decap) {
+        const uint64_t at = a.in_off ? in_off_ld : (uint64_t)i * a.in_stride;
+        const bool beyond = beyond_arena(at, len, a.in_limit);
+        if (in_batch && beyond) status_raise(a.status, STATUS_BOUNDS);
+        if (beyond || len < 32u) wg_res = BNK_WG_BAD_HEADER;
+        const uint4 h = ld16(wg_res == BNK_WG_OK && in_batch ? a.in + at : reinterpret_cast<const uint8_t *>(a.keys));
+        if (wg_res == BNK_WG_OK && h.x != 4u) wg_res = BNK_WG_BAD_HEADER;
+        if (wg_res == BNK_WG_OK) {
+            const uint32_t mask = (1u << a.wg.hash_bits) - 1u;
+            uint32_t slot = wg_hash_slot(h.y, a.wg.hash_bits);
+            wg_res = BNK_WG_UNKNOWN_INDEX;
+            // the table is never full: an empty slot ends the walk
+            for (uint32_t probe = 0; probe <= mask; probe++) {
+                const uint2 e = a.wg.index_hash[slot];
+                if (e.y == WG_HASH_EMPTY) break;
+                if (e.x == h.y) {
+                    wg_peer = e.y;
+                    wg_res = BNK_WG_OK;
+                    break;
+                }
+                slot = (slot + 1u) & mask;
+            }
+        }
+        wg_ctr = (uint64_t)h.z | (uint64_t)h.w << 32;
+        if (in_batch) {
+            const bool ok = wg_res == BNK_WG_OK;
+            a.wg.peer_out[i] = ok ? wg_peer : 0xFFFFFFFFu;
+            a.wg.counter_out[i] = ok ? wg_ctr : 0ull;
+            if (!ok) {
+                a.wg.result[i] = (uint8_t)wg_res;
+                a.wg.out_len[i] = 0;
+            }
+        }
+        len = len >= 16u ? len - 16u : 0u; // what goes through the cipher, tag included
+    }
     // Sealing with WireGuard's framing (a.wg.mode, with in_skip = out_skip = 16:
     // a packet's offset is where its header goes): the bytes after the
     // plaintext up to its padded length count as zeros without being in memory.
     const bool encap = !OPEN && a.wg.mode == WG_FUSE_ENCAP;
     const uint32_t len_plain = len;
     if (encap) len += wg_padding(len, a.wg.mtu);
-    const uint32_t pr = a.peer ? peer_ld : 0u;
-    const bool skipped = a.skip != nullptr && skip_ld != 0;
+    const uint32_t pr = decap ? wg_peer : a.peer ? peer_ld : 0u;
+    const bool skipped = (a.skip != nullptr && skip_ld != 0) || wg_res != BNK_WG_OK;
     const bool bad_peer = pr >= a.n_peers;
     const bool too_short = OPEN && len < 16u;
     const uint64_t in_at = (a.in_off ? in_off_ld : (uint64_t)i * a.in_stride) + a.in_skip;
@@ -651,7 +717,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // seal reads len and writes len + 16, open reads len (tag included) and writes len - 16
     const bool outside = beyond_arena(in_at, len, a.in_limit) ||
                          beyond_arena(out_at, OPEN ? (too_short ? 0u : len - 16u) : len + 16u, a.out_limit);
-    const uint64_t ctr = a.counters ? ctr_ld : a.counter0 + i;
+    const uint64_t ctr = decap ? wg_ctr : a.counters ? ctr_ld : a.counter0 + i;
     // a keypair that has used up its nonces sends nothing more (wireguard-go device/send.go)
     const bool spent = encap && ctr >= WG_REJECT_AFTER_MESSAGES;
     const bool have = in_batch && !skipped && !bad_peer && !too_short && !outside && !spent;
@@ -661,7 +727,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     if (in_batch && !skipped && (bad_peer || too_short || outside)) {
         if (bad_peer) status_raise(a.status, STATUS_PEER_RANGE);
         else if (outside) status_raise(a.status, STATUS_BOUNDS);
-        if (OPEN) a.verdict[i] = 0;
+        if (OPEN && a.verdict) a.verdict[i] = 0;
     }
     if (OPEN) len -= 16u;
     len = have ? len : 0u;
@@ -685,13 +751,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                             (((uintptr_t)src ^ (uintptr_t)dst) & 127u) == 0;
     const uint8_t *safe = reinterpret_cast<const uint8_t *>(a.keys);
     Head head;
-    head.on = OPEN && a.heads != nullptr;
+    head.on = OPEN && (a.heads != nullptr || decap);
     head.c0 = head.c1 = make_uint4(0, 0, 0, 0);
     if (__ballot(!lane_lines) != 0ull) body_lines<OPEN, false>(tile, lane, src, dst, len, len_in, safe, k, n1, n2, mac, x, head);
     else if (__ballot(len > 64u * SHORT_BLOCKS) == 0ull) body_short<OPEN>(tile, lane, src, dst, len, len_in, safe, k, n1, n2, mac, x, head);
     else body_lines<OPEN, true>(tile, lane, src, dst, len, len_in, safe, k, n1, n2, mac, x, head);
 
-    lane_finish<OPEN>(a, lane, have, i, len, src, dst, mac, head, in_batch && head.on ? a.heads + 32ull * t : nullptr);
+    lane_finish<OPEN>(a, lane, have, i, len, src, dst, mac, head, in_batch && a.heads ? a.heads + 32ull * t : nullptr,
+                      decap && in_batch && wg_res == BNK_WG_OK, pr);
 }
 
 // One wave = one packet, for batches too small to fill the chip with a packet
@@ -1004,7 +1071,9 @@ hipError_t launch_aead_open(const AeadArgs &a, hipStream_t s)
     if (a.n == 0) return hipSuccess;
     const dim3 waves((a.n + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK);
     if (a.wg.mode != WG_FUSE_OFF) {
-        if (a.wg.mode != WG_FUSE_DECAP || !aead_runs_spread(a)) return hipErrorInvalidValue;
+        if (a.wg.mode != WG_FUSE_DECAP) return hipErrorInvalidValue;
+        if (!aead_runs_spread(a)) return a.in_skip == 16u && a.out_skip == 0u ? launch_wave<true>(a, s) : hipErrorInvalidValue;
+        if (a.in_skip != 0u) return hipErrorInvalidValue;
         hipLaunchKernelGGL((aead_spread_kernel<true, true>), waves, dim3(256), 0, s, a);
     } else if (aead_runs_spread(a))
         hipLaunchKernelGGL((aead_spread_kernel<true, false>), waves, dim3(256), 0, s, a);

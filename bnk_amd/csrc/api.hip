@@ -386,7 +386,7 @@ void bnk_shutdown(bnk_ctx *ctx)
                           &ctx->wg_peer, &ctx->wg_counter, &ctx->wg_ctlen, &ctx->wg_result,
                           &ctx->wg_outlen, &ctx->wg_padded, &ctx->wg_wirelen, &ctx->wg_skip, &ctx->wg_sctr,
                           &ctx->wg_sval, &ctx->wg_pmax, &ctx->wg_lastb, &ctx->wg_rtable, &ctx->wg_rflags,
-                          &ctx->r_heads})
+                          &ctx->r_heads, &ctx->wg_hash})
             b->release();
         ctx->pin.release();
         if (ctx->wg_replay) (void)hipFree(ctx->wg_replay);

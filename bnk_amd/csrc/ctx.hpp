@@ -121,6 +121,8 @@ struct bnk_ctx {
     // anti-replay windows, one per row, and the scratch of a replay pass
     uint64_t *wg_replay = nullptr;
     uint32_t wg_replay_rows = 0;
+    bnk::DevBuf wg_hash;      // receiver index -> row, hash table form
+    uint32_t wg_hash_bits = 0;
     bool wg_replay_on = true;
     bool wg_unfused = false; // framing of lane-per-packet launches in kernels of its own
     bnk::DevBuf wg_sctr, wg_sval, wg_pmax, wg_lastb, wg_rtable, wg_rflags;

@@ -36,11 +36,21 @@ __host__ __device__ inline uint64_t ctr_add(uint64_t base, uint64_t rank, uint64
 // bytes long, padding included.  A lane-per-packet launch: in_skip and
 // out_skip say where the AEAD data starts within the slot or datagram (16 past
 // the header), any length.
+// Receiver index -> peer row as an open-addressing table of (index, row) pairs
+// with linear probing; an empty slot has row WG_HASH_EMPTY.
+constexpr uint32_t WG_HASH_EMPTY = 0xFFFFFFFFu;
+__host__ __device__ inline uint32_t wg_hash_slot(uint32_t index, uint32_t bits)
+{
+    return (index * 0x9E3779B1u) >> (32u - bits);
+}
+
 struct WgFuse {
     uint32_t mode;               // WG_FUSE_*
     uint32_t n_peers;            // rows of the peer tables
     uint32_t mtu;                // encapsulate: padding cap
-    const uint2 *index_sorted;   // decapsulate: (receiver index, peer), ascending
+    const uint2 *index_sorted;   // decapsulate, a wave per packet: (receiver index, peer), ascending
+    const uint2 *index_hash;     // decapsulate, a lane per packet: the same as a hash table of
+    uint32_t hash_bits;          // 2^hash_bits slots (wg_hash_slot)
     const uint2 *allowed;        // decapsulate: (net, mask) per peer
     const uint32_t *remote_index; // encapsulate: index the peer expects
     uint8_t *result;             // decapsulate: BNK_WG_* per packet

@@ -14,6 +14,8 @@ WgPeersDev peers_view(bnk_ctx *ctx)
 {
     WgPeersDev pe{};
     pe.index_sorted = ctx->wg_index.as<uint2>();
+    pe.index_hash = ctx->wg_hash.as<uint2>();
+    pe.hash_bits = ctx->wg_hash_bits;
     pe.remote_index = ctx->wg_remote.as<uint32_t>();
     pe.allowed = ctx->wg_allowed.as<uint2>();
     pe.send_ctr = ctx->wg_send_ctr.as<uint64_t>();
@@ -74,6 +76,36 @@ static int wg_build_index(bnk_ctx *ctx, const bnk_wg_peer *peers, uint32_t n, st
     return BNK_OK;
 }
 
+// The same map as an open-addressing hash table (see wg_hash_slot): at least
+// four slots per peer, so a lookup is one probe nine times in ten.
+static void wg_build_hash(const std::vector<uint2> &index, std::vector<uint2> *table, uint32_t *bits)
+{
+    uint32_t b = 6;
+    while (b < 31 && (1ull << b) < 4ull * index.size()) b++;
+    table->assign((size_t)1 << b, make_uint2(0, WG_HASH_EMPTY));
+    const uint32_t mask = (1u << b) - 1u;
+    for (const uint2 &e : index) {
+        uint32_t at = wg_hash_slot(e.x, b);
+        while ((*table)[at].y != WG_HASH_EMPTY) at = (at + 1u) & mask;
+        (*table)[at] = e;
+    }
+    *bits = b;
+}
+
+// Installs both forms of the receiver-index map.
+static int wg_upload_index(bnk_ctx *ctx, const std::vector<uint2> &index)
+{
+    std::vector<uint2> table;
+    uint32_t bits = 0;
+    wg_build_hash(index, &table, &bits);
+    int rc = upload(ctx, &ctx->wg_index, index.data(), index.size() * 8);
+    if (!rc) rc = upload(ctx, &ctx->wg_hash, table.data(), table.size() * 8);
+    if (rc) return rc;
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream)); // `table` goes away
+    ctx->wg_hash_bits = bits;
+    return BNK_OK;
+}
+
 extern "C" int bnk_wg_peers_set(bnk_ctx *ctx, const bnk_wg_peer *peers, uint32_t n)
 {
     BNK_API_TRY
@@ -105,7 +137,7 @@ extern "C" int bnk_wg_peers_set(bnk_ctx *ctx, const bnk_wg_peer *peers, uint32_t
         if (!same) ctr[i] = 0;
         fresh[i] = same ? 0 : 1; // the anti-replay window belongs to the keypair as well
     }
-    rc = upload(ctx, &ctx->wg_index, index.data(), (size_t)n * 8);
+    rc = wg_upload_index(ctx, index);
     if (!rc) rc = upload(ctx, &ctx->wg_remote, remote.data(), (size_t)n * 4);
     if (!rc) rc = upload(ctx, &ctx->wg_allowed, allowed.data(), (size_t)n * 8);
     if (!rc) rc = upload(ctx, &ctx->wg_send_ctr, ctr.data(), (size_t)n * 8);
@@ -142,7 +174,8 @@ extern "C" int bnk_wg_peer_set(bnk_ctx *ctx, uint32_t row, const bnk_wg_peer *pe
     const uint2 allowed = make_uint2(peer->allowed_net, peer->allowed_mask);
     const uint64_t zero = 0;
     hipStream_t s = ctx->stream;
-    HIPCHK(ctx, hipMemcpyAsync(ctx->wg_index.p, index.data(), index.size() * 8, hipMemcpyHostToDevice, s));
+    rc = wg_upload_index(ctx, index);
+    if (rc) return rc;
     HIPCHK(ctx, hipMemcpyAsync(ctx->wg_remote.as<uint32_t>() + row, &peer->remote_index, 4, hipMemcpyHostToDevice, s));
     HIPCHK(ctx, hipMemcpyAsync(ctx->wg_allowed.as<uint2>() + row, &allowed, 8, hipMemcpyHostToDevice, s));
     // this row's keypair is new: its nonces and its anti-replay window start
@@ -813,7 +846,6 @@ static int wg_decap_impl(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *o
                 return filter_range(lo, hi);
             }
         }
-        HIPCHK(ctx, launch_wg_parse(cw, pe, d_peer, d_counter, d_ctlen, d_result, ctx->d_status, ctx->stream));
         AeadArgs op{};
         op.spread_max = ctx->spread_max;
         op.keys = ctx->d_keys[BNK_KEYS_RECV];
@@ -829,10 +861,38 @@ static int wg_decap_impl(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *o
         op.out_off = ob.off;
         op.out_stride = out->stride;
         op.lens = d_ctlen;
+        op.out_limit = ob.limit;
+        if (!ctx->wg_unfused && !aead_runs_spread(op)) {
+            // a lane per packet: header checks, index lookup and what follows the
+            // open are the launch's own work too
+            op.lens = wb.lens;
+            op.len = wire->len;
+            op.in_limit = wb.limit;
+            op.wg.mode = WG_FUSE_DECAP;
+            op.wg.n_peers = pe.n;
+            op.wg.index_hash = pe.index_hash;
+            op.wg.hash_bits = pe.hash_bits;
+            op.wg.allowed = pe.allowed;
+            op.wg.result = d_result;
+            op.wg.out_len = d_out_len;
+            op.wg.peer_out = d_peer;
+            op.wg.counter_out = d_counter;
+            if (wire->lens && op.n > 64) {
+                // (32 bytes of every datagram are header and tag)
+                HIPCHK(ctx, launch_length_sort(wb.lens + lo, op.n, 32, ctx->order.as<uint32_t>() + lo,
+                                               ctx->hist.as<uint32_t>(), ctx->cursor.as<uint32_t>(), ctx->stream));
+                op.order = ctx->order.as<uint32_t>() + lo;
+            }
+            HIPCHK(ctx, launch_aead_open(op, ctx->stream));
+            if (int rr = replay_range(lo, hi)) return rr;
+            return filter_range(lo, hi);
+        }
+        // the framing in kernels of its own around a plain open
+        HIPCHK(ctx, launch_wg_parse(cw, pe, d_peer, d_counter, d_ctlen, d_result, ctx->d_status, ctx->stream));
         op.peer = d_peer;
         op.counters = d_counter;
         op.verdict = d_auth;
-        op.out_limit = ob.limit; // (the datagram's own bounds were checked by the parse)
+        // (the datagram's own bounds were checked by the parse)
         op.skip = d_result; // BNK_WG_OK is 0: header failures are not opened
         if (wire->lens && op.n > 64 && !aead_runs_spread(op)) {
             HIPCHK(ctx, launch_length_sort(d_ctlen + lo, op.n, 16, ctx->order.as<uint32_t>() + lo,

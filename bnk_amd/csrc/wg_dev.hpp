@@ -8,6 +8,8 @@ namespace bnk {
 
 struct WgPeersDev {
     const uint2 *index_sorted;   // (local receiver index, peer), ascending by index
+    const uint2 *index_hash;     // the same pairs in a hash table of 2^hash_bits slots (wg_hash_slot)
+    uint32_t hash_bits;
     const uint32_t *remote_index; // [n] index the peer expects in the header
     const uint2 *allowed;         // [n] (net, mask) of the peer's allowed IPv4 prefix
     uint64_t *send_ctr;           // [n] next nonce counter per peer

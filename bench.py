@@ -38,8 +38,8 @@ VALU_PEAK_TOPS = 39.3  # 256 CU x 64 lanes x 2.4 GHz, one int32 op per lane per 
 # Counter readings for one launch of aead_wave_kernel over 2^20 packets x 1420 B (mean of
 # seal and open), taken with rocprofv3 --pmc and kept in profiles/aead_wave_kernel_cfg2.md;
 # they change only when the kernel does.
-VALU_LANE_INSTR_PER_PACKET = 31276   # SQ_INSTS_VALU x 64 / 2^20
-TRAFFIC_BYTES_PER_LAUNCH = 3.187e9   # FETCH_SIZE + WRITE_SIZE, scaled by copy_kernel
+VALU_LANE_INSTR_PER_PACKET = 31315   # SQ_INSTS_VALU x 64 / 2^20
+TRAFFIC_BYTES_PER_LAUNCH = 3.132e9   # FETCH_SIZE + WRITE_SIZE, scaled by copy_kernel
 # the same for filter_check_kernel over 2^22 headers (profiles/filter_check_kernel_cfg4.md)
 FILTER_TRAFFIC_BYTES_PER_LAUNCH = 191.6e6
 
@@ -398,15 +398,20 @@ def bench_wg(args) -> dict:
     timed(args.warmup)
     ms = timed(args.steps)
     # the same steps with the framing in kernels of its own, and without the windows
-    ctx.wg_set_fused(False)
-    timed(1)
-    ms_separate = timed(args.steps)
-    ctx.wg_set_fused(True)
-    timed(1)
-    ms_again = timed(args.steps)  # clocks drift over a run: the first figure once more
-    ctx.wg_set_replay(False)
-    timed(1)
-    ms_no_windows = timed(args.steps)
+    variants = None
+    if not args.no_extras:
+        ctx.wg_set_fused(False)
+        timed(1)
+        ms_separate = timed(args.steps)
+        ctx.wg_set_fused(True)
+        timed(1)
+        ms_again = timed(args.steps)  # clocks drift over a run: the first figure once more
+        ctx.wg_set_replay(False)
+        timed(1)
+        ms_no_windows = timed(args.steps)
+        variants = {"framing_in_kernels_of_its_own": round(ms_separate, 4),
+                    "as_value_measured_again": round(ms_again, 4),
+                    "anti_replay_windows_off": round(ms_no_windows, 4)}
     last = arenas[done & 1][:n * stride].view(n, stride)[:, 16:16 + plen]
     assert bool((d_res == 0).all()) and bool((d_olen == plen).all()) and bool((d_gp == d_peer).all())
     assert bool((d_wl == wire_len).all()) and torch.equal(last, first_plain), "the packets did not survive the trips"
@@ -425,9 +430,7 @@ def bench_wg(args) -> dict:
                                "resident; every step sends what the step before received"
                                % (n, plen, wire_len, stride, n_peers), "packets": n},
         "mpkt_per_s_pair": round(n / (ms * 1e-3) / 1e6, 1),
-        "same_run_ms_per_step": {"framing_in_kernels_of_its_own": round(ms_separate, 4),
-                                 "as_value_measured_again": round(ms_again, 4),
-                                 "anti_replay_windows_off": round(ms_no_windows, 4)},
+        "same_run_ms_per_step": variants,
         "roofline_valu": {"achieved": round(2 * ops / (ms * 1e-3) / 1e12, 2), "peak": VALU_PEAK_TOPS,
                           "unit": "Top/s (int32 op-equivalents)",
                           "frac": round(2 * ops / (ms * 1e-3) / 1e12 / VALU_PEAK_TOPS, 4)},

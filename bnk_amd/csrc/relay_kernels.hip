@@ -91,6 +91,28 @@ static unsigned key_bits(uint32_t n_keys)
 using SortConfig = rocprim::radix_sort_config<rocprim::default_config, rocprim::default_config,
                                               rocprim::default_config, 32768>;
 
+constexpr uint32_t RANK_TABLE_MAX_KEYS = 4096;
+constexpr uint32_t TILE_RUNS_MAX = 32;
+constexpr size_t RANK_TABLE_MAX_BYTES = 64u << 20;
+
+struct RankPlan {
+    uint32_t runs;  // runs of 64 packets per tile
+    uint32_t tiles;
+    size_t bytes;   // the table, then one total per peer
+    bool fits;
+};
+
+static RankPlan rank_plan(uint32_t n, uint32_t n_keys)
+{
+    RankPlan p{};
+    // tiles as long as a wave can keep in registers, once there are enough of them to fill the chip
+    p.runs = std::min<uint32_t>(TILE_RUNS_MAX, std::max<uint32_t>(1u, n / (64u * 512u)));
+    p.tiles = (n + 64u * p.runs - 1u) / (64u * p.runs);
+    p.bytes = ((size_t)p.tiles + 1u) * n_keys * 4u;
+    p.fits = n_keys <= RANK_TABLE_MAX_KEYS && p.bytes <= RANK_TABLE_MAX_BYTES;
+    return p;
+}
+
 size_t relay_sort_tmp_bytes(uint32_t n, uint32_t n_keys)
 {
     size_t bytes = 0;
@@ -98,7 +120,13 @@ size_t relay_sort_tmp_bytes(uint32_t n, uint32_t n_keys)
                                     (const uint32_t *)nullptr, (uint32_t *)nullptr, (size_t)n, 0,
                                     key_bits(n_keys));
     // once the sort is done the same scratch holds one run start per key
-    return std::max(bytes, (size_t)n_keys * 4);
+    bytes = std::max(bytes, (size_t)n_keys * 4);
+    // the sort-free form's table, for this batch or any part of it (a part of fewer
+    // than 65,536 packets is cut into up to 1024 tiles)
+    const RankPlan plan = rank_plan(n, n_keys);
+    if (!plan.fits) return bytes;
+    const size_t rows = std::max<size_t>(plan.tiles, std::min<size_t>(n / 64u + 1u, 1024u)) + 1u;
+    return std::max(bytes, rows * n_keys * 4u);
 }
 
 __global__ void peer_rank_small_kernel(const uint32_t *peer, uint32_t n_keys, uint32_t n, uint64_t *ctr_base,
@@ -182,11 +210,137 @@ hipError_t launch_peer_rank_small(const uint32_t *peer, uint32_t n_keys, uint32_
     return hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------
+// The same counters without a sort, for peer tables of at most
+// RANK_TABLE_MAX_KEYS rows.  The batch is cut into tiles of TILE_RUNS runs of
+// 64 packets, one wave per tile.  rank_count_kernel counts each tile's packets
+// per peer into a row of a table; rank_scan_kernel turns every column (a
+// peer's counts, tile after tile) into exclusive prefixes and keeps the
+// totals; rank_assign_kernel loads its tile's row into LDS and walks the tile
+// run by run in batch order: a packet's rank is its peer's entry plus the
+// number of lower lanes of the run with the same peer, and one lane per peer
+// then moves the entry past the run.  Four launches over the keys, against
+// eight (two of them passes over key-index pairs) for the sort.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(64) void rank_count_kernel(const uint32_t *keys, uint32_t n, uint32_t n_keys,
+                                                        uint32_t runs, uint32_t *table)
+{
+    __shared__ uint32_t cnt[RANK_TABLE_MAX_KEYS];
+    const uint32_t lane = threadIdx.x;
+    for (uint32_t k = lane; k < n_keys; k += 64u) cnt[k] = 0;
+    __syncthreads();
+    const uint32_t first = blockIdx.x * runs * 64u;
+    for (uint32_t r = 0; r < runs; r++) {
+        const uint32_t i = first + r * 64u + lane;
+        const uint32_t key = i < n ? keys[i] : NO_PEER;
+        if (key < n_keys) atomicAdd(&cnt[key], 1u);
+    }
+    __syncthreads();
+    uint32_t *row = table + (size_t)blockIdx.x * n_keys;
+    for (uint32_t k = lane; k < n_keys; k += 64u) row[k] = cnt[k];
+}
+
+// One block per 64 peers: 16 groups of threads share the tiles between them.
+constexpr uint32_t SCAN_PEERS = 64, SCAN_PARTS = 16;
+__global__ __launch_bounds__(SCAN_PEERS * SCAN_PARTS) void rank_scan_kernel(uint32_t *table, uint32_t tiles,
+                                                                             uint32_t n_keys, uint32_t *total)
+{
+    __shared__ uint32_t part_sum[SCAN_PARTS][SCAN_PEERS];
+    const uint32_t x = threadIdx.x % SCAN_PEERS, y = threadIdx.x / SCAN_PEERS;
+    const uint32_t key = blockIdx.x * SCAN_PEERS + x;
+    const uint32_t per = (tiles + SCAN_PARTS - 1u) / SCAN_PARTS;
+    const uint32_t lo = min(y * per, tiles), hi = min(lo + per, tiles);
+    uint32_t sum = 0;
+    if (key < n_keys)
+        for (uint32_t t = lo; t < hi; t++) sum += table[(size_t)t * n_keys + key];
+    part_sum[y][x] = sum;
+    __syncthreads();
+    uint32_t run = 0;
+    for (uint32_t q = 0; q < y; q++) run += part_sum[q][x];
+    if (key < n_keys) {
+        for (uint32_t t = lo; t < hi; t++) {
+            uint32_t *e = table + (size_t)t * n_keys + key;
+            const uint32_t c = *e;
+            *e = run;
+            run += c;
+        }
+        if (y == SCAN_PARTS - 1u) total[key] = run;
+    }
+}
+
+__global__ __launch_bounds__(64) void rank_assign_kernel(const uint32_t *keys, uint32_t n, uint32_t n_keys,
+                                                         uint32_t runs, const uint32_t *table, unsigned bits,
+                                                         const uint64_t *ctr_base, uint64_t *ctr_out,
+                                                         uint64_t ctr_limit)
+{
+    __shared__ uint32_t before[RANK_TABLE_MAX_KEYS]; // packets of each peer ahead of the run at hand
+    const uint32_t lane = threadIdx.x;
+    const uint32_t *row = table + (size_t)blockIdx.x * n_keys;
+    for (uint32_t k = lane; k < n_keys; k += 64u) before[k] = row[k];
+    const uint32_t first = blockIdx.x * runs * 64u;
+    uint32_t key[TILE_RUNS_MAX];
+#pragma unroll
+    for (uint32_t r = 0; r < TILE_RUNS_MAX; r++) {
+        const uint32_t i = first + r * 64u + lane;
+        key[r] = r < runs && i < n ? keys[i] : NO_PEER;
+    }
+    __syncthreads();
+#pragma unroll
+    for (uint32_t r = 0; r < TILE_RUNS_MAX; r++) {
+        if (r >= runs) break; // uniform
+        const uint32_t kk = key[r];
+        const bool valid = kk < n_keys;
+        // the lanes of this run with my peer
+        unsigned long long same = __ballot(valid);
+        for (unsigned b = 0; b < bits; b++) {
+            const unsigned long long m = __ballot((kk >> b) & 1u);
+            same &= ((kk >> b) & 1u) ? m : ~m;
+        }
+        if (valid) {
+            const uint32_t lower = (uint32_t)__popcll(same & ((1ull << lane) - 1ull));
+            const uint32_t rank = before[kk] + lower;
+            ctr_out[first + r * 64u + lane] = ctr_add(ctr_base[kk], rank, ctr_limit);
+            // every lane has read the entry before any lane writes one: the lanes of a
+            // wave run in lockstep and LDS serves their accesses in order
+            if (lower == 0u) before[kk] += (uint32_t)__popcll(same);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
+__global__ __launch_bounds__(256) void rank_advance_kernel(const uint32_t *total, uint32_t n_keys,
+                                                           uint64_t *ctr_base, uint64_t ctr_limit)
+{
+    const uint32_t k = blockIdx.x * 256u + threadIdx.x;
+    if (k < n_keys && total[k] != 0u) ctr_base[k] = ctr_add(ctr_base[k], total[k], ctr_limit);
+}
+
+static hipError_t launch_peer_rank_table(const uint32_t *keys, const RankPlan &plan, void *tmp,
+                                         uint64_t *ctr_base, uint32_t n_keys, uint32_t n, uint64_t *ctr_out,
+                                         bool advance, uint64_t ctr_limit, hipStream_t s)
+{
+    uint32_t *table = static_cast<uint32_t *>(tmp);
+    uint32_t *total = table + (size_t)plan.tiles * n_keys;
+    hipLaunchKernelGGL(rank_count_kernel, dim3(plan.tiles), dim3(64), 0, s, keys, n, n_keys, plan.runs, table);
+    hipLaunchKernelGGL(rank_scan_kernel, dim3((n_keys + SCAN_PEERS - 1u) / SCAN_PEERS),
+                       dim3(SCAN_PEERS * SCAN_PARTS), 0, s, table, plan.tiles, n_keys, total);
+    hipLaunchKernelGGL(rank_assign_kernel, dim3(plan.tiles), dim3(64), 0, s, keys, n, n_keys, plan.runs, table,
+                       key_bits(n_keys), ctr_base, ctr_out, ctr_limit);
+    if (advance)
+        hipLaunchKernelGGL(rank_advance_kernel, dim3((n_keys + 255u) / 256u), dim3(256), 0, s, total, n_keys,
+                           ctr_base, ctr_limit);
+    return hipGetLastError();
+}
+
 hipError_t launch_peer_rank(uint32_t *keys, uint32_t *idx, uint32_t *skeys, uint32_t *sidx,
                             void *sort_tmp, size_t sort_tmp_bytes, uint64_t *ctr_base, uint32_t n_keys,
                             uint32_t n, uint64_t *ctr_out, bool advance, uint64_t ctr_limit, hipStream_t s)
 {
     if (n == 0) return hipSuccess;
+    const RankPlan plan = rank_plan(n, n_keys);
+    if (plan.fits && plan.bytes <= sort_tmp_bytes)
+        return launch_peer_rank_table(keys, plan, sort_tmp, ctr_base, n_keys, n, ctr_out, advance, ctr_limit, s);
     const dim3 grid((n + 255u) / 256u);
     hipError_t e = rocprim::radix_sort_pairs<SortConfig>(sort_tmp, sort_tmp_bytes, keys, skeys, idx, sidx, (size_t)n,
                                              0, key_bits(n_keys), s);

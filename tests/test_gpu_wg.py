@@ -192,6 +192,79 @@ def test_encap_uniform_slots_one_peer_and_padding_rules(fused, length, mtu):
     ctx.close()
 
 
+@pytest.mark.parametrize("n_peers", [700, 5000])
+def test_many_peers_counters_and_index_lookup(n_peers):
+    """A peer table of hundreds and of thousands of rows, batches large enough for
+    the lane-per-packet launches: send counters follow each peer's order in the
+    batch (700 rows: counted per tile; 5000: beyond what that holds in LDS, so
+    sorted), every datagram finds its sender through the hash form of the
+    receiver-index map (indices chosen to collide), and an index nobody owns is
+    told apart."""
+    from bnk_amd import lib
+    from oracle import binding as O
+    rng = np.random.default_rng(n_peers)
+    # local indices in a few clusters of consecutive numbers: long probe chains
+    local = (np.repeat(rng.integers(0, 1 << 32, 8, dtype=np.uint64), (n_peers + 7) // 8)[:n_peers]
+             + np.arange(n_peers, dtype=np.uint64) * 0x10000).astype(np.uint32)
+    assert np.unique(local).size == n_peers
+    remote = rng.integers(0, 1 << 32, n_peers, dtype=np.uint64).astype(np.uint32)
+    net = (0x64400000 + np.arange(n_peers, dtype=np.uint32)).astype(np.uint32)
+    peers = np.stack([local, remote, net, np.full(n_peers, 0xFFFFFFFF, np.uint32)], 1)
+    keys = rng.integers(0, 256, (n_peers, 32), dtype=np.uint8)
+    n, length, mtu = 9000, 44, 1420
+    stride = 112
+    peer = rng.integers(0, n_peers, n).astype(np.uint32)
+    peer[:50] = 3  # a run of one peer
+    arena = rng.integers(0, 256, n * stride, dtype=np.uint8)
+    v = arena.reshape(n, stride)
+    v[:, 16] = 0x45
+    v[:, 18], v[:, 19] = length >> 8, length & 255
+    for k in range(4):
+        v[:, 16 + 12 + k] = (net[peer] >> (24 - 8 * k)) & 255
+    plain = v[:, 16:16 + length].copy()
+    ctx = lib.Context(0)
+    ctx.keys_set(lib.KEYS_SEND, keys)
+    ctx.keys_set(lib.KEYS_RECV, keys)
+    # both ends in one table: what a peer expects in the header is what we look up
+    peers[:, 1] = peers[:, 0]
+    ctx.wg_peers_set(peers)
+    ctx.set_spread_max_packets(0)
+    wire_len = np.zeros(n, np.uint32)
+    ctx.wg_encap(lib.make_batch(arena, arena.nbytes, n, lib.MEM_HOST, stride=stride, length=length, peer=peer),
+                 mtu, wire_len)
+    padded = length + O.wg_padding(length, mtu)
+    assert (wire_len == 32 + padded).all()
+    hdr = v[:, :16].copy().view(np.uint32).reshape(n, 4)
+    assert (hdr[:, 0] == 4).all() and np.array_equal(hdr[:, 1], local[peer])
+    got_ctr = hdr[:, 2].astype(np.uint64) | hdr[:, 3].astype(np.uint64) << np.uint64(32)
+    assert np.array_equal(got_ctr, W.per_peer_sequence(peer, n_peers))
+    assert np.array_equal(ctx.wg_send_counters(n_peers), np.bincount(peer, minlength=n_peers).astype(np.uint64))
+    i = 4321
+    assert v[i, :32 + padded].tobytes() == O.wg_encap(plain[i].tobytes(), mtu, keys[peer[i]].tobytes(),
+                                                     int(local[peer[i]]), int(got_ctr[i]))
+    # back in: a few datagrams carry an index one off a real one
+    strangers = rng.permutation(n)[:40]
+    hdr_view = v[:, :16].view(np.uint32).reshape(n, 4)
+    free = np.setdiff1d(local[peer[strangers]] + np.uint32(1), local)
+    hdr_view[strangers[:free.size], 1] = free
+    strangers = strangers[:free.size]
+    out = np.zeros(n * stride, np.uint8)
+    res = np.full(n, 99, np.uint8)
+    out_len = np.zeros(n, np.uint32)
+    got_peer = np.zeros(n, np.uint32)
+    got_c = np.zeros(n, np.uint64)
+    ctx.wg_decap(lib.make_batch(arena, arena.nbytes, n, lib.MEM_HOST, stride=stride, length=32 + padded),
+                 lib.make_batch(out, out.nbytes, n, lib.MEM_HOST, stride=stride), res, out_len, got_peer, got_c)
+    want_res = np.zeros(n, np.uint8)
+    want_res[strangers] = lib.WG_UNKNOWN_INDEX
+    assert np.array_equal(res, want_res)
+    ok = want_res == 0
+    assert np.array_equal(got_peer[ok], peer[ok]) and (got_peer[~ok] == 0xFFFFFFFF).all()
+    assert np.array_equal(got_c[ok], got_ctr[ok]) and (out_len[ok] == length).all()
+    assert np.array_equal(out.reshape(n, stride)[ok, :length], plain[ok])
+    ctx.close()
+
+
 @pytest.mark.parametrize("fused", ["wave", "lane", "separate"])
 @pytest.mark.parametrize("inner", [0, 28, 1000, 1420])
 def test_decap_uniform_datagrams(fused, inner):

@@ -92,12 +92,15 @@ using SortConfig = rocprim::radix_sort_config<rocprim::default_config, rocprim::
                                               rocprim::default_config, 32768>;
 
 constexpr uint32_t RANK_TABLE_MAX_KEYS = 4096;
+constexpr uint32_t RANK_ROW_STEP = 256; // 64 lanes x 16 bytes
+constexpr uint32_t RANK_ROW_STEPS = RANK_TABLE_MAX_KEYS / RANK_ROW_STEP;
 constexpr uint32_t TILE_RUNS_MAX = 32;
 constexpr size_t RANK_TABLE_MAX_BYTES = 64u << 20;
 
 struct RankPlan {
     uint32_t runs;  // runs of 64 packets per tile
     uint32_t tiles;
+    uint32_t cols;  // entries per row of the table: the keys, rounded up to what a wave moves at once
     size_t bytes;   // the table, then one total per peer
     bool fits;
 };
@@ -105,10 +108,12 @@ struct RankPlan {
 static RankPlan rank_plan(uint32_t n, uint32_t n_keys)
 {
     RankPlan p{};
-    // tiles as long as a wave can keep in registers, once there are enough of them to fill the chip
-    p.runs = std::min<uint32_t>(TILE_RUNS_MAX, std::max<uint32_t>(1u, n / (64u * 512u)));
+    // about 2048 tiles (a wave each: enough to keep every CU busy), as long as a wave
+    // can hold its tile's keys in registers
+    p.runs = std::min<uint32_t>(TILE_RUNS_MAX, std::max<uint32_t>(1u, (n + 64u * 2048u - 1u) / (64u * 2048u)));
     p.tiles = (n + 64u * p.runs - 1u) / (64u * p.runs);
-    p.bytes = ((size_t)p.tiles + 1u) * n_keys * 4u;
+    p.cols = (n_keys + RANK_ROW_STEP - 1u) / RANK_ROW_STEP * RANK_ROW_STEP;
+    p.bytes = ((size_t)p.tiles + 1u) * p.cols * 4u;
     p.fits = n_keys <= RANK_TABLE_MAX_KEYS && p.bytes <= RANK_TABLE_MAX_BYTES;
     return p;
 }
@@ -121,12 +126,12 @@ size_t relay_sort_tmp_bytes(uint32_t n, uint32_t n_keys)
                                     key_bits(n_keys));
     // once the sort is done the same scratch holds one run start per key
     bytes = std::max(bytes, (size_t)n_keys * 4);
-    // the sort-free form's table, for this batch or any part of it (a part of fewer
-    // than 65,536 packets is cut into up to 1024 tiles)
+    // the sort-free form's table, for this batch or any part of it (a part is cut
+    // into up to 2048 tiles however small it is)
     const RankPlan plan = rank_plan(n, n_keys);
     if (!plan.fits) return bytes;
-    const size_t rows = std::max<size_t>(plan.tiles, std::min<size_t>(n / 64u + 1u, 1024u)) + 1u;
-    return std::max(bytes, rows * n_keys * 4u);
+    const size_t rows = std::max<size_t>(plan.tiles, std::min<size_t>(n / 64u + 1u, 2048u)) + 1u;
+    return std::max(bytes, rows * plan.cols * 4u);
 }
 
 __global__ void peer_rank_small_kernel(const uint32_t *peer, uint32_t n_keys, uint32_t n, uint64_t *ctr_base,
@@ -223,62 +228,15 @@ hipError_t launch_peer_rank_small(const uint32_t *peer, uint32_t n_keys, uint32_
 // eight (two of them passes over key-index pairs) for the sort.
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(64) void rank_count_kernel(const uint32_t *keys, uint32_t n, uint32_t n_keys,
-                                                        uint32_t runs, uint32_t *table)
+                                                        uint32_t cols, uint32_t runs, uint32_t *table)
 {
-    __shared__ uint32_t cnt[RANK_TABLE_MAX_KEYS];
+    __shared__ __attribute__((aligned(16))) uint32_t cnt[RANK_TABLE_MAX_KEYS];
     const uint32_t lane = threadIdx.x;
-    for (uint32_t k = lane; k < n_keys; k += 64u) cnt[k] = 0;
-    __syncthreads();
-    const uint32_t first = blockIdx.x * runs * 64u;
-    for (uint32_t r = 0; r < runs; r++) {
-        const uint32_t i = first + r * 64u + lane;
-        const uint32_t key = i < n ? keys[i] : NO_PEER;
-        if (key < n_keys) atomicAdd(&cnt[key], 1u);
-    }
-    __syncthreads();
-    uint32_t *row = table + (size_t)blockIdx.x * n_keys;
-    for (uint32_t k = lane; k < n_keys; k += 64u) row[k] = cnt[k];
-}
-
-// One block per 64 peers: 16 groups of threads share the tiles between them.
-constexpr uint32_t SCAN_PEERS = 64, SCAN_PARTS = 16;
-__global__ __launch_bounds__(SCAN_PEERS * SCAN_PARTS) void rank_scan_kernel(uint32_t *table, uint32_t tiles,
-                                                                             uint32_t n_keys, uint32_t *total)
-{
-    __shared__ uint32_t part_sum[SCAN_PARTS][SCAN_PEERS];
-    const uint32_t x = threadIdx.x % SCAN_PEERS, y = threadIdx.x / SCAN_PEERS;
-    const uint32_t key = blockIdx.x * SCAN_PEERS + x;
-    const uint32_t per = (tiles + SCAN_PARTS - 1u) / SCAN_PARTS;
-    const uint32_t lo = min(y * per, tiles), hi = min(lo + per, tiles);
-    uint32_t sum = 0;
-    if (key < n_keys)
-        for (uint32_t t = lo; t < hi; t++) sum += table[(size_t)t * n_keys + key];
-    part_sum[y][x] = sum;
-    __syncthreads();
-    uint32_t run = 0;
-    for (uint32_t q = 0; q < y; q++) run += part_sum[q][x];
-    if (key < n_keys) {
-        for (uint32_t t = lo; t < hi; t++) {
-            uint32_t *e = table + (size_t)t * n_keys + key;
-            const uint32_t c = *e;
-            *e = run;
-            run += c;
-        }
-        if (y == SCAN_PARTS - 1u) total[key] = run;
-    }
-}
-
-__global__ __launch_bounds__(64) void rank_assign_kernel(const uint32_t *keys, uint32_t n, uint32_t n_keys,
-                                                         uint32_t runs, const uint32_t *table, unsigned bits,
-                                                         const uint64_t *ctr_base, uint64_t *ctr_out,
-                                                         uint64_t ctr_limit)
-{
-    __shared__ uint32_t before[RANK_TABLE_MAX_KEYS]; // packets of each peer ahead of the run at hand
-    const uint32_t lane = threadIdx.x;
-    const uint32_t *row = table + (size_t)blockIdx.x * n_keys;
-    for (uint32_t k = lane; k < n_keys; k += 64u) before[k] = row[k];
+    uint4 *cnt4 = reinterpret_cast<uint4 *>(cnt);
+    for (uint32_t q = lane; q < cols / 4u; q += 64u) cnt4[q] = make_uint4(0, 0, 0, 0);
     const uint32_t first = blockIdx.x * runs * 64u;
     uint32_t key[TILE_RUNS_MAX];
+    // all of the tile's keys are on their way before the first one is counted
 #pragma unroll
     for (uint32_t r = 0; r < TILE_RUNS_MAX; r++) {
         const uint32_t i = first + r * 64u + lane;
@@ -286,8 +244,97 @@ __global__ __launch_bounds__(64) void rank_assign_kernel(const uint32_t *keys, u
     }
     __syncthreads();
 #pragma unroll
+    for (uint32_t r = 0; r < TILE_RUNS_MAX; r++)
+        if (key[r] < n_keys) atomicAdd(&cnt[key[r]], 1u);
+    __syncthreads();
+    uint4 *row = reinterpret_cast<uint4 *>(table + (size_t)blockIdx.x * cols);
+    for (uint32_t q = lane; q < cols / 4u; q += 64u) row[q] = cnt4[q];
+}
+
+// One block per 16 peers: 64 groups of threads share the tiles between them.
+constexpr uint32_t SCAN_PEERS = 16, SCAN_PARTS = 64;
+constexpr uint32_t SCAN_KEEP = 32; // tiles of a part held in registers between the two passes
+__global__ __launch_bounds__(SCAN_PEERS * SCAN_PARTS) void rank_scan_kernel(uint32_t *table, uint32_t tiles,
+                                                                             uint32_t n_keys, uint32_t cols,
+                                                                             uint32_t *total)
+{
+    __shared__ uint32_t part_sum[SCAN_PARTS][SCAN_PEERS];
+    const uint32_t x = threadIdx.x % SCAN_PEERS, y = threadIdx.x / SCAN_PEERS;
+    const uint32_t key = blockIdx.x * SCAN_PEERS + x;
+    const uint32_t per = (tiles + SCAN_PARTS - 1u) / SCAN_PARTS;
+    const uint32_t lo = min(y * per, tiles), hi = min(lo + per, tiles);
+    const bool mine = key < n_keys;
+    const bool keep = per <= SCAN_KEEP; // (the same for every thread)
+    uint32_t c[SCAN_KEEP];
+    uint32_t sum = 0;
+    if (keep) {
+        // every load of the part in flight at once
+#pragma unroll
+        for (uint32_t j = 0; j < SCAN_KEEP; j++) c[j] = mine && lo + j < hi ? table[(size_t)(lo + j) * cols + key] : 0u;
+#pragma unroll
+        for (uint32_t j = 0; j < SCAN_KEEP; j++) sum += c[j];
+    } else if (mine) {
+#pragma unroll 8
+        for (uint32_t t = lo; t < hi; t++) sum += table[(size_t)t * cols + key];
+    }
+    part_sum[y][x] = sum;
+    __syncthreads();
+    uint32_t run = 0;
+    for (uint32_t q = 0; q < y; q++) run += part_sum[q][x];
+    if (!mine) return;
+    if (keep) {
+#pragma unroll
+        for (uint32_t j = 0; j < SCAN_KEEP; j++) {
+            if (lo + j < hi) table[(size_t)(lo + j) * cols + key] = run;
+            run += c[j];
+        }
+    } else {
+        for (uint32_t t = lo; t < hi; t++) {
+            uint32_t *e = table + (size_t)t * cols + key;
+            const uint32_t v = *e;
+            *e = run;
+            run += v;
+        }
+    }
+    if (y == SCAN_PARTS - 1u) total[key] = run;
+}
+
+__global__ __launch_bounds__(64) void rank_assign_kernel(const uint32_t *keys, uint32_t n, uint32_t n_keys,
+                                                         uint32_t cols, uint32_t runs, const uint32_t *table,
+                                                         unsigned bits,
+                                                         const uint64_t *ctr_base, uint64_t *ctr_out,
+                                                         uint64_t ctr_limit)
+{
+    // packets of each peer ahead of the run at hand
+    __shared__ __attribute__((aligned(16))) uint32_t before[RANK_TABLE_MAX_KEYS];
+    const uint32_t lane = threadIdx.x;
+    {
+        // the tile's row, every load in flight before the first is used
+        const uint4 *row = reinterpret_cast<const uint4 *>(table + (size_t)blockIdx.x * cols);
+        uint4 v[RANK_ROW_STEPS];
+#pragma unroll
+        for (uint32_t q = 0; q < RANK_ROW_STEPS; q++)
+            v[q] = q * RANK_ROW_STEP < cols ? row[q * 64u + lane] : make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (uint32_t q = 0; q < RANK_ROW_STEPS; q++)
+            if (q * RANK_ROW_STEP < cols) reinterpret_cast<uint4 *>(before)[q * 64u + lane] = v[q];
+    }
+    const uint32_t first = blockIdx.x * runs * 64u;
+    uint32_t key[TILE_RUNS_MAX];
+    uint64_t base[TILE_RUNS_MAX];
+    // keys and the peers' bases are fetched up front: nothing inside the walk
+    // below waits for memory
+#pragma unroll
     for (uint32_t r = 0; r < TILE_RUNS_MAX; r++) {
-        if (r >= runs) break; // uniform
+        const uint32_t i = first + r * 64u + lane;
+        key[r] = r < runs && i < n ? keys[i] : NO_PEER;
+    }
+#pragma unroll
+    for (uint32_t r = 0; r < TILE_RUNS_MAX; r++) base[r] = key[r] < n_keys ? ctr_base[key[r]] : 0ull;
+    __syncthreads();
+#pragma unroll
+    for (uint32_t r = 0; r < TILE_RUNS_MAX; r++) {
+        if (r < runs) { // uniform
         const uint32_t kk = key[r];
         const bool valid = kk < n_keys;
         // the lanes of this run with my peer
@@ -299,13 +346,14 @@ __global__ __launch_bounds__(64) void rank_assign_kernel(const uint32_t *keys, u
         if (valid) {
             const uint32_t lower = (uint32_t)__popcll(same & ((1ull << lane) - 1ull));
             const uint32_t rank = before[kk] + lower;
-            ctr_out[first + r * 64u + lane] = ctr_add(ctr_base[kk], rank, ctr_limit);
+            ctr_out[first + r * 64u + lane] = ctr_add(base[r], rank, ctr_limit);
             // every lane has read the entry before any lane writes one: the lanes of a
             // wave run in lockstep and LDS serves their accesses in order
             if (lower == 0u) before[kk] += (uint32_t)__popcll(same);
         }
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
+        }
     }
 }
 
@@ -321,12 +369,13 @@ static hipError_t launch_peer_rank_table(const uint32_t *keys, const RankPlan &p
                                          bool advance, uint64_t ctr_limit, hipStream_t s)
 {
     uint32_t *table = static_cast<uint32_t *>(tmp);
-    uint32_t *total = table + (size_t)plan.tiles * n_keys;
-    hipLaunchKernelGGL(rank_count_kernel, dim3(plan.tiles), dim3(64), 0, s, keys, n, n_keys, plan.runs, table);
+    uint32_t *total = table + (size_t)plan.tiles * plan.cols;
+    hipLaunchKernelGGL(rank_count_kernel, dim3(plan.tiles), dim3(64), 0, s, keys, n, n_keys, plan.cols, plan.runs,
+                       table);
     hipLaunchKernelGGL(rank_scan_kernel, dim3((n_keys + SCAN_PEERS - 1u) / SCAN_PEERS),
-                       dim3(SCAN_PEERS * SCAN_PARTS), 0, s, table, plan.tiles, n_keys, total);
-    hipLaunchKernelGGL(rank_assign_kernel, dim3(plan.tiles), dim3(64), 0, s, keys, n, n_keys, plan.runs, table,
-                       key_bits(n_keys), ctr_base, ctr_out, ctr_limit);
+                       dim3(SCAN_PEERS * SCAN_PARTS), 0, s, table, plan.tiles, n_keys, plan.cols, total);
+    hipLaunchKernelGGL(rank_assign_kernel, dim3(plan.tiles), dim3(64), 0, s, keys, n, n_keys, plan.cols, plan.runs,
+                       table, key_bits(n_keys), ctr_base, ctr_out, ctr_limit);
     if (advance)
         hipLaunchKernelGGL(rank_advance_kernel, dim3((n_keys + 255u) / 256u), dim3(256), 0, s, total, n_keys,
                            ctr_base, ctr_limit);

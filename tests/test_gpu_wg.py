@@ -1237,3 +1237,90 @@ def test_wg_argument_errors():
     assert np.array_equal(wl_, [16 + 112 + 16] * 4)
     assert np.array_equal(ctx.wg_send_counters(2), [4, 0])
     ctx.close()
+
+
+def test_full_size_tunnel_round_trips_device_resident():
+    """2^20 MTU-sized packets across 1024 peers, device resident, the shape
+    bench.py --workload wg times (framing inside the lane-per-packet launches,
+    counters from the per-tile counting kernels, anti-replay windows on): two
+    encapsulate + decapsulate trips, the second carrying the first one's
+    counters on.  Counters follow each peer's order in the batch, every packet
+    comes back as it went in, a sample of datagrams is bit-exact against the
+    oracle, a trip of the same datagrams once more is all replays, and a few
+    tampered datagrams come back as exactly what was done to them."""
+    import torch
+    from bnk_amd import lib
+    from oracle import binding as O
+    dev = torch.device("cuda:0")
+    n, n_peers, plen, mtu, stride = 1 << 20, 1024, 1420, 1420, 1456
+    wire_len = 16 + plen + 16
+    keys = W.rand_bytes(W.stream_seed(2, 40), n_peers * 32).reshape(n_peers, 32)
+    idx = (np.arange(n_peers, dtype=np.uint32) * 7919 + 3).astype(np.uint32)
+    addr = (0x64400000 + np.arange(n_peers, dtype=np.uint32)).astype(np.uint32)
+    full = np.full(n_peers, 0xFFFFFFFF, np.uint32)
+    peer = W.rand_below(W.stream_seed(2, 41), n, n_peers).astype(np.uint32)
+    d_peer = torch.from_numpy(peer.astype(np.int32)).to(dev)
+    a = torch.zeros(n * stride + 16, dtype=torch.uint8, device=dev)
+    b = torch.zeros(n * stride + 16, dtype=torch.uint8, device=dev)
+    slots = a[:n * stride].view(n, stride)
+    slots.copy_(W.rand_bytes_torch(W.stream_seed(2, 42), n * stride, dev).view(n, stride))
+    slots[:, 16] = 0x45
+    slots[:, 18] = plen >> 8
+    slots[:, 19] = plen & 0xFF
+    src = torch.from_numpy(addr.astype(np.int64)).to(dev)[d_peer.long()]
+    for k in range(4):
+        slots[:, 28 + k] = ((src >> (24 - 8 * k)) & 0xFF).to(torch.uint8)
+    first_plain = slots[:, 16:16 + plen].clone()
+    d_wl = torch.zeros(n, dtype=torch.int32, device=dev)
+    d_res = torch.full((n,), 99, dtype=torch.uint8, device=dev)
+    d_olen = torch.zeros(n, dtype=torch.int32, device=dev)
+    d_gp = torch.zeros(n, dtype=torch.int32, device=dev)
+    d_gc = torch.zeros(n, dtype=torch.int64, device=dev)
+    torch.cuda.synchronize()
+    ctx = lib.Context(0)
+    ctx.keys_set(lib.KEYS_SEND, keys)
+    ctx.keys_set(lib.KEYS_RECV, keys)
+    ctx.wg_peers_set(np.stack([idx, idx, addr, full], 1))
+    nbytes = n * stride
+    seq = W.per_peer_sequence(peer, n_peers)
+    per_trip = np.bincount(peer, minlength=n_peers).astype(np.uint64)
+    sample = [0, 1, 4097, n // 2 + 5, n - 1]
+    arenas = (a, b)
+    for trip in range(2):
+        cur, nxt = arenas[trip & 1], arenas[1 - (trip & 1)]
+        plain_before = {i: cur[i * stride + 16:i * stride + 16 + plen].cpu().numpy().tobytes() for i in sample}
+        ctx.wg_encap(lib.make_batch(cur, nbytes, n, lib.MEM_DEVICE, stride=stride, length=plen, peer=d_peer),
+                     mtu, d_wl)
+        ctx.sync()
+        assert bool((d_wl == wire_len).all())
+        want_ctr = seq + per_trip[peer] * np.uint64(trip)
+        for i in sample:
+            want = O.wg_encap(plain_before[i], mtu, keys[peer[i]].tobytes(), int(idx[peer[i]]), int(want_ctr[i]))
+            assert cur[i * stride:i * stride + wire_len].cpu().numpy().tobytes() == want, (trip, i)
+        ctx.wg_decap(lib.make_batch(cur, nbytes, n, lib.MEM_DEVICE, stride=stride, length=wire_len),
+                     lib.make_batch(nxt[16:], nbytes, n, lib.MEM_DEVICE, stride=stride), d_res, d_olen, d_gp, d_gc)
+        ctx.sync()
+        assert bool((d_res == 0).all()) and bool((d_olen == plen).all()) and bool((d_gp == d_peer).all())
+        assert np.array_equal(d_gc.cpu().numpy().astype(np.uint64), want_ctr)
+        got = nxt[:n * stride].view(n, stride)[:, 16:16 + plen]
+        assert torch.equal(got, first_plain)
+    assert np.array_equal(ctx.wg_send_counters(n_peers), per_trip * np.uint64(2))
+    # the last trip's datagrams (still in `cur`) once more: every one is a replay; before
+    # that, tamper with a few: a flipped tag bit, a foreign index, a wrong type
+    bad_tag, bad_idx, bad_type = [7, 70000], [8, 900000], [9]
+    cv = cur[:n * stride].view(n, stride)
+    cv[bad_tag, wire_len - 1] ^= 0x10
+    cv[bad_idx, 5] ^= 0xFF
+    cv[bad_type, 0] = 1
+    torch.cuda.synchronize()
+    scratch_out = torch.zeros_like(a)
+    ctx.wg_decap(lib.make_batch(cur, nbytes, n, lib.MEM_DEVICE, stride=stride, length=wire_len),
+                 lib.make_batch(scratch_out[16:], nbytes, n, lib.MEM_DEVICE, stride=stride), d_res, d_olen, d_gp, d_gc)
+    ctx.sync()
+    want_res = np.full(n, lib.WG_REPLAY, np.uint8)
+    want_res[bad_tag] = lib.WG_AUTH_FAIL
+    want_res[bad_idx] = lib.WG_UNKNOWN_INDEX
+    want_res[bad_type] = lib.WG_BAD_HEADER
+    assert np.array_equal(d_res.cpu().numpy(), want_res)
+    assert bool((d_olen == 0).all())
+    ctx.close()

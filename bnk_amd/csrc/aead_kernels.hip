@@ -599,6 +599,10 @@ BNK_DEV void lane_finish(const AeadArgs &a, uint32_t lane, bool have, uint32_t i
         } else res = BNK_WG_BAD_IP;
         a.wg.result[i] = (uint8_t)res;
         a.wg.out_len[i] = out_len;
+        if (a.wg.replay_keys) {
+            a.wg.replay_keys[i - a.first] = res != BNK_WG_AUTH_FAIL ? pr : 0xFFFFFFFFu;
+            a.wg.replay_idx[i - a.first] = i - a.first;
+        }
     }
     if (OPEN && record) {
         // bytes 0-23 of the plaintext, its length, 1 if it is authentic: the lanes'
@@ -698,6 +702,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             if (!ok) {
                 a.wg.result[i] = (uint8_t)wg_res;
                 a.wg.out_len[i] = 0;
+                if (a.wg.replay_keys) {
+                    a.wg.replay_keys[i - a.first] = 0xFFFFFFFFu;
+                    a.wg.replay_idx[i - a.first] = i - a.first;
+                }
             }
         }
         len = len >= 16u ? len - 16u : 0u; // what goes through the cipher, tag included

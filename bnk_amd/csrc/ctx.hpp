@@ -123,6 +123,7 @@ struct bnk_ctx {
     uint32_t wg_replay_rows = 0;
     bnk::DevBuf wg_hash;      // receiver index -> row, hash table form
     uint32_t wg_hash_bits = 0;
+    uint32_t wg_replay_parity = 0; // WgReplayScratch::parity of the next pass over a large batch
     bool wg_replay_on = true;
     bool wg_unfused = false; // framing of lane-per-packet launches in kernels of its own
     bnk::DevBuf wg_sctr, wg_sval, wg_pmax, wg_lastb, wg_rtable, wg_rflags;

@@ -57,6 +57,8 @@ struct WgFuse {
     uint32_t *out_len;           // decapsulate: inner packet length
     uint32_t *peer_out;          // decapsulate: sender
     uint64_t *counter_out;       // decapsulate: its counter
+    uint32_t *replay_keys;       // decapsulate, a lane per packet, or nullptr: [i - first] = the sender
+    uint32_t *replay_idx;        // when the tag verified, else 0xFFFFFFFF; and i - first itself
     uint32_t *wire_len;          // encapsulate: datagram length
 };
 enum : uint32_t { WG_FUSE_OFF = 0, WG_FUSE_ENCAP = 1, WG_FUSE_DECAP = 2 };

@@ -761,9 +761,16 @@ static int wg_decap_impl(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *o
         for (DevBuf *buf : {&ctx->r_keys, &ctx->r_idx, &ctx->r_skeys, &ctx->r_sidx})
             HIPCHK(ctx, buf->reserve((size_t)biggest * 4));
         for (DevBuf *buf : {&ctx->wg_sctr, &ctx->wg_sval, &ctx->wg_pmax}) HIPCHK(ctx, buf->reserve((size_t)biggest * 8));
+        // the flag words and the first-occurrence table keep their resting state from pass
+        // to pass: set it when they are first allocated or grow
+        const void *had = ctx->wg_lastb.p;
         HIPCHK(ctx, ctx->wg_lastb.reserve((size_t)biggest + 64));
+        if (ctx->wg_lastb.p != had) HIPCHK(ctx, hipMemsetAsync(ctx->wg_lastb.p, 0, 64, ctx->stream));
         rsc.table_slots = wg_replay_table_slots(biggest);
+        had = ctx->wg_rtable.p;
         HIPCHK(ctx, ctx->wg_rtable.reserve((size_t)rsc.table_slots * 4));
+        if (ctx->wg_rtable.p != had)
+            HIPCHK(ctx, hipMemsetAsync(ctx->wg_rtable.p, 0xFF, ctx->wg_rtable.cap, ctx->stream));
         rsc.tmp_bytes = wg_replay_tmp_bytes(biggest, pe.n);
         HIPCHK(ctx, ctx->r_tmp.reserve(rsc.tmp_bytes + 16));
         rsc.keys = ctx->r_keys.as<uint32_t>();
@@ -780,10 +787,12 @@ static int wg_decap_impl(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *o
     }
     // wireguard-go's sequential receiver validates the counter of every
     // authentic packet before it looks inside: ahead of the inbound filter
-    auto replay_range = [&](uint32_t lo, uint32_t hi) -> int {
+    auto replay_range = [&](uint32_t lo, uint32_t hi, bool keys_from_open = false) -> int {
         if (!replay) return BNK_OK;
         WgReplayScratch c = rsc;
         c.table_slots = hi - lo > WG_REPLAY_SMALL_MAX ? wg_replay_table_slots(hi - lo) : 0;
+        if (c.table_slots) c.parity = ctx->wg_replay_parity++ & 1u;
+        c.keys_ready = keys_from_open;
         HIPCHK(ctx, launch_wg_replay(d_result + lo, d_out_len + lo, d_peer + lo, d_counter + lo, hi - lo, rpd, c,
                                      ctx->stream));
         return BNK_OK;
@@ -877,6 +886,12 @@ static int wg_decap_impl(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *o
             op.wg.out_len = d_out_len;
             op.wg.peer_out = d_peer;
             op.wg.counter_out = d_counter;
+            // the window pass sorts the authentic packets by peer: its keys come from here
+            const bool keys_here = replay && op.n > WG_REPLAY_SMALL_MAX;
+            if (keys_here) {
+                op.wg.replay_keys = rsc.keys;
+                op.wg.replay_idx = rsc.idx;
+            }
             if (wire->lens && op.n > 64) {
                 // (32 bytes of every datagram are header and tag)
                 HIPCHK(ctx, launch_length_sort(wb.lens + lo, op.n, 32, ctx->order.as<uint32_t>() + lo,
@@ -884,7 +899,7 @@ static int wg_decap_impl(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *o
                 op.order = ctx->order.as<uint32_t>() + lo;
             }
             HIPCHK(ctx, launch_aead_open(op, ctx->stream));
-            if (int rr = replay_range(lo, hi)) return rr;
+            if (int rr = replay_range(lo, hi, keys_here)) return rr;
             return filter_range(lo, hi);
         }
         // the framing in kernels of its own around a plain open

@@ -54,9 +54,13 @@ struct WgReplayScratch {
     uint32_t *keys, *idx, *skeys, *sidx;   // n words each
     uint64_t *sctr, *sval, *pmax;          // n each
     uint8_t *cls;                          // n
-    uint32_t *flags;                       // one word
-    uint32_t *table;                       // table_slots words, a power of two >= 2 n
+    uint32_t *flags;                       // two words, used in turn (parity): "this pass had late
+                                           // packets".  Both start out 0; a pass clears the other one
+    uint32_t parity;                       // 0 or 1, the other value in the next pass
+    uint32_t *table;                       // table_slots words, a power of two >= 2 n, all
+                                           // 0xFFFFFFFF between passes (a pass that used it clears it)
     uint32_t table_slots;
+    bool keys_ready;                       // keys[] and idx[] have been written by the open launch
     void *tmp;                             // wg_replay_tmp_bytes(n, n_peers)
     size_t tmp_bytes;
 };

@@ -424,6 +424,17 @@ uint32_t wg_replay_table_slots(uint32_t n)
     return s;
 }
 
+// Leaves the first-occurrence table empty for the next pass, which costs
+// nothing when this pass had no late packet (the usual case), and clears the
+// flag word the next pass will use (nobody reads that one now).
+__global__ __launch_bounds__(256) void replay_table_reset_kernel(uint32_t *table, uint32_t slots,
+                                                                 uint32_t *flags, uint32_t parity)
+{
+    if (blockIdx.x == 0 && threadIdx.x == 0) flags[parity ^ 1u] = 0u;
+    if (flags[parity] == 0u) return;
+    for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < slots; i += gridDim.x * 256u) table[i] = HASH_EMPTY;
+}
+
 hipError_t launch_wg_replay(uint8_t *result, uint32_t *out_len, const uint32_t *peer, const uint64_t *counter,
                             uint32_t n, const WgReplayDev &rp, const WgReplayScratch &sc, hipStream_t s)
 {
@@ -439,7 +450,8 @@ hipError_t launch_wg_replay(uint8_t *result, uint32_t *out_len, const uint32_t *
         return hipGetLastError();
     }
     const dim3 grid((n + 255u) / 256u);
-    hipLaunchKernelGGL(replay_keys_kernel, grid, dim3(256), 0, s, result, peer, rp.n_peers, n, sc.keys, sc.idx);
+    if (!sc.keys_ready)
+        hipLaunchKernelGGL(replay_keys_kernel, grid, dim3(256), 0, s, result, peer, rp.n_peers, n, sc.keys, sc.idx);
     size_t bytes = sc.tmp_bytes;
     hipError_t e = rocprim::radix_sort_pairs<SortConfig>(sc.tmp, bytes, sc.keys, sc.skeys, sc.idx, sc.sidx,
                                                          (size_t)n, 0, key_bits(rp.n_peers), s);
@@ -450,17 +462,16 @@ hipError_t launch_wg_replay(uint8_t *result, uint32_t *out_len, const uint32_t *
     e = rocprim::exclusive_scan_by_key(sc.tmp, bytes, sc.skeys, sc.sval, sc.pmax, (uint64_t)0, (size_t)n,
                                        rocprim::maximum<uint64_t>(), rocprim::equal_to<uint32_t>(), s);
     if (e != hipSuccess) return e;
-    e = launch_fill_u32(sc.table, sc.table_slots, HASH_EMPTY, s);
-    if (e != hipSuccess) return e;
-    e = launch_fill_u32(sc.flags, 1, 0u, s);
-    if (e != hipSuccess) return e;
     const uint32_t mask = sc.table_slots - 1u;
+    uint32_t *late_flag = sc.flags + sc.parity;
     hipLaunchKernelGGL(replay_classify_kernel, grid, dim3(256), 0, s, sc.skeys, sc.sidx, sc.sctr, sc.pmax,
-                       rp.state, n, sc.cls, sc.table, mask, sc.flags, result, out_len);
+                       rp.state, n, sc.cls, sc.table, mask, late_flag, result, out_len);
     hipLaunchKernelGGL(replay_claim_kernel, grid, dim3(256), 0, s, sc.skeys, sc.sctr, sc.cls, n, sc.table, mask,
-                       sc.flags);
+                       late_flag);
     hipLaunchKernelGGL(replay_late_kernel, grid, dim3(256), 0, s, sc.skeys, sc.sidx, sc.sctr, sc.cls, rp.state, n,
-                       sc.table, mask, sc.flags, result, out_len);
+                       sc.table, mask, late_flag, result, out_len);
+    hipLaunchKernelGGL(replay_table_reset_kernel, dim3(std::min<uint32_t>((sc.table_slots + 255u) / 256u, 2048u)),
+                       dim3(256), 0, s, sc.table, sc.table_slots, sc.flags, sc.parity);
     hipLaunchKernelGGL(replay_advance_kernel, grid, dim3(256), 0, s, sc.skeys, sc.sctr, sc.pmax, rp.state, n);
     hipLaunchKernelGGL(replay_mark_kernel, grid, dim3(256), 0, s, sc.skeys, sc.sctr, sc.cls, rp.state, n);
     return hipGetLastError();

@@ -106,7 +106,7 @@ def _expect(wires, rx, keys, filters):
     return res, olen, peer, ctr
 
 
-@pytest.mark.parametrize("mode", ["host_fused", "host_unfused", "device_large", "ring_fused"])
+@pytest.mark.parametrize("mode", ["host_fused", "host_unfused", "device_large", "device_separate", "ring_fused"])
 def test_replay_windows_match_the_sequential_filter(mode):
     import torch
     from bnk_amd import lib
@@ -117,18 +117,21 @@ def test_replay_windows_match_the_sequential_filter(mode):
     filters = [O.ReplayFilter() for _ in range(P)]
     last = [0] * P
     sizes = {"host_fused": [1, 64, 300, 1024, 700], "host_unfused": [300, 1024, 2000, 150],
-             "device_large": [5000, 1025, 9000, 3000], "ring_fused": [128, 900, 128]}[mode]
+             "device_large": [5000, 1025, 9000, 3000], "device_separate": [3000, 1025, 6000],
+             "ring_fused": [128, 900, 128]}[mode]
     seen = set()
     with lib.Context(0) as ctx:
         ctx.keys_set(lib.KEYS_RECV, keys)
         ctx.wg_peers_set(rx)
         if mode == "host_unfused":
             ctx.set_spread_max_packets(0)
+        if mode == "device_separate":
+            ctx.wg_set_fused(False)  # the framing, and the window pass's sort keys, from kernels of their own
         for b, n in enumerate(sizes):
             arena, offs, lens, wires, last = _batch(rng, tx, keys, n, last, near_limit=(b == 2))
             want = _expect(wires, rx, keys, filters)
             total = arena.nbytes
-            if mode == "device_large":
+            if mode in ("device_large", "device_separate"):
                 d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to("cuda:0")  # noqa: E731
                 d_arena, d_out = d(arena), torch.zeros(total, dtype=torch.uint8, device="cuda:0")
                 res = torch.zeros(n, dtype=torch.uint8, device="cuda:0")

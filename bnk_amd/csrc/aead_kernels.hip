@@ -600,8 +600,13 @@ BNK_DEV void lane_finish(const AeadArgs &a, uint32_t lane, bool have, uint32_t i
         a.wg.result[i] = (uint8_t)res;
         a.wg.out_len[i] = out_len;
         if (a.wg.replay_keys) {
-            a.wg.replay_keys[i - a.first] = res != BNK_WG_AUTH_FAIL ? pr : 0xFFFFFFFFu;
-            a.wg.replay_idx[i - a.first] = i - a.first;
+            const uint32_t sender = res != BNK_WG_AUTH_FAIL ? pr : 0xFFFFFFFFu;
+            if (a.wg.replay_index_bits) {
+                a.wg.replay_keys[i - a.first] = wg_replay_pack(sender, i - a.first, a.wg.replay_index_bits);
+            } else {
+                a.wg.replay_keys[i - a.first] = sender;
+                a.wg.replay_idx[i - a.first] = i - a.first;
+            }
         }
     }
     if (OPEN && record) {
@@ -703,8 +708,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 a.wg.result[i] = (uint8_t)wg_res;
                 a.wg.out_len[i] = 0;
                 if (a.wg.replay_keys) {
-                    a.wg.replay_keys[i - a.first] = 0xFFFFFFFFu;
-                    a.wg.replay_idx[i - a.first] = i - a.first;
+                    if (a.wg.replay_index_bits) {
+                        a.wg.replay_keys[i - a.first] = wg_replay_pack(0xFFFFFFFFu, i - a.first, a.wg.replay_index_bits);
+                    } else {
+                        a.wg.replay_keys[i - a.first] = 0xFFFFFFFFu;
+                        a.wg.replay_idx[i - a.first] = i - a.first;
+                    }
                 }
             }
         }

@@ -44,6 +44,14 @@ __host__ __device__ inline uint32_t wg_hash_slot(uint32_t index, uint32_t bits)
     return (index * 0x9E3779B1u) >> (32u - bits);
 }
 
+// Sender (0xFFFFFFFF: none) and position of a packet in one word: the position in the low
+// index_bits bits, the sender's low bits above them ("none" is then all ones, above every
+// sender, as long as the field is wider than the largest sender).
+__host__ __device__ inline uint32_t wg_replay_pack(uint32_t sender, uint32_t position, unsigned index_bits)
+{
+    return sender << index_bits | position;
+}
+
 struct WgFuse {
     uint32_t mode;               // WG_FUSE_*
     uint32_t n_peers;            // rows of the peer tables
@@ -58,7 +66,9 @@ struct WgFuse {
     uint32_t *peer_out;          // decapsulate: sender
     uint64_t *counter_out;       // decapsulate: its counter
     uint32_t *replay_keys;       // decapsulate, a lane per packet, or nullptr: [i - first] = the sender
-    uint32_t *replay_idx;        // when the tag verified, else 0xFFFFFFFF; and i - first itself
+    uint32_t *replay_idx;        // when the tag verified, else 0xFFFFFFFF; and i - first itself.  With
+    uint32_t replay_index_bits;  // replay_index_bits != 0 both in one word of replay_keys
+                                 // (wg_replay_pack) and replay_idx is not written
     uint32_t *wire_len;          // encapsulate: datagram length
 };
 enum : uint32_t { WG_FUSE_OFF = 0, WG_FUSE_ENCAP = 1, WG_FUSE_DECAP = 2 };

@@ -891,6 +891,7 @@ static int wg_decap_impl(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *o
             if (keys_here) {
                 op.wg.replay_keys = rsc.keys;
                 op.wg.replay_idx = rsc.idx;
+                op.wg.replay_index_bits = wg_replay_index_bits(op.n, pe.n);
             }
             if (wire->lens && op.n > 64) {
                 // (32 bytes of every datagram are header and tag)

@@ -65,6 +65,11 @@ struct WgReplayScratch {
     size_t tmp_bytes;
 };
 size_t wg_replay_tmp_bytes(uint32_t n, uint32_t n_peers);
+// When a sender and a position within a pass of n packets fit one word together: the bits
+// the position takes (the sender sits above them; see wg_replay_pack), else 0.  With it
+// WgReplayScratch::keys holds those words (and idx is scratch), without it keys and idx
+// hold senders and positions.
+unsigned wg_replay_index_bits(uint32_t n, uint32_t n_peers);
 uint32_t wg_replay_table_slots(uint32_t n);
 // Runs every packet whose result so far says "authentic" (anything but
 // BAD_HEADER, UNKNOWN_INDEX, AUTH_FAIL) through its peer's window, in batch

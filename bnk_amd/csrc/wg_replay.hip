@@ -104,6 +104,36 @@ __global__ __launch_bounds__(256) void replay_keys_kernel(const uint8_t *result,
     idx[i] = i;
 }
 
+// The same as one word per packet, sender above position (wg_replay_index_bits):
+// a stable sort on the sender's bits alone then moves half the bytes.
+__global__ __launch_bounds__(256) void replay_keys_packed_kernel(const uint8_t *result, const uint32_t *peer,
+                                                                 uint32_t n_peers, uint32_t n, unsigned index_bits,
+                                                                 uint32_t *packed)
+{
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i >= n) return;
+    const uint32_t p = peer[i];
+    packed[i] = wg_replay_pack((replay_subject(result[i]) && p < n_peers) ? p : NO_PEER, i, index_bits);
+}
+
+// Sender, position and counter of the packets in sorted order, from the sorted words.
+__global__ __launch_bounds__(256) void replay_unpack_kernel(const uint32_t *sorted, const uint64_t *counter,
+                                                            uint32_t n, unsigned index_bits, unsigned peer_bits,
+                                                            uint32_t *skeys, uint32_t *sidx, uint64_t *sctr,
+                                                            uint64_t *sval)
+{
+    const uint32_t p = blockIdx.x * 256u + threadIdx.x;
+    if (p >= n) return;
+    const uint32_t w = sorted[p];
+    const uint32_t none = (1u << peer_bits) - 1u, field = (w >> index_bits) & none;
+    const uint32_t i = w & ((1u << index_bits) - 1u);
+    const uint64_t c = field != none ? counter[i] : 0;
+    skeys[p] = field != none ? field : NO_PEER;
+    sidx[p] = i;
+    sctr[p] = c;
+    sval[p] = c < WG_REJECT_AFTER_MESSAGES ? c : 0;
+}
+
 // Counters in sorted order; a counter the filter turns away outright counts as
 // 0 for the running maximum (it never moves last).
 __global__ __launch_bounds__(256) void replay_gather_kernel(const uint32_t *skeys, const uint32_t *sidx,
@@ -405,16 +435,25 @@ hipError_t launch_wg_replay_reset(uint64_t *state, const uint8_t *flags, uint32_
     return hipGetLastError();
 }
 
+unsigned wg_replay_index_bits(uint32_t n, uint32_t n_peers)
+{
+    unsigned bits = 1;
+    while (bits < 32 && ((uint64_t)1 << bits) < n) bits++;
+    return bits + key_bits(n_peers) <= 32 ? bits : 0;
+}
+
 size_t wg_replay_tmp_bytes(uint32_t n, uint32_t n_peers)
 {
-    size_t a = 0, b = 0;
+    size_t a = 0, b = 0, c = 0;
+    (void)rocprim::radix_sort_keys<SortConfig>(nullptr, c, (const uint32_t *)nullptr, (uint32_t *)nullptr, (size_t)n,
+                                               0, 32);
     (void)rocprim::radix_sort_pairs<SortConfig>(nullptr, a, (const uint32_t *)nullptr, (uint32_t *)nullptr,
                                                 (const uint32_t *)nullptr, (uint32_t *)nullptr, (size_t)n, 0,
                                                 key_bits(n_peers));
     (void)rocprim::exclusive_scan_by_key(nullptr, b, (const uint32_t *)nullptr, (const uint64_t *)nullptr,
                                          (uint64_t *)nullptr, (uint64_t)0, (size_t)n,
                                          rocprim::maximum<uint64_t>(), rocprim::equal_to<uint32_t>());
-    return std::max(a, b);
+    return std::max(std::max(a, b), c);
 }
 
 uint32_t wg_replay_table_slots(uint32_t n)
@@ -450,14 +489,29 @@ hipError_t launch_wg_replay(uint8_t *result, uint32_t *out_len, const uint32_t *
         return hipGetLastError();
     }
     const dim3 grid((n + 255u) / 256u);
-    if (!sc.keys_ready)
-        hipLaunchKernelGGL(replay_keys_kernel, grid, dim3(256), 0, s, result, peer, rp.n_peers, n, sc.keys, sc.idx);
     size_t bytes = sc.tmp_bytes;
-    hipError_t e = rocprim::radix_sort_pairs<SortConfig>(sc.tmp, bytes, sc.keys, sc.skeys, sc.idx, sc.sidx,
-                                                         (size_t)n, 0, key_bits(rp.n_peers), s);
-    if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(replay_gather_kernel, grid, dim3(256), 0, s, sc.skeys, sc.sidx, counter, n, sc.sctr,
-                       sc.sval);
+    hipError_t e = hipSuccess;
+    const unsigned peer_bits = key_bits(rp.n_peers);
+    if (const unsigned index_bits = wg_replay_index_bits(n, rp.n_peers)) {
+        // one word per packet: keys[] in, idx[] out
+        if (!sc.keys_ready)
+            hipLaunchKernelGGL(replay_keys_packed_kernel, grid, dim3(256), 0, s, result, peer, rp.n_peers, n,
+                               index_bits, sc.keys);
+        e = rocprim::radix_sort_keys<SortConfig>(sc.tmp, bytes, sc.keys, sc.idx, (size_t)n, index_bits,
+                                                 index_bits + peer_bits, s);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(replay_unpack_kernel, grid, dim3(256), 0, s, sc.idx, counter, n, index_bits, peer_bits,
+                           sc.skeys, sc.sidx, sc.sctr, sc.sval);
+    } else {
+        if (!sc.keys_ready)
+            hipLaunchKernelGGL(replay_keys_kernel, grid, dim3(256), 0, s, result, peer, rp.n_peers, n, sc.keys,
+                               sc.idx);
+        e = rocprim::radix_sort_pairs<SortConfig>(sc.tmp, bytes, sc.keys, sc.skeys, sc.idx, sc.sidx, (size_t)n, 0,
+                                                  peer_bits, s);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(replay_gather_kernel, grid, dim3(256), 0, s, sc.skeys, sc.sidx, counter, n, sc.sctr,
+                           sc.sval);
+    }
     bytes = sc.tmp_bytes;
     e = rocprim::exclusive_scan_by_key(sc.tmp, bytes, sc.skeys, sc.sval, sc.pmax, (uint64_t)0, (size_t)n,
                                        rocprim::maximum<uint64_t>(), rocprim::equal_to<uint32_t>(), s);

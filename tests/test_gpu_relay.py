@@ -20,15 +20,18 @@ def _note(ctx, ora, w):
 
 
 @pytest.mark.parametrize("mem", ["host", "ring"])
-@pytest.mark.parametrize("n,n_peers", [(12000, 64), (900, 64), (40000, 64), (12000, 5000), (40000, 5000)])
+@pytest.mark.parametrize("n,n_peers", [(12000, 64), (900, 64), (40000, 64), (12000, 5000), (40000, 5000),
+                                       (150000, 700)])
 def test_relay_matches_oracle_host_path(mem, n, n_peers):
     """"ring": both arenas lie in pinned rings of the context, which batches of
     a few megabytes relay in place without staging copies.  900 packets also
     take the wave-per-packet kernels and the one-launch counter assignment;
     40000 (14 MB) go through in overlapped chunks, each continuing the
-    counters of the one before.  With 64 peers the outbound counters come from
-    the per-tile counting kernels, with 5000 (beyond what those hold in LDS)
-    from the sort."""
+    counters of the one before; 150000 (52 MB) in chunks large enough for the
+    lane-per-packet launches, the header records and the counting kernels,
+    chunk by chunk.  With 64 or 700 peers the outbound counters come from the
+    per-tile counting kernels, with 5000 (beyond what those hold in LDS) from
+    the sort."""
     from bnk_amd import lib
     from oracle import binding as O
     w = W.relay_workload(n=n, n_peers=n_peers, n_rules=512)

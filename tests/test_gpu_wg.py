@@ -994,16 +994,19 @@ def test_encap_then_decap_round_trip_full_size():
     rx.close()
 
 
-def test_large_host_rings_take_the_chunked_route():
+@pytest.mark.parametrize("n", [24000, 96000])
+def test_large_host_rings_take_the_chunked_route(n):
     """Host rings of several chunks' worth (pinned, as a tunnel would use them):
     encapsulate in place and decapsulate chunk by chunk with upload, kernels
     and download overlapped; results equal the device-resident path's and a
-    sample equals the oracle."""
+    sample equals the oracle.  24000 packets make chunks small enough for a
+    wave per packet, 96000 chunks of 6000 that take a lane per packet (framing
+    and window-pass keys from the AEAD launches, chunk by chunk)."""
     import torch
     from bnk_amd import lib
     from oracle import binding as O
     rng = np.random.default_rng(31)
-    n, n_peers, stride = 24000, 64, 1536
+    n_peers, stride = 64, 1536
     keys = rng.integers(0, 256, (n_peers, 32), dtype=np.uint8)
     idx_a = (np.arange(n_peers, dtype=np.uint32) * 7919 + 3).astype(np.uint32)
     idx_b = (np.arange(n_peers, dtype=np.uint32) * 104729 + 11).astype(np.uint32)

@@ -407,7 +407,9 @@ __global__ __launch_bounds__(SMALL) void replay_small_kernel(uint8_t *result, ui
         if (c < WG_REJECT_AFTER_MESSAGES && c > nl) nl = c;
         advance_window(st, nl);
     }
-    __threadfence();
+    // (one workgroup does all of this: waiting for its stores to be acknowledged is
+    // enough; a device-wide fence would write the whole L2 back)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads(); // the cleared blocks are in place before bits go in
     if (reached) {
         const uint64_t final_last = *reinterpret_cast<volatile uint64_t *>(st);

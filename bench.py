@@ -8,7 +8,7 @@ value is plaintext Gbit/s through the seal+open pair on one MI355X.
 
 Prints ONE JSON line.  Besides the contract fields it carries
   roofline       the binding one: int32 VALU instructions issued by the dominant kernel
-                 (aead_wave_kernel) against the lane-op peak, with the survey's op model beside it
+                 (aead_wave_kernel) against the lane-op peak, with an op-equivalent model beside it
   roofline_hbm   the same launches as algorithmic bytes against the HBM peak
   cpu_baseline   the CPU oracle timed on this box's host cores (bounded sample)
   cpu_baseline_openssl  the same sample through OpenSSL's assembly, when libcrypto is there
@@ -866,7 +866,7 @@ def main() -> int:
             "traffic": TRAFFIC_BYTES_PER_LAUNCH if counters_apply else None,
             "traffic_source": "profiles/aead_wave_kernel_cfg2.md (FETCH_SIZE and WRITE_SIZE under "
                               "rocprofv3 --pmc, scaled by copy_kernel; not re-measured in this run)",
-            # the survey's op model beside it: it prices a 64-bit multiply-add at 4 and
+            # an op-equivalent model beside it (976 per ChaCha20 block + 16 per data block, 142 per Poly1305 block + 40): it prices a 64-bit multiply-add at 4 and
             # assumes 25 of them per Poly1305 block (radix 2^26), the kernel issues 20
             # (radix 2^32), so this ratio is not bounded by 1 and is no roofline fraction
             "op_equivalent_model": {

@@ -106,7 +106,7 @@ def test_aead_rfc_2_8_2():
 def test_aead_zero_key_empty_is_keepalive_tag():
     # empty plaintext, empty AAD: Poly1305 over the single length block of
     # zeros -- the body of a WireGuard keepalive under an all-zero key.  The
-    # value is what OpenSSL (via node) produced when the survey was written;
+    # value is what OpenSSL (via node) produced when this vector was first recorded;
     # the big-integer transcription must agree.
     want = H("4eb972c9a8fb3a1b382bb4d36f5ffad1")
     assert rfc.aead_seal(bytes(32), bytes(12), b"") == want

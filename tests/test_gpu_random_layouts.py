@@ -1,0 +1,83 @@
+"""Large device-resident batches with seeded random lengths, alignments and
+peers: sealed arenas equal the oracle's byte for byte (bytes between packets
+included), forged tags are rejected and their plaintext left as zeros, every
+other packet opens to what was sealed.  Each seed picks a length mix (uniform
+random up to 1500, the IMIX sizes, short packets only, or block and line
+boundaries with a 4100-byte packet among them) and a layout (slots at 1-, 4-,
+16- or 128-byte alignment), so the aligned, short, unaligned and generic
+paths of the lane-per-packet kernels all see ragged input."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_lengths_and_alignments_match_the_oracle(seed):
+    import torch
+    from bnk_amd import lib
+    from oracle import binding as O
+    rng = np.random.default_rng(1000 + seed)
+    dev = torch.device("cuda:0")
+    n_peers = 33
+    keys = rng.integers(0, 256, (n_peers, 32), dtype=np.uint8)
+    n = int(rng.choice([30000, 70000]))
+    kind = seed % 4
+    if kind == 0:
+        lens = rng.integers(0, 1501, n)
+    elif kind == 1:
+        lens = rng.choice([60, 576, 1420], n, p=[7 / 12, 4 / 12, 1 / 12])
+    elif kind == 2:
+        lens = rng.integers(0, 130, n)
+    else:
+        lens = rng.choice([0, 1, 15, 16, 17, 63, 64, 65, 127, 128, 129, 1419, 1420, 4100], n)
+    lens = lens.astype(np.uint32)
+    align = [1, 4, 16, 128][(seed // 4 + seed) % 4]
+    if align == 1:
+        gap = rng.integers(0, 16, n)
+    elif align == 4:
+        gap = rng.integers(0, 4, n) * 4
+    else:
+        gap = np.zeros(n, np.int64)
+    unit = 128 if align == 128 else 16
+    room = ((lens.astype(np.int64) + 16 + unit - 1) // unit) * unit + (16 if align < 16 else 0)
+    off = (np.concatenate([[0], np.cumsum(room)[:-1]]) + gap).astype(np.uint64)
+    total = int(room.sum()) + 32
+    plain = rng.integers(0, 256, total, dtype=np.uint8)
+    peer = rng.integers(0, n_peers, n).astype(np.uint32)
+    ctrs = rng.integers(0, 1 << 63, n, dtype=np.uint64)
+    want = np.full(total, 0x5A, np.uint8)
+    O.seal_batch(keys, peer, ctrs, plain, off, lens, want, off, 8)
+    d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)  # noqa: E731
+    d_plain = d(plain)
+    d_sealed = torch.full((total,), 0x5A, dtype=torch.uint8, device=dev)
+    d_off, d_len, d_ctl = d(off.astype(np.int64)), d(lens.astype(np.int32)), d((lens + 16).astype(np.int32))
+    d_peer, d_ctr = d(peer.astype(np.int32)), d(ctrs.astype(np.int64))
+    with lib.Context(0) as ctx:
+        ctx.keys_set(lib.KEYS_SEND, keys)
+        ctx.keys_set(lib.KEYS_RECV, keys)
+        ctx.seal(lib.make_batch(d_plain, total, n, lib.MEM_DEVICE, offsets=d_off, lens=d_len, peer=d_peer,
+                                counters=d_ctr),
+                 lib.make_batch(d_sealed, total, n, lib.MEM_DEVICE, offsets=d_off))
+        ctx.sync()
+        got = d_sealed.cpu().numpy()
+        bad = np.flatnonzero(got != want)
+        assert bad.size == 0, f"kind {kind} align {align}: first differing byte at {bad[:4]}"
+        forged = rng.permutation(n)[:40]
+        pos = off[forged].astype(np.int64) + lens[forged].astype(np.int64) + 3
+        d_sealed[d(pos)] ^= 0x40
+        d_back = torch.full((total,), 0xA5, dtype=torch.uint8, device=dev)
+        d_v = torch.full((n,), 9, dtype=torch.uint8, device=dev)
+        ctx.open(lib.make_batch(d_sealed, total, n, lib.MEM_DEVICE, offsets=d_off, lens=d_ctl, peer=d_peer,
+                                counters=d_ctr),
+                 lib.make_batch(d_back, total, n, lib.MEM_DEVICE, offsets=d_off), d_v)
+        ctx.sync()
+    exp_v = np.ones(n, np.uint8)
+    exp_v[forged] = 0
+    assert np.array_equal(d_v.cpu().numpy(), exp_v)
+    expect = np.full(total, 0xA5, np.uint8)
+    length, at = lens.astype(np.int64), off.astype(np.int64)
+    for k in range(int(length.max())):
+        sel = length > k
+        expect[at[sel] + k] = np.where(exp_v[sel] == 1, plain[at[sel] + k], 0)
+    assert np.array_equal(d_back.cpu().numpy(), expect)

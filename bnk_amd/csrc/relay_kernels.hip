@@ -37,8 +37,11 @@ __global__ __launch_bounds__(256) void relay_verdict_kernel(
     }
     verdict[i] = v;
     keys[i] = key;
-    idx[i] = i;
-    ctr_out[i] = 0;
+    // (the counting kernels need no positions and write every packet's counter themselves)
+    if (idx) {
+        idx[i] = i;
+        ctr_out[i] = 0;
+    }
 }
 
 // Where each peer's run starts in the sorted sequence.
@@ -138,6 +141,10 @@ __global__ void peer_rank_small_kernel(const uint32_t *peer, uint32_t n_keys, ui
                                        uint64_t *ctr_out, int advance, int no_peer_ok, unsigned bits,
                                        uint64_t ctr_limit, uint32_t *status);
 
+static hipError_t launch_peer_rank_table(const uint32_t *keys, const RankPlan &plan, void *tmp,
+                                         uint64_t *ctr_base, uint32_t n_keys, uint32_t n, uint64_t *ctr_out,
+                                         bool advance, uint64_t ctr_limit, bool zero_others, hipStream_t s);
+
 hipError_t launch_relay_assign(const uint8_t *auth, const uint8_t *pass, const uint32_t *peer_out,
                                const uint64_t *ctr_base_out, uint32_t n_peers_out, uint32_t n,
                                uint32_t *keys, uint32_t *idx, uint32_t *skeys, uint32_t *sidx,
@@ -146,8 +153,10 @@ hipError_t launch_relay_assign(const uint8_t *auth, const uint8_t *pass, const u
 {
     if (n == 0) return hipSuccess;
     const dim3 grid((n + 255u) / 256u);
+    const RankPlan plan = rank_plan(n, n_peers_out);
+    const bool counting = n > PEER_RANK_SMALL_MAX && plan.fits && plan.bytes <= sort_tmp_bytes;
     hipLaunchKernelGGL(relay_verdict_kernel, grid, dim3(256), 0, s, auth, pass, peer_out, n_peers_out,
-                       n, keys, idx, verdict, ctr_out, status);
+                       n, keys, counting ? (uint32_t *)nullptr : idx, verdict, ctr_out, status);
     if (n <= PEER_RANK_SMALL_MAX) {
         // keys[] is the peer of each survivor and all ones for the rest
         hipLaunchKernelGGL(peer_rank_small_kernel, dim3(1), dim3(PEER_RANK_SMALL_MAX), 0, s, keys, n_peers_out,
@@ -155,6 +164,9 @@ hipError_t launch_relay_assign(const uint8_t *auth, const uint8_t *pass, const u
                            key_bits(n_peers_out), 0ull, status);
         return hipGetLastError();
     }
+    if (counting)
+        return launch_peer_rank_table(keys, plan, sort_tmp, const_cast<uint64_t *>(ctr_base_out), n_peers_out, n,
+                                      ctr_out, advance, 0ull, true, s);
     return launch_peer_rank(keys, idx, skeys, sidx, sort_tmp, sort_tmp_bytes,
                             const_cast<uint64_t *>(ctr_base_out), n_peers_out, n, ctr_out, advance, 0ull, s);
 }
@@ -303,7 +315,7 @@ __global__ __launch_bounds__(64) void rank_assign_kernel(const uint32_t *keys, u
                                                          uint32_t cols, uint32_t runs, const uint32_t *table,
                                                          unsigned bits,
                                                          const uint64_t *ctr_base, uint64_t *ctr_out,
-                                                         uint64_t ctr_limit)
+                                                         uint64_t ctr_limit, int zero_others)
 {
     // packets of each peer ahead of the run at hand
     __shared__ __attribute__((aligned(16))) uint32_t before[RANK_TABLE_MAX_KEYS];
@@ -350,6 +362,8 @@ __global__ __launch_bounds__(64) void rank_assign_kernel(const uint32_t *keys, u
             // every lane has read the entry before any lane writes one: the lanes of a
             // wave run in lockstep and LDS serves their accesses in order
             if (lower == 0u) before[kk] += (uint32_t)__popcll(same);
+        } else if (zero_others && first + r * 64u + lane < n) {
+            ctr_out[first + r * 64u + lane] = 0; // a packet without a peer gets no counter
         }
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -366,7 +380,7 @@ __global__ __launch_bounds__(256) void rank_advance_kernel(const uint32_t *total
 
 static hipError_t launch_peer_rank_table(const uint32_t *keys, const RankPlan &plan, void *tmp,
                                          uint64_t *ctr_base, uint32_t n_keys, uint32_t n, uint64_t *ctr_out,
-                                         bool advance, uint64_t ctr_limit, hipStream_t s)
+                                         bool advance, uint64_t ctr_limit, bool zero_others, hipStream_t s)
 {
     uint32_t *table = static_cast<uint32_t *>(tmp);
     uint32_t *total = table + (size_t)plan.tiles * plan.cols;
@@ -375,7 +389,7 @@ static hipError_t launch_peer_rank_table(const uint32_t *keys, const RankPlan &p
     hipLaunchKernelGGL(rank_scan_kernel, dim3((n_keys + SCAN_PEERS - 1u) / SCAN_PEERS),
                        dim3(SCAN_PEERS * SCAN_PARTS), 0, s, table, plan.tiles, n_keys, plan.cols, total);
     hipLaunchKernelGGL(rank_assign_kernel, dim3(plan.tiles), dim3(64), 0, s, keys, n, n_keys, plan.cols, plan.runs,
-                       table, key_bits(n_keys), ctr_base, ctr_out, ctr_limit);
+                       table, key_bits(n_keys), ctr_base, ctr_out, ctr_limit, zero_others ? 1 : 0);
     if (advance)
         hipLaunchKernelGGL(rank_advance_kernel, dim3((n_keys + 255u) / 256u), dim3(256), 0, s, total, n_keys,
                            ctr_base, ctr_limit);
@@ -389,7 +403,8 @@ hipError_t launch_peer_rank(uint32_t *keys, uint32_t *idx, uint32_t *skeys, uint
     if (n == 0) return hipSuccess;
     const RankPlan plan = rank_plan(n, n_keys);
     if (plan.fits && plan.bytes <= sort_tmp_bytes)
-        return launch_peer_rank_table(keys, plan, sort_tmp, ctr_base, n_keys, n, ctr_out, advance, ctr_limit, s);
+        return launch_peer_rank_table(keys, plan, sort_tmp, ctr_base, n_keys, n, ctr_out, advance, ctr_limit, false,
+                                      s);
     const dim3 grid((n + 255u) / 256u);
     hipError_t e = rocprim::radix_sort_pairs<SortConfig>(sort_tmp, sort_tmp_bytes, keys, skeys, idx, sidx, (size_t)n,
                                              0, key_bits(n_keys), s);

@@ -116,35 +116,186 @@ __global__ __launch_bounds__(256) void replay_keys_packed_kernel(const uint8_t *
     packed[i] = wg_replay_pack((replay_subject(result[i]) && p < n_peers) ? p : NO_PEER, i, index_bits);
 }
 
-// Sender, position and counter of the packets in sorted order, from the sorted words.
-__global__ __launch_bounds__(256) void replay_unpack_kernel(const uint32_t *sorted, const uint64_t *counter,
-                                                            uint32_t n, unsigned index_bits, unsigned peer_bits,
-                                                            uint32_t *skeys, uint32_t *sidx, uint64_t *sctr,
-                                                            uint64_t *sval)
+// ---------------------------------------------------------------------------
+// Running maximum per peer in sorted order: pmax[p] = the largest sval of the
+// earlier positions with p's key, 0 when there is none.  A segmented exclusive
+// max-scan, the segments being the peers' runs.  Three steps: every block of
+// SEG_BLOCK positions reduces to what it hands on (seg_carry_kernel), one block
+// scans those (seg_carry_scan_kernel), and every block scans itself again with
+// what it was handed (inside replay_classify_kernel, which needs the values).
+// ---------------------------------------------------------------------------
+constexpr uint32_t SEG_BLOCK = 1024;
+
+__device__ __forceinline__ uint64_t shfl_up64(uint64_t v, unsigned off)
 {
-    const uint32_t p = blockIdx.x * 256u + threadIdx.x;
-    if (p >= n) return;
-    const uint32_t w = sorted[p];
-    const uint32_t none = (1u << peer_bits) - 1u, field = (w >> index_bits) & none;
-    const uint32_t i = w & ((1u << index_bits) - 1u);
-    const uint64_t c = field != none ? counter[i] : 0;
-    skeys[p] = field != none ? field : NO_PEER;
-    sidx[p] = i;
-    sctr[p] = c;
-    sval[p] = c < WG_REJECT_AFTER_MESSAGES ? c : 0;
+    const uint32_t lo = (uint32_t)__shfl_up((int)(uint32_t)v, off, 64);
+    const uint32_t hi = (uint32_t)__shfl_up((int)(uint32_t)(v >> 32), off, 64);
+    return (uint64_t)hi << 32 | lo;
 }
 
-// Counters in sorted order; a counter the filter turns away outright counts as
-// 0 for the running maximum (it never moves last).
-__global__ __launch_bounds__(256) void replay_gather_kernel(const uint32_t *skeys, const uint32_t *sidx,
-                                                            const uint64_t *counter, uint32_t n,
-                                                            uint64_t *sctr, uint64_t *sval)
+struct SegScan {
+    uint64_t excl;    // maximum over my run's earlier positions within the block
+    bool open;        // my run began before the block (and I am not its head)
+    uint64_t prev;    // what the position before me ends with (0 for the block's first)
+    uint64_t total;   // the block's last run, maximum over its positions in the block
+    bool total_open;  // the block holds no head at all
+};
+
+// For a block of SEG_BLOCK threads in position order; head: my key differs from
+// the position before me.
+__device__ __forceinline__ SegScan seg_block_scan(uint64_t v, bool head)
 {
-    const uint32_t p = blockIdx.x * 256u + threadIdx.x;
-    if (p >= n) return;
-    const uint64_t c = skeys[p] != NO_PEER ? counter[sidx[p]] : 0;
-    sctr[p] = c;
-    sval[p] = c < WG_REJECT_AFTER_MESSAGES ? c : 0;
+    __shared__ uint64_t wave_x[SEG_BLOCK / 64];
+    __shared__ uint32_t wave_f[SEG_BLOCK / 64];
+    const uint32_t lane = threadIdx.x & 63u, wv = threadIdx.x >> 6;
+    // inclusive within the wave: x = maximum back to my run's head or the wave's
+    // first lane, f = a head lies in that span
+    uint64_t x = v;
+    uint32_t f = head ? 1u : 0u;
+#pragma unroll
+    for (unsigned off = 1; off < 64; off <<= 1) {
+        const uint64_t xo = shfl_up64(x, off);
+        const uint32_t fo = (uint32_t)__shfl_up((int)f, off, 64);
+        if (lane >= off && !f) {
+            x = xo > x ? xo : x;
+            f = fo;
+        }
+    }
+    if (lane == 63u) {
+        wave_x[wv] = x;
+        wave_f[wv] = f;
+    }
+    __syncthreads();
+    // the same over the waves' last lanes, by the first wave
+    if (wv == 0) {
+        uint64_t ax = lane < SEG_BLOCK / 64 ? wave_x[lane] : 0;
+        uint32_t af = lane < SEG_BLOCK / 64 ? wave_f[lane] : 1u;
+#pragma unroll
+        for (unsigned off = 1; off < SEG_BLOCK / 64; off <<= 1) {
+            const uint64_t xo = shfl_up64(ax, off);
+            const uint32_t fo = (uint32_t)__shfl_up((int)af, off, 64);
+            if (lane >= off && !af) {
+                ax = xo > ax ? xo : ax;
+                af = fo;
+            }
+        }
+        if (lane < SEG_BLOCK / 64) {
+            wave_x[lane] = ax;
+            wave_f[lane] = af;
+        }
+    }
+    __syncthreads();
+    const uint64_t before_x = wv ? wave_x[wv - 1] : 0; // up to the last lane of the wave before mine
+    const uint32_t before_f = wv ? wave_f[wv - 1] : 0u;
+    if (!f) {
+        x = before_x > x ? before_x : x;
+        f = before_f;
+    }
+    // exclusive: what the position before me holds
+    uint64_t px = shfl_up64(x, 1);
+    uint32_t pf = (uint32_t)__shfl_up((int)f, 1, 64);
+    if (lane == 0) {
+        px = before_x;
+        pf = before_f;
+    }
+    SegScan r;
+    r.excl = head ? 0 : px;
+    r.open = !head && !pf;
+    r.prev = px;
+    r.total = wave_x[SEG_BLOCK / 64 - 1];
+    r.total_open = wave_f[SEG_BLOCK / 64 - 1] == 0u;
+    return r;
+}
+
+__device__ __forceinline__ bool seg_head(const uint32_t *skeys, uint32_t p, uint32_t n, uint32_t key)
+{
+    return p >= n || p == 0u || skeys[p - 1u] != key;
+}
+
+// Sender, position and counter of the packets in sorted order, from the sorted
+// words, and what each block of positions hands on to the running maximum
+// (carry_x, carry_open: see seg_carry_scan_kernel).
+__global__ __launch_bounds__(SEG_BLOCK) void replay_unpack_kernel(const uint32_t *sorted, const uint64_t *counter,
+                                                                  uint32_t n, unsigned index_bits, unsigned peer_bits,
+                                                                  uint32_t *skeys, uint32_t *sidx, uint64_t *sctr,
+                                                                  uint64_t *sval, uint64_t *carry_x,
+                                                                  uint32_t *carry_open)
+{
+    const uint32_t p = blockIdx.x * SEG_BLOCK + threadIdx.x;
+    const uint32_t none = (1u << peer_bits) - 1u;
+    uint32_t field = none, before = none;
+    uint64_t v = 0;
+    if (p < n) {
+        const uint32_t w = sorted[p];
+        field = (w >> index_bits) & none;
+        if (p) before = (sorted[p - 1u] >> index_bits) & none;
+        const uint32_t i = w & ((1u << index_bits) - 1u);
+        const uint64_t c = field != none ? counter[i] : 0;
+        v = c < WG_REJECT_AFTER_MESSAGES ? c : 0;
+        skeys[p] = field != none ? field : NO_PEER;
+        sidx[p] = i;
+        sctr[p] = c;
+        sval[p] = v;
+    }
+    const SegScan r = seg_block_scan(v, p >= n || p == 0u || before != field);
+    if (threadIdx.x == 0) {
+        carry_x[blockIdx.x] = r.total;
+        carry_open[blockIdx.x] = r.total_open ? 1u : 0u;
+    }
+}
+
+// Counters in sorted order (a counter the filter turns away outright counts as
+// 0 for the running maximum: it never moves last), and the blocks' carries.
+__global__ __launch_bounds__(SEG_BLOCK) void replay_gather_kernel(const uint32_t *skeys, const uint32_t *sidx,
+                                                                  const uint64_t *counter, uint32_t n,
+                                                                  uint64_t *sctr, uint64_t *sval, uint64_t *carry_x,
+                                                                  uint32_t *carry_open)
+{
+    const uint32_t p = blockIdx.x * SEG_BLOCK + threadIdx.x;
+    const uint32_t key = p < n ? skeys[p] : NO_PEER;
+    uint64_t v = 0;
+    if (p < n) {
+        const uint64_t c = key != NO_PEER ? counter[sidx[p]] : 0;
+        v = c < WG_REJECT_AFTER_MESSAGES ? c : 0;
+        sctr[p] = c;
+        sval[p] = v;
+    }
+    const SegScan r = seg_block_scan(v, seg_head(skeys, p, n, key));
+    if (threadIdx.x == 0) {
+        carry_x[blockIdx.x] = r.total;
+        carry_open[blockIdx.x] = r.total_open ? 1u : 0u;
+    }
+}
+
+// carry_x[b] becomes what block b is handed: the maximum of the run that runs
+// into it, over the blocks before it.  One block; each thread takes a stretch
+// of consecutive blocks.
+__global__ __launch_bounds__(SEG_BLOCK) void seg_carry_scan_kernel(uint64_t *carry_x, const uint32_t *carry_open,
+                                                                   uint32_t blocks)
+{
+    const uint32_t per = (blocks + SEG_BLOCK - 1u) / SEG_BLOCK;
+    const uint32_t lo = min(threadIdx.x * per, blocks), hi = min(lo + per, blocks);
+    // my stretch as one element: its value, and whether no head lies in it
+    uint64_t x = 0;
+    bool open = true;
+    for (uint32_t b = lo; b < hi; b++) {
+        const uint64_t v = carry_x[b];
+        if (carry_open[b]) x = v > x ? v : x;
+        else {
+            x = v;
+            open = false;
+        }
+    }
+    const SegScan r = seg_block_scan(x, !open);
+    // my first block is handed what the stretch before mine ends with (a head inside
+    // my stretch cuts off what follows it, not the blocks before it)
+    uint64_t run = r.prev;
+    for (uint32_t b = lo; b < hi; b++) {
+        const uint64_t v = carry_x[b];
+        const bool o = carry_open[b] != 0u;
+        carry_x[b] = run;
+        run = o ? (v > run ? v : run) : v;
+    }
 }
 
 // What the window decides about a packet without looking at other packets'
@@ -161,20 +312,29 @@ __device__ __forceinline__ uint32_t table_home(uint32_t key, uint64_t c, uint32_
 // Classifies every packet; turns away what never reaches the bit test; enters
 // the late ones into the table (slot = earliest sorted position carrying that
 // peer and counter) and raises flags[0] when there are any.
-__global__ __launch_bounds__(256) void replay_classify_kernel(const uint32_t *skeys, const uint32_t *sidx,
-                                                              const uint64_t *sctr, const uint64_t *pmax,
-                                                              const uint64_t *state, uint32_t n, uint8_t *cls,
-                                                              uint32_t *table, uint32_t mask, uint32_t *flags,
-                                                              uint8_t *result, uint32_t *out_len)
+__global__ __launch_bounds__(SEG_BLOCK) void replay_classify_kernel(const uint32_t *skeys, const uint32_t *sidx,
+                                                                    const uint64_t *sctr, const uint64_t *sval,
+                                                                    const uint64_t *carry, uint64_t *pmax,
+                                                                    const uint64_t *state, uint32_t n, uint8_t *cls,
+                                                                    uint32_t *table, uint32_t mask, uint32_t *flags,
+                                                                    uint8_t *result, uint32_t *out_len)
 {
-    const uint32_t p = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t p = blockIdx.x * SEG_BLOCK + threadIdx.x;
+    const uint32_t key = p < n ? skeys[p] : NO_PEER;
+    // the running maximum of my peer's earlier counters (every thread of the block takes part)
+    const SegScan seg = seg_block_scan(p < n ? sval[p] : 0, seg_head(skeys, p, n, key));
     if (p >= n) return;
-    const uint32_t key = skeys[p];
+    uint64_t before = seg.excl;
+    if (seg.open) {
+        const uint64_t handed = carry[blockIdx.x];
+        before = handed > before ? handed : before;
+    }
+    pmax[p] = before;
     uint8_t k = RP_NONE;
     if (key != NO_PEER) {
         const uint64_t c = sctr[p];
         const uint64_t last0 = state[(size_t)key * WG_REPLAY_WORDS];
-        const uint64_t last = last0 > pmax[p] ? last0 : pmax[p];
+        const uint64_t last = last0 > before ? last0 : before;
         if (reaches_bit_test(c, last)) k = c > last ? RP_AHEAD : RP_LATE;
         if (k == RP_NONE) {
             const uint32_t i = sidx[p];
@@ -452,9 +612,7 @@ size_t wg_replay_tmp_bytes(uint32_t n, uint32_t n_peers)
     (void)rocprim::radix_sort_pairs<SortConfig>(nullptr, a, (const uint32_t *)nullptr, (uint32_t *)nullptr,
                                                 (const uint32_t *)nullptr, (uint32_t *)nullptr, (size_t)n, 0,
                                                 key_bits(n_peers));
-    (void)rocprim::exclusive_scan_by_key(nullptr, b, (const uint32_t *)nullptr, (const uint64_t *)nullptr,
-                                         (uint64_t *)nullptr, (uint64_t)0, (size_t)n,
-                                         rocprim::maximum<uint64_t>(), rocprim::equal_to<uint32_t>());
+    b = ((size_t)(n + SEG_BLOCK - 1u) / SEG_BLOCK) * 12u + 16u; // the scan's block carries
     return std::max(std::max(a, b), c);
 }
 
@@ -494,6 +652,10 @@ hipError_t launch_wg_replay(uint8_t *result, uint32_t *out_len, const uint32_t *
     size_t bytes = sc.tmp_bytes;
     hipError_t e = hipSuccess;
     const unsigned peer_bits = key_bits(rp.n_peers);
+    // (what the blocks hand on to the running maximum goes into the sort's scratch, free by then)
+    const uint32_t seg_blocks = (n + SEG_BLOCK - 1u) / SEG_BLOCK;
+    uint64_t *carry_x = static_cast<uint64_t *>(sc.tmp);
+    uint32_t *carry_open = reinterpret_cast<uint32_t *>(carry_x + seg_blocks);
     if (const unsigned index_bits = wg_replay_index_bits(n, rp.n_peers)) {
         // one word per packet: keys[] in, idx[] out
         if (!sc.keys_ready)
@@ -502,8 +664,8 @@ hipError_t launch_wg_replay(uint8_t *result, uint32_t *out_len, const uint32_t *
         e = rocprim::radix_sort_keys<SortConfig>(sc.tmp, bytes, sc.keys, sc.idx, (size_t)n, index_bits,
                                                  index_bits + peer_bits, s);
         if (e != hipSuccess) return e;
-        hipLaunchKernelGGL(replay_unpack_kernel, grid, dim3(256), 0, s, sc.idx, counter, n, index_bits, peer_bits,
-                           sc.skeys, sc.sidx, sc.sctr, sc.sval);
+        hipLaunchKernelGGL(replay_unpack_kernel, dim3(seg_blocks), dim3(SEG_BLOCK), 0, s, sc.idx, counter, n,
+                           index_bits, peer_bits, sc.skeys, sc.sidx, sc.sctr, sc.sval, carry_x, carry_open);
     } else {
         if (!sc.keys_ready)
             hipLaunchKernelGGL(replay_keys_kernel, grid, dim3(256), 0, s, result, peer, rp.n_peers, n, sc.keys,
@@ -511,17 +673,16 @@ hipError_t launch_wg_replay(uint8_t *result, uint32_t *out_len, const uint32_t *
         e = rocprim::radix_sort_pairs<SortConfig>(sc.tmp, bytes, sc.keys, sc.skeys, sc.idx, sc.sidx, (size_t)n, 0,
                                                   peer_bits, s);
         if (e != hipSuccess) return e;
-        hipLaunchKernelGGL(replay_gather_kernel, grid, dim3(256), 0, s, sc.skeys, sc.sidx, counter, n, sc.sctr,
-                           sc.sval);
+        hipLaunchKernelGGL(replay_gather_kernel, dim3(seg_blocks), dim3(SEG_BLOCK), 0, s, sc.skeys, sc.sidx, counter,
+                           n, sc.sctr, sc.sval, carry_x, carry_open);
     }
-    bytes = sc.tmp_bytes;
-    e = rocprim::exclusive_scan_by_key(sc.tmp, bytes, sc.skeys, sc.sval, sc.pmax, (uint64_t)0, (size_t)n,
-                                       rocprim::maximum<uint64_t>(), rocprim::equal_to<uint32_t>(), s);
-    if (e != hipSuccess) return e;
+    // the running maximum per peer: the scan of the blocks' carries, and the rest inside the
+    // classifying launch
+    hipLaunchKernelGGL(seg_carry_scan_kernel, dim3(1), dim3(SEG_BLOCK), 0, s, carry_x, carry_open, seg_blocks);
     const uint32_t mask = sc.table_slots - 1u;
     uint32_t *late_flag = sc.flags + sc.parity;
-    hipLaunchKernelGGL(replay_classify_kernel, grid, dim3(256), 0, s, sc.skeys, sc.sidx, sc.sctr, sc.pmax,
-                       rp.state, n, sc.cls, sc.table, mask, late_flag, result, out_len);
+    hipLaunchKernelGGL(replay_classify_kernel, dim3(seg_blocks), dim3(SEG_BLOCK), 0, s, sc.skeys, sc.sidx, sc.sctr,
+                       sc.sval, carry_x, sc.pmax, rp.state, n, sc.cls, sc.table, mask, late_flag, result, out_len);
     hipLaunchKernelGGL(replay_claim_kernel, grid, dim3(256), 0, s, sc.skeys, sc.sctr, sc.cls, n, sc.table, mask,
                        late_flag);
     hipLaunchKernelGGL(replay_late_kernel, grid, dim3(256), 0, s, sc.skeys, sc.sidx, sc.sctr, sc.cls, rp.state, n,

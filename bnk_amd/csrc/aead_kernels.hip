@@ -160,6 +160,18 @@ constexpr uint32_t WAVES_PER_BLOCK = 4;
 constexpr uint32_t SHORT_BLOCKS = 2;
 constexpr uint32_t SHORT_ROW = 144;          // 8 cells + 16 pad
 
+// v: the cell's 16 bytes, read from `cell` beforehand (before the keystream block was
+// computed, so that the LDS read is not waited for)
+template <bool OPEN>
+BNK_DEV void crypt_cell_v(Poly32 &mac, const uint32_t (&x)[16], int j, const uint4 v, uint8_t *cell)
+{
+    const uint4 o = make_uint4(v.x ^ x[4 * j], v.y ^ x[4 * j + 1], v.z ^ x[4 * j + 2],
+                               v.w ^ x[4 * j + 3]);
+    if (OPEN) mac.block(v.x, v.y, v.z, v.w);
+    else mac.block(o.x, o.y, o.z, o.w);
+    *reinterpret_cast<uint4 *>(cell) = o;
+}
+
 template <bool OPEN>
 BNK_DEV void crypt_cell(Poly32 &mac, const uint32_t (&x)[16], int j, uint8_t *cell)
 {
@@ -377,12 +389,17 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
 #define BNK_ISSUE_ALL(q, m) pre##q = BNK_LD(csrc[q] + 128u * (m))
 #define BNK_COMMIT(q, m) if (BNK_INSIDE_LD(q, m)) *BNK_SLOT(q, m) = pre##q
 #define BNK_COMMIT_ALL(q, m) *BNK_SLOT(q, m) = pre##q
-#define BNK_STORE(q, m)                                                                     \
-    do {                                                                                    \
-        const uint4 out_##q = *BNK_SLOT(q, m); /* read first, unconditionally: same reason */ \
-        if (BNK_INSIDE(q, m)) BNK_ST(cdst[q] + 128u * (m), out_##q);                         \
-    } while (0)
-#define BNK_STORE_ALL(q, m) BNK_ST(cdst[q] + 128u * (m), *BNK_SLOT(q, m))
+    // A finished line leaves in two parts: out of the ring into registers
+    // (unconditionally, for the same reason), and to memory only after the next
+    // line's loads have been issued.  The wave's memory operations complete in
+    // the order they were issued and one counter covers loads and stores, so a
+    // wait for a line's loads also waits for every store issued after them:
+    // stores issued just before the wait (a finished line, then straight on to
+    // the next line's arrival) cost 24-31 % of a wave's time; issued after the
+    // following loads, the next wait that covers them is a whole step away.
+#define BNK_TAKE(q, m) out##q = *BNK_SLOT(q, m)
+#define BNK_PUT(q, m) if (BNK_INSIDE(q, m)) BNK_ST(cdst[q] + 128u * (m), out##q)
+#define BNK_PUT_ALL(q, m) BNK_ST(cdst[q] + 128u * (m), out##q)
 #define BNK_EIGHT(OP, m)                                                                    \
     do {                                                                                    \
         OP(0, m); OP(1, m); OP(2, m); OP(3, m); OP(4, m); OP(5, m); OP(6, m); OP(7, m);     \
@@ -394,7 +411,7 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
     } while (0)
 #define BNK_ISSUE_LINE(m) BNK_LINE(BNK_ISSUE, m)
 #define BNK_COMMIT_LINE(m) BNK_LINE(BNK_COMMIT, m)
-    auto store_line = [&](uint32_t m) __attribute__((always_inline)) { BNK_LINE(BNK_STORE, m); };
+    uint4 out0 = pre0, out1 = pre0, out2 = pre0, out3 = pre0, out4 = pre0, out5 = pre0, out6 = pre0, out7 = pre0;
 
     uint8_t *row = tile + lane * RING_ROW;
     BNK_ISSUE_LINE(0u);
@@ -403,22 +420,35 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
     mac.init(x);
     BNK_COMMIT_LINE(0u);
     BNK_ISSUE_LINE(1u);
-    // iteration s: line s+1 enters the ring, line s+2 starts flying, packet
-    // bytes [128s, 128s+128) are processed, line s is written back; the extra
-    // last iteration only writes back the final line
-    for (uint32_t s = 0; s <= maxsteps; s++) {
+    // iteration s: line s-1 (complete since the step before) leaves the ring,
+    // line s+1 enters it, line s+2 starts flying, line s-1 goes to memory,
+    // packet bytes [128s, 128s+128) are processed; the extra last iteration
+    // only writes back the final line
+    for (uint32_t s = 0; s <= maxsteps + 1; s++) {
+        if (s >= 1) BNK_EIGHT(BNK_TAKE, s - 1);
+        wave_sync();
         BNK_COMMIT_LINE(s + 1);
         if (s + 2 <= maxsteps) BNK_ISSUE_LINE(s + 2);
+        if (s >= 1) {
+            if (s - 1 >= m_lo && s - 1 < m_hi) BNK_EIGHT(BNK_PUT_ALL, s - 1);
+            else BNK_EIGHT(BNK_PUT, s - 1);
+        }
         wave_sync();
         if (s < steps) {
             if (8u * s + 8u <= ncell_in) {
                 // all eight cells of this step are whole cells of the packet
 #pragma unroll 1
                 for (uint32_t h = 0; h < 2; h++) {
-                    chacha_block(k, 2u * s + h + 1, n1, n2, x);
                     const uint32_t r0 = c0 + 8u * s + 4u * h;
-#pragma unroll
-                    for (int j = 0; j < 4; j++) crypt_cell<OPEN>(mac, x, j, row + (((r0 + j) & 15u) << 4));
+                    uint8_t *const cell0 = row + ((r0 & 15u) << 4), *const cell1 = row + (((r0 + 1u) & 15u) << 4);
+                    uint8_t *const cell2 = row + (((r0 + 2u) & 15u) << 4), *const cell3 = row + (((r0 + 3u) & 15u) << 4);
+                    const uint4 v0 = *reinterpret_cast<const uint4 *>(cell0), v1 = *reinterpret_cast<const uint4 *>(cell1);
+                    const uint4 v2 = *reinterpret_cast<const uint4 *>(cell2), v3 = *reinterpret_cast<const uint4 *>(cell3);
+                    chacha_block(k, 2u * s + h + 1, n1, n2, x);
+                    crypt_cell_v<OPEN>(mac, x, 0, v0, cell0);
+                    crypt_cell_v<OPEN>(mac, x, 1, v1, cell1);
+                    crypt_cell_v<OPEN>(mac, x, 2, v2, cell2);
+                    crypt_cell_v<OPEN>(mac, x, 3, v3, cell3);
                 }
             } else {
 #pragma unroll 1
@@ -447,8 +477,6 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
             if (OPEN && s == 0) capture_head(head, row + (c0 << 4), row + (((c0 + 1u) & 15u) << 4));
         }
         wave_sync();
-        store_line(s);
-        wave_sync();
     }
 #undef BNK_INSIDE
 #undef BNK_LD
@@ -459,8 +487,9 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
 #undef BNK_ISSUE_ALL
 #undef BNK_COMMIT
 #undef BNK_COMMIT_ALL
-#undef BNK_STORE
-#undef BNK_STORE_ALL
+#undef BNK_TAKE
+#undef BNK_PUT
+#undef BNK_PUT_ALL
 #undef BNK_EIGHT
 #undef BNK_LINE
 #undef BNK_ISSUE_LINE

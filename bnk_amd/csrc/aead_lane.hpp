@@ -25,12 +25,53 @@ namespace bnk {
 BNK_DEV uint32_t rotl32(uint32_t v, int c) { return v << c | v >> (32 - c); }
 // low 32 bits of (hi:lo) >> s, 0 < s < 32 (one v_alignbit_b32 on the GPU)
 BNK_DEV uint32_t funnel(uint32_t hi, uint32_t lo, int s) { return lo >> s | hi << (32 - s); }
+// a + b + cin (cin 0 or 1) as 32 bits and a carry
+BNK_DEV uint32_t addc32(uint32_t a, uint32_t b, uint32_t cin, uint32_t &cout)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    unsigned int co;
+    const uint32_t r = __builtin_addc(a, b, cin, &co);
+    cout = co;
+    return r;
+#else
+    const uint64_t t = (uint64_t)a + b + cin;
+    cout = (uint32_t)(t >> 32);
+    return (uint32_t)t;
+#endif
+}
 
+#if defined(__HIP_DEVICE_COMPILE__)
+// Four quarter rounds side by side.  A SIMD issues adds and xors of two waves
+// together but rotates (v_alignbit_b32) of one wave at a time, and serves its
+// older wave first: the younger wave's rotates then wait about four of the
+// older wave's issue slots each.  The four rotates of a step therefore run at
+// raised wave priority, so that whichever wave is rotating owns the SIMD and the
+// other fills in with its adds and xors (measured on the bare quarter-round
+// stream at two waves per SIMD: 41.9 -> 50.1 T lane-instructions/s).
+#define BNK_ROT4(n, a, b, c, d)                                                        \
+    asm volatile("s_setprio 1\n\t"                                                     \
+                 "v_alignbit_b32 %0, %0, %0, " #n "\n\tv_alignbit_b32 %1, %1, %1, " #n "\n\t" \
+                 "v_alignbit_b32 %2, %2, %2, " #n "\n\tv_alignbit_b32 %3, %3, %3, " #n "\n\t" \
+                 "s_setprio 0"                                                         \
+                 : "+v"(a), "+v"(b), "+v"(c), "+v"(d))
+#define BNK_QR4(a0, b0, c0, d0, a1, b1, c1, d1, a2, b2, c2, d2, a3, b3, c3, d3)       \
+    a0 += b0; a1 += b1; a2 += b2; a3 += b3; d0 ^= a0; d1 ^= a1; d2 ^= a2; d3 ^= a3;    \
+    BNK_ROT4(16, d0, d1, d2, d3);                                                      \
+    c0 += d0; c1 += d1; c2 += d2; c3 += d3; b0 ^= c0; b1 ^= c1; b2 ^= c2; b3 ^= c3;    \
+    BNK_ROT4(20, b0, b1, b2, b3);                                                      \
+    a0 += b0; a1 += b1; a2 += b2; a3 += b3; d0 ^= a0; d1 ^= a1; d2 ^= a2; d3 ^= a3;    \
+    BNK_ROT4(24, d0, d1, d2, d3);                                                      \
+    c0 += d0; c1 += d1; c2 += d2; c3 += d3; b0 ^= c0; b1 ^= c1; b2 ^= c2; b3 ^= c3;    \
+    BNK_ROT4(25, b0, b1, b2, b3)
+#else
 #define BNK_QR(a, b, c, d)                          \
     a += b; d ^= a; d = rotl32(d, 16);              \
     c += d; b ^= c; b = rotl32(b, 12);              \
     a += b; d ^= a; d = rotl32(d, 8);               \
     c += d; b ^= c; b = rotl32(b, 7)
+#define BNK_QR4(a0, b0, c0, d0, a1, b1, c1, d1, a2, b2, c2, d2, a3, b3, c3, d3)       \
+    BNK_QR(a0, b0, c0, d0); BNK_QR(a1, b1, c1, d1); BNK_QR(a2, b2, c2, d2); BNK_QR(a3, b3, c3, d3)
+#endif
 
 // RFC 8439 section 2.3 with the WireGuard nonce: words 13..15 of the state
 // are 0, counter low, counter high.
@@ -43,14 +84,8 @@ BNK_DEV void chacha_block(const uint32_t (&k)[8], uint32_t blk, uint32_t n1,
     x[12] = blk; x[13] = 0; x[14] = n1; x[15] = n2;
 #pragma unroll 1
     for (int r = 0; r < 10; r++) {
-        BNK_QR(x[0], x[4], x[8], x[12]);
-        BNK_QR(x[1], x[5], x[9], x[13]);
-        BNK_QR(x[2], x[6], x[10], x[14]);
-        BNK_QR(x[3], x[7], x[11], x[15]);
-        BNK_QR(x[0], x[5], x[10], x[15]);
-        BNK_QR(x[1], x[6], x[11], x[12]);
-        BNK_QR(x[2], x[7], x[8], x[13]);
-        BNK_QR(x[3], x[4], x[9], x[14]);
+        BNK_QR4(x[0], x[4], x[8], x[12], x[1], x[5], x[9], x[13], x[2], x[6], x[10], x[14], x[3], x[7], x[11], x[15]);
+        BNK_QR4(x[0], x[5], x[10], x[15], x[1], x[6], x[11], x[12], x[2], x[7], x[8], x[13], x[3], x[4], x[9], x[14]);
     }
     x[0] += 0x61707865u; x[1] += 0x3320646eu; x[2] += 0x79622d32u; x[3] += 0x6b206574u;
 #pragma unroll
@@ -168,36 +203,53 @@ struct Poly32 {
     }
 
     // One full 16-byte block (little-endian words w0..w3) with bit 128 set.
+    // Additions go 32 bits at a time with an explicit carry (add-with-carry
+    // instructions on the GPU; written as 64-bit sums the compiler builds each
+    // zero-extended operand with a move first: 68 instructions a block against 47).
+    // The block runs at raised wave priority for the same reason as the rotates of
+    // ChaCha20: nearly all of it is multiplies and carries, which a SIMD takes
+    // from one wave at a time.
     BNK_DEV void block(uint32_t w0, uint32_t w1, uint32_t w2, uint32_t w3)
     {
-        uint64_t t;
-        t = (uint64_t)h0 + w0;             const uint32_t a0 = (uint32_t)t;
-        t = (uint64_t)h1 + w1 + (t >> 32); const uint32_t a1 = (uint32_t)t;
-        t = (uint64_t)h2 + w2 + (t >> 32); const uint32_t a2 = (uint32_t)t;
-        t = (uint64_t)h3 + w3 + (t >> 32); const uint32_t a3 = (uint32_t)t;
-        const uint32_t a4 = h4 + (uint32_t)(t >> 32) + 1u; // at most 9
+#if defined(__HIP_DEVICE_COMPILE__)
+        __builtin_amdgcn_s_setprio(1);
+#endif
+        uint32_t c;
+        const uint32_t a0 = addc32(h0, w0, 0, c);
+        const uint32_t a1 = addc32(h1, w1, c, c);
+        const uint32_t a2 = addc32(h2, w2, c, c);
+        const uint32_t a3 = addc32(h3, w3, c, c);
+        const uint32_t a4 = h4 + 1u + c; // at most 9
 
-        // a_i < 2^32, r_j < 2^28, s_j < 1.25 * 2^28: four terms stay below 2^63
-        uint64_t d0 = (uint64_t)a0 * r0 + (uint64_t)a1 * s3 + (uint64_t)a2 * s2 + (uint64_t)a3 * s1;
-        uint64_t d1 = (uint64_t)a0 * r1 + (uint64_t)a1 * r0 + (uint64_t)a2 * s3 + (uint64_t)a3 * s2 +
-                      (uint64_t)(a4 * s1);
-        uint64_t d2 = (uint64_t)a0 * r2 + (uint64_t)a1 * r1 + (uint64_t)a2 * r0 + (uint64_t)a3 * s3 +
-                      (uint64_t)(a4 * s2);
-        uint64_t d3 = (uint64_t)a0 * r3 + (uint64_t)a1 * r2 + (uint64_t)a2 * r1 + (uint64_t)a3 * r0 +
-                      (uint64_t)(a4 * s3);
+        // a_i < 2^32, r_j < 2^28, s_j < 1.25 * 2^28: four terms stay below 2^63,
+        // and a4 * s_j below 2^32
+        const uint64_t d0 = (uint64_t)a0 * r0 + (uint64_t)a1 * s3 + (uint64_t)a2 * s2 + (uint64_t)a3 * s1;
+        const uint64_t d1 = (uint64_t)a0 * r1 + (uint64_t)a1 * r0 + (uint64_t)a2 * s3 + (uint64_t)a3 * s2 +
+                            (uint64_t)a4 * s1;
+        const uint64_t d2 = (uint64_t)a0 * r2 + (uint64_t)a1 * r1 + (uint64_t)a2 * r0 + (uint64_t)a3 * s3 +
+                            (uint64_t)a4 * s2;
+        const uint64_t d3 = (uint64_t)a0 * r3 + (uint64_t)a1 * r2 + (uint64_t)a2 * r1 + (uint64_t)a3 * r0 +
+                            (uint64_t)a4 * s3;
         uint32_t e4 = a4 * r0; // stays at 2^128; below 2^32 because a4 <= 9
 
-        d1 += d0 >> 32;
-        d2 += d1 >> 32;
-        d3 += d2 >> 32;
-        e4 += (uint32_t)(d3 >> 32);
+        // each column's upper half goes into the next column
+        const uint32_t l1 = addc32((uint32_t)d1, (uint32_t)(d0 >> 32), 0, c);
+        const uint32_t u1 = (uint32_t)(d1 >> 32) + c;
+        const uint32_t l2 = addc32((uint32_t)d2, u1, 0, c);
+        const uint32_t u2 = (uint32_t)(d2 >> 32) + c;
+        const uint32_t l3 = addc32((uint32_t)d3, u2, 0, c);
+        const uint32_t u3 = (uint32_t)(d3 >> 32) + c;
+        e4 += u3;
         // everything at and above 2^130 comes back times 5
-        const uint32_t c = (e4 >> 2) * 5u;
-        t = (uint64_t)(uint32_t)d0 + c;             h0 = (uint32_t)t;
-        t = (uint64_t)(uint32_t)d1 + (t >> 32);     h1 = (uint32_t)t;
-        t = (uint64_t)(uint32_t)d2 + (t >> 32);     h2 = (uint32_t)t;
-        t = (uint64_t)(uint32_t)d3 + (t >> 32);     h3 = (uint32_t)t;
-        h4 = (e4 & 3u) + (uint32_t)(t >> 32);
+        const uint32_t f = (e4 >> 2) * 5u;
+        h0 = addc32((uint32_t)d0, f, 0, c);
+        h1 = addc32(l1, 0, c, c);
+        h2 = addc32(l2, 0, c, c);
+        h3 = addc32(l3, 0, c, c);
+        h4 = (e4 & 3u) + c;
+#if defined(__HIP_DEVICE_COMPILE__)
+        __builtin_amdgcn_s_setprio(0);
+#endif
     }
 
     // tag = ((h mod 2^130-5) + s) mod 2^128 as four little-endian words

@@ -551,11 +551,15 @@ BNK_DEV void body_short(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
 #pragma unroll 1
     for (uint32_t b = 0; b < SHORT_BLOCKS; b++) {
         if (64u * b < len) {
+            // the block's four cells leave LDS while the keystream block is computed
+            uint4 v[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) v[j] = *reinterpret_cast<const uint4 *>(row + ((4u * b + j) << 4));
             chacha_block(k, b + 1, n1, n2, x);
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 const uint32_t kc = 4u * b + j;
-                if (kc < ncell_in) crypt_cell<OPEN>(mac, x, j, row + (kc << 4));
+                if (kc < ncell_in) crypt_cell_v<OPEN>(mac, x, j, v[j], row + (kc << 4));
                 else if (kc < ncell || (kc == ncell && (len & 15u))) {
                     const uint32_t m_out = kc < ncell ? 16u : len & 15u;
                     const uint32_t m_in = len_in > 16u * kc ? min(len_in - 16u * kc, m_out) : 0u;

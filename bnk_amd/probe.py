@@ -39,3 +39,29 @@ def copy(nbytes: int, iters: int, device: int = 0) -> float:
     if rc != 0:
         raise RuntimeError(f"bnkp_copy failed: {rc}")
     return float(r.value)
+
+
+PAIR_KINDS = {"v_add_u32": 0, "v_xor_b32": 1, "v_alignbit_b32": 2, "v_mad_u64_u32": 3,
+              "v_addc_co_u32": 4, "v_lshlrev_b32": 5, "v_lshrrev_b32": 6, "v_mov_b32": 7}
+
+
+def pair(kind_a: str, kind_b: str | None, iters: int = 20000, device: int = 0) -> tuple[float, float]:
+    """Nanoseconds per instruction of two streams that share each SIMD (waves 0-3 of a
+    workgroup run kind_a, waves 4-7 kind_b; None: the first four run alone)."""
+    a, b = C.c_double(), C.c_double()
+    rc = load().bnkp_pair(C.c_int(device), C.c_int(PAIR_KINDS[kind_a]),
+                          C.c_int(-1 if kind_b is None else PAIR_KINDS[kind_b]), C.c_uint32(iters),
+                          C.byref(a), C.byref(b))
+    if rc != 0:
+        raise RuntimeError(f"bnkp_pair failed: {rc}")
+    return float(a.value), float(b.value)
+
+
+def mix(raised_priority: bool, waves_per_simd: int, iters: int = 500, device: int = 0) -> float:
+    """VALU lane-ops per second of the ChaCha20 quarter-round stream."""
+    r = C.c_double()
+    rc = load().bnkp_mix(C.c_int(device), C.c_int(1 if raised_priority else 0), C.c_int(waves_per_simd),
+                         C.c_uint32(iters), C.byref(r))
+    if rc != 0:
+        raise RuntimeError(f"bnkp_mix failed: {rc}")
+    return float(r.value)

@@ -24,6 +24,21 @@ int bnkp_valu(int device, int op, uint32_t iters, double *ops_per_sec);
  * times (copy_kernel) and reports bytes read plus bytes written per second. */
 int bnkp_copy(int device, size_t bytes, uint32_t iters, double *bytes_per_sec);
 
+/* Two instruction streams sharing each SIMD: one workgroup of eight waves per
+ * CU, waves 0-3 run kind_a and waves 4-7 (one on each SIMD beside the first
+ * four) kind_b, or nothing with kind_b = -1.  Kinds: 0 v_add_u32, 1 v_xor_b32,
+ * 2 v_alignbit_b32, 3 v_mad_u64_u32, 4 v_addc_co_u32, 5 v_lshlrev_b32,
+ * 6 v_lshrrev_b32, 7 v_mov_b32.  Reports each group's nanoseconds per
+ * instruction over its own stream (the second group's figure includes the
+ * time it runs alone after the first has finished, if it is the slower). */
+int bnkp_pair(int device, int kind_a, int kind_b, uint32_t iters, double *ns_a, double *ns_b);
+
+/* The ChaCha20 quarter-round stream (adds, xors and rotates 1:1:1 in groups of
+ * four) with `waves_per_simd` waves resident per SIMD, waves coming and going
+ * as in a long launch; with raised_priority the four rotates of a group run
+ * between s_setprio 1 and s_setprio 0.  Reports VALU lane-ops per second. */
+int bnkp_mix(int device, int raised_priority, int waves_per_simd, uint32_t iters, double *ops_per_sec);
+
 #ifdef __cplusplus
 }
 #endif

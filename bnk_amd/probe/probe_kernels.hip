@@ -92,6 +92,114 @@ static hipError_t launch_copy(const void *src, void *dst, size_t bytes, uint32_t
     return hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------
+// How a SIMD shares its issue between two waves.
+//
+// pair_kernel: one workgroup of eight waves per CU, so that waves w and w + 4
+// share a SIMD; the first four run one instruction kind, the second four
+// another, and each group reports how long its own stream took.
+// mix_kernel: the ChaCha20 quarter-round stream (four adds, four xors, four
+// rotates, each group depending on the one before) in many short-lived
+// workgroups, a chosen number resident per CU, with or without raised wave
+// priority around the rotates.
+// ---------------------------------------------------------------------------
+#define P_ADD(a, b) asm volatile("v_add_u32 %0, %0, %1" : "+v"(a) : "v"(b))
+#define P_XOR(a, b) asm volatile("v_xor_b32 %0, %0, %1" : "+v"(a) : "v"(b))
+#define P_ROT(a, n) asm volatile("v_alignbit_b32 %0, %0, %0, " #n : "+v"(a))
+
+constexpr int PAIR_KINDS = 8;
+template <int K>
+__device__ __forceinline__ void pair_stream(uint32_t iters, uint32_t (&x)[8], uint32_t b, uint32_t m, uint64_t (&q)[8])
+{
+    for (uint32_t it = 0; it < iters; it++) {
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+#pragma unroll
+            for (int c = 0; c < 8; c++) {
+                if (K == 0) P_ADD(x[c], b);
+                if (K == 1) P_XOR(x[c], b);
+                if (K == 2) P_ROT(x[c], 7);
+                if (K == 3) asm volatile("v_mad_u64_u32 %0, vcc, %1, %2, %0" : "+v"(q[c]) : "v"(b), "v"(m) : "vcc");
+                if (K == 4) asm volatile("v_addc_co_u32 %0, vcc, %0, %1, vcc" : "+v"(x[c]) : "v"(b) : "vcc");
+                if (K == 5) asm volatile("v_lshlrev_b32 %0, 7, %0" : "+v"(x[c]));
+                if (K == 6) asm volatile("v_lshrrev_b32 %0, 7, %0" : "+v"(x[c]));
+                if (K == 7) asm volatile("v_mov_b32 %0, %1" : "+v"(x[c]) : "v"(b));
+            }
+        }
+    }
+}
+
+template <int KA, int KB>
+__global__ __launch_bounds__(512) void pair_kernel(uint32_t iters, uint32_t *out, uint64_t *ticks)
+{
+    extern __shared__ uint32_t pair_lds[];
+    const uint32_t tid = blockIdx.x * 512u + threadIdx.x;
+    uint32_t x[8];
+    uint64_t q[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) { x[i] = tid * 2654435761u + i; q[i] = x[i]; }
+    uint32_t b = tid | 1u, m = 0x9e3779b9u;
+    asm volatile("" : "+v"(b), "+v"(m));
+    const bool second = threadIdx.x >= 256;
+    __syncthreads();
+    const uint64_t t0 = wall_clock64();
+    if (!second) pair_stream<KA>(iters, x, b, m, q);
+    else if (KB >= 0) pair_stream<(KB >= 0 ? KB : 0)>(iters, x, b, m, q);
+    const uint64_t t1 = wall_clock64();
+    uint32_t acc = 0;
+#pragma unroll
+    for (int i = 0; i < 8; i++) acc ^= x[i] ^ (uint32_t)q[i] ^ (uint32_t)(q[i] >> 32);
+    out[tid] = acc + pair_lds[threadIdx.x & 1u];
+    if (blockIdx.x == 0 && (threadIdx.x == 0 || threadIdx.x == 256)) ticks[second ? 1 : 0] = t1 - t0;
+}
+
+template <int KA, int KB>
+static hipError_t pair_dispatch(int ka, int kb, uint32_t iters, uint32_t blocks, uint32_t *out, uint64_t *ticks, hipStream_t s)
+{
+    if (ka == KA && kb == KB) {
+        // more than half a CU's LDS: one workgroup per CU
+        const uint32_t lds_bytes = 96u * 1024u;
+        hipError_t e = hipFuncSetAttribute((const void *)pair_kernel<KA, KB>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL((pair_kernel<KA, KB>), dim3(blocks), dim3(512), lds_bytes, s, iters, out, ticks);
+        return hipGetLastError();
+    }
+    if constexpr (KB + 1 < PAIR_KINDS) return pair_dispatch<KA, KB + 1>(ka, kb, iters, blocks, out, ticks, s);
+    else if constexpr (KA + 1 < PAIR_KINDS) return pair_dispatch<KA + 1, -1>(ka, kb, iters, blocks, out, ticks, s);
+    return hipErrorInvalidValue;
+}
+
+template <int PRIO>
+__global__ __launch_bounds__(256) void mix_kernel(uint32_t iters, uint32_t *out)
+{
+    extern __shared__ uint32_t mix_lds[];
+    const uint32_t tid = blockIdx.x * 256u + threadIdx.x;
+    uint32_t x[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) x[i] = tid * 2654435761u + i;
+#define P_STEP(a0, a1, a2, a3, b0, b1, b2, b3, d0, d1, d2, d3, n)                                \
+    P_ADD(x[a0], x[b0]); P_ADD(x[a1], x[b1]); P_ADD(x[a2], x[b2]); P_ADD(x[a3], x[b3]);         \
+    P_XOR(x[d0], x[a0]); P_XOR(x[d1], x[a1]); P_XOR(x[d2], x[a2]); P_XOR(x[d3], x[a3]);         \
+    if (PRIO) asm volatile("s_setprio 1");                                                      \
+    P_ROT(x[d0], n); P_ROT(x[d1], n); P_ROT(x[d2], n); P_ROT(x[d3], n);                         \
+    if (PRIO) asm volatile("s_setprio 0");
+    for (uint32_t it = 0; it < iters; it++) {
+        P_STEP(0, 1, 2, 3, 4, 5, 6, 7, 12, 13, 14, 15, 16)
+        P_STEP(8, 9, 10, 11, 12, 13, 14, 15, 4, 5, 6, 7, 20)
+        P_STEP(0, 1, 2, 3, 4, 5, 6, 7, 12, 13, 14, 15, 24)
+        P_STEP(8, 9, 10, 11, 12, 13, 14, 15, 4, 5, 6, 7, 25)
+        P_STEP(0, 1, 2, 3, 5, 6, 7, 4, 15, 12, 13, 14, 16)
+        P_STEP(10, 11, 8, 9, 15, 12, 13, 14, 5, 6, 7, 4, 20)
+        P_STEP(0, 1, 2, 3, 5, 6, 7, 4, 15, 12, 13, 14, 24)
+        P_STEP(10, 11, 8, 9, 15, 12, 13, 14, 5, 6, 7, 4, 25)
+    }
+    uint32_t acc = 0;
+#pragma unroll
+    for (int i = 0; i < 16; i++) acc ^= x[i];
+    out[tid & 0xFFFFFu] = acc + mix_lds[threadIdx.x & 1u];
+}
+constexpr uint32_t MIX_INSTR_PER_ITER = 96;
+
 template <int OP>
 static hipError_t probe_dispatch(int op, uint32_t iters, uint32_t blocks, uint32_t *out, hipStream_t s)
 {
@@ -180,6 +288,80 @@ extern "C" int bnkp_copy(int device, size_t bytes, uint32_t iters, double *bytes
 fail:
     if (src) (void)hipFree(src);
     if (dst) (void)hipFree(dst);
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    if (s) (void)hipStreamDestroy(s);
+    return rc;
+}
+
+extern "C" int bnkp_pair(int device, int kind_a, int kind_b, uint32_t iters, double *ns_a, double *ns_b)
+{
+    if (!ns_a || !ns_b || iters == 0 || kind_a < 0 || kind_a >= PAIR_KINDS || kind_b < -1 || kind_b >= PAIR_KINDS) return -1;
+    hipDeviceProp_t prop;
+    hipStream_t s = nullptr;
+    uint32_t *out = nullptr;
+    uint64_t *ticks = nullptr;
+    uint64_t h[2] = {0, 0};
+    int rc = -3;
+    uint32_t blocks = 0;
+    PROBE_CHK(hipSetDevice(device));
+    PROBE_CHK(hipGetDeviceProperties(&prop, device));
+    blocks = (uint32_t)prop.multiProcessorCount;
+    PROBE_CHK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    PROBE_CHK(hipMalloc((void **)&out, (size_t)blocks * 512 * 4));
+    PROBE_CHK(hipMalloc((void **)&ticks, 16));
+    PROBE_CHK(hipMemsetAsync(ticks, 0, 16, s));
+    PROBE_CHK((pair_dispatch<0, -1>(kind_a, kind_b, 64, blocks, out, ticks, s))); // warm-up
+    PROBE_CHK((pair_dispatch<0, -1>(kind_a, kind_b, iters, blocks, out, ticks, s)));
+    PROBE_CHK(hipStreamSynchronize(s));
+    PROBE_CHK(hipMemcpy(h, ticks, 16, hipMemcpyDeviceToHost));
+    // the realtime counter runs at 100 MHz; 64 instructions per pass of the stream
+    *ns_a = (double)h[0] * 10.0 / ((double)iters * 64.0);
+    *ns_b = kind_b >= 0 ? (double)h[1] * 10.0 / ((double)iters * 64.0) : 0.0;
+    rc = 0;
+fail:
+    if (out) (void)hipFree(out);
+    if (ticks) (void)hipFree(ticks);
+    if (s) (void)hipStreamDestroy(s);
+    return rc;
+}
+
+extern "C" int bnkp_mix(int device, int raised_priority, int waves_per_simd, uint32_t iters, double *ops_per_sec)
+{
+    if (!ops_per_sec || iters == 0 || waves_per_simd < 1 || waves_per_simd > 8) return -1;
+    hipDeviceProp_t prop;
+    hipStream_t s = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    uint32_t *out = nullptr;
+    float ms = 0;
+    int rc = -3;
+    uint32_t blocks = 0, lds_bytes = 0;
+    const void *fn = raised_priority ? (const void *)mix_kernel<1> : (const void *)mix_kernel<0>;
+    PROBE_CHK(hipSetDevice(device));
+    PROBE_CHK(hipGetDeviceProperties(&prop, device));
+    // workgroups of four waves, one per SIMD; their LDS allocation limits how many a CU
+    // holds at a time; 32 rounds of them, so that waves come and go as in a long launch
+    lds_bytes = ((uint32_t)prop.maxSharedMemoryPerMultiProcessor / (uint32_t)waves_per_simd) & ~1023u;
+    if (lds_bytes > 160u * 1024u) lds_bytes = 160u * 1024u;
+    blocks = (uint32_t)prop.multiProcessorCount * (uint32_t)waves_per_simd * 32u;
+    PROBE_CHK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+    PROBE_CHK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    PROBE_CHK(hipEventCreate(&e0));
+    PROBE_CHK(hipEventCreate(&e1));
+    PROBE_CHK(hipMalloc((void **)&out, (size_t)(1u << 20) * 4));
+    for (int pass = 0; pass < 2; pass++) { // the first pass warms up
+        PROBE_CHK(hipEventRecord(e0, s));
+        if (raised_priority) hipLaunchKernelGGL(mix_kernel<1>, dim3(blocks), dim3(256), lds_bytes, s, iters, out);
+        else hipLaunchKernelGGL(mix_kernel<0>, dim3(blocks), dim3(256), lds_bytes, s, iters, out);
+        PROBE_CHK(hipGetLastError());
+        PROBE_CHK(hipEventRecord(e1, s));
+        PROBE_CHK(hipEventSynchronize(e1));
+    }
+    PROBE_CHK(hipEventElapsedTime(&ms, e0, e1));
+    *ops_per_sec = (double)blocks * 256.0 * (double)iters * MIX_INSTR_PER_ITER / ((double)ms * 1e-3);
+    rc = 0;
+fail:
+    if (out) (void)hipFree(out);
     if (e0) (void)hipEventDestroy(e0);
     if (e1) (void)hipEventDestroy(e1);
     if (s) (void)hipStreamDestroy(s);

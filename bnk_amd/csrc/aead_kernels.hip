@@ -436,20 +436,19 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
         wave_sync();
         if (s < steps) {
             if (8u * s + 8u <= ncell_in) {
-                // all eight cells of this step are whole cells of the packet
-#pragma unroll 1
-                for (uint32_t h = 0; h < 2; h++) {
-                    const uint32_t r0 = c0 + 8u * s + 4u * h;
-                    uint8_t *const cell0 = row + ((r0 & 15u) << 4), *const cell1 = row + (((r0 + 1u) & 15u) << 4);
-                    uint8_t *const cell2 = row + (((r0 + 2u) & 15u) << 4), *const cell3 = row + (((r0 + 3u) & 15u) << 4);
-                    const uint4 v0 = *reinterpret_cast<const uint4 *>(cell0), v1 = *reinterpret_cast<const uint4 *>(cell1);
-                    const uint4 v2 = *reinterpret_cast<const uint4 *>(cell2), v3 = *reinterpret_cast<const uint4 *>(cell3);
-                    chacha_block(k, 2u * s + h + 1, n1, n2, x);
-                    crypt_cell_v<OPEN>(mac, x, 0, v0, cell0);
-                    crypt_cell_v<OPEN>(mac, x, 1, v1, cell1);
-                    crypt_cell_v<OPEN>(mac, x, 2, v2, cell2);
-                    crypt_cell_v<OPEN>(mac, x, 3, v3, cell3);
-                }
+                // all eight cells of this step are whole cells of the packet: its two
+                // keystream blocks side by side
+                uint32_t y[16];
+                const uint32_t r0 = c0 + 8u * s;
+                // the first block's cells leave LDS while the keystream is computed
+                uint4 v[4];
+#pragma unroll
+                for (int j = 0; j < 4; j++) v[j] = *reinterpret_cast<const uint4 *>(row + (((r0 + j) & 15u) << 4));
+                chacha_block2(k, 2u * s + 1u, n1, n2, x, y);
+#pragma unroll
+                for (int j = 0; j < 4; j++) crypt_cell_v<OPEN>(mac, x, j, v[j], row + (((r0 + j) & 15u) << 4));
+#pragma unroll
+                for (int j = 0; j < 4; j++) crypt_cell<OPEN>(mac, y, j, row + (((r0 + 4u + j) & 15u) << 4));
             } else {
 #pragma unroll 1
                 for (uint32_t h = 0; h < 2; h++) {

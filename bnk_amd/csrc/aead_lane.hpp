@@ -63,6 +63,26 @@ BNK_DEV uint32_t addc32(uint32_t a, uint32_t b, uint32_t cin, uint32_t &cout)
     BNK_ROT4(24, d0, d1, d2, d3);                                                      \
     c0 += d0; c1 += d1; c2 += d2; c3 += d3; b0 ^= c0; b1 ^= c1; b2 ^= c2; b3 ^= c3;    \
     BNK_ROT4(25, b0, b1, b2, b3)
+// The same for two blocks side by side: eight rotates per pair of priority changes.
+#define BNK_ROT8(n, a, b, c, d, e, f, g, h)                                            \
+    asm volatile("s_setprio 1\n\t"                                                     \
+                 "v_alignbit_b32 %0, %0, %0, " #n "\n\tv_alignbit_b32 %1, %1, %1, " #n "\n\t" \
+                 "v_alignbit_b32 %2, %2, %2, " #n "\n\tv_alignbit_b32 %3, %3, %3, " #n "\n\t" \
+                 "v_alignbit_b32 %4, %4, %4, " #n "\n\tv_alignbit_b32 %5, %5, %5, " #n "\n\t" \
+                 "v_alignbit_b32 %6, %6, %6, " #n "\n\tv_alignbit_b32 %7, %7, %7, " #n "\n\t" \
+                 "s_setprio 0"                                                         \
+                 : "+v"(a), "+v"(b), "+v"(c), "+v"(d), "+v"(e), "+v"(f), "+v"(g), "+v"(h))
+#define BNK_HALF8(x, y, a0, b0, d0, a1, b1, d1, a2, b2, d2, a3, b3, d3, n)             \
+    x[a0] += x[b0]; x[a1] += x[b1]; x[a2] += x[b2]; x[a3] += x[b3];                    \
+    x[d0] ^= x[a0]; x[d1] ^= x[a1]; x[d2] ^= x[a2]; x[d3] ^= x[a3];                    \
+    y[a0] += y[b0]; y[a1] += y[b1]; y[a2] += y[b2]; y[a3] += y[b3];                    \
+    y[d0] ^= y[a0]; y[d1] ^= y[a1]; y[d2] ^= y[a2]; y[d3] ^= y[a3];                    \
+    BNK_ROT8(n, x[d0], x[d1], x[d2], x[d3], y[d0], y[d1], y[d2], y[d3])
+#define BNK_QR8(x, y, a0, b0, c0, d0, a1, b1, c1, d1, a2, b2, c2, d2, a3, b3, c3, d3)  \
+    BNK_HALF8(x, y, a0, b0, d0, a1, b1, d1, a2, b2, d2, a3, b3, d3, 16);               \
+    BNK_HALF8(x, y, c0, d0, b0, c1, d1, b1, c2, d2, b2, c3, d3, b3, 20);               \
+    BNK_HALF8(x, y, a0, b0, d0, a1, b1, d1, a2, b2, d2, a3, b3, d3, 24);               \
+    BNK_HALF8(x, y, c0, d0, b0, c1, d1, b1, c2, d2, b2, c3, d3, b3, 25)
 #else
 #define BNK_QR(a, b, c, d)                          \
     a += b; d ^= a; d = rotl32(d, 16);              \
@@ -71,6 +91,9 @@ BNK_DEV uint32_t addc32(uint32_t a, uint32_t b, uint32_t cin, uint32_t &cout)
     c += d; b ^= c; b = rotl32(b, 7)
 #define BNK_QR4(a0, b0, c0, d0, a1, b1, c1, d1, a2, b2, c2, d2, a3, b3, c3, d3)       \
     BNK_QR(a0, b0, c0, d0); BNK_QR(a1, b1, c1, d1); BNK_QR(a2, b2, c2, d2); BNK_QR(a3, b3, c3, d3)
+#define BNK_QR8(x, y, a0, b0, c0, d0, a1, b1, c1, d1, a2, b2, c2, d2, a3, b3, c3, d3)  \
+    BNK_QR4(x[a0], x[b0], x[c0], x[d0], x[a1], x[b1], x[c1], x[d1], x[a2], x[b2], x[c2], x[d2], x[a3], x[b3], x[c3], x[d3]); \
+    BNK_QR4(y[a0], y[b0], y[c0], y[d0], y[a1], y[b1], y[c1], y[d1], y[a2], y[b2], y[c2], y[d2], y[a3], y[b3], y[c3], y[d3])
 #endif
 
 // RFC 8439 section 2.3 with the WireGuard nonce: words 13..15 of the state
@@ -91,6 +114,26 @@ BNK_DEV void chacha_block(const uint32_t (&k)[8], uint32_t blk, uint32_t n1,
 #pragma unroll
     for (int i = 0; i < 8; i++) x[4 + i] += k[i];
     x[12] += blk; x[14] += n1; x[15] += n2;
+}
+
+// Blocks blk and blk + 1 at once, their rounds interleaved.
+BNK_DEV void chacha_block2(const uint32_t (&k)[8], uint32_t blk, uint32_t n1, uint32_t n2,
+                           uint32_t (&x)[16], uint32_t (&y)[16])
+{
+    x[0] = y[0] = 0x61707865u; x[1] = y[1] = 0x3320646eu; x[2] = y[2] = 0x79622d32u; x[3] = y[3] = 0x6b206574u;
+#pragma unroll
+    for (int i = 0; i < 8; i++) x[4 + i] = y[4 + i] = k[i];
+    x[12] = blk; y[12] = blk + 1u; x[13] = y[13] = 0; x[14] = y[14] = n1; x[15] = y[15] = n2;
+#pragma unroll 1
+    for (int r = 0; r < 10; r++) {
+        BNK_QR8(x, y, 0, 4, 8, 12, 1, 5, 9, 13, 2, 6, 10, 14, 3, 7, 11, 15);
+        BNK_QR8(x, y, 0, 5, 10, 15, 1, 6, 11, 12, 2, 7, 8, 13, 3, 4, 9, 14);
+    }
+    x[0] += 0x61707865u; x[1] += 0x3320646eu; x[2] += 0x79622d32u; x[3] += 0x6b206574u;
+    y[0] += 0x61707865u; y[1] += 0x3320646eu; y[2] += 0x79622d32u; y[3] += 0x6b206574u;
+#pragma unroll
+    for (int i = 0; i < 8; i++) { x[4 + i] += k[i]; y[4 + i] += k[i]; }
+    x[12] += blk; y[12] += blk + 1u; x[14] += n1; y[14] += n1; x[15] += n2; y[15] += n2;
 }
 
 // Poly1305 (RFC 8439 section 2.5), radix 2^26.

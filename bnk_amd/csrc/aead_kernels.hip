@@ -533,8 +533,9 @@ BNK_DEV void body_short(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
 #pragma unroll
         for (int q = 0; q < 8; q++) pre[1][q] = ld16a(jcell[q] + 8u < nld[q] ? csrc[q] + 128u : safe);
     }
-    // keystream block 0 (the Poly1305 key) while the loads fly
-    chacha_block(k, 0, n1, n2, x);
+    // keystream blocks 0 (the Poly1305 key) and 1 side by side while the loads fly
+    uint32_t y[16];
+    chacha_block2(k, 0, n1, n2, x, y);
     mac.init(x);
 #pragma unroll
     for (int q = 0; q < 8; q++)
@@ -547,25 +548,32 @@ BNK_DEV void body_short(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
     }
     wave_sync();
     uint8_t *row = tile + lane * SHORT_ROW;
-#pragma unroll 1
-    for (uint32_t b = 0; b < SHORT_BLOCKS; b++) {
-        if (64u * b < len) {
-            // the block's four cells leave LDS while the keystream block is computed
-            uint4 v[4];
+    // block b's four cells with keystream ks
+    auto crypt_block = [&](uint32_t b, const uint32_t (&ks)[16], const uint4 (&v)[4]) __attribute__((always_inline)) {
 #pragma unroll
-            for (int j = 0; j < 4; j++) v[j] = *reinterpret_cast<const uint4 *>(row + ((4u * b + j) << 4));
-            chacha_block(k, b + 1, n1, n2, x);
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const uint32_t kc = 4u * b + j;
-                if (kc < ncell_in) crypt_cell_v<OPEN>(mac, x, j, v[j], row + (kc << 4));
-                else if (kc < ncell || (kc == ncell && (len & 15u))) {
-                    const uint32_t m_out = kc < ncell ? 16u : len & 15u;
-                    const uint32_t m_in = len_in > 16u * kc ? min(len_in - 16u * kc, m_out) : 0u;
-                    crypt_tail_lds<OPEN>(mac, x, j, row + (kc << 4), dst + 16u * kc, m_in, m_out);
-                }
+        for (int j = 0; j < 4; j++) {
+            const uint32_t kc = 4u * b + j;
+            if (kc < ncell_in) crypt_cell_v<OPEN>(mac, ks, j, v[j], row + (kc << 4));
+            else if (kc < ncell || (kc == ncell && (len & 15u))) {
+                const uint32_t m_out = kc < ncell ? 16u : len & 15u;
+                const uint32_t m_in = len_in > 16u * kc ? min(len_in - 16u * kc, m_out) : 0u;
+                crypt_tail_lds<OPEN>(mac, ks, j, row + (kc << 4), dst + 16u * kc, m_in, m_out);
             }
         }
+    };
+    static_assert(SHORT_BLOCKS == 2, "the short path is written out for two data blocks");
+    uint4 v[4];
+    if (len != 0) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) v[j] = *reinterpret_cast<const uint4 *>(row + (j << 4));
+        crypt_block(0, y, v);
+    }
+    if (len > 64u) {
+        // the second block's cells leave LDS while its keystream is computed
+#pragma unroll
+        for (int j = 0; j < 4; j++) v[j] = *reinterpret_cast<const uint4 *>(row + ((4 + j) << 4));
+        chacha_block(k, 2, n1, n2, x);
+        crypt_block(1, x, v);
     }
     if (OPEN) capture_head(head, row, row + 16);
     wave_sync();

@@ -65,6 +65,7 @@ BNK_DEV void st16a_out(uint8_t *p, uint4 v)
 
 BNK_DEV uint8_t ld8(const uint8_t *p) { return *reinterpret_cast<const BNK_GLOBAL uint8_t *>((uintptr_t)p); }
 BNK_DEV void st8(uint8_t *p, uint8_t v) { *reinterpret_cast<BNK_GLOBAL uint8_t *>((uintptr_t)p) = v; }
+BNK_DEV void st4a(uint8_t *p, uint32_t v) { *reinterpret_cast<BNK_GLOBAL uint32_t *>((uintptr_t)p) = v; }
 
 typedef uint32_t __attribute__((aligned(1))) u32_unaligned;
 typedef uint16_t __attribute__((aligned(1))) u16_unaligned;
@@ -315,7 +316,17 @@ BNK_DEV void body_generic(uint8_t *tile, uint32_t lane, const uint8_t *src, uint
 // Otherwise the stream starts at the packet itself (any alignment, source and
 // destination independent): the same pipeline over 128-byte pieces of the
 // packet, which then straddle two lines each.
-template <bool OPEN, bool ALIGNED>
+// SHIFT (not ALIGNED, every destination of the wave 4-byte aligned): the input
+// comes in as such pieces, but the output leaves as whole aligned 16-byte cells
+// of the destination's own 128-byte lines.  A lane that moves such a cell reads
+// the two ring cells it straddles and picks its four words from their eight;
+// the first and the last cell of a packet, which it shares with its neighbours,
+// leave word by word.  (Misaligned 16-byte stores run at half rate and leave
+// every line in two parts.)  A destination line lags the packet's pieces by up to
+// 124 bytes, so a piece enters the ring one step later than otherwise: just
+// before it is needed, after the line that still holds the end of the piece
+// two before it has left.
+template <bool OPEN, bool ALIGNED, bool SHIFT = false>
 BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_t *dst, uint32_t len,
                         uint32_t len_in, const uint8_t *safe, const uint32_t (&k)[8], uint32_t n1, uint32_t n2,
                         Poly32 &mac, uint32_t (&x)[16], Head &head)
@@ -337,6 +348,9 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
     const uint8_t *csrc[8];
     uint8_t *cdst[8];
     uint32_t cfirst[8], cend[8], cend_ld[8];
+    int32_t pofs[8];
+    uint32_t whole[8];
+    bool odd1[8], odd2[8];
 #pragma unroll
     for (int q = 0; q < 8; q++) {
         const int owner = 8 * q + (int)(lane >> 3);
@@ -348,6 +362,15 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
         // (a cell that is not aligned may reach into the next page: only aligned ones
         // are fetched beyond the packet's last byte)
         cend_ld[q] = cfirst[q] + ((olen + (ALIGNED ? 15u : 0u)) >> 4);
+        if (SHIFT) {
+            const uint64_t od = shfl64((uint64_t)(uintptr_t)dst, owner);
+            const uint32_t skd = (uint32_t)od & 127u;
+            cdst[q] = reinterpret_cast<uint8_t *>(od - skd) + 16u * sub; // my cell of the line holding the packet's first byte
+            pofs[q] = (int32_t)(16u * sub) - (int32_t)skd;               // where that cell starts within the packet
+            whole[q] = olen & ~15u;                                      // bytes of it that go through the ring
+            odd1[q] = (pofs[q] & 4) != 0;
+            odd2[q] = (pofs[q] & 8) != 0;
+        }
     }
     uint32_t maxsteps = steps;
 #pragma unroll
@@ -400,6 +423,34 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
 #define BNK_TAKE(q, m) out##q = *BNK_SLOT(q, m)
 #define BNK_PUT(q, m) if (BNK_INSIDE(q, m)) BNK_ST(cdst[q] + 128u * (m), out##q)
 #define BNK_PUT_ALL(q, m) BNK_ST(cdst[q] + 128u * (m), out##q)
+    // SHIFT: my cell of destination line m starts pofs[q] + 128 m bytes into the packet
+    // (before it when negative), a multiple of 4: ring cells at and after that place,
+    // and of their eight words the four from word (offset / 4) % 4 on
+#define BNK_TAKE_SHIFT(q, m)                                                                \
+    do {                                                                                    \
+        const int32_t at_##q = pofs[q] + (int32_t)(128u * (m));                             \
+        const uint32_t cl_##q = (uint32_t)(at_##q >> 4);                                    \
+        const uint4 lo_##q = *reinterpret_cast<const uint4 *>(mycell + 8u * q * RING_ROW + ((cl_##q & 15u) << 4));        \
+        const uint4 hi_##q = *reinterpret_cast<const uint4 *>(mycell + 8u * q * RING_ROW + (((cl_##q + 1u) & 15u) << 4)); \
+        const uint32_t u0_##q = odd1[q] ? lo_##q.y : lo_##q.x, u1_##q = odd1[q] ? lo_##q.z : lo_##q.y;                    \
+        const uint32_t u2_##q = odd1[q] ? lo_##q.w : lo_##q.z, u3_##q = odd1[q] ? hi_##q.x : lo_##q.w;                    \
+        const uint32_t u4_##q = odd1[q] ? hi_##q.y : hi_##q.x, u5_##q = odd1[q] ? hi_##q.z : hi_##q.y;                    \
+        out##q = make_uint4(odd2[q] ? u2_##q : u0_##q, odd2[q] ? u3_##q : u1_##q, odd2[q] ? u4_##q : u2_##q,             \
+                            odd2[q] ? u5_##q : u3_##q);                                     \
+    } while (0)
+#define BNK_PUT_SHIFT(q, m)                                                                 \
+    do {                                                                                    \
+        const uint32_t at_##q = (uint32_t)(pofs[q] + (int32_t)(128u * (m)));                \
+        uint8_t *const to_##q = cdst[q] + 128u * (m);                                       \
+        if (at_##q < whole[q] && at_##q + 12u < whole[q]) st16a_out(to_##q, out##q);        \
+        else {                                                                              \
+            if (at_##q < whole[q]) st4a(to_##q, out##q.x);                                  \
+            if (at_##q + 4u < whole[q]) st4a(to_##q + 4, out##q.y);                         \
+            if (at_##q + 8u < whole[q]) st4a(to_##q + 8, out##q.z);                         \
+            if (at_##q + 12u < whole[q]) st4a(to_##q + 12, out##q.w);                       \
+        }                                                                                   \
+    } while (0)
+#define BNK_PUT_SHIFT_ALL(q, m) st16a_out(cdst[q] + 128u * (m), out##q)
 #define BNK_EIGHT(OP, m)                                                                    \
     do {                                                                                    \
         OP(0, m); OP(1, m); OP(2, m); OP(3, m); OP(4, m); OP(5, m); OP(6, m); OP(7, m);     \
@@ -418,19 +469,30 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
     // keystream block 0 (the Poly1305 key) is computed while the first line flies
     chacha_block(k, 0, n1, n2, x);
     mac.init(x);
-    BNK_COMMIT_LINE(0u);
-    BNK_ISSUE_LINE(1u);
+    // (with SHIFT a piece enters the ring, and the next one starts flying, one step later)
+    constexpr uint32_t AHEAD = SHIFT ? 0u : 1u;
+    if (!SHIFT) {
+        BNK_COMMIT_LINE(0u);
+        BNK_ISSUE_LINE(1u);
+    }
     // iteration s: line s-1 (complete since the step before) leaves the ring,
     // line s+1 enters it, line s+2 starts flying, line s-1 goes to memory,
     // packet bytes [128s, 128s+128) are processed; the extra last iteration
     // only writes back the final line
     for (uint32_t s = 0; s <= maxsteps + 1; s++) {
-        if (s >= 1) BNK_EIGHT(BNK_TAKE, s - 1);
-        wave_sync();
-        BNK_COMMIT_LINE(s + 1);
-        if (s + 2 <= maxsteps) BNK_ISSUE_LINE(s + 2);
         if (s >= 1) {
-            if (s - 1 >= m_lo && s - 1 < m_hi) BNK_EIGHT(BNK_PUT_ALL, s - 1);
+            if (SHIFT) BNK_EIGHT(BNK_TAKE_SHIFT, s - 1);
+            else BNK_EIGHT(BNK_TAKE, s - 1);
+        }
+        wave_sync();
+        BNK_COMMIT_LINE(s + AHEAD);
+        if (s + AHEAD + 1u <= maxsteps) BNK_ISSUE_LINE(s + AHEAD + 1u);
+        if (s >= 1) {
+            if (SHIFT) {
+                // whole lines of every packet of the wave: not the first, and ending within its whole cells
+                if (s - 1 >= 1u && s - 1 < m_hi) BNK_EIGHT(BNK_PUT_SHIFT_ALL, s - 1);
+                else BNK_EIGHT(BNK_PUT_SHIFT, s - 1);
+            } else if (s - 1 >= m_lo && s - 1 < m_hi) BNK_EIGHT(BNK_PUT_ALL, s - 1);
             else BNK_EIGHT(BNK_PUT, s - 1);
         }
         wave_sync();
@@ -489,6 +551,9 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
 #undef BNK_TAKE
 #undef BNK_PUT
 #undef BNK_PUT_ALL
+#undef BNK_TAKE_SHIFT
+#undef BNK_PUT_SHIFT
+#undef BNK_PUT_SHIFT_ALL
 #undef BNK_EIGHT
 #undef BNK_LINE
 #undef BNK_ISSUE_LINE
@@ -810,7 +875,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     Head head;
     head.on = OPEN && (a.heads != nullptr || decap);
     head.c0 = head.c1 = make_uint4(0, 0, 0, 0);
-    if (__ballot(!lane_lines) != 0ull) body_lines<OPEN, false>(tile, lane, src, dst, len, len_in, safe, k, n1, n2, mac, x, head);
+    if (__ballot(!lane_lines) != 0ull) {
+        if (__ballot(((uintptr_t)dst & 3u) != 0) == 0ull)
+            body_lines<OPEN, false, true>(tile, lane, src, dst, len, len_in, safe, k, n1, n2, mac, x, head);
+        else body_lines<OPEN, false>(tile, lane, src, dst, len, len_in, safe, k, n1, n2, mac, x, head);
+    }
     else if (__ballot(len > 64u * SHORT_BLOCKS) == 0ull) body_short<OPEN>(tile, lane, src, dst, len, len_in, safe, k, n1, n2, mac, x, head);
     else body_lines<OPEN, true>(tile, lane, src, dst, len, len_in, safe, k, n1, n2, mac, x, head);
 

@@ -469,6 +469,8 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
     // keystream block 0 (the Poly1305 key) is computed while the first line flies
     chacha_block(k, 0, n1, n2, x);
     mac.init(x);
+    ChachaShared shared;
+    if (!OPEN) chacha_shared(k, n1, n2, shared);
     // (with SHIFT a piece enters the ring, and the next one starts flying, one step later)
     constexpr uint32_t AHEAD = SHIFT ? 0u : 1u;
     if (!SHIFT) {
@@ -506,7 +508,8 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
                 uint4 v[4];
 #pragma unroll
                 for (int j = 0; j < 4; j++) v[j] = *reinterpret_cast<const uint4 *>(row + (((r0 + j) & 15u) << 4));
-                chacha_block2(k, 2u * s + 1u, n1, n2, x, y);
+                if (OPEN) chacha_block2(k, 2u * s + 1u, n1, n2, x, y);
+                else chacha_block2_shared(k, shared, 2u * s + 1u, n1, n2, x, y);
 #pragma unroll
                 for (int j = 0; j < 4; j++) crypt_cell_v<OPEN>(mac, x, j, v[j], row + (((r0 + j) & 15u) << 4));
 #pragma unroll

@@ -136,6 +136,63 @@ BNK_DEV void chacha_block2(const uint32_t (&k)[8], uint32_t blk, uint32_t n1, ui
     x[12] += blk; y[12] += blk + 1u; x[14] += n1; y[14] += n1; x[15] += n2; y[15] += n2;
 }
 
+// What the blocks of one packet share: the block counter sits in the first column of
+// the state, so the first column round leaves the other three columns the same for
+// every block, and the first addition of the first column as well.
+struct ChachaShared {
+    uint32_t a0;     // constant 0 + key word 0
+    uint32_t col[12]; // words 1, 5, 9, 13, 2, 6, 10, 14, 3, 7, 11, 15 after the first column round
+};
+
+BNK_DEV void chacha_shared(const uint32_t (&k)[8], uint32_t n1, uint32_t n2, ChachaShared &sh)
+{
+    const uint32_t c[4] = {0x61707865u, 0x3320646eu, 0x79622d32u, 0x6b206574u};
+    const uint32_t n[4] = {0, 0, n1, n2};
+    sh.a0 = c[0] + k[0];
+#pragma unroll
+    for (int j = 1; j < 4; j++) {
+        uint32_t a = c[j], b = k[j], cc = k[4 + j], d = n[j];
+        a += b; d ^= a; d = rotl32(d, 16);
+        cc += d; b ^= cc; b = rotl32(b, 12);
+        a += b; d ^= a; d = rotl32(d, 8);
+        cc += d; b ^= cc; b = rotl32(b, 7);
+        sh.col[4 * (j - 1)] = a; sh.col[4 * (j - 1) + 1] = b; sh.col[4 * (j - 1) + 2] = cc; sh.col[4 * (j - 1) + 3] = d;
+    }
+}
+
+// chacha_block2 from what the packet's blocks share: the first column round is only
+// the counter's column, once per block.
+BNK_DEV void chacha_block2_shared(const uint32_t (&k)[8], const ChachaShared &sh, uint32_t blk, uint32_t n1,
+                                  uint32_t n2, uint32_t (&x)[16], uint32_t (&y)[16])
+{
+    x[0] = y[0] = sh.a0;
+    x[12] = rotl32(blk ^ x[0], 16); y[12] = rotl32((blk + 1u) ^ y[0], 16);
+    x[8] = k[4] + x[12]; y[8] = k[4] + y[12];
+    x[4] = rotl32(k[0] ^ x[8], 12); y[4] = rotl32(k[0] ^ y[8], 12);
+    x[0] += x[4]; y[0] += y[4];
+    x[12] = rotl32(x[12] ^ x[0], 8); y[12] = rotl32(y[12] ^ y[0], 8);
+    x[8] += x[12]; y[8] += y[12];
+    x[4] = rotl32(x[4] ^ x[8], 7); y[4] = rotl32(y[4] ^ y[8], 7);
+#pragma unroll
+    for (int j = 1; j < 4; j++) {
+        x[j] = y[j] = sh.col[4 * (j - 1)];
+        x[4 + j] = y[4 + j] = sh.col[4 * (j - 1) + 1];
+        x[8 + j] = y[8 + j] = sh.col[4 * (j - 1) + 2];
+        x[12 + j] = y[12 + j] = sh.col[4 * (j - 1) + 3];
+    }
+    BNK_QR8(x, y, 0, 5, 10, 15, 1, 6, 11, 12, 2, 7, 8, 13, 3, 4, 9, 14);
+#pragma unroll 1
+    for (int r = 1; r < 10; r++) {
+        BNK_QR8(x, y, 0, 4, 8, 12, 1, 5, 9, 13, 2, 6, 10, 14, 3, 7, 11, 15);
+        BNK_QR8(x, y, 0, 5, 10, 15, 1, 6, 11, 12, 2, 7, 8, 13, 3, 4, 9, 14);
+    }
+    x[0] += 0x61707865u; x[1] += 0x3320646eu; x[2] += 0x79622d32u; x[3] += 0x6b206574u;
+    y[0] += 0x61707865u; y[1] += 0x3320646eu; y[2] += 0x79622d32u; y[3] += 0x6b206574u;
+#pragma unroll
+    for (int i = 0; i < 8; i++) { x[4 + i] += k[i]; y[4 + i] += k[i]; }
+    x[12] += blk; y[12] += blk + 1u; x[14] += n1; y[14] += n1; x[15] += n2; y[15] += n2;
+}
+
 // Poly1305 (RFC 8439 section 2.5), radix 2^26.
 struct Poly26 {
     uint32_t r0, r1, r2, r3, r4;

@@ -210,7 +210,20 @@ int main()
         bool ok = true;
         for (int i = 0; i < 16; i++) ok = ok && x[i] == ld32(want + 4 * i);
         expect(ok, "chacha_block against the oracle");
-        (void)y;
+        // two blocks side by side, plainly and from what a packet's blocks share
+        uint8_t want2[64];
+        bnko_chacha20_block(key, blk + 1u, nonce, want2);
+        uint32_t x2[16];
+        chacha_block2(k, blk, (uint32_t)ctr, (uint32_t)(ctr >> 32), x2, y);
+        ok = true;
+        for (int i = 0; i < 16; i++) ok = ok && x2[i] == ld32(want + 4 * i) && y[i] == ld32(want2 + 4 * i);
+        expect(ok, "chacha_block2 against the oracle");
+        ChachaShared sh;
+        chacha_shared(k, (uint32_t)ctr, (uint32_t)(ctr >> 32), sh);
+        chacha_block2_shared(k, sh, blk, (uint32_t)ctr, (uint32_t)(ctr >> 32), x2, y);
+        ok = true;
+        for (int i = 0; i < 16; i++) ok = ok && x2[i] == ld32(want + 4 * i) && y[i] == ld32(want2 + 4 * i);
+        expect(ok, "chacha_block2_shared against the oracle");
     }
     run_poly<Poly26>("Poly26");
     run_poly<Poly32>("Poly32");

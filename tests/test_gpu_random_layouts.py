@@ -81,3 +81,85 @@ def test_random_lengths_and_alignments_match_the_oracle(seed):
         sel = length > k
         expect[at[sel] + k] = np.where(exp_v[sel] == 1, plain[at[sel] + k], 0)
     assert np.array_equal(d_back.cpu().numpy(), expect)
+
+
+def _layout(rng, lens, extra, align, fixed_gap=None):
+    """Slots back to back, each holding lens[i] + extra bytes, starting at a multiple of 16
+    plus a gap that is a multiple of `align` below 16 (or `fixed_gap` for every packet)."""
+    room = ((lens.astype(np.int64) + extra + 15) // 16) * 16 + 16
+    if fixed_gap is not None:
+        gap = np.full(len(lens), fixed_gap, np.int64)
+    elif align >= 16:
+        gap = np.zeros(len(lens), np.int64)
+    else:
+        gap = rng.integers(0, 16 // align, len(lens)) * align
+    off = (np.concatenate([[0], np.cumsum(room)[:-1]]) + gap).astype(np.uint64)
+    return off, int(room.sum()) + 32
+
+
+@pytest.mark.parametrize("src_align,dst_align,src_gap,dst_gap", [
+    (1, 4, None, None),   # input anywhere, output on words: whole destination cells, word-shifted
+    (4, 1, None, None),   # output anywhere: misaligned stores
+    (4, 4, None, None),   # both on words, each packet with skews of its own
+    (16, 4, None, None),
+    (4, 16, None, None),
+    (4, 4, 4, 12),        # one skew for every packet of the batch, different on the two sides
+    (16, 16, None, None), # both on cells but in different places within their lines
+])
+def test_source_and_destination_laid_out_independently(src_align, dst_align, src_gap, dst_gap):
+    """Seal and open between arenas whose packets sit at unrelated alignments: sealed
+    bytes equal the oracle's, the bytes between packets stay as they were, forged tags
+    are rejected and everything else opens to the plaintext."""
+    import torch
+    from bnk_amd import lib
+    from oracle import binding as O
+    rng = np.random.default_rng(4242 + 16 * src_align + dst_align)
+    dev = torch.device("cuda:0")
+    n, n_peers = 40000, 17
+    keys = rng.integers(0, 256, (n_peers, 32), dtype=np.uint8)
+    lens = rng.choice([0, 1, 3, 16, 17, 60, 63, 64, 65, 127, 128, 129, 255, 576, 1419, 1420, 1500], n).astype(np.uint32)
+    off_p, total_p = _layout(rng, lens, 0, src_align, src_gap)
+    off_s, total_s = _layout(rng, lens, 16, dst_align, dst_gap)
+    if src_align == 16 and dst_align == 16:
+        off_s = off_s + np.uint64(48)  # cells on both sides, 48 bytes apart within their lines
+        total_s += 48
+    plain = rng.integers(0, 256, total_p, dtype=np.uint8)
+    peer = rng.integers(0, n_peers, n).astype(np.uint32)
+    ctrs = rng.integers(0, 1 << 63, n, dtype=np.uint64)
+    want = np.full(total_s, 0x5A, np.uint8)
+    O.seal_batch(keys, peer, ctrs, plain, off_p, lens, want, off_s, 8)
+    d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)  # noqa: E731
+    d_plain = d(plain)
+    d_sealed = torch.full((total_s,), 0x5A, dtype=torch.uint8, device=dev)
+    d_offp, d_offs = d(off_p.astype(np.int64)), d(off_s.astype(np.int64))
+    d_len, d_ctl = d(lens.astype(np.int32)), d((lens + 16).astype(np.int32))
+    d_peer, d_ctr = d(peer.astype(np.int32)), d(ctrs.astype(np.int64))
+    with lib.Context(0) as ctx:
+        ctx.keys_set(lib.KEYS_SEND, keys)
+        ctx.keys_set(lib.KEYS_RECV, keys)
+        ctx.seal(lib.make_batch(d_plain, total_p, n, lib.MEM_DEVICE, offsets=d_offp, lens=d_len, peer=d_peer,
+                                counters=d_ctr),
+                 lib.make_batch(d_sealed, total_s, n, lib.MEM_DEVICE, offsets=d_offs))
+        ctx.sync()
+        got = d_sealed.cpu().numpy()
+        bad = np.flatnonzero(got != want)
+        assert bad.size == 0, f"first differing sealed byte at {bad[:4]}"
+        forged = rng.permutation(n)[:30]
+        pos = off_s[forged].astype(np.int64) + lens[forged].astype(np.int64) + 5
+        d_sealed[d(pos)] ^= 0x01
+        # open back into an arena laid out like the plaintext's
+        d_back = torch.full((total_p,), 0xA5, dtype=torch.uint8, device=dev)
+        d_v = torch.full((n,), 9, dtype=torch.uint8, device=dev)
+        ctx.open(lib.make_batch(d_sealed, total_s, n, lib.MEM_DEVICE, offsets=d_offs, lens=d_ctl, peer=d_peer,
+                                counters=d_ctr),
+                 lib.make_batch(d_back, total_p, n, lib.MEM_DEVICE, offsets=d_offp), d_v)
+        ctx.sync()
+    exp_v = np.ones(n, np.uint8)
+    exp_v[forged] = 0
+    assert np.array_equal(d_v.cpu().numpy(), exp_v)
+    expect = np.full(total_p, 0xA5, np.uint8)
+    length, at = lens.astype(np.int64), off_p.astype(np.int64)
+    for k in range(int(length.max())):
+        sel = length > k
+        expect[at[sel] + k] = np.where(exp_v[sel] == 1, plain[at[sel] + k], 0)
+    assert np.array_equal(d_back.cpu().numpy(), expect)

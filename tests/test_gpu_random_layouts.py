@@ -163,3 +163,51 @@ def test_source_and_destination_laid_out_independently(src_align, dst_align, src
         sel = length > k
         expect[at[sel] + k] = np.where(exp_v[sel] == 1, plain[at[sel] + k], 0)
     assert np.array_equal(d_back.cpu().numpy(), expect)
+
+
+@pytest.mark.parametrize("align", [4, 16, 1])
+def test_seal_and_open_in_place(align):
+    """One arena for both sides: every packet is sealed where it lies (its slot has
+    room for the tag) and opened there again."""
+    import torch
+    from bnk_amd import lib
+    from oracle import binding as O
+    rng = np.random.default_rng(777 + align)
+    dev = torch.device("cuda:0")
+    n, n_peers = 50000, 5
+    keys = rng.integers(0, 256, (n_peers, 32), dtype=np.uint8)
+    lens = rng.choice([0, 2, 16, 31, 60, 64, 100, 128, 130, 576, 1420, 1421], n).astype(np.uint32)
+    off, total = _layout(rng, lens, 16, align)
+    arena = rng.integers(0, 256, total, dtype=np.uint8)
+    peer = rng.integers(0, n_peers, n).astype(np.uint32)
+    ctrs = rng.integers(0, 1 << 63, n, dtype=np.uint64)
+    want = arena.copy()
+    O.seal_batch(keys, peer, ctrs, arena, off, lens, want, off, 8)
+    d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)  # noqa: E731
+    d_arena = d(arena)
+    d_off, d_len, d_ctl = d(off.astype(np.int64)), d(lens.astype(np.int32)), d((lens + 16).astype(np.int32))
+    d_peer, d_ctr = d(peer.astype(np.int32)), d(ctrs.astype(np.int64))
+    d_v = torch.zeros(n, dtype=torch.uint8, device=dev)
+    with lib.Context(0) as ctx:
+        ctx.keys_set(lib.KEYS_SEND, keys)
+        ctx.keys_set(lib.KEYS_RECV, keys)
+        ctx.seal(lib.make_batch(d_arena, total, n, lib.MEM_DEVICE, offsets=d_off, lens=d_len, peer=d_peer,
+                                counters=d_ctr),
+                 lib.make_batch(d_arena, total, n, lib.MEM_DEVICE, offsets=d_off))
+        ctx.sync()
+        got = d_arena.cpu().numpy()
+        bad = np.flatnonzero(got != want)
+        assert bad.size == 0, f"first differing sealed byte at {bad[:4]}"
+        ctx.open(lib.make_batch(d_arena, total, n, lib.MEM_DEVICE, offsets=d_off, lens=d_ctl, peer=d_peer,
+                                counters=d_ctr),
+                 lib.make_batch(d_arena, total, n, lib.MEM_DEVICE, offsets=d_off), d_v)
+        ctx.sync()
+    assert bool(d_v.all())
+    back = d_arena.cpu().numpy()
+    # the plaintext is back; the 16 bytes after it still hold the tag
+    at, length = off.astype(np.int64), lens.astype(np.int64)
+    expect = want.copy()
+    for k in range(int(length.max())):
+        sel = length > k
+        expect[at[sel] + k] = arena[at[sel] + k]
+    assert np.array_equal(back, expect)

@@ -15,7 +15,8 @@ Prints ONE JSON line.  Besides the contract fields it carries
   cpu_baseline_openssl  the same sample through OpenSSL's assembly, when libcrypto is there
   packed_layout  the same packets back to back (no slot 16-byte aligned)
   extra          the ACL filter rate (configuration 4) with its own roofline and CPU
-                 baseline, and what one call costs on 128 packets in pinned host rings
+                 baseline, what one call costs on 128 packets in pinned host rings, and the
+                 rates of configurations 3 and 5 and of the transport framing
 
 --workload filter | imix | relay | wg | host | latency | copy | sizes | issue print one line for that
 workload alone; --no-extras leaves out everything but the timed launches (for traces).
@@ -1047,6 +1048,19 @@ def main() -> int:
         "workload": lat["config"]["workload"],
         **lat["per_batch_size_us"]["128"],
     }
+    # the other configurations the path is specified on, each a short run of its own
+    # workload (their full lines: --workload imix | relay | wg)
+    others = {}
+    oargs = argparse.Namespace(**vars(args))
+    oargs.steps, oargs.warmup, oargs.no_cpu_baseline, oargs.no_extras = 10, 2, True, True
+    for name, fn in (("cfg3_imix", bench_imix), ("cfg5_relay", bench_relay), ("transport_framing", bench_wg)):
+        try:
+            r = fn(oargs)
+            others[name] = {"metric": r["metric"], "value": r["value"], "unit": r["unit"],
+                            "ms_per_step": r["ms_per_step"], "workload": r["config"]["workload"]}
+        except Exception as e:  # a side measurement must not take the headline line with it
+            others[name] = {"error": "%s: %s" % (type(e).__name__, e)}
+    out["extra"]["other_configurations"] = others
     print(json.dumps(out))
     return 0
 

@@ -470,7 +470,7 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
     chacha_block(k, 0, n1, n2, x);
     mac.init(x);
     ChachaShared shared;
-    if (!OPEN) chacha_shared(k, n1, n2, shared);
+    chacha_shared(k, n1, n2, shared);
     // (with SHIFT a piece enters the ring, and the next one starts flying, one step later)
     constexpr uint32_t AHEAD = SHIFT ? 0u : 1u;
     if (!SHIFT) {
@@ -504,14 +504,20 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
                 // keystream blocks side by side
                 uint32_t y[16];
                 const uint32_t r0 = c0 + 8u * s;
-                // the first block's cells leave LDS while the keystream is computed
-                uint4 v[4];
+                if (OPEN) {
+                    // (open has no registers for reading cells ahead of the keystream)
+                    chacha_block2_shared(k, shared, 2u * s + 1u, n1, n2, x, y);
 #pragma unroll
-                for (int j = 0; j < 4; j++) v[j] = *reinterpret_cast<const uint4 *>(row + (((r0 + j) & 15u) << 4));
-                if (OPEN) chacha_block2(k, 2u * s + 1u, n1, n2, x, y);
-                else chacha_block2_shared(k, shared, 2u * s + 1u, n1, n2, x, y);
+                    for (int j = 0; j < 4; j++) crypt_cell<OPEN>(mac, x, j, row + (((r0 + j) & 15u) << 4));
+                } else {
+                    // the first block's cells leave LDS while the keystream is computed
+                    uint4 v[4];
 #pragma unroll
-                for (int j = 0; j < 4; j++) crypt_cell_v<OPEN>(mac, x, j, v[j], row + (((r0 + j) & 15u) << 4));
+                    for (int j = 0; j < 4; j++) v[j] = *reinterpret_cast<const uint4 *>(row + (((r0 + j) & 15u) << 4));
+                    chacha_block2_shared(k, shared, 2u * s + 1u, n1, n2, x, y);
+#pragma unroll
+                    for (int j = 0; j < 4; j++) crypt_cell_v<OPEN>(mac, x, j, v[j], row + (((r0 + j) & 15u) << 4));
+                }
 #pragma unroll
                 for (int j = 0; j < 4; j++) crypt_cell<OPEN>(mac, y, j, row + (((r0 + 4u + j) & 15u) << 4));
             } else {

@@ -133,20 +133,28 @@ BNK_DEV void wave_sync()
 }
 
 // One wave = 64 packets, one lane per packet for the arithmetic.  Memory is
-// touched cooperatively through a per-wave LDS tile, in one of two ways.
+// touched cooperatively through a per-wave LDS tile (body_lines, body_short,
+// body_generic).
 //
 // Line path (every packet of the wave 16-byte aligned, source and destination
 // at the same offset within a 128-byte line): the wave moves whole aligned
 // 128-byte lines, eight adjacent lanes per line, so every HBM/L2 access is a
 // full line touched exactly once.  A packet rarely starts on a line boundary,
 // so each LDS row is a ring of two lines: step s consumes packet bytes
-// [128s, 128s+128), which live in lines s and s+1 of the packet; line s+1 is
-// fetched just before step s, line s is complete and written back just after.
-// Only the 16-byte cells that belong to the packet are ever read or written,
-// so neighbours sharing a line are never disturbed.
+// [128s, 128s+128), which live in lines s and s+1 of the packet; line s+2 is
+// on its way into registers meanwhile, line s is complete after the step and
+// leaves before line s+2 takes its place.  Only the 16-byte cells that belong
+// to the packet are ever read or written, so neighbours sharing a line are
+// never disturbed.
 //
-// Generic path (anything else): 64 bytes per packet per step, four adjacent
-// lanes per packet, any byte alignment.
+// Unaligned path (any other layout): the same ring over 128-byte pieces of the
+// packet itself, at whatever alignment it has; where every destination of the
+// wave is 4-byte aligned the output still leaves as whole aligned cells of the
+// destination's lines (see body_lines).
+//
+// Generic path (packets beyond the wave-per-packet kernel's reach in small
+// batches): 64 bytes per packet per step, four adjacent lanes per packet, any
+// byte alignment.
 constexpr uint32_t LDS_ROW = 80;    // generic: 64 data bytes + 16 pad
 constexpr uint32_t RING_ROW = 272;  // line path: 2 x 128-byte lines + 16 pad
 constexpr uint32_t WAVES_PER_BLOCK = 4;

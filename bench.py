@@ -47,7 +47,7 @@ VALU_SINGLE_ISSUE_TOPS = 39.3
 # Counter readings for one launch of aead_wave_kernel over 2^20 packets x 1420 B (mean of
 # seal and open), taken with rocprofv3 --pmc and kept in profiles/aead_wave_kernel_cfg2.md;
 # they change only when the kernel does.
-VALU_LANE_INSTR_PER_PACKET = 28288   # SQ_INSTS_VALU x 64 / 2^20
+VALU_LANE_INSTR_PER_PACKET = 27703   # SQ_INSTS_VALU x 64 / 2^20
 VALU_SINGLE_ISSUE_SHARE = 0.40       # of them: v_alignbit_b32, v_mad_u64_u32, v_add_co/v_addc_co (counted in the kernel's loops)
 TRAFFIC_BYTES_PER_LAUNCH = 3.177e9   # FETCH_SIZE + WRITE_SIZE, scaled by copy_kernel
 # the same for filter_check_kernel over 2^22 headers (profiles/filter_check_kernel_cfg4.md)

@@ -617,7 +617,11 @@ BNK_DEV void body_short(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
     }
     // keystream blocks 0 (the Poly1305 key) and 1 side by side while the loads fly
     uint32_t y[16];
-    chacha_block2(k, 0, n1, n2, x, y);
+    {
+        ChachaShared shared;
+        chacha_shared(k, n1, n2, shared);
+        chacha_block2_shared(k, shared, 0, n1, n2, x, y);
+    }
     mac.init(x);
 #pragma unroll
     for (int q = 0; q < 8; q++)

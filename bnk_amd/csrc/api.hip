@@ -1,6 +1,9 @@
 // C ABI of libbnkhip.so (see include/bnkhip.h): argument checking, staging of
 // host batches through the context's device buffers, kernel launches.
 #include "api_common.hpp"
+
+#include <atomic>
+#include <chrono>
 #include "filter_host.hpp"
 
 using namespace bnk;
@@ -160,7 +163,7 @@ int aead_batch_host_direct(bnk_ctx *ctx, bool open, const bnk_batch *in, const b
     HIPCHK(ctx, open ? launch_aead_open(a, ctx->stream) : launch_aead_seal(a, ctx->stream));
     // host batches have had their peer indices checked above, so the kernel
     // has nothing to report through the status word
-    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    if (int wrc = wait_stream(ctx)) return wrc;
     if (open) memcpy(verdict, p_verdict, n);
     return BNK_OK;
 }
@@ -283,10 +286,46 @@ int aead_batch(bnk_ctx *ctx, bool open, const bnk_batch *in, const bnk_batch *ou
     return BNK_OK;
 }
 
-// Waits for the stream, then reads and clears the status words.
-int take_status(bnk_ctx *ctx, uint32_t *status)
+// Waits for everything enqueued on the context stream so far.  After a short kernel
+// hipStreamSynchronize returns 13 us after the launch; a one-thread launch behind the
+// work that writes this wait's number into pinned memory, with the host watching that
+// word, is seen after 9.6 us (the stream's order puts the write behind everything before
+// it, results in host memory included).  The watch is bounded: whatever takes longer than
+// WAIT_WATCH_US is waited for the ordinary way, which also reports a failed launch.
+constexpr int64_t WAIT_WATCH_US = 100;
+int wait_stream(bnk_ctx *ctx)
 {
+    const uint32_t seq = ++ctx->wait_seq;
+    if (launch_fill_u32(ctx->d_status + STATUS_DONE_WORD, 1, seq, ctx->stream) == hipSuccess) {
+        volatile uint32_t *done = ctx->h_status + STATUS_DONE_WORD;
+        const auto t0 = std::chrono::steady_clock::now();
+        for (;;) {
+            for (int spin = 0; spin < 64; spin++) {
+                if (*done == seq) {
+                    std::atomic_thread_fence(std::memory_order_acquire);
+                    return BNK_OK;
+                }
+                __builtin_ia32_pause();
+            }
+            if (std::chrono::duration_cast<std::chrono::microseconds>(std::chrono::steady_clock::now() - t0).count() >
+                WAIT_WATCH_US)
+                break;
+        }
+    }
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    return BNK_OK;
+}
+
+// Waits for the stream, then reads and clears the status words.  after_kernel: the
+// last thing enqueued is a kernel (behind a copy the watched word comes later than the
+// copy's own completion does).
+int take_status(bnk_ctx *ctx, uint32_t *status, bool after_kernel)
+{
+    if (after_kernel) {
+        if (int rc = wait_stream(ctx)) return rc;
+    } else {
+        HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    }
     volatile uint32_t *h = ctx->h_status;
     *status = (h[STATUS_PEER_RANGE] ? STATUS_PEER_RANGE : 0u) | (h[STATUS_FLOWS_FULL] ? STATUS_FLOWS_FULL : 0u) |
               (h[STATUS_BOUNDS] ? STATUS_BOUNDS : 0u);

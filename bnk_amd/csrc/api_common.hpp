@@ -445,8 +445,11 @@ int aead_batch(bnk_ctx *ctx, bool open, const bnk_batch *in, const bnk_batch *ou
 // (noalloc_api.hip): looks up its address on `device` (which must be current).
 int noalloc_setup(bnk_ctx *ctx, int device);
 
-// Reads and clears the device status word (waits for the stream).
-int take_status(bnk_ctx *ctx, uint32_t *status);
+// Waits for everything enqueued on the context stream so far.
+int wait_stream(bnk_ctx *ctx);
+// Reads and clears the device status word (waits for the stream; after_kernel: through
+// wait_stream, for a call whose last enqueued operation is a kernel).
+int take_status(bnk_ctx *ctx, uint32_t *status, bool after_kernel = false);
 // Maps status bits to an error code (BNK_OK when clear).
 int status_to_rc(bnk_ctx *ctx, uint32_t status);
 

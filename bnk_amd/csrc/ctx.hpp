@@ -108,6 +108,7 @@ struct bnk_ctx {
     struct Ring { uintptr_t host; uint8_t *dev; size_t bytes; };
     std::vector<Ring> rings;
     uint32_t *h_status = nullptr; // pinned status words the kernels write
+    uint32_t wait_seq = 0;        // number of the last wait_stream(), see STATUS_DONE_WORD
     uint32_t spread_max = bnk::SPREAD_MAX_PACKETS; // see AeadArgs::spread_max
     // fused relay: plaintext scratch, per-packet flags, sort buffers, staged arrays
     bnk::DevBuf r_plain, r_auth, r_pass, r_keys, r_idx, r_skeys, r_sidx, r_tmp;

@@ -197,7 +197,7 @@ int run_staged(bnk_ctx *ctx, bool check, FilterArgs &a, uint8_t *h_verdict, uint
         // CheckInbound reports nothing through the status word
         a.verdict = ctx->pin.dev(h_verdict);
         HIPCHK(ctx, launch_filter_check(a, f->max_blocks, ctx->stream));
-        HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+        if (int wrc = wait_stream(ctx)) return wrc;
         memcpy(verdict, h_verdict, a.n);
         return BNK_OK;
     } else {
@@ -207,7 +207,7 @@ int run_staged(bnk_ctx *ctx, bool check, FilterArgs &a, uint8_t *h_verdict, uint
         HIPCHK(ctx, hipMemcpyAsync(verdict, a.verdict, a.n, hipMemcpyDeviceToHost, ctx->stream));
     }
     uint32_t status = 0;
-    int rc = take_status(ctx, &status);
+    int rc = take_status(ctx, &status, !check);
     if (rc) return rc;
     return status_to_rc(ctx, status);
 }

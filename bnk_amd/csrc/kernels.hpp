@@ -119,6 +119,9 @@ constexpr uint32_t SPREAD_MAX_PACKETS = 4096;
 // with no copy.
 enum : uint32_t { STATUS_PEER_RANGE = 1u, STATUS_FLOWS_FULL = 2u, STATUS_BOUNDS = 4u };
 constexpr uint32_t STATUS_WORDS = 8; // word [bit value] holds that condition
+// Word 7 of the same block is no condition: a one-thread launch writes the number of the
+// wait it ends there, for the host to watch (wait_stream in api.hip).
+constexpr uint32_t STATUS_DONE_WORD = 7;
 
 // True when [off, off + len) does not fit an arena of `limit` bytes (limit 0: not checked).
 __host__ __device__ inline bool beyond_arena(uint64_t off, uint64_t len, uint64_t limit)

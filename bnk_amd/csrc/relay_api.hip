@@ -332,7 +332,8 @@ extern "C" int bnk_relay_fused_batch(bnk_ctx *ctx, const bnk_batch *in, const ui
     if (!host) return BNK_OK;
     if (direct) {
         // both peer arrays were checked above: nothing comes back through the status word
-        HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+        rc = wait_stream(ctx);
+        if (rc) return rc;
         memcpy(verdict, h_verdict, n);
         memcpy(ctr_out, h_ctr_out, (size_t)n * 8);
         return BNK_OK;

@@ -529,10 +529,11 @@ static int wg_encap_impl(bnk_ctx *ctx, const bnk_batch *slots, uint32_t mtu, uin
             // back through the status word
             uint32_t status = 0;
             if (note) {
-                rc = take_status(ctx, &status);
+                rc = take_status(ctx, &status, true);
                 if (rc) return rc;
             } else {
-                HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+                rc = wait_stream(ctx);
+                if (rc) return rc;
             }
             memcpy(wire_len, h_wire_len, (size_t)n * 4);
             return status_to_rc(ctx, status);
@@ -938,7 +939,8 @@ static int wg_decap_impl(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *o
         if (direct) {
             // the peer index of every opened packet comes from the table lookup:
             // nothing comes back through the status word
-            HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+            rc = wait_stream(ctx);
+            if (rc) return rc;
             memcpy(result, h_result, n);
             memcpy(out_len, h_out_len, (size_t)n * 4);
             memcpy(peer, h_peer, (size_t)n * 4);

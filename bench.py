@@ -916,6 +916,7 @@ def main() -> int:
                 "ops_per_packet": ops_aead(L), "achieved": round(achieved_tops, 2),
                 "unit": "Top/s (int32 op-equivalents)",
                 "ratio_to_single_issue_rate": round(achieved_tops / VALU_SINGLE_ISSUE_TOPS, 4),
+                "ratio_to_peak": round(achieved_tops / VALU_PEAK_TOPS, 4),
             },
             "measured_ceilings_tops": probes,
         },

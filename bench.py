@@ -761,8 +761,10 @@ def bench_issue(args) -> dict:
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=30,
+                    help="untimed steps first: a chip that was idle needs some 50 ms of work to reach the "
+                         "clocks it then holds (the first 20 steps run about 5 %% slower)")
     ap.add_argument("--packets", type=int, default=1 << 20)
     ap.add_argument("--workload", default="aead", choices=["aead", "filter", "imix", "relay", "wg", "host", "latency", "copy", "sizes", "issue"],
                     help="aead (default, the headline line, with the ACL filter rate as an extra); "
@@ -1053,7 +1055,7 @@ def main() -> int:
     # workload (their full lines: --workload imix | relay | wg)
     others = {}
     oargs = argparse.Namespace(**vars(args))
-    oargs.steps, oargs.warmup, oargs.no_cpu_baseline, oargs.no_extras = 10, 2, True, True
+    oargs.steps, oargs.warmup, oargs.no_cpu_baseline, oargs.no_extras = 20, 20, True, True
     for name, fn in (("cfg3_imix", bench_imix), ("cfg5_relay", bench_relay), ("transport_framing", bench_wg)):
         try:
             r = fn(oargs)

@@ -146,7 +146,7 @@ hipError_t launch_aead_open(const AeadArgs &a, hipStream_t s);
 // device scratch of LEN_BINS and LEN_CURSOR_WORDS words; hist must be all zeros on entry and
 // is all zeros again when the grouping has run.
 constexpr uint32_t LEN_BINS = 1032;
-constexpr uint32_t LEN_CURSOR_WORDS = LEN_BINS;
+constexpr uint32_t LEN_CURSOR_WORDS = LEN_BINS + 8;
 hipError_t launch_length_sort(const uint32_t *lens, uint32_t n, uint32_t tag_bytes,
                               uint32_t *order, uint32_t *hist, uint32_t *cursor,
                               hipStream_t s);

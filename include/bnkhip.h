@@ -165,7 +165,7 @@ int bnk_aead_open_batch(bnk_ctx *ctx, const bnk_batch *in,
  * under HIP graph capture, tight serving loops, harnesses that forbid
  * hipMalloc.  It has no counterpart in the reference.  The call allocates
  * nothing: the scratch the length grouping needs lives in a file-scope device
- * array of BNK_NOALLOC_MAX_PACKETS + 2064 words (4 MiB + 8 KiB per GPU, held
+ * array of BNK_NOALLOC_MAX_PACKETS + 2072 words (4 MiB + 8 KiB per GPU, held
  * until the process ends).  Device-resident batches only (in->mem and out->mem
  * BNK_MEM_DEVICE), at most BNK_NOALLOC_MAX_PACKETS packets, otherwise
  * BNK_E_INVAL.  Results are those of bnk_aead_seal_batch.  Every call on a GPU

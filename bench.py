@@ -867,6 +867,16 @@ def main() -> int:
     lane_instr = n * VALU_LANE_INSTR_PER_PACKET
     achieved_lane_tops = lane_instr / (kern_ms * 1e-3) / 1e12
     counters_apply = n == 1 << 20
+    # Two measured ceilings beside the nominal ones: the kernel's arithmetic with no
+    # packet movement (the product's lane code on constants in registers) at 1-4 waves
+    # per SIMD, and a plain copy.  The kernel runs two waves per SIMD.
+    blocks_per_packet = (L + 63) // 64 + 1
+    kernel_gblocks = n * blocks_per_packet / (kern_ms * 1e-3) / 1e9
+    arithmetic_alone = copy_gbs = None
+    if not args.no_extras:
+        arithmetic_alone = {str(w): round(probe.aead_compute(True, w) / 1e9, 1) for w in (1, 2, 3, 4)}
+        copy_gbs = probe.copy(1 << 30, 10) / 1e9
+    traffic_gbs = TRAFFIC_BYTES_PER_LAUNCH / (kern_ms * 1e-3) / 1e9 if counters_apply else None
 
     out = {
         "metric": "aead_seal_open_gbit_per_s_1420B",
@@ -921,6 +931,13 @@ def main() -> int:
                 "ratio_to_peak": round(achieved_tops / VALU_PEAK_TOPS, 4),
             },
             "measured_ceilings_tops": probes,
+            # 64-byte blocks (ChaCha20 block + xor + four Poly1305 blocks) per second: the
+            # kernel, and the same arithmetic alone by waves resident per SIMD
+            "arithmetic_alone": None if arithmetic_alone is None else {
+                "unit": "G 64-byte blocks/s", "kernel": round(kernel_gblocks, 1),
+                "by_waves_per_simd": arithmetic_alone,
+                "kernel_over_two_waves_per_simd": round(kernel_gblocks / arithmetic_alone["2"], 4),
+            },
         },
         "roofline_hbm": {
             "bound": "hbm", "kernel": "aead_wave_kernel",
@@ -929,6 +946,12 @@ def main() -> int:
             "traffic": TRAFFIC_BYTES_PER_LAUNCH if counters_apply else None,
             "traffic_source": "profiles/aead_wave_kernel_cfg2.md (not re-measured in this run)",
             "bytes_per_launch": alg_bytes, "avg_launch_ms": round(kern_ms, 4),
+            # what a plain copy of 1 GiB reaches on this box (bytes read + written), and the
+            # kernel's counter traffic per second against it
+            "measured_copy_gb_per_s": None if copy_gbs is None else round(copy_gbs, 1),
+            "traffic_gb_per_s": None if traffic_gbs is None else round(traffic_gbs, 1),
+            "traffic_over_measured_copy": None if copy_gbs is None or traffic_gbs is None
+            else round(traffic_gbs / copy_gbs, 4),
         },
     }
 

@@ -65,3 +65,13 @@ def mix(raised_priority: bool, waves_per_simd: int, iters: int = 500, device: in
     if rc != 0:
         raise RuntimeError(f"bnkp_mix failed: {rc}")
     return float(r.value)
+
+
+def aead_compute(paired: bool, waves_per_simd: int, data_blocks: int = 48, device: int = 0) -> float:
+    """64-byte blocks per second of the AEAD arithmetic with no packet movement."""
+    r = C.c_double()
+    rc = load().bnkp_aead_compute(C.c_int(device), C.c_int(1 if paired else 0), C.c_int(waves_per_simd),
+                                  C.c_uint32(data_blocks), C.byref(r))
+    if rc != 0:
+        raise RuntimeError(f"bnkp_aead_compute failed: {rc}")
+    return float(r.value)

@@ -39,6 +39,15 @@ int bnkp_pair(int device, int kind_a, int kind_b, uint32_t iters, double *ns_a, 
  * between s_setprio 1 and s_setprio 0.  Reports VALU lane-ops per second. */
 int bnkp_mix(int device, int raised_priority, int waves_per_simd, uint32_t iters, double *ops_per_sec);
 
+/* The AEAD kernel's arithmetic alone (the product's lane code: per 64 bytes a
+ * ChaCha20 block, the xor and four Poly1305 blocks, a packet per lane, the
+ * data a constant in registers) with `waves_per_simd` (1..4) waves resident
+ * per SIMD; paired: two keystream blocks side by side as in the kernel's
+ * 128-byte steps.  data_blocks (even) per lane.  Reports 64-byte blocks per
+ * second, the packet's key block included: the kernel's rate if moving the
+ * packets cost nothing. */
+int bnkp_aead_compute(int device, int paired, int waves_per_simd, uint32_t data_blocks, double *blocks_per_sec);
+
 #ifdef __cplusplus
 }
 #endif

@@ -211,3 +211,37 @@ def test_seal_and_open_in_place(align):
         sel = length > k
         expect[at[sel] + k] = arena[at[sel] + k]
     assert np.array_equal(back, expect)
+
+
+@pytest.mark.parametrize("n", [1 << 20, (1 << 20) + 1])
+def test_length_grouping_on_either_side_of_its_launch_shapes(n):
+    """2^20 packets are grouped by length in two launches (every scatter block scans the
+    histogram itself), one packet more in three (a scan launch in between).  Two batches
+    in a row through one context, the second with other lengths: both sealed arenas equal
+    the oracle's, so each shape also left the histogram cleared for the next grouping."""
+    import torch
+    from bnk_amd import lib
+    from oracle import binding as O
+    rng = np.random.default_rng(77 + (n & 1))
+    dev = torch.device("cuda:0")
+    n_peers = 5
+    keys = rng.integers(0, 256, (n_peers, 32), dtype=np.uint8)
+    d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)  # noqa: E731
+    with lib.Context(0) as ctx:
+        ctx.keys_set(lib.KEYS_SEND, keys)
+        for top in (40, 150):
+            lens = rng.integers(0, top + 1, n).astype(np.uint32)
+            off, total = _layout(rng, lens, 16, 16)
+            plain = rng.integers(0, 256, total, dtype=np.uint8)
+            peer = rng.integers(0, n_peers, n).astype(np.uint32)
+            ctrs = rng.integers(0, 1 << 63, n, dtype=np.uint64)
+            want = np.full(total, 0x5A, np.uint8)
+            O.seal_batch(keys, peer, ctrs, plain, off, lens, want, off, 8)
+            d_sealed = torch.full((total,), 0x5A, dtype=torch.uint8, device=dev)
+            d_off = d(off.astype(np.int64))
+            ctx.seal(lib.make_batch(d(plain), total, n, lib.MEM_DEVICE, offsets=d_off, lens=d(lens.astype(np.int32)),
+                                    peer=d(peer.astype(np.int32)), counters=d(ctrs.astype(np.int64))),
+                     lib.make_batch(d_sealed, total, n, lib.MEM_DEVICE, offsets=d_off))
+            ctx.sync()
+            bad = np.flatnonzero(d_sealed.cpu().numpy() != want)
+            assert bad.size == 0, f"lengths up to {top}: first differing byte at {bad[:4]}"

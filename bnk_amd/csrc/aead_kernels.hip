@@ -804,7 +804,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     uint32_t wg_res = BNK_WG_OK;
     if (decap) {
         const uint64_t at = a.in_off ? in_off_ld : (uint64_t)i * a.in_stride;
-        const bool beyond = beyond_arena(at, len, a.in_limit);
+        // the datagram where it is read, and the plaintext where it would be written
+        const bool beyond = beyond_arena(at, len, a.in_limit) ||
+                            beyond_arena((a.out_off ? out_off_ld : (uint64_t)i * a.out_stride) + a.out_skip,
+                                         len >= 32u ? len - 32u : 0u, a.out_limit);
         if (in_batch && beyond) status_raise(a.status, STATUS_BOUNDS);
         if (beyond || len < 32u) wg_res = BNK_WG_BAD_HEADER;
         const uint4 h = ld16(wg_res == BNK_WG_OK && in_batch ? a.in + at : reinterpret_cast<const uint8_t *>(a.keys));
@@ -850,7 +853,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // plaintext up to its padded length count as zeros without being in memory.
     const bool encap = !OPEN && a.wg.mode == WG_FUSE_ENCAP;
     const uint32_t len_plain = len;
-    if (encap) len += wg_padding(len, a.wg.mtu);
+    // a length word of a device-resident batch may be garbage: one so large that
+    // the sums below would wrap is beyond any arena
+    const bool wraps = len > MAX_PACKET_BYTES;
+    if (encap && !wraps) len += wg_padding(len, a.wg.mtu);
     const uint32_t pr = decap ? wg_peer : a.peer ? peer_ld : 0u;
     const bool skipped = (a.skip != nullptr && skip_ld != 0) || wg_res != BNK_WG_OK;
     const bool bad_peer = pr >= a.n_peers;
@@ -859,7 +865,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const uint64_t out_at = (a.out_off ? out_off_ld : (uint64_t)i * a.out_stride) + a.out_skip;
     // seal reads len and writes len + 16, open reads len (tag included) and writes len - 16
     const bool outside = beyond_arena(in_at, len, a.in_limit) ||
-                         beyond_arena(out_at, OPEN ? (too_short ? 0u : len - 16u) : len + 16u, a.out_limit);
+                         beyond_arena(out_at, OPEN ? (too_short ? 0u : len - 16u) : (uint64_t)len + 16u, a.out_limit) ||
+                         (wraps && (a.in_limit | a.out_limit) != 0);
     const uint64_t ctr = decap ? wg_ctr : a.counters ? ctr_ld : a.counter0 + i;
     // a keypair that has used up its nonces sends nothing more (wireguard-go device/send.go)
     const bool spent = encap && ctr >= WG_REJECT_AFTER_MESSAGES;
@@ -945,7 +952,8 @@ __global__ __launch_bounds__(256) void aead_spread_kernel(AeadArgs a)
         const uint64_t in_at = (uint64_t)(src - a.in), out_at = (uint64_t)(dst - a.out);
         const bool short_ct = OPEN && len < 16u;
         if (beyond_arena(in_at, len, a.in_limit) ||
-            beyond_arena(out_at, OPEN ? (short_ct ? 0u : len - 16u) : len + 16u, a.out_limit)) {
+            beyond_arena(out_at, OPEN ? (short_ct ? 0u : len - 16u) : (uint64_t)len + 16u, a.out_limit) ||
+            (len > MAX_PACKET_BYTES && (a.in_limit | a.out_limit) != 0)) {
             if (lane == 0 && !(a.skip && a.skip[i] != 0)) {
                 status_raise(a.status, STATUS_BOUNDS);
                 if (OPEN) a.verdict[i] = 0;
@@ -1438,6 +1446,24 @@ hipError_t launch_fill_u32(uint32_t *p, uint32_t n, uint32_t v, hipStream_t s)
 {
     if (n == 0) return hipSuccess;
     hipLaunchKernelGGL(fill_u32_kernel, dim3((n + 255u) / 256u), dim3(256), 0, s, p, n, v);
+    return hipGetLastError();
+}
+
+// The last launch of a host call that waits by watching a word in pinned host
+// memory: everything the stream ran before this kernel has completed when it
+// starts (kernels of one stream do not overlap, and a kernel's end makes its
+// stores visible at system scope); the fence and the release store at system
+// scope state that order for this store as well, so a host that sees `v` in the
+// word also sees every result the earlier kernels wrote to host memory.
+__global__ void done_word_kernel(uint32_t *word, uint32_t v)
+{
+    __threadfence_system();
+    __hip_atomic_store(word, v, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+hipError_t launch_done_word(uint32_t *word, uint32_t v, hipStream_t s)
+{
+    hipLaunchKernelGGL(done_word_kernel, dim3(1), dim3(1), 0, s, word, v);
     return hipGetLastError();
 }
 

@@ -231,7 +231,7 @@ int aead_batch(bnk_ctx *ctx, bool open, const bnk_batch *in, const bnk_batch *ou
         a.counters = in->counters;
         a.verdict = verdict;
         // offsets and lengths in device memory cannot be checked here: the lanes do it
-        if (in->offsets || in->lens) {
+        if (in->offsets || in->lens || out->offsets) {
             a.in_limit = in->bytes;
             a.out_limit = out->bytes;
         }
@@ -289,20 +289,30 @@ int aead_batch(bnk_ctx *ctx, bool open, const bnk_batch *in, const bnk_batch *ou
 // Waits for everything enqueued on the context stream so far.  After a short kernel
 // hipStreamSynchronize returns 13 us after the launch; a one-thread launch behind the
 // work that writes this wait's number into pinned memory, with the host watching that
-// word, is seen after 9.6 us (the stream's order puts the write behind everything before
-// it, results in host memory included).  The watch is bounded: whatever takes longer than
-// WAIT_WATCH_US is waited for the ordinary way, which also reports a failed launch.
+// word, is seen after 9.6 us.  Why the results are there when the word is: the stream
+// runs its kernels one after the other, so the earlier kernels (which wrote verdicts,
+// lengths and status words to pinned host memory) have ended, and their stores have
+// been released at system scope, before done_word_kernel starts; that kernel fences and
+// stores the word with release semantics at system scope; the host reads it with an
+// acquire fence before it touches the results.  The watch is bounded: whatever takes
+// longer than WAIT_WATCH_US is waited for the ordinary way.  A launch that failed is
+// reported by hipGetLastError on either path; a fault inside a kernel ends the process
+// on this runtime whichever way the host waits.  BNK_WAIT_SYNC=1 in the environment at
+// bnk_init switches the watch off (every wait is hipStreamSynchronize).
 constexpr int64_t WAIT_WATCH_US = 100;
 int wait_stream(bnk_ctx *ctx)
 {
     const uint32_t seq = ++ctx->wait_seq;
-    if (launch_fill_u32(ctx->d_status + STATUS_DONE_WORD, 1, seq, ctx->stream) == hipSuccess) {
+    if (!ctx->wait_sync_only &&
+        launch_done_word(ctx->d_status + STATUS_DONE_WORD, seq, ctx->stream) == hipSuccess) {
         volatile uint32_t *done = ctx->h_status + STATUS_DONE_WORD;
         const auto t0 = std::chrono::steady_clock::now();
         for (;;) {
             for (int spin = 0; spin < 64; spin++) {
-                if (*done == seq) {
+                // (numbers are handed out in stream order: a later one also means done)
+                if ((int32_t)(*done - seq) >= 0) {
                     std::atomic_thread_fence(std::memory_order_acquire);
+                    HIPCHK(ctx, hipGetLastError());
                     return BNK_OK;
                 }
                 __builtin_ia32_pause();
@@ -382,9 +392,12 @@ int bnk_init(int device_ordinal, bnk_ctx **out)
         return bail("hipStreamCreate", e);
     if ((e = hipEventCreate(&ctx->ev0)) != hipSuccess) return bail("hipEventCreate", e);
     if ((e = hipEventCreate(&ctx->ev1)) != hipSuccess) return bail("hipEventCreate", e);
+    if ((e = hipEventCreateWithFlags(&ctx->ev_noalloc, hipEventDisableTiming)) != hipSuccess)
+        return bail("hipEventCreate", e);
     if ((e = hipHostMalloc((void **)&ctx->h_status, 64, hipHostMallocDefault)) != hipSuccess)
         return bail("hipHostMalloc", e);
     memset(ctx->h_status, 0, 64);
+    if (const char *ws = getenv("BNK_WAIT_SYNC")) ctx->wait_sync_only = ws[0] != '\0' && ws[0] != '0';
     if ((e = hipHostGetDevicePointer((void **)&ctx->d_status, ctx->h_status, 0)) != hipSuccess)
         return bail("hipHostGetDevicePointer", e);
     // the length grouping's histogram starts out cleared and every grouping
@@ -416,6 +429,7 @@ void bnk_shutdown(bnk_ctx *ctx)
         ctx->alive = false;
         (void)hipSetDevice(ctx->device);
         if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+        noalloc_forget(ctx);
         for (DevBuf *b : {&ctx->in_arena, &ctx->out_arena, &ctx->off_in, &ctx->off_out, &ctx->lens,
                           &ctx->peer, &ctx->counters, &ctx->verdict, &ctx->order, &ctx->hist,
                           &ctx->cursor, &ctx->misc, &ctx->r_plain, &ctx->r_auth, &ctx->r_pass,
@@ -441,6 +455,7 @@ void bnk_shutdown(bnk_ctx *ctx)
         if (ctx->s_down) (void)hipStreamDestroy(ctx->s_down);
         if (ctx->ev0) (void)hipEventDestroy(ctx->ev0);
         if (ctx->ev1) (void)hipEventDestroy(ctx->ev1);
+        if (ctx->ev_noalloc) (void)hipEventDestroy(ctx->ev_noalloc);
         if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
     }
     delete ctx;

@@ -444,6 +444,8 @@ int aead_batch(bnk_ctx *ctx, bool open, const bnk_batch *in, const bnk_batch *ou
 // The file-scope device scratch of the entry point that allocates nothing
 // (noalloc_api.hip): looks up its address on `device` (which must be current).
 int noalloc_setup(bnk_ctx *ctx, int device);
+// Drops a context that is being shut down from the record of who used the scratch last.
+void noalloc_forget(bnk_ctx *ctx);
 
 // Waits for everything enqueued on the context stream so far.
 int wait_stream(bnk_ctx *ctx);

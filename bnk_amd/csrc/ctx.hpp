@@ -89,6 +89,7 @@ struct bnk_ctx {
     int device = -1;
     hipStream_t stream = nullptr;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    hipEvent_t ev_noalloc = nullptr; // recorded behind every bnk_aead_seal_batch_noalloc of this context
     // chunked host batches: upload and download streams, one event pair per chunk
     hipStream_t s_up = nullptr, s_down = nullptr;
     std::vector<hipEvent_t> ev_up, ev_done;
@@ -109,6 +110,7 @@ struct bnk_ctx {
     std::vector<Ring> rings;
     uint32_t *h_status = nullptr; // pinned status words the kernels write
     uint32_t wait_seq = 0;        // number of the last wait_stream(), see STATUS_DONE_WORD
+    bool wait_sync_only = false;  // BNK_WAIT_SYNC=1: wait with hipStreamSynchronize, never by watching the word
     uint32_t spread_max = bnk::SPREAD_MAX_PACKETS; // see AeadArgs::spread_max
     // fused relay: plaintext scratch, per-packet flags, sort buffers, staged arrays
     bnk::DevBuf r_plain, r_auth, r_pass, r_keys, r_idx, r_skeys, r_sidx, r_tmp;

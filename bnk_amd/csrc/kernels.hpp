@@ -73,6 +73,10 @@ struct WgFuse {
 };
 enum : uint32_t { WG_FUSE_OFF = 0, WG_FUSE_ENCAP = 1, WG_FUSE_DECAP = 2 };
 constexpr uint32_t WG_FUSE_MAX_LEN = 63u * 64u;
+// No packet is longer than this: a length word above it (only a device-resident
+// batch can carry one unseen) is treated as reaching beyond the arena, so that
+// length + tag and length + padding never wrap 32 bits.
+constexpr uint32_t MAX_PACKET_BYTES = 0x7FFFFFFFu;
 
 // Device-side view of one AEAD launch.  All pointers are device pointers.
 struct AeadArgs {
@@ -153,6 +157,8 @@ hipError_t launch_length_sort(const uint32_t *lens, uint32_t n, uint32_t tag_byt
 
 // p[0..n) = v on the stream (a kernel, so it is safe under graph capture).
 hipError_t launch_fill_u32(uint32_t *p, uint32_t n, uint32_t v, hipStream_t s);
+// One thread behind everything queued so far: fence, then store v to *word at system scope.
+hipError_t launch_done_word(uint32_t *word, uint32_t v, hipStream_t s);
 
 // Fused relay bookkeeping (relay_kernels.hip).  After open (auth[i]) and the
 // filter (pass[i]): verdicts, then per-peer batch-order counters for the

@@ -25,6 +25,11 @@ namespace {
 constexpr int MAX_DEVICES = 64;
 std::mutex g_mu;
 uint32_t *g_scratch_ptr[MAX_DEVICES]; // per device: each GPU holds its own copy of the array
+// Who used a device's array last, and the event that context recorded behind its
+// launches: another context makes its stream wait for that event before it
+// touches the array, so that calls of different contexts on one GPU take turns
+// instead of interleaving their groupings on the same words.
+bnk_ctx *g_last_user[MAX_DEVICES];
 
 } // namespace
 
@@ -43,6 +48,14 @@ int noalloc_setup(bnk_ctx *ctx, int device)
     return BNK_OK;
 }
 
+// A context that goes away takes its event with it (its stream has been waited for).
+void noalloc_forget(bnk_ctx *ctx)
+{
+    if (ctx->device < 0 || ctx->device >= MAX_DEVICES) return;
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (g_last_user[ctx->device] == ctx) g_last_user[ctx->device] = nullptr;
+}
+
 } // namespace bnk
 
 extern "C" int bnk_aead_seal_batch_noalloc(bnk_ctx *ctx, const bnk_batch *in, const bnk_batch *out)
@@ -55,15 +68,19 @@ extern "C" int bnk_aead_seal_batch_noalloc(bnk_ctx *ctx, const bnk_batch *in, co
         return fail(ctx, BNK_E_INVAL, "bnk_aead_seal_batch_noalloc takes device-resident batches only");
     if (in->n > BNK_NOALLOC_MAX_PACKETS)
         return fail(ctx, BNK_E_INVAL, "bnk_aead_seal_batch_noalloc: more than BNK_NOALLOC_MAX_PACKETS packets");
-    uint32_t *ptr;
-    {
-        std::lock_guard<std::mutex> lk(g_mu);
-        ptr = g_scratch_ptr[ctx->device];
-    }
+    // held while the call enqueues its work (it does not wait for it), so that two
+    // contexts' waits and records on a device pair up in one order
+    std::lock_guard<std::mutex> lk(g_mu);
+    uint32_t *ptr = g_scratch_ptr[ctx->device];
     if (!ptr) return fail(ctx, BNK_E_STATE, "device scratch was not set up");
+    bnk_ctx *last = g_last_user[ctx->device];
+    if (last && last != ctx) HIPCHK(ctx, hipStreamWaitEvent(ctx->stream, last->ev_noalloc, 0));
     // The array keeps the last call's contents: the histogram starts as zeros
     // (static storage) and every length grouping clears it again before it ends
     // (a kernel, no memset), order[] and cursor[] are written before they are read.
-    return aead_batch(ctx, false, in, out, nullptr, ptr);
+    const int rc = aead_batch(ctx, false, in, out, nullptr, ptr);
+    // (also after a failure: part of the work may have been enqueued)
+    if (hipEventRecord(ctx->ev_noalloc, ctx->stream) == hipSuccess) g_last_user[ctx->device] = ctx;
+    return rc;
     BNK_API_CATCH(ctx)
 }

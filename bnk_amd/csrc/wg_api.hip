@@ -174,19 +174,30 @@ extern "C" int bnk_wg_peer_set(bnk_ctx *ctx, uint32_t row, const bnk_wg_peer *pe
     const uint2 allowed = make_uint2(peer->allowed_net, peer->allowed_mask);
     const uint64_t zero = 0;
     hipStream_t s = ctx->stream;
-    rc = wg_upload_index(ctx, index);
-    if (rc) return rc;
-    HIPCHK(ctx, hipMemcpyAsync(ctx->wg_remote.as<uint32_t>() + row, &peer->remote_index, 4, hipMemcpyHostToDevice, s));
-    HIPCHK(ctx, hipMemcpyAsync(ctx->wg_allowed.as<uint2>() + row, &allowed, 8, hipMemcpyHostToDevice, s));
-    // this row's keypair is new: its nonces and its anti-replay window start
-    // over; every other row goes on
-    HIPCHK(ctx, hipMemcpyAsync(ctx->wg_send_ctr.as<uint64_t>() + row, &zero, 8, hipMemcpyHostToDevice, s));
-    HIPCHK(ctx, hipMemsetAsync(ctx->wg_replay + (size_t)row * WG_REPLAY_WORDS, 0, (size_t)WG_REPLAY_WORDS * 8, s));
-    if (key_send32)
-        HIPCHK(ctx, hipMemcpyAsync(ctx->d_keys[BNK_KEYS_SEND] + 8u * row, key_send32, 32, hipMemcpyHostToDevice, s));
-    if (key_recv32)
-        HIPCHK(ctx, hipMemcpyAsync(ctx->d_keys[BNK_KEYS_RECV] + 8u * row, key_recv32, 32, hipMemcpyHostToDevice, s));
-    HIPCHK(ctx, hipStreamSynchronize(s));
+    // Everything about the row goes up before the index that makes it findable;
+    // a failure part-way leaves tables that disagree, and a half-installed table
+    // is no table (as in bnk_wg_peers_set).
+    auto install = [&]() -> int {
+        HIPCHK(ctx, hipMemcpyAsync(ctx->wg_remote.as<uint32_t>() + row, &peer->remote_index, 4, hipMemcpyHostToDevice, s));
+        HIPCHK(ctx, hipMemcpyAsync(ctx->wg_allowed.as<uint2>() + row, &allowed, 8, hipMemcpyHostToDevice, s));
+        // this row's keypair is new: its nonces and its anti-replay window start
+        // over; every other row goes on
+        HIPCHK(ctx, hipMemcpyAsync(ctx->wg_send_ctr.as<uint64_t>() + row, &zero, 8, hipMemcpyHostToDevice, s));
+        HIPCHK(ctx, hipMemsetAsync(ctx->wg_replay + (size_t)row * WG_REPLAY_WORDS, 0, (size_t)WG_REPLAY_WORDS * 8, s));
+        if (key_send32)
+            HIPCHK(ctx, hipMemcpyAsync(ctx->d_keys[BNK_KEYS_SEND] + 8u * row, key_send32, 32, hipMemcpyHostToDevice, s));
+        if (key_recv32)
+            HIPCHK(ctx, hipMemcpyAsync(ctx->d_keys[BNK_KEYS_RECV] + 8u * row, key_recv32, 32, hipMemcpyHostToDevice, s));
+        if (int irc = wg_upload_index(ctx, index)) return irc;
+        HIPCHK(ctx, hipStreamSynchronize(s));
+        return BNK_OK;
+    };
+    rc = install();
+    if (rc) {
+        ctx->n_wg_peers = 0;
+        ctx->wg_rows.clear();
+        return rc;
+    }
     ctx->wg_rows.swap(rows);
     return BNK_OK;
     BNK_API_CATCH(ctx)

@@ -164,7 +164,8 @@ __global__ __launch_bounds__(256) void wg_encap_prep_kernel(WgBatch b, uint8_t *
     const uint64_t c = pr < pe.n ? counter[i] : 0;
     const uint64_t at = b.off ? b.off[i] : (uint64_t)i * b.stride;
     const uint32_t pad = wg_padding(len, mtu);
-    const bool outside = beyond_arena(at, 16ull + len + pad + 16ull, b.limit);
+    const bool outside = beyond_arena(at, 16ull + len + pad + 16ull, b.limit) ||
+                         (len > MAX_PACKET_BYTES && b.limit != 0); // len + pad must not wrap
     if (outside) status_raise(status, STATUS_BOUNDS);
     if (pr >= pe.n || c >= WG_REJECT_AFTER_MESSAGES || outside) {
         skip[i] = 1;

@@ -18,7 +18,14 @@
  *   - calls on one context are serialised by an internal mutex, so Go may
  *     call from many goroutines (the reference serialises its filter the same
  *     way, internal/filter/filter.go:34,122,190);
- *   - there is no CPU fallback: without a gfx950 device bnk_init fails.
+ *   - there is no CPU fallback: without a gfx950 device bnk_init fails;
+ *   - a BNK_MEM_HOST call that ends with a kernel waits for it by watching a
+ *     word in pinned memory that a last one-thread launch writes, spinning on
+ *     the calling core for up to 100 us before it falls back to
+ *     hipStreamSynchronize (BNK_WAIT_SYNC=1 in the environment at bnk_init:
+ *     always the latter).  A launch that fails is reported by the call that
+ *     made it; BNK_MEM_DEVICE calls only enqueue, so what goes wrong while
+ *     their work runs is reported by the next call that waits (bnk_sync).
  */
 #ifndef BNKHIP_H
 #define BNKHIP_H
@@ -169,9 +176,10 @@ int bnk_aead_open_batch(bnk_ctx *ctx, const bnk_batch *in,
  * until the process ends).  Device-resident batches only (in->mem and out->mem
  * BNK_MEM_DEVICE), at most BNK_NOALLOC_MAX_PACKETS packets, otherwise
  * BNK_E_INVAL.  Results are those of bnk_aead_seal_batch.  Every call on a GPU
- * shares that GPU's array, so two such calls must not overlap on one GPU
- * (calls on one context are serialised on its stream; calls on different
- * contexts of the same GPU race unless the caller orders them). */
+ * shares that GPU's array: calls on one context are serialised on its stream,
+ * and a call on another context of the same GPU first makes its stream wait
+ * (hipStreamWaitEvent, no host wait) for the event the previous user recorded
+ * behind its launches, so such calls take turns on the device. */
 #define BNK_NOALLOC_MAX_PACKETS (1u << 20)
 int bnk_aead_seal_batch_noalloc(bnk_ctx *ctx, const bnk_batch *in,
                                 const bnk_batch *out);

@@ -108,6 +108,105 @@ def test_seal_and_open_skip_packets_outside_the_arena(n, spread_max):
         assert np.array_equal(back.arena(), expect)
 
 
+@pytest.mark.parametrize("n,spread_max", [(300, 4096), (300, 0), (9000, 4096)])
+def test_uniform_input_with_device_output_offsets_is_checked(n, spread_max):
+    """The input is a uniform stride and length (nothing of it lies in device
+    arrays), only the output offsets do: the lanes still check where they write."""
+    import torch
+    from bnk_amd import lib
+    from oracle import binding as O
+    rng = np.random.default_rng(5)
+    L, stride = 200, 224
+    key = rng.integers(0, 256, (1, 32), dtype=np.uint8)
+    plain = rng.integers(0, 256, n * stride, dtype=np.uint8)
+    off = (np.arange(n, dtype=np.uint64) * stride)
+    lens = np.full(n, L, np.uint32)
+    zeros = np.zeros(n, np.uint32)
+    ctrs = np.arange(n, dtype=np.uint64) + 9
+    want = np.full(n * stride, 0x5A, np.uint8)
+    O.seal_batch(key, zeros, ctrs, plain, off, lens, want, off, 4)
+    bad = np.array([2, n // 2, n - 1])
+    out_off = off.copy()
+    out_off[bad[0]] = n * stride + (1 << 33)
+    out_off[bad[1]] = n * stride - L - 8      # ciphertext fits, the tag does not
+    out_off[bad[2]] = n * stride              # starts at the arena's end
+    good = np.ones(n, bool)
+    good[bad] = False
+    with lib.Context(0) as ctx:
+        ctx.set_spread_max_packets(spread_max)
+        ctx.keys_set(lib.KEYS_SEND, key)
+        ctx.keys_set(lib.KEYS_RECV, key)
+        src, dst = Banded(plain), Banded(np.full(n * stride, 0x5A, np.uint8))
+        d_out_off = _dev(out_off.astype(np.int64))
+        torch.cuda.synchronize()
+        ctx.seal(lib.make_batch(src.ptr, plain.nbytes, n, lib.MEM_DEVICE, stride=stride, length=L, counter0=9),
+                 lib.make_batch(dst.ptr, plain.nbytes, n, lib.MEM_DEVICE, offsets=d_out_off))
+        _expect_inval(ctx)
+        assert src.guards_intact() and dst.guards_intact()
+        expect = np.full(n * stride, 0x5A, np.uint8)
+        for i in np.flatnonzero(good):
+            o = int(off[i])
+            expect[o:o + L + 16] = want[o:o + L + 16]
+        assert np.array_equal(dst.arena(), expect)
+
+        # open of the oracle's sealed packets, plaintexts to checked offsets
+        sealed, back = Banded(want), Banded(np.full(n * stride, 0xA5, np.uint8))
+        out_off[bad[1]] = n * stride - L + 3  # the plaintext itself sticks out
+        d_out_off = _dev(out_off.astype(np.int64))
+        v = torch.full((n,), 7, dtype=torch.uint8, device="cuda:0")
+        torch.cuda.synchronize()
+        ctx.open(lib.make_batch(sealed.ptr, plain.nbytes, n, lib.MEM_DEVICE, stride=stride, length=L + 16,
+                                counter0=9),
+                 lib.make_batch(back.ptr, plain.nbytes, n, lib.MEM_DEVICE, offsets=d_out_off), v)
+        _expect_inval(ctx)
+        assert sealed.guards_intact() and back.guards_intact()
+        assert np.array_equal(v.cpu().numpy(), good.astype(np.uint8))
+        expect = np.full(n * stride, 0xA5, np.uint8)
+        for i in np.flatnonzero(good):
+            o = int(off[i])
+            expect[o:o + L] = plain[o:o + L]
+        assert np.array_equal(back.arena(), expect)
+
+
+@pytest.mark.parametrize("n,spread_max", [(300, 4096), (9000, 4096)])
+def test_length_words_near_2_to_32_do_not_wrap_past_the_check(n, spread_max):
+    """len + 16 and len + padding are not 32-bit sums: a length word of
+    0xFFFFFFF0 or more in an arena of any size is refused, not wrapped to a
+    small number that passes."""
+    import torch
+    from bnk_amd import lib
+    from oracle import binding as O
+    b = W.aead_imix(43, n, n_peers=4)
+    keys = np.ascontiguousarray(b.keys)
+    total = b.plain.nbytes
+    want = np.zeros_like(b.plain)
+    O.seal_batch(keys, b.peer, b.counters, b.plain, b.off, b.lens, want, b.off, 4)
+    bad = np.array([1, n // 2, n - 2])
+    lens = b.lens.copy()
+    lens[bad] = [0xFFFFFFF0, 0xFFFFFFFF, 0xFFFFFFF5]
+    good = np.ones(n, bool)
+    good[bad] = False
+    with lib.Context(0) as ctx:
+        ctx.set_spread_max_packets(spread_max)
+        ctx.keys_set(lib.KEYS_SEND, keys)
+        src, dst = Banded(b.plain), Banded(np.full(total, 0x5A, np.uint8))
+        d_off, d_lens = _dev(b.off.astype(np.int64)), _dev(lens.view(np.int32))
+        d_peer, d_ctr = _dev(b.peer.astype(np.int32)), _dev(b.counters.astype(np.int64))
+        torch.cuda.synchronize()
+        # the declared arena size is beyond 4 GiB, so that only a wrapped sum could pass
+        # for the offenders (the good packets all lie within the real allocation)
+        ctx.seal(lib.make_batch(src.ptr, 1 << 33, n, lib.MEM_DEVICE, offsets=d_off, lens=d_lens, peer=d_peer,
+                                counters=d_ctr),
+                 lib.make_batch(dst.ptr, 1 << 33, n, lib.MEM_DEVICE, offsets=d_off))
+        _expect_inval(ctx)
+        assert src.guards_intact() and dst.guards_intact()
+        expect = np.full(total, 0x5A, np.uint8)
+        for i in np.flatnonzero(good):
+            o, L = int(b.off[i]), int(b.lens[i]) + 16
+            expect[o:o + L] = want[o:o + L]
+        assert np.array_equal(dst.arena(), expect)
+
+
 def test_filter_skips_packets_outside_the_arena():
     import torch
     from bnk_amd import lib

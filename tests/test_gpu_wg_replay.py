@@ -214,3 +214,126 @@ def test_a_rekeyed_peer_starts_with_an_empty_window_and_the_switch_turns_windows
         assert decap(ctx, [dg(2, 9), dg(2, 9)]) == [lib.WG_OK, lib.WG_OK]
         ctx.wg_set_replay(True)
         assert decap(ctx, [dg(2, 9), dg(2, 9)]) == [lib.WG_OK, lib.WG_REPLAY]
+
+
+def _traffic(tx_ctx, tx_peers, n_a, n_b, n_total, inner_len, jump_rows, rng):
+    """Datagrams for a large decapsulating batch without a per-packet oracle:
+    two encapsulated batches (between them some peers' send counters jump ahead
+    by more than a window, so that the first batch's packets of those peers are
+    too old once a second-batch packet has been seen), then a shuffled mix of
+    both with repeats.  Returns the wire arena, offsets, lengths, and each
+    datagram's sender and counter as the sending side knows them."""
+    from bnk_amd import lib
+    n_peers = len(tx_peers)
+    slot = (16 + inner_len + 15 + 16 + 15) & ~15
+    per = []
+    for k, n in enumerate((n_a, n_b)):
+        peer = rng.integers(0, n_peers, n).astype(np.uint32)
+        # half of either batch belongs to the peers that jump, so that they have old
+        # packets to be refused and new ones to refuse them
+        peer[: n // 2] = rng.choice(jump_rows, n // 2).astype(np.uint32)
+        arena = rng.integers(0, 256, n * slot, dtype=np.uint8)
+        for i in range(n):
+            o = i * slot + 16
+            arena[o] = 0x45
+            arena[o + 2:o + 4] = np.frombuffer(int(inner_len).to_bytes(2, "big"), np.uint8)
+            arena[o + 12:o + 16] = np.frombuffer(int(tx_peers[int(peer[i])][2]).to_bytes(4, "big"), np.uint8)
+        wl = np.zeros(n, np.uint32)
+        if k == 1:
+            for r in jump_rows:
+                tx_ctx.wg_send_counter_set(int(r), 9000 + int(r) % 7)
+        tx_ctx.wg_encap(lib.make_batch(arena, arena.nbytes, n, lib.MEM_HOST, stride=slot, length=inner_len,
+                                       peer=peer), 1420, wl)
+        assert (wl == 16 + ((inner_len + 15) & ~15) + 16).all()
+        per.append((arena.reshape(n, slot), peer, int(wl[0])))
+    wire_len = per[0][2]
+    src = np.concatenate([per[0][0], per[1][0]])[:, :wire_len]
+    src_peer = np.concatenate([per[0][1], per[1][1]])
+    pick = np.concatenate([np.arange(n_a + n_b), rng.integers(0, n_a + n_b, n_total - n_a - n_b)])
+    rng.shuffle(pick)
+    stride = (wire_len + 15) & ~15
+    wire = np.zeros((n_total, stride), np.uint8)
+    wire[:, :wire_len] = src[pick]
+    ctr = wire[:, 8:16].copy().view("<u8").reshape(-1)
+    return wire.reshape(-1), stride, wire_len, src_peer[pick], ctr
+
+
+def _window_expectation(peer, ctr, n_peers_seen):
+    from bnk_amd import lib
+    from oracle import binding as O
+    filters = {}
+    want = np.zeros(len(peer), np.uint8)
+    for i in range(len(peer)):
+        f = filters.setdefault(int(peer[i]), O.ReplayFilter())
+        want[i] = lib.WG_OK if f.validate(int(ctr[i])) else lib.WG_REPLAY
+    return want
+
+
+def test_window_pass_with_more_peers_than_a_packed_sort_key_holds():
+    """70,000 peers and 40,000 packets: the sender's number and the packet's
+    position no longer fit one 32-bit sort key, so the window pass sorts
+    (sender, position) pairs.  Expected results come from the sequential
+    filter fed, in batch order, the senders and counters the sending side
+    assigned."""
+    import torch
+    from bnk_amd import lib
+    rng = np.random.default_rng(77)
+    n_peers, n_total = 70000, 40000
+    tx = [(10 + 3 * i, 500000 + 5 * i, 0x64400000 + i, 0xFFFFFFFF) for i in range(n_peers)]
+    rx = [(p[1], p[0], p[2], p[3]) for p in tx]
+    keys = rng.integers(0, 256, (n_peers, 32), dtype=np.uint8)
+    jump_rows = rng.choice(n_peers, 300, replace=False)
+    with lib.Context(0) as txc, lib.Context(0) as rxc:
+        txc.keys_set(lib.KEYS_SEND, keys)
+        txc.wg_peers_set(tx)
+        rxc.keys_set(lib.KEYS_RECV, keys)
+        rxc.wg_peers_set(rx)
+        wire, stride, wire_len, peer, ctr = _traffic(txc, tx, 12000, 8000, n_total, 40, jump_rows, rng)
+        want = _window_expectation(peer, ctr, n_peers)
+        d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to("cuda:0")  # noqa: E731
+        d_wire, d_out = d(wire), torch.zeros(wire.nbytes, dtype=torch.uint8, device="cuda:0")
+        res = torch.zeros(n_total, dtype=torch.uint8, device="cuda:0")
+        olen = torch.zeros(n_total, dtype=torch.int32, device="cuda:0")
+        gp = torch.zeros(n_total, dtype=torch.int32, device="cuda:0")
+        gc = torch.zeros(n_total, dtype=torch.int64, device="cuda:0")
+        torch.cuda.synchronize()
+        rxc.wg_decap(lib.make_batch(d_wire, wire.nbytes, n_total, lib.MEM_DEVICE, stride=stride, length=wire_len),
+                     lib.make_batch(d_out, wire.nbytes, n_total, lib.MEM_DEVICE, stride=stride), res, olen, gp, gc)
+        rxc.sync()
+        assert np.array_equal(gp.cpu().numpy().astype(np.uint32), peer)
+        assert np.array_equal(gc.cpu().numpy().astype(np.uint64), ctr)
+        got = res.cpu().numpy()
+        bad = np.flatnonzero(got != want)
+        assert bad.size == 0, f"result differs at {bad[:5]}: got {got[bad[:5]]} want {want[bad[:5]]}"
+        assert (want == lib.WG_REPLAY).sum() > 1000 and (want == lib.WG_OK).sum() > 1000
+        assert np.array_equal(olen.cpu().numpy() != 0, want == lib.WG_OK)
+
+
+def test_window_pass_of_a_host_batch_that_goes_through_in_chunks():
+    """A host batch beyond the size that runs in one piece is cut into chunks,
+    each with a window pass of its own continuing the one before: results are
+    those of the sequential filter over the whole batch in order."""
+    from bnk_amd import lib
+    rng = np.random.default_rng(78)
+    n_peers, n_total = 40, 14000
+    tx = [(100 + 3 * i, 9000 + 5 * i, 0x64400000 + i, 0xFFFFFFFF) for i in range(n_peers)]
+    rx = [(p[1], p[0], p[2], p[3]) for p in tx]
+    keys = rng.integers(0, 256, (n_peers, 32), dtype=np.uint8)
+    with lib.Context(0) as txc, lib.Context(0) as rxc:
+        txc.keys_set(lib.KEYS_SEND, keys)
+        txc.wg_peers_set(tx)
+        rxc.keys_set(lib.KEYS_RECV, keys)
+        rxc.wg_peers_set(rx)
+        wire, stride, wire_len, peer, ctr = _traffic(txc, tx, 6000, 5000, n_total, 1400, np.arange(0, n_peers, 3),
+                                                     rng)
+        assert wire.nbytes > (16 << 20)  # well beyond two chunks' worth
+        want = _window_expectation(peer, ctr, n_peers)
+        out = np.zeros(wire.nbytes, np.uint8)
+        res, olen = np.zeros(n_total, np.uint8), np.zeros(n_total, np.uint32)
+        gp, gc = np.zeros(n_total, np.uint32), np.zeros(n_total, np.uint64)
+        rxc.wg_decap(lib.make_batch(wire, wire.nbytes, n_total, lib.MEM_HOST, stride=stride, length=wire_len),
+                     lib.make_batch(out, out.nbytes, n_total, lib.MEM_HOST, stride=stride), res, olen, gp, gc)
+        assert np.array_equal(gp, peer) and np.array_equal(gc, ctr)
+        bad = np.flatnonzero(res != want)
+        assert bad.size == 0, f"result differs at {bad[:5]}: got {res[bad[:5]]} want {want[bad[:5]]}"
+        assert (want == lib.WG_REPLAY).sum() > 1000 and (want == lib.WG_OK).sum() > 1000

@@ -18,7 +18,7 @@ Prints ONE JSON line.  Besides the contract fields it carries
                  baseline, what one call costs on 128 packets in pinned host rings, and the
                  rates of configurations 3 and 5 and of the transport framing
 
---workload filter | imix | relay | wg | host | latency | copy | sizes | issue print one line for that
+--workload filter | imix | relay | wg | host | latency | callers | copy | sizes | issue print one line for that
 workload alone; --no-extras leaves out everything but the timed launches (for traces).
 """
 from __future__ import annotations
@@ -662,6 +662,75 @@ def bench_latency(args) -> dict:
     }
 
 
+def bench_callers(args) -> dict:
+    """The reference's calling pattern: T threads, each one per-peer goroutine's worth of
+    blocking calls of 128 packets x 1420 B from its own part of a pinned ring
+    (internal/filter/filter.go:160-186, internal/magicsock/bind.go:326-328, 372-377), through
+    the library as it is (one call at a time behind the context lock) and with the library
+    merging them (bnk_set_coalesce).  The load generator is native code over the C ABI
+    (bnk_amd/host/bnk_callers.cpp): Python threads would measure the interpreter lock."""
+    import ctypes as C
+    import numpy as np
+    from bnk_amd import lib, workloads as W
+    so = C.CDLL(os.path.join(ROOT, "bnk_amd", "libbnkcallers.so"))
+
+    class Result(C.Structure):
+        _fields_ = [("seconds", C.c_double), ("calls", C.c_uint64), ("packets", C.c_uint64),
+                    ("plaintext_bytes", C.c_uint64), ("out_p50_us", C.c_double), ("out_p99_us", C.c_double),
+                    ("out_max_us", C.c_double), ("in_p50_us", C.c_double), ("in_p99_us", C.c_double),
+                    ("in_max_us", C.c_double), ("rc", C.c_int), ("mismatches", C.c_uint64),
+                    ("filtered", C.c_uint64)]
+
+    t_max, per_call, rounds, warm = 16, 128, max(args.steps, 20) * 4, 10
+    window_packets, wait_us = 4096, 30
+    ctx = lib.Context(0)
+    keys = W.rand_bytes(W.stream_seed(2, 7), t_max * 32).reshape(t_max, 32)
+    ctx.keys_set(lib.KEYS_SEND, keys)
+    ctx.keys_set(lib.KEYS_RECV, keys)
+    # a peer table that loops back: what a peer sends is addressed to itself
+    ctx.wg_peers_set([(0x1000 + 37 * t, 0x1000 + 37 * t, W.CGNAT_BASE + t, 0xFFFFFFFF) for t in range(t_max)])
+    ctx.filter_set_rules([([(W.CGNAT_BASE, 10)], "tcp", [(8000, 8000)])])
+    now = 1_700_000_000 * 10**9
+    rows = []
+    for workload, name, legs in ((0, "seal + open", ("seal", "open")),
+                                 (1, "NoteOutbound + encapsulate, decapsulate + CheckInbound",
+                                  ("note_encap", "decap_filter"))):
+        for threads in (1, 4, 16):
+            for merged in (False, True):
+                ctx.set_coalesce(window_packets if merged else 0, wait_us)
+                s0 = ctx.coalesce_stats()
+                r = Result()
+                rc = so.bnkc_run(C.c_void_p(ctx._h.value), C.c_int(workload), C.c_uint32(threads),
+                                 C.c_uint32(per_call), C.c_uint32(L), C.c_uint32(rounds), C.c_uint32(warm),
+                                 C.c_int64(now), C.byref(r))
+                if rc != 0 or r.mismatches:
+                    raise RuntimeError("callers workload failed: rc %d, %d mismatches" % (rc, r.mismatches))
+                s1 = ctx.coalesce_stats()
+                calls, batches = s1["calls"] - s0["calls"], s1["batches"] - s0["batches"]
+                rows.append({
+                    "calls": name, "threads": threads, "mode": "merged" if merged else "direct",
+                    "gbit_per_s_round_trip": round(r.plaintext_bytes * 8e-9 / r.seconds, 1),
+                    "gbit_per_s_per_direction": round(2 * r.plaintext_bytes * 8e-9 / r.seconds, 1),
+                    "us_per_call": {legs[0]: {"p50": round(r.out_p50_us, 1), "p99": round(r.out_p99_us, 1)},
+                                    legs[1]: {"p50": round(r.in_p50_us, 1), "p99": round(r.in_p99_us, 1)}},
+                    "calls_per_launch": round(calls / batches, 2) if batches else 1.0,
+                    "windows": batches,
+                    "windows_that_waited_in_vain": s1["timed_out"] - s0["timed_out"],
+                })
+    ctx.set_coalesce(0)
+    ctx.close()
+    best = max((x for x in rows if x["threads"] == 16 and x["mode"] == "merged" and x["calls"] == "seal + open"),
+               key=lambda x: x["gbit_per_s_round_trip"])
+    return {"metric": "callers_seal_open_gbit_per_s_16_threads_merged", "value": best["gbit_per_s_round_trip"],
+            "unit": "Gbit/s", "n_gpus": 1, "higher_is_better": True, "data": "synthetic", "dtype": "u32",
+            "config": {"workload": "T threads x blocking calls of %d packets x %d B in one pinned ring, each thread "
+                                   "a round trip per round (plaintext counted once per round trip); direct = one "
+                                   "call at a time behind the context lock, merged = bnk_set_coalesce(%d packets, "
+                                   "%d us)" % (per_call, L, window_packets, wait_us),
+                       "rounds": rounds, "host_cpus": os.cpu_count()},
+            "rows": rows}
+
+
 def bench_sizes(args) -> dict:
     """Seal and open of 2^20 packets of one common length, for each of a list
     of lengths (--sizes, default the three IMIX sizes): how far short packets
@@ -766,7 +835,7 @@ def main() -> int:
                     help="untimed steps first: a chip that was idle needs some 50 ms of work to reach the "
                          "clocks it then holds (the first 20 steps run about 5 %% slower)")
     ap.add_argument("--packets", type=int, default=1 << 20)
-    ap.add_argument("--workload", default="aead", choices=["aead", "filter", "imix", "relay", "wg", "host", "latency", "copy", "sizes", "issue"],
+    ap.add_argument("--workload", default="aead", choices=["aead", "filter", "imix", "relay", "wg", "host", "latency", "callers", "copy", "sizes", "issue"],
                     help="aead (default, the headline line, with the ACL filter rate as an extra); "
                          "filter / imix / relay / wg / host / latency / copy print one line for that workload alone")
     ap.add_argument("--sizes", default="60,576,1420", help="sizes: packet lengths, comma separated")
@@ -795,7 +864,8 @@ def main() -> int:
         return 2
     if args.workload != "aead":
         out = {"filter": bench_filter, "imix": bench_imix, "relay": bench_relay,
-               "wg": bench_wg, "host": bench_host, "latency": bench_latency, "copy": bench_copy, "issue": bench_issue,
+               "wg": bench_wg, "host": bench_host, "latency": bench_latency, "callers": bench_callers,
+               "copy": bench_copy, "issue": bench_issue,
                "sizes": bench_sizes}[args.workload](args)
         print(json.dumps(out))
         return 0
@@ -1074,6 +1144,19 @@ def main() -> int:
         "workload": lat["config"]["workload"],
         **lat["per_batch_size_us"]["128"],
     }
+    # the same calls from 16 threads at once, the way wireguard-go's per-peer goroutines
+    # make them, one at a time behind the context lock and merged by the library
+    try:
+        cargs = argparse.Namespace(**vars(args))
+        cargs.steps = 20
+        cal = bench_callers(cargs)
+        out["extra"]["callers_16_threads_x_128_packets"] = {
+            "unit": "Gbit/s of plaintext through a round trip (both calls); us per call",
+            "workload": cal["config"]["workload"],
+            "rows": [r for r in cal["rows"] if r["threads"] == 16],
+        }
+    except Exception as e:  # a side measurement must not take the headline line with it
+        out["extra"]["callers_16_threads_x_128_packets"] = {"error": "%s: %s" % (type(e).__name__, e)}
     # the other configurations the path is specified on, each a short run of its own
     # workload (their full lines: --workload imix | relay | wg)
     others = {}

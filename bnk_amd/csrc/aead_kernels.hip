@@ -984,13 +984,22 @@ __global__ __launch_bounds__(256) void aead_spread_kernel(AeadArgs a)
     const uint32_t at = 64u * (lane - 1u);
     const uint32_t mine = (lane == 0 || at >= data_len) ? 0u : min(data_len - at, 64u);
     const uint32_t there = (lane == 0 || at >= data_there) ? 0u : min(data_there - at, 64u);
-    uint32_t m[16];
+    // The wave fetches the packet in pieces of 1 KB, lane l taking bytes [16 l,
+    // 16 l + 16) of each piece, so that an instruction reads 1 KB in a row; the
+    // lanes pick their own 64-byte blocks out of LDS further down.  (A lane
+    // fetching its own block reads 16 bytes every 64: sixty-four small requests
+    // an instruction, which a packet that lies in host memory pays for with a
+    // read of its own over the link for each.)
+    uint4 pre[4];
 #pragma unroll
     for (int j = 0; j < 4; j++) {
+        const uint32_t off = 1024u * j + 16u * lane;
         uint4 v = make_uint4(0, 0, 0, 0);
-        if (there >= 16u * (j + 1)) v = ld16(data + at + 16 * j);
-        else if (there > 16u * j) v = ld_partial(data + at + 16 * j, there - 16u * j);
-        m[4 * j] = v.x; m[4 * j + 1] = v.y; m[4 * j + 2] = v.z; m[4 * j + 3] = v.w;
+        if (1024u * j < data_there) { // (the same for the whole wave)
+            if (off + 16u <= data_there) v = ld16(data + off);
+            else if (off < data_there) v = ld_partial(data + off, data_there - off);
+        }
+        pre[j] = v;
     }
     uint4 want_tag = make_uint4(0, 0, 0, 0);
     if (OPEN && (WG ? len >= 32u && len - 32u <= WG_FUSE_MAX_LEN : len >= 16u && data_len <= SPREAD_MAX_LEN))
@@ -1094,6 +1103,22 @@ __global__ __launch_bounds__(256) void aead_spread_kernel(AeadArgs a)
 
     // (the packet's bytes are already on their way: see the top of the kernel)
     chacha_block(k, lane, n1, n2, x);
+    // Block b of the packet lies at stage + 80 b (rows padded against bank
+    // conflicts): written in the order the pieces came in, read a block per lane.
+    uint8_t *stage = tile_all[threadIdx.x >> 6];
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+        if (1024u * j < data_there)
+            *reinterpret_cast<uint4 *>(stage + (16u * j + (lane >> 2)) * LDS_ROW + 16u * (lane & 3u)) = pre[j];
+    wave_sync();
+    uint32_t m[16];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        uint4 v = make_uint4(0, 0, 0, 0);
+        // (bytes of a cell beyond the data were fetched as zeros)
+        if (there > 16u * j) v = *reinterpret_cast<const uint4 *>(stage + (lane - 1u) * LDS_ROW + 16u * j);
+        m[4 * j] = v.x; m[4 * j + 1] = v.y; m[4 * j + 2] = v.z; m[4 * j + 3] = v.w;
+    }
     // the one-time key is lane 0's block
     const Fe26 r = fe_clamped_r((uint32_t)__builtin_amdgcn_readlane((int)x[0], 0),
                                 (uint32_t)__builtin_amdgcn_readlane((int)x[1], 0),
@@ -1176,13 +1201,24 @@ __global__ __launch_bounds__(256) void aead_spread_kernel(AeadArgs a)
             a.wg.counter_out[i] = ctr;
         }
     }
-    // ---- my bytes out; a rejected packet leaves zeros (chacha20poly1305.Open) ----
+    // ---- the bytes out, the way they came in: blocks into LDS, pieces of 1 KB in
+    // a row out of it; a rejected packet leaves zeros (chacha20poly1305.Open) ----
+    wave_sync();
 #pragma unroll
     for (int j = 0; j < 4; j++) {
         const uint4 v = reject ? make_uint4(0, 0, 0, 0)
                                : make_uint4(o[4 * j], o[4 * j + 1], o[4 * j + 2], o[4 * j + 3]);
-        if (mine >= 16u * (j + 1)) st16(dst + at + 16 * j, v);
-        else if (mine > 16u * j) st_partial(dst + at + 16 * j, v, mine - 16u * j);
+        if (mine > 16u * j) *reinterpret_cast<uint4 *>(stage + (lane - 1u) * LDS_ROW + 16u * j) = v;
+    }
+    wave_sync();
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const uint32_t off = 1024u * j + 16u * lane;
+        if (1024u * j < data_len && off < data_len) {
+            const uint4 v = *reinterpret_cast<const uint4 *>(stage + (16u * j + (lane >> 2)) * LDS_ROW + 16u * (lane & 3u));
+            if (off + 16u <= data_len) st16(dst + off, v);
+            else st_partial(dst + off, v, data_len - off);
+        }
     }
 }
 

@@ -105,13 +105,18 @@ int aead_batch_host_direct(bnk_ctx *ctx, bool open, const bnk_batch *in, const b
     if (rc) return rc;
     rc = scan_host_layout(ctx, out, in, open ? -16 : 16, &sout, "out");
     if (rc) return rc;
-    if (sin.size() > DIRECT_MAX_BYTES) return 1;
+    // A launch of a wave per packet reads every packet where it lies, so only the
+    // packets' own bytes count; a lane per packet first fetches the whole span.
+    a.lens = in->lens; // (for aead_runs_spread only whether there is one matters; set properly below)
+    const uint64_t moved = aead_runs_spread(a) ? host_payload_bytes(in) : sin.size();
+    if (moved > DIRECT_MAX_BYTES) return 1;
     rc = check_index_range(ctx, in->peer, n, a.n_peers, "peer index", "the key table");
     if (rc) return rc;
 
     // pinned staging: three 8-byte arrays, three 4-byte arrays, verdict bytes
-    HIPCHK(ctx, ctx->pin.reserve((size_t)n * 37 + 64));
-    uint8_t *pin = ctx->pin.as<uint8_t>();
+    PinBuf &stage = *ctx->pin_cur;
+    HIPCHK(ctx, stage.reserve((size_t)n * 37 + 64));
+    uint8_t *pin = stage.as<uint8_t>();
     uint64_t *p_in_off = (uint64_t *)pin, *p_out_off = p_in_off + n, *p_ctr = p_out_off + n;
     uint32_t *p_lens = (uint32_t *)(p_ctr + n), *p_peer = p_lens + n, *p_order = p_peer + n;
     uint8_t *p_verdict = (uint8_t *)(p_order + n);
@@ -121,7 +126,7 @@ int aead_batch_host_direct(bnk_ctx *ctx, bool open, const bnk_batch *in, const b
     // into device memory by one wide copy kernel, at the same position within a
     // 128-byte line so that whole lines can be moved.  Either way the output
     // goes straight into the ring, where stores need no round trip.
-    a.lens = in->lens ? ctx->pin.dev(p_lens) : nullptr;
+    a.lens = in->lens ? stage.dev(p_lens) : nullptr;
     if (aead_runs_spread(a)) {
         a.in = d_in + sin.lo;
     } else {
@@ -133,14 +138,14 @@ int aead_batch_host_direct(bnk_ctx *ctx, bool open, const bnk_batch *in, const b
     a.out = d_out;
     if (in->offsets) {
         for (uint32_t i = 0; i < n; i++) p_in_off[i] = in->offsets[i] - sin.lo;
-        a.in_off = ctx->pin.dev(p_in_off);
+        a.in_off = stage.dev(p_in_off);
     }
-    if (out->offsets) { memcpy(p_out_off, out->offsets, (size_t)n * 8); a.out_off = ctx->pin.dev(p_out_off); }
-    if (in->counters) { memcpy(p_ctr, in->counters, (size_t)n * 8); a.counters = ctx->pin.dev(p_ctr); }
-    if (in->peer) { memcpy(p_peer, in->peer, (size_t)n * 4); a.peer = ctx->pin.dev(p_peer); }
+    if (out->offsets) { memcpy(p_out_off, out->offsets, (size_t)n * 8); a.out_off = stage.dev(p_out_off); }
+    if (in->counters) { memcpy(p_ctr, in->counters, (size_t)n * 8); a.counters = stage.dev(p_ctr); }
+    if (in->peer) { memcpy(p_peer, in->peer, (size_t)n * 4); a.peer = stage.dev(p_peer); }
     if (in->lens) {
         memcpy(p_lens, in->lens, (size_t)n * 4);
-        a.lens = ctx->pin.dev(p_lens);
+        a.lens = stage.dev(p_lens);
         if (n > 64 && !aead_runs_spread(a)) {
             // lanes of a wave should run equal block counts: longest first
             const uint32_t tag = open ? 16 : 0;
@@ -155,17 +160,15 @@ int aead_batch_host_direct(bnk_ctx *ctx, bool open, const bnk_batch *in, const b
                 for (uint32_t i = 0; i < n; i++) at[most - blocks(i) + 1]++;
                 for (uint32_t b = 0; b <= most; b++) at[b + 1] += at[b];
                 for (uint32_t i = 0; i < n; i++) p_order[at[most - blocks(i)]++] = i;
-                a.order = ctx->pin.dev(p_order);
+                a.order = stage.dev(p_order);
             }
         }
     }
-    if (open) a.verdict = ctx->pin.dev(p_verdict);
+    if (open) a.verdict = stage.dev(p_verdict);
     HIPCHK(ctx, open ? launch_aead_open(a, ctx->stream) : launch_aead_seal(a, ctx->stream));
     // host batches have had their peer indices checked above, so the kernel
     // has nothing to report through the status word
-    if (int wrc = wait_stream(ctx)) return wrc;
-    if (open) memcpy(verdict, p_verdict, n);
-    return BNK_OK;
+    return finish_direct(ctx, false, {{verdict, p_verdict, open ? (size_t)n : 0}});
 }
 
 // Device batches cannot be walked on the host; check what is uniform.
@@ -300,17 +303,26 @@ int aead_batch(bnk_ctx *ctx, bool open, const bnk_batch *in, const bnk_batch *ou
 // on this runtime whichever way the host waits.  BNK_WAIT_SYNC=1 in the environment at
 // bnk_init switches the watch off (every wait is hipStreamSynchronize).
 constexpr int64_t WAIT_WATCH_US = 100;
-int wait_stream(bnk_ctx *ctx)
+int post_ticket(bnk_ctx *ctx, uint32_t *ticket)
 {
     const uint32_t seq = ++ctx->wait_seq;
-    if (!ctx->wait_sync_only &&
-        launch_done_word(ctx->d_status + STATUS_DONE_WORD, seq, ctx->stream) == hipSuccess) {
+    *ticket = seq;
+    HIPCHK(ctx, launch_done_word(ctx->d_status + STATUS_DONE_WORD, seq, ctx->stream));
+    return BNK_OK;
+}
+
+// May be called without the context lock: it reads the watched word and, past
+// the watch, waits for the stream as a whole (which then includes whatever
+// other callers have enqueued behind the ticket).
+int wait_ticket(bnk_ctx *ctx, uint32_t ticket)
+{
+    if (!ctx->wait_sync_only) {
         volatile uint32_t *done = ctx->h_status + STATUS_DONE_WORD;
         const auto t0 = std::chrono::steady_clock::now();
         for (;;) {
             for (int spin = 0; spin < 64; spin++) {
                 // (numbers are handed out in stream order: a later one also means done)
-                if ((int32_t)(*done - seq) >= 0) {
+                if ((int32_t)(*done - ticket) >= 0) {
                     std::atomic_thread_fence(std::memory_order_acquire);
                     HIPCHK(ctx, hipGetLastError());
                     return BNK_OK;
@@ -326,6 +338,35 @@ int wait_stream(bnk_ctx *ctx)
     return BNK_OK;
 }
 
+int wait_stream(bnk_ctx *ctx)
+{
+    uint32_t ticket;
+    if (ctx->wait_sync_only || post_ticket(ctx, &ticket) != BNK_OK) {
+        HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+        return BNK_OK;
+    }
+    return wait_ticket(ctx, ticket);
+}
+
+int finish_direct(bnk_ctx *ctx, bool with_status, std::initializer_list<Deferred> copies)
+{
+    if (ctx->defer) {
+        for (const Deferred &c : copies)
+            if (c.bytes) ctx->defer->push_back(c);
+        ctx->defer_status = with_status;
+        return BNK_DEFERRED;
+    }
+    uint32_t status = 0;
+    if (with_status) {
+        if (int rc = take_status(ctx, &status, true)) return rc;
+    } else {
+        if (int rc = wait_stream(ctx)) return rc;
+    }
+    for (const Deferred &c : copies)
+        if (c.bytes) memcpy(c.dst, c.src, c.bytes);
+    return status_to_rc(ctx, status);
+}
+
 // Waits for the stream, then reads and clears the status words.  after_kernel: the
 // last thing enqueued is a kernel (behind a copy the watched word comes later than the
 // copy's own completion does).
@@ -336,15 +377,21 @@ int take_status(bnk_ctx *ctx, uint32_t *status, bool after_kernel)
     } else {
         HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
     }
+    *status = read_status_words(ctx);
+    return BNK_OK;
+}
+
+uint32_t read_status_words(bnk_ctx *ctx)
+{
     volatile uint32_t *h = ctx->h_status;
-    *status = (h[STATUS_PEER_RANGE] ? STATUS_PEER_RANGE : 0u) | (h[STATUS_FLOWS_FULL] ? STATUS_FLOWS_FULL : 0u) |
-              (h[STATUS_BOUNDS] ? STATUS_BOUNDS : 0u);
-    if (*status) {
+    const uint32_t status = (h[STATUS_PEER_RANGE] ? STATUS_PEER_RANGE : 0u) |
+                            (h[STATUS_FLOWS_FULL] ? STATUS_FLOWS_FULL : 0u) | (h[STATUS_BOUNDS] ? STATUS_BOUNDS : 0u);
+    if (status) {
         h[STATUS_PEER_RANGE] = 0;
         h[STATUS_FLOWS_FULL] = 0;
         h[STATUS_BOUNDS] = 0;
     }
-    return BNK_OK;
+    return status;
 }
 
 int status_to_rc(bnk_ctx *ctx, uint32_t status)
@@ -442,6 +489,7 @@ void bnk_shutdown(bnk_ctx *ctx)
                           &ctx->r_heads, &ctx->wg_hash})
             b->release();
         ctx->pin.release();
+        for (HostStage &st : ctx->stages) st.pin.release();
         if (ctx->wg_replay) (void)hipFree(ctx->wg_replay);
         for (const bnk_ctx::Ring &r : ctx->rings) (void)hipHostFree(reinterpret_cast<void *>(r.host));
         ctx->rings.clear();
@@ -494,6 +542,7 @@ int bnk_ring_alloc(bnk_ctx *ctx, size_t bytes, void **host_pinned)
         (void)hipGetLastError();
     }
     try {
+        std::lock_guard<std::mutex> rl(ctx->rings_mu);
         ctx->rings.push_back({(uintptr_t)*host_pinned, (uint8_t *)dev, bytes});
     } catch (...) {
         (void)hipHostFree(*host_pinned);
@@ -511,11 +560,14 @@ int bnk_ring_free(bnk_ctx *ctx, void *host_pinned)
     if (g.rc) return g.rc;
     if (!host_pinned) return BNK_OK;
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
-    for (size_t i = 0; i < ctx->rings.size(); i++)
-        if (ctx->rings[i].host == (uintptr_t)host_pinned) {
-            ctx->rings.erase(ctx->rings.begin() + i);
-            break;
-        }
+    {
+        std::lock_guard<std::mutex> rl(ctx->rings_mu);
+        for (size_t i = 0; i < ctx->rings.size(); i++)
+            if (ctx->rings[i].host == (uintptr_t)host_pinned) {
+                ctx->rings.erase(ctx->rings.begin() + i);
+                break;
+            }
+    }
     HIPCHK(ctx, hipHostFree(host_pinned));
     return BNK_OK;
     BNK_API_CATCH(ctx)
@@ -622,6 +674,11 @@ int bnk_keys_set(bnk_ctx *ctx, int which, const uint8_t *keys32, uint32_t n_peer
 int bnk_aead_seal_batch(bnk_ctx *ctx, const bnk_batch *in, const bnk_batch *out)
 {
     BNK_API_TRY
+    {
+        CoRequest rq{CO_SEAL, in, out, 0, 0, nullptr, nullptr, nullptr, nullptr};
+        int crc;
+        if (out && coalesce_submit(ctx, rq, &crc)) return crc;
+    }
     Guard g(ctx);
     if (g.rc) return g.rc;
     return aead_batch(ctx, false, in, out, nullptr, nullptr);
@@ -631,6 +688,11 @@ int bnk_aead_seal_batch(bnk_ctx *ctx, const bnk_batch *in, const bnk_batch *out)
 int bnk_aead_open_batch(bnk_ctx *ctx, const bnk_batch *in, const bnk_batch *out, uint8_t *verdict)
 {
     BNK_API_TRY
+    {
+        CoRequest rq{CO_OPEN, in, out, 0, 0, verdict, nullptr, nullptr, nullptr};
+        int crc;
+        if (out && coalesce_submit(ctx, rq, &crc)) return crc;
+    }
     Guard g(ctx);
     if (g.rc) return g.rc;
     return aead_batch(ctx, true, in, out, verdict, nullptr);

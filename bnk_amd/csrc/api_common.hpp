@@ -6,6 +6,7 @@
 
 #include <algorithm>
 #include <functional>
+#include <initializer_list>
 #include <new>
 #include <string>
 
@@ -102,6 +103,15 @@ inline int scan_host_layout(bnk_ctx *ctx, const bnk_batch *lay, const bnk_batch 
         span->add(off, off + (uint64_t)len);
     }
     return BNK_OK;
+}
+
+// Sum of the packet lengths of a host batch.
+inline uint64_t host_payload_bytes(const bnk_batch *b)
+{
+    if (!b->lens) return (uint64_t)b->n * b->len;
+    uint64_t sum = 0;
+    for (uint32_t i = 0; i < b->n; i++) sum += b->lens[i];
+    return sum;
 }
 
 // Every index of a host array must name a row of a table with `rows` rows.
@@ -441,17 +451,40 @@ struct HostPipe {
 int aead_batch(bnk_ctx *ctx, bool open, const bnk_batch *in, const bnk_batch *out, uint8_t *verdict,
                uint32_t *sort_scratch);
 
+// bnk_wg_encap_batch (wg_api.hip), with NoteOutbound at *note_now on the plaintexts first
+// when note_now is given; and bnk_wg_decap_batch, with CheckInbound at *check_now on the
+// delivered packets afterwards when check_now is given.  The context lock is held.
+int wg_encap_impl(bnk_ctx *ctx, const bnk_batch *slots, uint32_t mtu, uint32_t *wire_len, const int64_t *note_now);
+int wg_decap_impl(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *out, uint8_t *result, uint32_t *out_len,
+                  uint32_t *peer, uint64_t *counter, const int64_t *check_now);
+
 // The file-scope device scratch of the entry point that allocates nothing
 // (noalloc_api.hip): looks up its address on `device` (which must be current).
 int noalloc_setup(bnk_ctx *ctx, int device);
 // Drops a context that is being shut down from the record of who used the scratch last.
 void noalloc_forget(bnk_ctx *ctx);
 
+// What a small-batch route returns in deferred mode (bnk_ctx::defer) instead of BNK_OK:
+// its work is enqueued, its results are not there yet.  Never crosses the C ABI.
+constexpr int BNK_DEFERRED = 2;
+
 // Waits for everything enqueued on the context stream so far.
 int wait_stream(bnk_ctx *ctx);
+// The same in two steps, for a caller that gives up the context lock in between:
+// post_ticket enqueues the one-thread launch that ends the work so far and
+// returns its number; wait_ticket waits for that number (or a later one).
+int post_ticket(bnk_ctx *ctx, uint32_t *ticket);
+int wait_ticket(bnk_ctx *ctx, uint32_t ticket);
+// The end of a small-batch route whose kernels wrote their results to pinned
+// staging: waits for the stream (reading the status words when with_status),
+// then copies the results out -- or, when the context is in deferred mode,
+// only notes the copies for whoever waits later.
+int finish_direct(bnk_ctx *ctx, bool with_status, std::initializer_list<Deferred> copies);
 // Reads and clears the device status word (waits for the stream; after_kernel: through
 // wait_stream, for a call whose last enqueued operation is a kernel).
 int take_status(bnk_ctx *ctx, uint32_t *status, bool after_kernel = false);
+// Reads and clears the status words (the stream must have been waited for).
+uint32_t read_status_words(bnk_ctx *ctx);
 // Maps status bits to an error code (BNK_OK when clear).
 int status_to_rc(bnk_ctx *ctx, uint32_t status);
 

@@ -4,11 +4,13 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
 #include <mutex>
 #include <string>
 #include <vector>
 
 #include "../../include/bnkhip.h"
+#include "coalesce.hpp"
 #include "kernels.hpp"
 
 namespace bnk {
@@ -81,6 +83,23 @@ struct PinBuf {
 
 struct FilterState; // filter_host.hpp
 
+// A result array a kernel leaves in pinned staging, to be copied to the
+// caller's array once the stream has reached the end of the call.
+struct Deferred {
+    void *dst;
+    const void *src;
+    size_t bytes;
+};
+
+// Staging of one merged window (coalesce.hpp): windows are enqueued one behind
+// the other and each is waited for outside the context lock, so each needs
+// staging of its own until its work is done.
+struct HostStage {
+    PinBuf pin;
+    std::atomic<bool> busy{false}; // taken by a window's leader until it has copied its results out
+};
+constexpr uint32_t HOST_STAGES = 4;
+
 } // namespace bnk
 
 struct bnk_ctx {
@@ -104,10 +123,20 @@ struct bnk_ctx {
     bnk::DevBuf in_arena, out_arena, off_in, off_out, lens, peer, counters, verdict;
     bnk::DevBuf order, hist, cursor, misc;
     bnk::PinBuf pin;
+    // Which pinned staging the small-batch routes of the call being enqueued
+    // use, and whether that call returns as soon as its work is enqueued (defer
+    // non-null: the result copies are appended there and the caller waits for
+    // the stream itself, see finish_direct and coalesce.hip) or waits itself.
+    bnk::PinBuf *pin_cur = &pin;
+    std::vector<bnk::Deferred> *defer = nullptr;
+    bool defer_status = false; // the deferred call wants the status words read when it is done
+    bnk::HostStage stages[bnk::HOST_STAGES];
     // Pinned rings handed out by bnk_ring_alloc: kernels may read and write
     // them in place (small host batches skip the copies).
     struct Ring { uintptr_t host; uint8_t *dev; size_t bytes; };
     std::vector<Ring> rings;
+    std::mutex rings_mu; // held (with mu) while `rings` changes, and alone by readers that do not hold mu
+    bnk::Coalescer co;   // merging of small host calls, see coalesce.hpp
     uint32_t *h_status = nullptr; // pinned status words the kernels write
     uint32_t wait_seq = 0;        // number of the last wait_stream(), see STATUS_DONE_WORD
     bool wait_sync_only = false;  // BNK_WAIT_SYNC=1: wait with hipStreamSynchronize, never by watching the word

@@ -73,6 +73,8 @@ struct FilterArgs {
                           // an IP header with options
     const uint32_t *order; // with heads, or nullptr
     uint8_t *verdict;     // check only
+    uint8_t *wg_result;   // check only, or nullptr: the BNK_WG_* results of the decapsulation that
+                          // delivered these packets; a denied packet's BNK_WG_OK becomes BNK_WG_FILTERED
     uint32_t *status;
     int64_t now;
     uint32_t n, stride, len;

@@ -25,6 +25,7 @@
 // marker bit form the key word, so 0 can mean "empty" and a slot is claimed
 // with one 64-bit compare-and-swap.  Deleted entries keep their key and carry
 // expiry FLOW_TOMB.
+#include "../../include/bnkhip.h"
 #include "filter_dev.hpp"
 #include "kernels.hpp"
 
@@ -382,7 +383,11 @@ __global__ __launch_bounds__(FILTER_THREADS, 8) void filter_check_kernel(FilterA
                 break;
             }
         }
-        if (t < a.n) a.verdict[i] = pass;
+        if (t < a.n) {
+            a.verdict[i] = pass;
+            // a packet WireGuard delivered and this filter denied (BNK_WG_OK is 0)
+            if (a.wg_result && !pass && a.wg_result[i] == 0) a.wg_result[i] = BNK_WG_FILTERED;
+        }
     }
 }
 

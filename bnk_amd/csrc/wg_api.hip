@@ -252,8 +252,8 @@ extern "C" int bnk_wg_send_counters(bnk_ctx *ctx, uint64_t *out, uint32_t n)
 
 // bnk_wg_encap_batch, with NoteOutbound at *note_now on the plaintexts first
 // when note_now is given.
-static int wg_encap_impl(bnk_ctx *ctx, const bnk_batch *slots, uint32_t mtu, uint32_t *wire_len,
-                         const int64_t *note_now)
+int bnk::wg_encap_impl(bnk_ctx *ctx, const bnk_batch *slots, uint32_t mtu, uint32_t *wire_len,
+                       const int64_t *note_now)
 {
     int rc = check_batch_common(ctx, slots, "slots");
     if (rc) return rc;
@@ -313,15 +313,18 @@ static int wg_encap_impl(bnk_ctx *ctx, const bnk_batch *slots, uint32_t mtu, uin
                     return fail(ctx, BNK_E_INVAL, "slots: packet " + std::to_string(i) + " lies outside the arena");
                 sp.add(off, off + need);
             }
-            if (sp.size() <= DIRECT_MAX_BYTES) {
+            // (a wave per packet reads each slot where it lies; a lane per packet
+            // first fetches the whole span)
+            if ((wave_per_packet ? host_payload_bytes(slots) : sp.size()) <= DIRECT_MAX_BYTES) {
                 span = sp;
                 ring_out = d_ring + span.lo;
             }
         }
     }
     if (ring_out) {
-        HIPCHK(ctx, ctx->pin.reserve((size_t)n * 20 + 64));
-        uint64_t *p_off = ctx->pin.as<uint64_t>();
+        PinBuf &stage = *ctx->pin_cur;
+        HIPCHK(ctx, stage.reserve((size_t)n * 20 + 64));
+        uint64_t *p_off = stage.as<uint64_t>();
         uint32_t *p_lens = (uint32_t *)(p_off + n), *p_peer = p_lens + n;
         h_wire_len = p_peer + n;
         if (wave_per_packet) {
@@ -335,11 +338,11 @@ static int wg_encap_impl(bnk_ctx *ctx, const bnk_batch *slots, uint32_t mtu, uin
         }
         if (slots->offsets) {
             for (uint32_t i = 0; i < n; i++) p_off[i] = slots->offsets[i] - span.lo;
-            b.off = ctx->pin.dev(p_off);
+            b.off = stage.dev(p_off);
         }
-        if (slots->lens) { memcpy(p_lens, slots->lens, (size_t)n * 4); b.lens = ctx->pin.dev(p_lens); }
-        if (slots->peer) { memcpy(p_peer, slots->peer, (size_t)n * 4); d_peer = ctx->pin.dev(p_peer); }
-        d_wire_len = ctx->pin.dev(h_wire_len);
+        if (slots->lens) { memcpy(p_lens, slots->lens, (size_t)n * 4); b.lens = stage.dev(p_lens); }
+        if (slots->peer) { memcpy(p_peer, slots->peer, (size_t)n * 4); d_peer = stage.dev(p_peer); }
+        d_wire_len = stage.dev(h_wire_len);
     } else if (host) {
         HIPCHK(ctx, ctx->wg_wirelen.reserve((size_t)n * 4));
         d_wire_len = ctx->wg_wirelen.as<uint32_t>();
@@ -538,16 +541,7 @@ static int wg_encap_impl(bnk_ctx *ctx, const bnk_batch *slots, uint32_t mtu, uin
         if (ring_out) {
             // peer indices were checked above: only a flow table overflow could come
             // back through the status word
-            uint32_t status = 0;
-            if (note) {
-                rc = take_status(ctx, &status, true);
-                if (rc) return rc;
-            } else {
-                rc = wait_stream(ctx);
-                if (rc) return rc;
-            }
-            memcpy(wire_len, h_wire_len, (size_t)n * 4);
-            return status_to_rc(ctx, status);
+            return finish_direct(ctx, note, {{wire_len, h_wire_len, (size_t)n * 4}});
         }
         HIPCHK(ctx, hipMemcpyAsync((uint8_t *)slots->base + span.lo, ctx->in_arena.p, span.size(),
                                    hipMemcpyDeviceToHost, ctx->stream));
@@ -562,6 +556,11 @@ static int wg_encap_impl(bnk_ctx *ctx, const bnk_batch *slots, uint32_t mtu, uin
 extern "C" int bnk_wg_encap_batch(bnk_ctx *ctx, const bnk_batch *slots, uint32_t mtu, uint32_t *wire_len)
 {
     BNK_API_TRY
+    {
+        CoRequest rq{CO_ENCAP, slots, nullptr, mtu, 0, nullptr, wire_len, nullptr, nullptr};
+        int crc;
+        if (coalesce_submit(ctx, rq, &crc)) return crc;
+    }
     Guard g(ctx);
     if (g.rc) return g.rc;
     return wg_encap_impl(ctx, slots, mtu, wire_len, nullptr);
@@ -572,6 +571,11 @@ extern "C" int bnk_wg_note_encap_batch(bnk_ctx *ctx, const bnk_batch *slots, uin
                                        uint32_t *wire_len)
 {
     BNK_API_TRY
+    {
+        CoRequest rq{CO_NOTE_ENCAP, slots, nullptr, mtu, now_ns, nullptr, wire_len, nullptr, nullptr};
+        int crc;
+        if (coalesce_submit(ctx, rq, &crc)) return crc;
+    }
     Guard g(ctx);
     if (g.rc) return g.rc;
     return wg_encap_impl(ctx, slots, mtu, wire_len, &now_ns);
@@ -580,8 +584,8 @@ extern "C" int bnk_wg_note_encap_batch(bnk_ctx *ctx, const bnk_batch *slots, uin
 
 // bnk_wg_decap_batch, with CheckInbound at *check_now on the delivered
 // packets afterwards when check_now is given.
-static int wg_decap_impl(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *out, uint8_t *result,
-                         uint32_t *out_len, uint32_t *peer, uint64_t *counter, const int64_t *check_now)
+int bnk::wg_decap_impl(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *out, uint8_t *result,
+                       uint32_t *out_len, uint32_t *peer, uint64_t *counter, const int64_t *check_now)
 {
     int rc = check_batch_common(ctx, wire, "wire");
     if (rc) return rc;
@@ -652,10 +656,11 @@ static int wg_decap_impl(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *o
             if (rc) return rc;
             rc = scan_host_layout(ctx, out, &w2, -32, &sout, "out");
             if (rc) return rc;
-            if (sin.size() <= DIRECT_MAX_BYTES) {
+            if ((wave_per_packet ? host_payload_bytes(&w2) : sin.size()) <= DIRECT_MAX_BYTES) {
                 direct = true;
-                HIPCHK(ctx, ctx->pin.reserve((size_t)n * 37 + 64));
-                uint64_t *p_in_off = ctx->pin.as<uint64_t>(), *p_out_off = p_in_off + n;
+                PinBuf &stage = *ctx->pin_cur;
+                HIPCHK(ctx, stage.reserve((size_t)n * 37 + 64));
+                uint64_t *p_in_off = stage.as<uint64_t>(), *p_out_off = p_in_off + n;
                 h_counter = p_out_off + n;
                 uint32_t *p_lens = (uint32_t *)(h_counter + n);
                 h_out_len = p_lens + n;
@@ -672,15 +677,15 @@ static int wg_decap_impl(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *o
                 }
                 if (wire->offsets) {
                     for (uint32_t i = 0; i < n; i++) p_in_off[i] = wire->offsets[i] - sin.lo;
-                    wb.off = ctx->pin.dev(p_in_off);
+                    wb.off = stage.dev(p_in_off);
                 }
-                if (wire->lens) { memcpy(p_lens, wire->lens, (size_t)n * 4); wb.lens = ctx->pin.dev(p_lens); }
+                if (wire->lens) { memcpy(p_lens, wire->lens, (size_t)n * 4); wb.lens = stage.dev(p_lens); }
                 ob.base = d_outr;
-                if (out->offsets) { memcpy(p_out_off, out->offsets, (size_t)n * 8); ob.off = ctx->pin.dev(p_out_off); }
-                d_result = ctx->pin.dev(h_result);
-                d_out_len = ctx->pin.dev(h_out_len);
-                d_peer = ctx->pin.dev(h_peer);
-                d_counter = ctx->pin.dev(h_counter);
+                if (out->offsets) { memcpy(p_out_off, out->offsets, (size_t)n * 8); ob.off = stage.dev(p_out_off); }
+                d_result = stage.dev(h_result);
+                d_out_len = stage.dev(h_out_len);
+                d_peer = stage.dev(h_peer);
+                d_counter = stage.dev(h_counter);
             }
         }
     }
@@ -827,8 +832,8 @@ static int wg_decap_impl(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *o
         fa.n = hi - lo;
         fa.rules = f->ridx;
         fa.flows = f->flows;
+        fa.wg_result = d_result + lo;
         HIPCHK(ctx, launch_filter_check(fa, f->max_blocks, ctx->stream));
-        HIPCHK(ctx, launch_wg_mark_filtered(d_result + lo, d_pass + lo, hi - lo, ctx->stream));
         return BNK_OK;
     };
 
@@ -950,13 +955,10 @@ static int wg_decap_impl(bnk_ctx *ctx, const bnk_batch *wire, const bnk_batch *o
         if (direct) {
             // the peer index of every opened packet comes from the table lookup:
             // nothing comes back through the status word
-            rc = wait_stream(ctx);
-            if (rc) return rc;
-            memcpy(result, h_result, n);
-            memcpy(out_len, h_out_len, (size_t)n * 4);
-            memcpy(peer, h_peer, (size_t)n * 4);
-            memcpy(counter, h_counter, (size_t)n * 8);
-            return BNK_OK;
+            return finish_direct(ctx, false, {{result, h_result, (size_t)n},
+                                              {out_len, h_out_len, (size_t)n * 4},
+                                              {peer, h_peer, (size_t)n * 4},
+                                              {counter, h_counter, (size_t)n * 8}});
         }
         HIPCHK(ctx, hipMemcpyAsync((uint8_t *)out->base + st.sout.lo, st.d_out, st.sout.size(),
                                    hipMemcpyDeviceToHost, ctx->stream));
@@ -975,6 +977,11 @@ extern "C" int bnk_wg_decap_batch(bnk_ctx *ctx, const bnk_batch *wire, const bnk
                                   uint8_t *result, uint32_t *out_len, uint32_t *peer, uint64_t *counter)
 {
     BNK_API_TRY
+    {
+        CoRequest rq{CO_DECAP, wire, out, 0, 0, result, out_len, peer, counter};
+        int crc;
+        if (coalesce_submit(ctx, rq, &crc)) return crc;
+    }
     Guard g(ctx);
     if (g.rc) return g.rc;
     return wg_decap_impl(ctx, wire, out, result, out_len, peer, counter, nullptr);
@@ -986,6 +993,11 @@ extern "C" int bnk_wg_decap_filter_batch(bnk_ctx *ctx, const bnk_batch *wire, co
                                          uint32_t *peer, uint64_t *counter)
 {
     BNK_API_TRY
+    {
+        CoRequest rq{CO_DECAP_FILTER, wire, out, 0, now_ns, result, out_len, peer, counter};
+        int crc;
+        if (coalesce_submit(ctx, rq, &crc)) return crc;
+    }
     Guard g(ctx);
     if (g.rc) return g.rc;
     return wg_decap_impl(ctx, wire, out, result, out_len, peer, counter, &now_ns);

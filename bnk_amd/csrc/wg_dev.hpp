@@ -80,7 +80,5 @@ hipError_t launch_wg_replay(uint8_t *result, uint32_t *out_len, const uint32_t *
 // Clears the windows of the rows whose flag is set.
 hipError_t launch_wg_replay_reset(uint64_t *state, const uint8_t *flags, uint32_t n_peers, hipStream_t s);
 
-// result[i] = BNK_WG_FILTERED where it was BNK_WG_OK and pass[i] == 0.
-hipError_t launch_wg_mark_filtered(uint8_t *result, const uint8_t *pass, uint32_t n, hipStream_t s);
 
 } // namespace bnk

@@ -182,21 +182,7 @@ __global__ __launch_bounds__(256) void wg_encap_prep_kernel(WgBatch b, uint8_t *
     wire_len[i] = 16u + len + pad + 16u;
 }
 
-// A packet WireGuard delivered and the inbound filter denied.
-__global__ __launch_bounds__(256) void wg_mark_filtered_kernel(uint8_t *result, const uint8_t *pass, uint32_t n)
-{
-    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
-    if (i < n && result[i] == BNK_WG_OK && pass[i] == 0) result[i] = BNK_WG_FILTERED;
-}
-
 static dim3 grid_of(uint32_t n) { return dim3((n + 255u) / 256u); }
-
-hipError_t launch_wg_mark_filtered(uint8_t *result, const uint8_t *pass, uint32_t n, hipStream_t s)
-{
-    if (n == 0) return hipSuccess;
-    hipLaunchKernelGGL(wg_mark_filtered_kernel, grid_of(n), dim3(256), 0, s, result, pass, n);
-    return hipGetLastError();
-}
 
 hipError_t launch_wg_parse(const WgBatch &b, const WgPeersDev &pe, uint32_t *peer, uint64_t *counter,
                            uint32_t *ct_len, uint8_t *result, uint32_t *status, hipStream_t s)

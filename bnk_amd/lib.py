@@ -50,6 +50,16 @@ class Rule(C.Structure):
                 ("proto", C.c_uint8), ("pad", C.c_uint8 * 3)]
 
 
+class CoalesceStats(C.Structure):
+    """struct bnk_coalesce_stats"""
+    _fields_ = [(k, C.c_uint64) for k in ("calls", "packets", "batches", "largest_batch", "largest_callers",
+                                          "full_windows", "timed_out", "retried", "gather_ns", "enqueue_ns",
+                                          "wait_ns")]
+
+    def as_dict(self) -> dict:
+        return {k: int(getattr(self, k)) for k, _ in self._fields_}
+
+
 _lib = None
 
 
@@ -210,6 +220,17 @@ class Context:
         self._rings = getattr(self, "_rings", {})
         self._rings[arr.ctypes.data] = p.value
         return arr
+
+    def set_coalesce(self, max_packets: int, max_wait_us: int = 30, expect_callers: int = 0) -> None:
+        """Merging of small host calls from several threads into one batch
+        (max_packets 0: off).  Results per call are unchanged."""
+        self._chk(self._lib.bnk_set_coalesce(self._h, C.c_uint32(max_packets), C.c_uint32(max_wait_us),
+                                             C.c_uint32(expect_callers)))
+
+    def coalesce_stats(self) -> dict:
+        st = CoalesceStats()
+        self._chk(self._lib.bnk_coalesce_stats_get(self._h, C.byref(st)))
+        return st.as_dict()
 
     def set_spread_max_packets(self, max_packets: int) -> None:
         """Batches of at most this many packets run one wave per packet

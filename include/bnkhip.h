@@ -142,6 +142,63 @@ void *bnk_stream(bnk_ctx *ctx);
  * counterpart in the reference. */
 int bnk_set_spread_max_packets(bnk_ctx *ctx, uint32_t max_packets);
 
+/* ---- merging of small host calls ----------------------------------------
+ *
+ * wireguard-go calls with at most 128 packets at a time, from one goroutine
+ * per peer: filteredTUN.Write once per peer batch
+ * (internal/filter/filter.go:171-186), Bind.Send "concurrently by per-peer
+ * goroutines" (internal/magicsock/bind.go:326-328; batch size bind.go:372-377).
+ * A context runs one call at a time, so at that calling pattern every call
+ * pays a launch and a wait for 180 KB.  With merging on, BNK_MEM_HOST calls of
+ * bnk_aead_seal_batch, bnk_aead_open_batch, bnk_wg_encap_batch,
+ * bnk_wg_note_encap_batch, bnk_wg_decap_batch and bnk_wg_decap_filter_batch
+ * that arrive from different threads while the context is busy (or within
+ * max_wait_us of each other once callers have been seen to come in groups)
+ * are run as one batch; every caller blocks until that batch is done and gets
+ * exactly its own results.  Nothing changes in any signature.
+ *
+ * A call takes part when its arenas lie inside pinned rings of the context
+ * (bnk_ring_alloc; callers of one window must use the same ring or pair of
+ * rings, each its own part of it) and it has at most max(128, max_packets/4)
+ * packets; any other call runs by itself as before.  Per call the results are
+ * those of some serial order of the merged calls: each call's packets stay in
+ * order and calls are taken in arrival order, so send counters and anti-replay
+ * windows, which depend on the order of one peer's packets, are as if the calls
+ * had run one after the other (a peer's calls come from one thread and do not
+ * overlap).  Calls of a window that carry a now_ns share the latest of theirs.
+ * A call whose arguments a direct call would refuse (BNK_E_INVAL, BNK_E_RANGE,
+ * BNK_E_STATE) is refused alone, with its own message.
+ *
+ * max_packets: size at which a window is run without waiting further (4096
+ * keeps a window within what one launch of a wave per packet takes); 0
+ * switches merging off (the default).  max_wait_us: how long the first caller
+ * of a window waits for company: half of the callers that are inside these
+ * entry points at that moment, and never fewer than expect_callers (0 or 1:
+ * no such floor; for an application that knows how many threads call and
+ * wants them in one launch); a caller that is alone does not wait at all.
+ * Added latency per call is at most max_wait_us plus
+ * the time the batch before takes, which a direct call would have waited for
+ * on the context's lock as well.
+ * No counterpart in the reference (wireguard-go fans its AEAD out over CPU
+ * cores instead). */
+int bnk_set_coalesce(bnk_ctx *ctx, uint32_t max_packets, uint32_t max_wait_us,
+                     uint32_t expect_callers);
+
+typedef struct bnk_coalesce_stats {
+    uint64_t calls;           /* calls that joined a window */
+    uint64_t packets;         /* their packets */
+    uint64_t batches;         /* windows run */
+    uint64_t largest_batch;   /* packets in the largest window */
+    uint64_t largest_callers; /* calls in the window that merged most */
+    uint64_t full_windows;    /* closed because max_packets was reached */
+    uint64_t timed_out;       /* leader waited max_wait_us and went without the expected company */
+    uint64_t retried;         /* windows refused as a whole, whose callers then ran by themselves */
+    uint64_t gather_ns;       /* summed over windows: from the first caller's arrival to the window's close */
+    uint64_t enqueue_ns;      /* ... the context lock held to stage and launch the merged batch */
+    uint64_t wait_ns;         /* ... from there until the batch's results were back */
+} bnk_coalesce_stats;
+int bnk_coalesce_stats_get(bnk_ctx *ctx, bnk_coalesce_stats *out);
+
 /* ---- transport AEAD ---------------------------------------------------- */
 
 /* Loads n_peers 32-byte ChaCha20-Poly1305 keys (host memory) into key table

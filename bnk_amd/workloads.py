@@ -484,6 +484,20 @@ def relay_workload(cfg: int = 5, n: int = 1 << 22, n_peers: int = 4096, n_rules:
                          forged_fraction=forged_fraction, now_ns=T0_NS)
 
 
+def relay_forged_bits(w: RelayWorkload, cfg: int = 5):
+    """Which packets of the relay's inbound traffic carry a forged tag, and
+    how: (packet indices, byte position of the flipped bit in the sealed arena,
+    the bit as a mask).  forged_fraction of the packets, one seeded bit of the
+    16-byte tag each."""
+    b = w.batch
+    n = b.n
+    k = int(w.forged_fraction * n)
+    which = permutation(stream_seed(cfg, 5), n)[:k].astype(np.int64)
+    bit = rand_below(stream_seed(cfg, 6), k, 128)
+    pos = b.off[which].astype(np.int64) + b.lens[which].astype(np.int64) + (bit >> 3).astype(np.int64)
+    return which, pos, (1 << (bit & 7)).astype(np.uint8)
+
+
 def relay_plain_torch(w: RelayWorkload, device):
     """Plaintext arena of a relay_workload(..., payload=False), built on
     ``device``: the IMIX payload with each packet's 28 header bytes written in."""

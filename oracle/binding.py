@@ -13,7 +13,8 @@ import subprocess
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_SO = os.path.join(_HERE, "libbnkoracle.so")
+# BNK_ORACLE_SO: another build of the same library (the sanitizer build, oracle/san/)
+_SO = os.environ.get("BNK_ORACLE_SO") or os.path.join(_HERE, "libbnkoracle.so")
 
 
 def build() -> str:

@@ -192,11 +192,9 @@ def test_relay_full_size_device_resident_properties():
                             counters=d_ctr),
              lib.make_batch(sealed, total, n, lib.MEM_DEVICE, offsets=d_off))
     ctx.sync()
-    k = int(w.forged_fraction * n)
-    which = W.permutation(W.stream_seed(5, 5), n)[:k].astype(np.int64)
-    bit = W.rand_below(W.stream_seed(5, 6), k, 128)
-    pos = b.off[which].astype(np.int64) + b.lens[which].astype(np.int64) + (bit >> 3).astype(np.int64)
-    sealed[d(pos)] ^= d((1 << (bit & 7)).astype(np.uint8))
+    which, pos, mask = W.relay_forged_bits(w)
+    k = which.shape[0]
+    sealed[d(pos)] ^= d(mask)
     forged = np.zeros(n, bool)
     forged[which] = True
     torch.cuda.synchronize()

@@ -52,6 +52,24 @@ VALU_SINGLE_ISSUE_SHARE = 0.40       # of them: v_alignbit_b32, v_mad_u64_u32, v
 TRAFFIC_BYTES_PER_LAUNCH = 3.177e9   # FETCH_SIZE + WRITE_SIZE, scaled by copy_kernel
 # the same for filter_check_kernel over 2^22 headers (profiles/filter_check_kernel_cfg4.md)
 FILTER_TRAFFIC_BYTES_PER_LAUNCH = 191.6e6
+# The counter readings above describe the kernel sources as they were when the readings
+# were taken: sha256 (first 16 hex digits) over the files named, in order.  When a file has
+# changed since, the JSON line says "counters_stale": true beside the figures derived from
+# them, until the profile is taken again and the hash here replaced
+# (`python bench.py --source-hashes` prints the current ones).
+AEAD_COUNTER_SOURCES = ("bnk_amd/csrc/aead_kernels.hip", "bnk_amd/csrc/aead_lane.hpp", "bnk_amd/csrc/kernels.hpp")
+AEAD_COUNTERS_TAKEN_ON = "0000000000000000"
+FILTER_COUNTER_SOURCES = ("bnk_amd/csrc/filter_kernels.hip", "bnk_amd/csrc/filter_dev.hpp")
+FILTER_COUNTERS_TAKEN_ON = "0000000000000000"
+
+
+def source_hash(files) -> str:
+    import hashlib
+    h = hashlib.sha256()
+    for f in files:
+        with open(os.path.join(ROOT, f), "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:16]
 
 
 def ops_chacha(length: int) -> int:
@@ -126,6 +144,7 @@ def bench_filter(args) -> dict:
                    "packets": n, "rules": 4096, "allowed_fraction": round(allowed, 4)},
         "roofline": {"bound": "hbm", "kernel": "filter_check_kernel", "achieved": round(gbs, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+                     "counters_stale": source_hash(FILTER_COUNTER_SOURCES) != FILTER_COUNTERS_TAKEN_ON,
                      "traffic": FILTER_TRAFFIC_BYTES_PER_LAUNCH if n == 1 << 22 else None,
                      "traffic_source": "profiles/filter_check_kernel_cfg4.md (FETCH_SIZE and WRITE_SIZE under "
                                        "rocprofv3 --pmc, scaled by copy_kernel; not re-measured in this run)",
@@ -849,7 +868,13 @@ def main() -> int:
                          "kernel trace of the run holds the timed launches only")
     ap.add_argument("--cpu-sample", type=int, default=0,
                     help="packets in the CPU baseline sample (0 = sized for ~10 s)")
+    ap.add_argument("--source-hashes", action="store_true",
+                    help="print the hashes of the kernel sources the pasted counter readings belong to, and exit")
     args = ap.parse_args()
+    if args.source_hashes:
+        print(json.dumps({"AEAD_COUNTERS_TAKEN_ON": source_hash(AEAD_COUNTER_SOURCES),
+                          "FILTER_COUNTERS_TAKEN_ON": source_hash(FILTER_COUNTER_SOURCES)}))
+        return 0
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no cross-GPU step and every box "
               "here has one GPU; run with --gpus 1", file=sys.stderr)
@@ -983,6 +1008,7 @@ def main() -> int:
             # per SIMD per four cycles, the rate of the rotates, multiplies and carries
             "frac_of_single_issue_rate": round(achieved_lane_tops / VALU_SINGLE_ISSUE_TOPS, 4),
             "single_issue_share_of_instructions": VALU_SINGLE_ISSUE_SHARE,
+            "counters_stale": source_hash(AEAD_COUNTER_SOURCES) != AEAD_COUNTERS_TAKEN_ON,
             "instructions_per_packet": VALU_LANE_INSTR_PER_PACKET,
             "instructions_source": "SQ_INSTS_VALU per launch x 64 / packets, rocprofv3 --pmc, mean of the "
                                    "seal and the open launch (profiles/aead_wave_kernel_cfg2.md); "
@@ -1013,6 +1039,7 @@ def main() -> int:
             "bound": "hbm", "kernel": "aead_wave_kernel",
             "achieved": round(achieved_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": round(achieved_gbs / HBM_PEAK_GBS, 4),
+            "counters_stale": source_hash(AEAD_COUNTER_SOURCES) != AEAD_COUNTERS_TAKEN_ON,
             "traffic": TRAFFIC_BYTES_PER_LAUNCH if counters_apply else None,
             "traffic_source": "profiles/aead_wave_kernel_cfg2.md (not re-measured in this run)",
             "bytes_per_launch": alg_bytes, "avg_launch_ms": round(kern_ms, 4),

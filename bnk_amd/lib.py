@@ -13,7 +13,8 @@ import os
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-SO_PATH = os.path.join(_HERE, "libbnkhip.so")
+# BNK_HIP_SO: another build of the same library (an experiment beside the in-tree one)
+SO_PATH = os.environ.get("BNK_HIP_SO") or os.path.join(_HERE, "libbnkhip.so")
 
 MEM_HOST, MEM_DEVICE = 0, 1
 KEYS_SEND, KEYS_RECV = 0, 1

@@ -119,10 +119,11 @@ __global__ __launch_bounds__(256) void replay_keys_packed_kernel(const uint8_t *
 // ---------------------------------------------------------------------------
 // Running maximum per peer in sorted order: pmax[p] = the largest sval of the
 // earlier positions with p's key, 0 when there is none.  A segmented exclusive
-// max-scan, the segments being the peers' runs.  Three steps: every block of
-// SEG_BLOCK positions reduces to what it hands on (seg_carry_kernel), one block
-// scans those (seg_carry_scan_kernel), and every block scans itself again with
-// what it was handed (inside replay_classify_kernel, which needs the values).
+// max-scan, the segments being the peers' runs.  Two steps: every block of
+// SEG_BLOCK positions reduces to what it hands on (in the launch that puts the
+// counters into sorted order), and every block scans itself again, together
+// with the carries of the blocks before it back to the nearest head (seg_handed;
+// inside replay_classify_kernel, which needs the values).
 // ---------------------------------------------------------------------------
 constexpr uint32_t SEG_BLOCK = 1024;
 
@@ -214,7 +215,7 @@ __device__ __forceinline__ bool seg_head(const uint32_t *skeys, uint32_t p, uint
 
 // Sender, position and counter of the packets in sorted order, from the sorted
 // words, and what each block of positions hands on to the running maximum
-// (carry_x, carry_open: see seg_carry_scan_kernel).
+// (carry_x: the maximum over the block's last run; carry_open: the block holds no head).
 __global__ __launch_bounds__(SEG_BLOCK) void replay_unpack_kernel(const uint32_t *sorted, const uint64_t *counter,
                                                                   uint32_t n, unsigned index_bits, unsigned peer_bits,
                                                                   uint32_t *skeys, uint32_t *sidx, uint64_t *sctr,
@@ -267,76 +268,70 @@ __global__ __launch_bounds__(SEG_BLOCK) void replay_gather_kernel(const uint32_t
     }
 }
 
-// carry_x[b] becomes what block b is handed: the maximum of the run that runs
-// into it, over the blocks before it.  One block; each thread takes a stretch
-// of consecutive blocks.
-__global__ __launch_bounds__(SEG_BLOCK) void seg_carry_scan_kernel(uint64_t *carry_x, const uint32_t *carry_open,
-                                                                   uint32_t blocks)
+// What block b is handed: the maximum of the run that runs into it, over the
+// blocks before it -- the blocks' carries from the nearest one that holds a
+// head onwards.  Every thread of the block takes part; the carries are read
+// SEG_BLOCK at a time, going back (a run seldom spans more than a few blocks).
+__device__ __forceinline__ uint64_t seg_handed(const uint64_t *carry_x, const uint32_t *carry_open, uint32_t b)
 {
-    const uint32_t per = (blocks + SEG_BLOCK - 1u) / SEG_BLOCK;
-    const uint32_t lo = min(threadIdx.x * per, blocks), hi = min(lo + per, blocks);
-    // my stretch as one element: its value, and whether no head lies in it
-    uint64_t x = 0;
-    bool open = true;
-    for (uint32_t b = lo; b < hi; b++) {
-        const uint64_t v = carry_x[b];
-        if (carry_open[b]) x = v > x ? v : x;
-        else {
-            x = v;
-            open = false;
-        }
+    uint64_t acc = 0;
+    for (uint32_t hi = b; hi > 0u;) {
+        // blocks hi - SEG_BLOCK .. hi - 1, right-aligned: what falls before block 0 is neutral
+        const int64_t at = (int64_t)hi - (int64_t)SEG_BLOCK + (int64_t)threadIdx.x;
+        const uint64_t v = at >= 0 ? carry_x[at] : 0;
+        const bool head = at >= 0 && carry_open[at] == 0u;
+        __syncthreads(); // the scan before this one has been read out of its LDS words
+        const SegScan r = seg_block_scan(v, head);
+        acc = r.total > acc ? r.total : acc;
+        if (!r.total_open) break;
+        hi = hi > SEG_BLOCK ? hi - SEG_BLOCK : 0u;
     }
-    const SegScan r = seg_block_scan(x, !open);
-    // my first block is handed what the stretch before mine ends with (a head inside
-    // my stretch cuts off what follows it, not the blocks before it)
-    uint64_t run = r.prev;
-    for (uint32_t b = lo; b < hi; b++) {
-        const uint64_t v = carry_x[b];
-        const bool o = carry_open[b] != 0u;
-        carry_x[b] = run;
-        run = o ? (v > run ? v : run) : v;
-    }
+    return acc;
 }
 
 // What the window decides about a packet without looking at other packets'
 // counters: turned away outright, ahead of everything before it (fresh for
-// certain), or inside the window at or below an earlier counter ("late": fresh
-// unless that counter was seen before).
-enum : uint8_t { RP_NONE = 0, RP_AHEAD = 1, RP_LATE = 2 };
+// certain), inside the window with its bit set before the batch (a repeat for
+// certain), or inside the window at or below an earlier counter with the bit
+// clear ("late": fresh unless an earlier packet of the batch carried the
+// counter too).
+enum : uint8_t { RP_NONE = 0, RP_AHEAD = 1, RP_LATE = 2, RP_SEEN = 3 };
 
 __device__ __forceinline__ uint32_t table_home(uint32_t key, uint64_t c, uint32_t mask)
 {
     return (uint32_t)mix(c ^ ((uint64_t)key << 40) ^ key) & mask;
 }
 
-// Classifies every packet; turns away what never reaches the bit test; enters
-// the late ones into the table (slot = earliest sorted position carrying that
-// peer and counter) and raises flags[0] when there are any.
+// The running maximum of every packet's peer (a segmented scan within the block
+// plus what the block is handed), the packet's class, REPLAY for what never
+// reaches the bit test and for what the window had seen before the batch; late
+// packets enter the table (slot = earliest sorted position among the late
+// packets carrying that peer and counter) and raise flags[0].
 __global__ __launch_bounds__(SEG_BLOCK) void replay_classify_kernel(const uint32_t *skeys, const uint32_t *sidx,
                                                                     const uint64_t *sctr, const uint64_t *sval,
-                                                                    const uint64_t *carry, uint64_t *pmax,
+                                                                    const uint64_t *carry_x,
+                                                                    const uint32_t *carry_open, uint64_t *pmax,
                                                                     const uint64_t *state, uint32_t n, uint8_t *cls,
                                                                     uint32_t *table, uint32_t mask, uint32_t *flags,
                                                                     uint8_t *result, uint32_t *out_len)
 {
     const uint32_t p = blockIdx.x * SEG_BLOCK + threadIdx.x;
     const uint32_t key = p < n ? skeys[p] : NO_PEER;
-    // the running maximum of my peer's earlier counters (every thread of the block takes part)
     const SegScan seg = seg_block_scan(p < n ? sval[p] : 0, seg_head(skeys, p, n, key));
+    const uint64_t handed = seg_handed(carry_x, carry_open, blockIdx.x);
     if (p >= n) return;
     uint64_t before = seg.excl;
-    if (seg.open) {
-        const uint64_t handed = carry[blockIdx.x];
-        before = handed > before ? handed : before;
-    }
+    if (seg.open && handed > before) before = handed;
     pmax[p] = before;
     uint8_t k = RP_NONE;
     if (key != NO_PEER) {
         const uint64_t c = sctr[p];
-        const uint64_t last0 = state[(size_t)key * WG_REPLAY_WORDS];
+        const uint64_t *st = state + (size_t)key * WG_REPLAY_WORDS;
+        const uint64_t last0 = st[0];
         const uint64_t last = last0 > before ? last0 : before;
         if (reaches_bit_test(c, last)) k = c > last ? RP_AHEAD : RP_LATE;
-        if (k == RP_NONE) {
+        if (k == RP_LATE && c <= last0 && seen_before(st, c)) k = RP_SEEN;
+        if (k == RP_NONE || k == RP_SEEN) {
             const uint32_t i = sidx[p];
             result[i] = BNK_WG_REPLAY;
             out_len[i] = 0;
@@ -357,47 +352,56 @@ __global__ __launch_bounds__(SEG_BLOCK) void replay_classify_kernel(const uint32
     cls[p] = k;
 }
 
-// A late packet may repeat a packet that was ahead when it came: those look
-// their counter up and take the slot over when they are the earlier one.
-// Nothing to do in a batch without late packets.
-__global__ __launch_bounds__(256) void replay_claim_kernel(const uint32_t *skeys, const uint64_t *sctr,
-                                                           const uint8_t *cls, uint32_t n, uint32_t *table,
-                                                           uint32_t mask, const uint32_t *flags)
+// Did an earlier packet of p's run raise the run's maximum to exactly c (c > 0)?
+// Such a packet carried c and reached the bit test.  The running maximum before
+// each position does not fall along a run, so the first position whose value
+// reaches c is found by doubling steps back from p and halving in between;
+// position q's packet carried c iff the value before q + 1 is c.
+__device__ __forceinline__ bool raised_to(const uint32_t *skeys, const uint64_t *pmax, uint32_t p, uint32_t key,
+                                          uint64_t c)
 {
-    if (flags[0] == 0u) return;
-    const uint32_t p = blockIdx.x * 256u + threadIdx.x;
-    if (p >= n || cls[p] != RP_AHEAD) return;
-    const uint32_t key = skeys[p];
-    const uint64_t c = sctr[p];
-    uint32_t h = table_home(key, c, mask);
-    for (;;) {
-        const uint32_t at = table[h];
-        if (at == HASH_EMPTY) return; // no late packet carries my counter
-        if (skeys[at] == key && sctr[at] == c) {
-            atomicMin(&table[h], p);
-            return;
+    if (pmax[p] < c) return false;
+    // invariant: below lo the value is under c or the run has not begun; at hi it is at least c
+    uint32_t hi = p, lo = 0;
+    for (uint32_t step = 1;; step <<= 1) {
+        if (step > hi) break;
+        const uint32_t q = hi - step;
+        if (skeys[q] != key || pmax[q] < c) {
+            lo = q + 1u;
+            break;
         }
-        h = (h + 1u) & mask;
+        hi = q;
+        if (step >= 0x80000000u) break;
     }
+    while (lo < hi) {
+        const uint32_t mid = lo + (hi - lo) / 2u;
+        if (skeys[mid] == key && pmax[mid] >= c) hi = mid;
+        else lo = mid + 1u;
+    }
+    return pmax[hi] == c;
 }
 
-// A late packet is fresh when its counter was not seen before the batch and no
-// earlier packet of the batch carried it.
-__global__ __launch_bounds__(256) void replay_late_kernel(const uint32_t *skeys, const uint32_t *sidx,
-                                                          const uint64_t *sctr, const uint8_t *cls,
-                                                          const uint64_t *state, uint32_t n,
-                                                          const uint32_t *table, uint32_t mask,
-                                                          const uint32_t *flags, uint8_t *result,
-                                                          uint32_t *out_len)
+// Two things no packet of the other needs: a late packet is fresh when no
+// earlier packet of the batch carried its counter -- neither a late one (the
+// table holds the first of those) nor one that was ahead when it came (those
+// raised the running maximum to their counter) -- and the last packet of each
+// peer's run brings that peer's window to where `last` ends up (clearing the
+// blocks it passed over; the class of every packet was settled against the
+// windows as the batch found them by the launch before this one).
+__global__ __launch_bounds__(256) void replay_late_advance_kernel(const uint32_t *skeys, const uint32_t *sidx,
+                                                                  const uint64_t *sctr, const uint64_t *pmax,
+                                                                  const uint8_t *cls, uint64_t *state, uint32_t n,
+                                                                  const uint32_t *table, uint32_t mask,
+                                                                  const uint32_t *flags, uint8_t *result,
+                                                                  uint32_t *out_len)
 {
-    if (flags[0] == 0u) return;
     const uint32_t p = blockIdx.x * 256u + threadIdx.x;
-    if (p >= n || cls[p] != RP_LATE) return;
+    if (p >= n) return;
     const uint32_t key = skeys[p];
+    if (key == NO_PEER) return;
     const uint64_t c = sctr[p];
-    const uint64_t *st = state + (size_t)key * WG_REPLAY_WORDS;
-    bool fresh = !(c <= st[0] && seen_before(st, c));
-    if (fresh) {
+    if (flags[0] != 0u && cls[p] == RP_LATE) {
+        bool fresh = true;
         uint32_t h = table_home(key, c, mask);
         for (;;) {
             const uint32_t at = table[h];
@@ -408,25 +412,15 @@ __global__ __launch_bounds__(256) void replay_late_kernel(const uint32_t *skeys,
             }
             h = (h + 1u) & mask;
         }
+        // (counter 0 is never ahead of anything: every packet carrying it is in the table)
+        if (fresh && c != 0u && raised_to(skeys, pmax, p, key, c)) fresh = false;
+        if (!fresh) {
+            const uint32_t i = sidx[p];
+            result[i] = BNK_WG_REPLAY;
+            out_len[i] = 0;
+        }
     }
-    if (!fresh) {
-        const uint32_t i = sidx[p];
-        result[i] = BNK_WG_REPLAY;
-        out_len[i] = 0;
-    }
-}
-
-// The last packet of each peer's run knows where that peer's `last` ends up.
-__global__ __launch_bounds__(256) void replay_advance_kernel(const uint32_t *skeys, const uint64_t *sctr,
-                                                             const uint64_t *pmax, uint64_t *state,
-                                                             uint32_t n)
-{
-    const uint32_t p = blockIdx.x * 256u + threadIdx.x;
-    if (p >= n) return;
-    const uint32_t key = skeys[p];
-    if (key == NO_PEER) return;
     if (p + 1u < n && skeys[p + 1u] == key) return;
-    const uint64_t c = sctr[p];
     uint64_t last = pmax[p];
     if (c < WG_REJECT_AFTER_MESSAGES && c > last) last = c;
     advance_window(state + (size_t)key * WG_REPLAY_WORDS, last);
@@ -437,9 +431,18 @@ __global__ __launch_bounds__(256) void replay_advance_kernel(const uint32_t *ske
 // share their peer and their block of 64 counters: a lane whose left neighbour
 // differs gathers the bits of the lanes behind it that agree with it and
 // issues one atomic for all of them.
+//
+// The same launch leaves the first-occurrence table empty for the next pass
+// (nothing to do when this pass had no late packet, the usual case) and clears
+// the flag word the next pass will use (nobody reads that one now).
 __global__ __launch_bounds__(256) void replay_mark_kernel(const uint32_t *skeys, const uint64_t *sctr,
-                                                          const uint8_t *cls, uint64_t *state, uint32_t n)
+                                                          const uint8_t *cls, uint64_t *state, uint32_t n,
+                                                          uint32_t *table, uint32_t slots, uint32_t *flags,
+                                                          uint32_t parity)
 {
+    if (blockIdx.x == 0 && threadIdx.x == 0) flags[parity ^ 1u] = 0u;
+    if (flags[parity] != 0u)
+        for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < slots; i += gridDim.x * 256u) table[i] = HASH_EMPTY;
     const uint32_t p = blockIdx.x * 256u + threadIdx.x;
     const uint32_t lane = threadIdx.x & 63u;
     uint32_t key = NO_PEER;
@@ -623,17 +626,6 @@ uint32_t wg_replay_table_slots(uint32_t n)
     return s;
 }
 
-// Leaves the first-occurrence table empty for the next pass, which costs
-// nothing when this pass had no late packet (the usual case), and clears the
-// flag word the next pass will use (nobody reads that one now).
-__global__ __launch_bounds__(256) void replay_table_reset_kernel(uint32_t *table, uint32_t slots,
-                                                                 uint32_t *flags, uint32_t parity)
-{
-    if (blockIdx.x == 0 && threadIdx.x == 0) flags[parity ^ 1u] = 0u;
-    if (flags[parity] == 0u) return;
-    for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < slots; i += gridDim.x * 256u) table[i] = HASH_EMPTY;
-}
-
 hipError_t launch_wg_replay(uint8_t *result, uint32_t *out_len, const uint32_t *peer, const uint64_t *counter,
                             uint32_t n, const WgReplayDev &rp, const WgReplayScratch &sc, hipStream_t s)
 {
@@ -676,21 +668,16 @@ hipError_t launch_wg_replay(uint8_t *result, uint32_t *out_len, const uint32_t *
         hipLaunchKernelGGL(replay_gather_kernel, dim3(seg_blocks), dim3(SEG_BLOCK), 0, s, sc.skeys, sc.sidx, counter,
                            n, sc.sctr, sc.sval, carry_x, carry_open);
     }
-    // the running maximum per peer: the scan of the blocks' carries, and the rest inside the
-    // classifying launch
-    hipLaunchKernelGGL(seg_carry_scan_kernel, dim3(1), dim3(SEG_BLOCK), 0, s, carry_x, carry_open, seg_blocks);
+    // the running maximum per peer is finished inside the classifying launch
     const uint32_t mask = sc.table_slots - 1u;
     uint32_t *late_flag = sc.flags + sc.parity;
     hipLaunchKernelGGL(replay_classify_kernel, dim3(seg_blocks), dim3(SEG_BLOCK), 0, s, sc.skeys, sc.sidx, sc.sctr,
-                       sc.sval, carry_x, sc.pmax, rp.state, n, sc.cls, sc.table, mask, late_flag, result, out_len);
-    hipLaunchKernelGGL(replay_claim_kernel, grid, dim3(256), 0, s, sc.skeys, sc.sctr, sc.cls, n, sc.table, mask,
-                       late_flag);
-    hipLaunchKernelGGL(replay_late_kernel, grid, dim3(256), 0, s, sc.skeys, sc.sidx, sc.sctr, sc.cls, rp.state, n,
-                       sc.table, mask, late_flag, result, out_len);
-    hipLaunchKernelGGL(replay_table_reset_kernel, dim3(std::min<uint32_t>((sc.table_slots + 255u) / 256u, 2048u)),
-                       dim3(256), 0, s, sc.table, sc.table_slots, sc.flags, sc.parity);
-    hipLaunchKernelGGL(replay_advance_kernel, grid, dim3(256), 0, s, sc.skeys, sc.sctr, sc.pmax, rp.state, n);
-    hipLaunchKernelGGL(replay_mark_kernel, grid, dim3(256), 0, s, sc.skeys, sc.sctr, sc.cls, rp.state, n);
+                       sc.sval, carry_x, carry_open, sc.pmax, rp.state, n, sc.cls, sc.table, mask, late_flag, result,
+                       out_len);
+    hipLaunchKernelGGL(replay_late_advance_kernel, grid, dim3(256), 0, s, sc.skeys, sc.sidx, sc.sctr, sc.pmax, sc.cls,
+                       rp.state, n, sc.table, mask, late_flag, result, out_len);
+    hipLaunchKernelGGL(replay_mark_kernel, grid, dim3(256), 0, s, sc.skeys, sc.sctr, sc.cls, rp.state, n, sc.table,
+                       sc.table_slots, sc.flags, sc.parity);
     return hipGetLastError();
 }
 

@@ -233,11 +233,11 @@ def _traffic(tx_ctx, tx_peers, n_a, n_b, n_total, inner_len, jump_rows, rng):
         # packets to be refused and new ones to refuse them
         peer[: n // 2] = rng.choice(jump_rows, n // 2).astype(np.uint32)
         arena = rng.integers(0, 256, n * slot, dtype=np.uint8)
-        for i in range(n):
-            o = i * slot + 16
-            arena[o] = 0x45
-            arena[o + 2:o + 4] = np.frombuffer(int(inner_len).to_bytes(2, "big"), np.uint8)
-            arena[o + 12:o + 16] = np.frombuffer(int(tx_peers[int(peer[i])][2]).to_bytes(4, "big"), np.uint8)
+        rows = arena.reshape(n, slot)
+        rows[:, 16] = 0x45
+        rows[:, 18], rows[:, 19] = inner_len >> 8, inner_len & 255
+        allowed = np.array([t[2] for t in tx_peers], np.uint32)[peer]
+        rows[:, 28:32] = allowed.astype(">u4").view(np.uint8).reshape(n, 4)
         wl = np.zeros(n, np.uint32)
         if k == 1:
             for r in jump_rows:
@@ -337,3 +337,55 @@ def test_window_pass_of_a_host_batch_that_goes_through_in_chunks():
         bad = np.flatnonzero(res != want)
         assert bad.size == 0, f"result differs at {bad[:5]}: got {res[bad[:5]]} want {want[bad[:5]]}"
         assert (want == lib.WG_REPLAY).sum() > 1000 and (want == lib.WG_OK).sum() > 1000
+
+
+def test_window_pass_where_one_peer_fills_more_blocks_than_one_look_back_reads():
+    """Two peers, one of them sending nearly everything: its run in sorted order
+    spans well over a thousand blocks of 1024 positions, so the running maximum
+    a block is handed comes from carries read in more than one step, and a late
+    repeat of a counter that was ahead when it first came is found by a search
+    that goes back across many blocks."""
+    import torch
+    from bnk_amd import lib
+    rng = np.random.default_rng(79)
+    n_total = 2_300_000
+    tx = [(100, 9000, 0x64400000, 0xFFFFFFFF), (103, 9005, 0x64400001, 0xFFFFFFFF)]
+    rx = [(p[1], p[0], p[2], p[3]) for p in tx]
+    keys = rng.integers(0, 256, (2, 32), dtype=np.uint8)
+    with lib.Context(0) as txc, lib.Context(0) as rxc:
+        txc.keys_set(lib.KEYS_SEND, keys)
+        txc.wg_peers_set(tx)
+        rxc.keys_set(lib.KEYS_RECV, keys)
+        rxc.wg_peers_set(rx)
+        # (no jump: a window is far shorter than the batch, so most early packets are too old
+        # by the time they come, the rest repeat or are fresh)
+        wire, stride, wire_len, peer, ctr = _traffic(txc, tx, 700_000, 500_000, n_total, 40, np.array([0]), rng)
+        # the first 1.2 million in sending order, so that long stretches are ahead of everything
+        # before them, then the shuffled mix with its repeats
+        order = np.argsort(ctr[:1_200_000], kind="stable")
+        w2 = wire.reshape(n_total, stride)
+        w2[:1_200_000] = w2[:1_200_000][order]
+        peer[:1_200_000], ctr[:1_200_000] = peer[:1_200_000][order], ctr[:1_200_000][order]
+        assert (peer == 0).sum() > 1_500_000
+        want = _window_expectation(peer, ctr, 2)
+        d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to("cuda:0")  # noqa: E731
+        d_wire, d_out = d(wire), torch.zeros(wire.nbytes, dtype=torch.uint8, device="cuda:0")
+        res = torch.zeros(n_total, dtype=torch.uint8, device="cuda:0")
+        olen = torch.zeros(n_total, dtype=torch.int32, device="cuda:0")
+        gp = torch.zeros(n_total, dtype=torch.int32, device="cuda:0")
+        gc = torch.zeros(n_total, dtype=torch.int64, device="cuda:0")
+        torch.cuda.synchronize()
+        rxc.wg_decap(lib.make_batch(d_wire, wire.nbytes, n_total, lib.MEM_DEVICE, stride=stride, length=wire_len),
+                     lib.make_batch(d_out, wire.nbytes, n_total, lib.MEM_DEVICE, stride=stride), res, olen, gp, gc)
+        rxc.sync()
+        assert np.array_equal(gp.cpu().numpy().astype(np.uint32), peer)
+        assert np.array_equal(gc.cpu().numpy().astype(np.uint64), ctr)
+        got = res.cpu().numpy()
+        bad = np.flatnonzero(got != want)
+        assert bad.size == 0, f"result differs at {bad[:5]}: got {got[bad[:5]]} want {want[bad[:5]]}"
+        assert (want == lib.WG_REPLAY).sum() > 100_000 and (want == lib.WG_OK).sum() > 100_000
+        # the same datagrams again: the windows have seen or passed every counter
+        rxc.wg_decap(lib.make_batch(d_wire, wire.nbytes, n_total, lib.MEM_DEVICE, stride=stride, length=wire_len),
+                     lib.make_batch(d_out, wire.nbytes, n_total, lib.MEM_DEVICE, stride=stride), res, olen, gp, gc)
+        rxc.sync()
+        assert (res.cpu().numpy() == lib.WG_REPLAY).all()

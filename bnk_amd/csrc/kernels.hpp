@@ -184,6 +184,15 @@ hipError_t launch_peer_rank(uint32_t *keys, uint32_t *idx, uint32_t *skeys, uint
                             void *sort_tmp, size_t sort_tmp_bytes, uint64_t *ctr_base, uint32_t n_keys,
                             uint32_t n, uint64_t *ctr_out, bool advance, uint64_t ctr_limit, hipStream_t s);
 
+// The same straight from a caller's peer array, without a sort, where the peer
+// table is small enough for the counting form (peer_rank_counts says whether;
+// tmp as for launch_peer_rank): a peer index beyond the table raises
+// STATUS_PEER_RANGE in *status and gets counter 0.
+bool peer_rank_counts(uint32_t n, uint32_t n_keys, size_t tmp_bytes);
+hipError_t launch_peer_rank_counting(const uint32_t *peer, void *tmp, uint64_t *ctr_base, uint32_t n_keys, uint32_t n,
+                                     uint64_t *ctr_out, bool advance, uint64_t ctr_limit, uint32_t *status,
+                                     hipStream_t s);
+
 // Copy of a byte span whose two ends share their alignment within 16 bytes,
 // one aligned 16-byte piece per lane (used to fetch small spans of pinned
 // host memory).

@@ -104,7 +104,7 @@ struct RankPlan {
     uint32_t runs;  // runs of 64 packets per tile
     uint32_t tiles;
     uint32_t cols;  // entries per row of the table: the keys, rounded up to what a wave moves at once
-    size_t bytes;   // the table, then one total per peer
+    size_t bytes;   // the table, then one total per peer, then every peer's counter as the batch found it
     bool fits;
 };
 
@@ -116,7 +116,7 @@ static RankPlan rank_plan(uint32_t n, uint32_t n_keys)
     p.runs = std::min<uint32_t>(TILE_RUNS_MAX, std::max<uint32_t>(1u, (n + 64u * 2048u - 1u) / (64u * 2048u)));
     p.tiles = (n + 64u * p.runs - 1u) / (64u * p.runs);
     p.cols = (n_keys + RANK_ROW_STEP - 1u) / RANK_ROW_STEP * RANK_ROW_STEP;
-    p.bytes = ((size_t)p.tiles + 1u) * p.cols * 4u;
+    p.bytes = ((size_t)p.tiles + 1u) * p.cols * 4u + (size_t)p.cols * 8u;
     p.fits = n_keys <= RANK_TABLE_MAX_KEYS && p.bytes <= RANK_TABLE_MAX_BYTES;
     return p;
 }
@@ -134,7 +134,7 @@ size_t relay_sort_tmp_bytes(uint32_t n, uint32_t n_keys)
     const RankPlan plan = rank_plan(n, n_keys);
     if (!plan.fits) return bytes;
     const size_t rows = std::max<size_t>(plan.tiles, std::min<size_t>(n / 64u + 1u, 2048u)) + 1u;
-    return std::max(bytes, rows * plan.cols * 4u);
+    return std::max(bytes, rows * plan.cols * 4u + (size_t)plan.cols * 8u);
 }
 
 __global__ void peer_rank_small_kernel(const uint32_t *peer, uint32_t n_keys, uint32_t n, uint64_t *ctr_base,
@@ -143,7 +143,8 @@ __global__ void peer_rank_small_kernel(const uint32_t *peer, uint32_t n_keys, ui
 
 static hipError_t launch_peer_rank_table(const uint32_t *keys, const RankPlan &plan, void *tmp,
                                          uint64_t *ctr_base, uint32_t n_keys, uint32_t n, uint64_t *ctr_out,
-                                         bool advance, uint64_t ctr_limit, bool zero_others, hipStream_t s);
+                                         bool advance, uint64_t ctr_limit, bool zero_others, uint32_t *status,
+                                         hipStream_t s);
 
 hipError_t launch_relay_assign(const uint8_t *auth, const uint8_t *pass, const uint32_t *peer_out,
                                const uint64_t *ctr_base_out, uint32_t n_peers_out, uint32_t n,
@@ -166,7 +167,7 @@ hipError_t launch_relay_assign(const uint8_t *auth, const uint8_t *pass, const u
     }
     if (counting)
         return launch_peer_rank_table(keys, plan, sort_tmp, const_cast<uint64_t *>(ctr_base_out), n_peers_out, n,
-                                      ctr_out, advance, 0ull, true, s);
+                                      ctr_out, advance, 0ull, true, nullptr, s);
     return launch_peer_rank(keys, idx, skeys, sidx, sort_tmp, sort_tmp_bytes,
                             const_cast<uint64_t *>(ctr_base_out), n_peers_out, n, ctr_out, advance, 0ull, s);
 }
@@ -236,11 +237,14 @@ hipError_t launch_peer_rank_small(const uint32_t *peer, uint32_t n_keys, uint32_
 // totals; rank_assign_kernel loads its tile's row into LDS and walks the tile
 // run by run in batch order: a packet's rank is its peer's entry plus the
 // number of lower lanes of the run with the same peer, and one lane per peer
-// then moves the entry past the run.  Four launches over the keys, against
-// eight (two of them passes over key-index pairs) for the sort.
+// then moves the entry past the run.  The scan also moves the peers' counters
+// past the batch, leaving the values it found for the assigning launch.
+// Three launches over the keys, against eight (two of them passes over
+// key-index pairs) for the sort.
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(64) void rank_count_kernel(const uint32_t *keys, uint32_t n, uint32_t n_keys,
-                                                        uint32_t cols, uint32_t runs, uint32_t *table)
+                                                        uint32_t cols, uint32_t runs, uint32_t *table,
+                                                        uint32_t *status)
 {
     __shared__ __attribute__((aligned(16))) uint32_t cnt[RANK_TABLE_MAX_KEYS];
     const uint32_t lane = threadIdx.x;
@@ -256,8 +260,11 @@ __global__ __launch_bounds__(64) void rank_count_kernel(const uint32_t *keys, ui
     }
     __syncthreads();
 #pragma unroll
-    for (uint32_t r = 0; r < TILE_RUNS_MAX; r++)
+    for (uint32_t r = 0; r < TILE_RUNS_MAX; r++) {
         if (key[r] < n_keys) atomicAdd(&cnt[key[r]], 1u);
+        // (keys straight from a caller's peer array: one beyond the table gets no counter and is reported)
+        else if (status && r < runs && first + r * 64u + lane < n) status_raise(status, STATUS_PEER_RANGE);
+    }
     __syncthreads();
     uint4 *row = reinterpret_cast<uint4 *>(table + (size_t)blockIdx.x * cols);
     for (uint32_t q = lane; q < cols / 4u; q += 64u) row[q] = cnt4[q];
@@ -268,7 +275,9 @@ constexpr uint32_t SCAN_PEERS = 16, SCAN_PARTS = 64;
 constexpr uint32_t SCAN_KEEP = 32; // tiles of a part held in registers between the two passes
 __global__ __launch_bounds__(SCAN_PEERS * SCAN_PARTS) void rank_scan_kernel(uint32_t *table, uint32_t tiles,
                                                                              uint32_t n_keys, uint32_t cols,
-                                                                             uint32_t *total)
+                                                                             uint32_t *total, uint64_t *ctr_base,
+                                                                             uint64_t *base_was, int advance,
+                                                                             uint64_t ctr_limit)
 {
     __shared__ uint32_t part_sum[SCAN_PARTS][SCAN_PEERS];
     const uint32_t x = threadIdx.x % SCAN_PEERS, y = threadIdx.x / SCAN_PEERS;
@@ -308,7 +317,14 @@ __global__ __launch_bounds__(SCAN_PEERS * SCAN_PARTS) void rank_scan_kernel(uint
             run += v;
         }
     }
-    if (y == SCAN_PARTS - 1u) total[key] = run;
+    if (y == SCAN_PARTS - 1u) {
+        // the peer's counter as the batch found it stays behind for the assigning launch;
+        // the counter itself moves past what the batch takes
+        total[key] = run;
+        const uint64_t was = ctr_base[key];
+        base_was[key] = was;
+        if (advance && run != 0u) ctr_base[key] = ctr_add(was, run, ctr_limit);
+    }
 }
 
 __global__ __launch_bounds__(64) void rank_assign_kernel(const uint32_t *keys, uint32_t n, uint32_t n_keys,
@@ -371,29 +387,38 @@ __global__ __launch_bounds__(64) void rank_assign_kernel(const uint32_t *keys, u
     }
 }
 
-__global__ __launch_bounds__(256) void rank_advance_kernel(const uint32_t *total, uint32_t n_keys,
-                                                           uint64_t *ctr_base, uint64_t ctr_limit)
-{
-    const uint32_t k = blockIdx.x * 256u + threadIdx.x;
-    if (k < n_keys && total[k] != 0u) ctr_base[k] = ctr_add(ctr_base[k], total[k], ctr_limit);
-}
-
 static hipError_t launch_peer_rank_table(const uint32_t *keys, const RankPlan &plan, void *tmp,
                                          uint64_t *ctr_base, uint32_t n_keys, uint32_t n, uint64_t *ctr_out,
-                                         bool advance, uint64_t ctr_limit, bool zero_others, hipStream_t s)
+                                         bool advance, uint64_t ctr_limit, bool zero_others, uint32_t *status,
+                                         hipStream_t s)
 {
     uint32_t *table = static_cast<uint32_t *>(tmp);
     uint32_t *total = table + (size_t)plan.tiles * plan.cols;
+    uint64_t *base_was = reinterpret_cast<uint64_t *>(total + plan.cols);
     hipLaunchKernelGGL(rank_count_kernel, dim3(plan.tiles), dim3(64), 0, s, keys, n, n_keys, plan.cols, plan.runs,
-                       table);
+                       table, status);
     hipLaunchKernelGGL(rank_scan_kernel, dim3((n_keys + SCAN_PEERS - 1u) / SCAN_PEERS),
-                       dim3(SCAN_PEERS * SCAN_PARTS), 0, s, table, plan.tiles, n_keys, plan.cols, total);
+                       dim3(SCAN_PEERS * SCAN_PARTS), 0, s, table, plan.tiles, n_keys, plan.cols, total, ctr_base,
+                       base_was, advance ? 1 : 0, ctr_limit);
     hipLaunchKernelGGL(rank_assign_kernel, dim3(plan.tiles), dim3(64), 0, s, keys, n, n_keys, plan.cols, plan.runs,
-                       table, key_bits(n_keys), ctr_base, ctr_out, ctr_limit, zero_others ? 1 : 0);
-    if (advance)
-        hipLaunchKernelGGL(rank_advance_kernel, dim3((n_keys + 255u) / 256u), dim3(256), 0, s, total, n_keys,
-                           ctr_base, ctr_limit);
+                       table, key_bits(n_keys), base_was, ctr_out, ctr_limit, zero_others ? 1 : 0);
     return hipGetLastError();
+}
+
+bool peer_rank_counts(uint32_t n, uint32_t n_keys, size_t tmp_bytes)
+{
+    const RankPlan plan = rank_plan(n, n_keys);
+    return n > PEER_RANK_SMALL_MAX && plan.fits && plan.bytes <= tmp_bytes;
+}
+
+hipError_t launch_peer_rank_counting(const uint32_t *peer, void *tmp, uint64_t *ctr_base, uint32_t n_keys, uint32_t n,
+                                     uint64_t *ctr_out, bool advance, uint64_t ctr_limit, uint32_t *status,
+                                     hipStream_t s)
+{
+    if (n == 0) return hipSuccess;
+    // (a packet whose peer lies beyond the table gets counter 0, as one without a peer does)
+    return launch_peer_rank_table(peer, rank_plan(n, n_keys), tmp, ctr_base, n_keys, n, ctr_out, advance, ctr_limit,
+                                  true, status, s);
 }
 
 hipError_t launch_peer_rank(uint32_t *keys, uint32_t *idx, uint32_t *skeys, uint32_t *sidx,
@@ -404,7 +429,7 @@ hipError_t launch_peer_rank(uint32_t *keys, uint32_t *idx, uint32_t *skeys, uint
     const RankPlan plan = rank_plan(n, n_keys);
     if (plan.fits && plan.bytes <= sort_tmp_bytes)
         return launch_peer_rank_table(keys, plan, sort_tmp, ctr_base, n_keys, n, ctr_out, advance, ctr_limit, false,
-                                      s);
+                                      nullptr, s);
     const dim3 grid((n + 255u) / 256u);
     hipError_t e = rocprim::radix_sort_pairs<SortConfig>(sort_tmp, sort_tmp_bytes, keys, skeys, idx, sidx, (size_t)n,
                                              0, key_bits(n_keys), s);

@@ -417,6 +417,9 @@ int bnk::wg_encap_impl(bnk_ctx *ctx, const bnk_batch *slots, uint32_t mtu, uint3
     if (n <= PEER_RANK_SMALL_MAX) {
         HIPCHK(ctx, launch_peer_rank_small(d_peer, pe.n, n, pe.send_ctr, d_ctr, true, WG_REJECT_AFTER_MESSAGES,
                                            ctx->d_status, ctx->stream));
+    } else if (d_peer && peer_rank_counts(n, pe.n, tmp_bytes)) {
+        HIPCHK(ctx, launch_peer_rank_counting(d_peer, ctx->r_tmp.p, pe.send_ctr, pe.n, n, d_ctr, true,
+                                              WG_REJECT_AFTER_MESSAGES, ctx->d_status, ctx->stream));
     } else {
         HIPCHK(ctx, launch_wg_keys(d_peer, pe.n, n, ctx->r_keys.as<uint32_t>(), ctx->r_idx.as<uint32_t>(),
                                    ctx->d_status, ctx->stream));

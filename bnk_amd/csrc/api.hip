@@ -439,6 +439,9 @@ int bnk_init(int device_ordinal, bnk_ctx **out)
         return bail("hipStreamCreate", e);
     if ((e = hipEventCreate(&ctx->ev0)) != hipSuccess) return bail("hipEventCreate", e);
     if ((e = hipEventCreate(&ctx->ev1)) != hipSuccess) return bail("hipEventCreate", e);
+    for (auto &t : ctx->tally_host) t.store(0, std::memory_order_relaxed);
+    if ((e = hipMalloc((void **)&ctx->d_tally, TALLY_SLOTS * 8)) != hipSuccess) return bail("hipMalloc", e);
+    if ((e = hipMemset(ctx->d_tally, 0, TALLY_SLOTS * 8)) != hipSuccess) return bail("hipMemset", e);
     if ((e = hipEventCreateWithFlags(&ctx->ev_noalloc, hipEventDisableTiming)) != hipSuccess)
         return bail("hipEventCreate", e);
     if ((e = hipHostMalloc((void **)&ctx->h_status, 64, hipHostMallocDefault)) != hipSuccess)
@@ -491,6 +494,7 @@ void bnk_shutdown(bnk_ctx *ctx)
         ctx->pin.release();
         for (HostStage &st : ctx->stages) st.pin.release();
         if (ctx->wg_replay) (void)hipFree(ctx->wg_replay);
+        if (ctx->d_tally) (void)hipFree(ctx->d_tally);
         for (const bnk_ctx::Ring &r : ctx->rings) (void)hipHostFree(reinterpret_cast<void *>(r.host));
         ctx->rings.clear();
         for (int w = 0; w < 2; w++)
@@ -677,11 +681,16 @@ int bnk_aead_seal_batch(bnk_ctx *ctx, const bnk_batch *in, const bnk_batch *out)
     {
         CoRequest rq{CO_SEAL, in, out, 0, 0, nullptr, nullptr, nullptr, nullptr};
         int crc;
-        if (out && coalesce_submit(ctx, rq, &crc)) return crc;
+        if (out && coalesce_submit(ctx, rq, &crc)) {
+            if (crc == BNK_OK) tally_add(ctx, TALLY_SEALED, in->n);
+            return crc;
+        }
     }
     Guard g(ctx);
     if (g.rc) return g.rc;
-    return aead_batch(ctx, false, in, out, nullptr, nullptr);
+    const int rc = aead_batch(ctx, false, in, out, nullptr, nullptr);
+    if (rc == BNK_OK) tally_add(ctx, TALLY_SEALED, in->n);
+    return rc;
     BNK_API_CATCH(ctx)
 }
 
@@ -691,11 +700,16 @@ int bnk_aead_open_batch(bnk_ctx *ctx, const bnk_batch *in, const bnk_batch *out,
     {
         CoRequest rq{CO_OPEN, in, out, 0, 0, verdict, nullptr, nullptr, nullptr};
         int crc;
-        if (out && coalesce_submit(ctx, rq, &crc)) return crc;
+        if (out && coalesce_submit(ctx, rq, &crc)) {
+            if (crc == BNK_OK) (void)tally_results(ctx, TALLY_OPEN, verdict, in->n, BNK_MEM_HOST);
+            return crc;
+        }
     }
     Guard g(ctx);
     if (g.rc) return g.rc;
-    return aead_batch(ctx, true, in, out, verdict, nullptr);
+    const int rc = aead_batch(ctx, true, in, out, verdict, nullptr);
+    if (rc == BNK_OK) return tally_results(ctx, TALLY_OPEN, verdict, in->n, in->mem);
+    return rc;
     BNK_API_CATCH(ctx)
 }
 

@@ -404,7 +404,9 @@ int bnk_filter_check_inbound_batch(bnk_ctx *ctx, const bnk_batch *pkts, int64_t 
     BNK_API_TRY
     Guard g(ctx);
     if (g.rc) return g.rc;
-    return filter_batch(ctx, true, pkts, now_ns, verdict);
+    const int rc = filter_batch(ctx, true, pkts, now_ns, verdict);
+    if (rc == BNK_OK && pkts) return tally_results(ctx, TALLY_CHECK, verdict, pkts->n, pkts->mem);
+    return rc;
     BNK_API_CATCH(ctx)
 }
 
@@ -424,7 +426,9 @@ int bnk_filter_check_inbound_ptrs(bnk_ctx *ctx, const uint8_t *const *pkts, cons
     BNK_API_TRY
     Guard g(ctx);
     if (g.rc) return g.rc;
-    return filter_ptrs(ctx, true, pkts, lens, n, now_ns, verdict);
+    const int rc = filter_ptrs(ctx, true, pkts, lens, n, now_ns, verdict);
+    if (rc == BNK_OK) return tally_results(ctx, TALLY_CHECK, verdict, n, BNK_MEM_HOST);
+    return rc;
     BNK_API_CATCH(ctx)
 }
 

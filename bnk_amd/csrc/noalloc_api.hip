@@ -81,6 +81,7 @@ extern "C" int bnk_aead_seal_batch_noalloc(bnk_ctx *ctx, const bnk_batch *in, co
     const int rc = aead_batch(ctx, false, in, out, nullptr, ptr);
     // (also after a failure: part of the work may have been enqueued)
     if (hipEventRecord(ctx->ev_noalloc, ctx->stream) == hipSuccess) g_last_user[ctx->device] = ctx;
+    if (rc == BNK_OK) tally_add(ctx, TALLY_SEALED, in->n); // (a host-side count: nothing is launched or allocated)
     return rc;
     BNK_API_CATCH(ctx)
 }

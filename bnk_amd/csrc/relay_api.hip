@@ -13,14 +13,10 @@ using namespace bnk;
 // the bytes between packets, the output arena up, and the output down).
 constexpr uint32_t RELAY_CHUNKS = 8;
 
-extern "C" int bnk_relay_fused_batch(bnk_ctx *ctx, const bnk_batch *in, const uint32_t *peer_out,
-                                     const uint64_t *ctr_base_out, uint32_t n_peers_out,
-                                     int64_t now_ns, const bnk_batch *out, uint8_t *verdict,
-                                     uint64_t *ctr_out)
+static int relay_impl(bnk_ctx *ctx, const bnk_batch *in, const uint32_t *peer_out, const uint64_t *ctr_base_out,
+                      uint32_t n_peers_out, int64_t now_ns, const bnk_batch *out, uint8_t *verdict,
+                      uint64_t *ctr_out)
 {
-    BNK_API_TRY
-    Guard g(ctx);
-    if (g.rc) return g.rc;
     int rc = check_batch_common(ctx, in, "in");
     if (rc) return rc;
     rc = check_batch_common(ctx, out, "out");
@@ -347,5 +343,19 @@ extern "C" int bnk_relay_fused_batch(bnk_ctx *ctx, const bnk_batch *in, const ui
     rc = take_status(ctx, &status);
     if (rc) return rc;
     return status_to_rc(ctx, status);
+}
+
+extern "C" int bnk_relay_fused_batch(bnk_ctx *ctx, const bnk_batch *in, const uint32_t *peer_out,
+                                     const uint64_t *ctr_base_out, uint32_t n_peers_out,
+                                     int64_t now_ns, const bnk_batch *out, uint8_t *verdict,
+                                     uint64_t *ctr_out)
+{
+    BNK_API_TRY
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    const int rc = relay_impl(ctx, in, peer_out, ctr_base_out, n_peers_out, now_ns, out, verdict, ctr_out);
+    // (every packet relayed was opened and re-sealed on the way)
+    if (rc == BNK_OK) return tally_results(ctx, TALLY_RELAY, verdict, in->n, in->mem);
+    return rc;
     BNK_API_CATCH(ctx)
 }

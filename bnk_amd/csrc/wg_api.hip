@@ -562,11 +562,16 @@ extern "C" int bnk_wg_encap_batch(bnk_ctx *ctx, const bnk_batch *slots, uint32_t
     {
         CoRequest rq{CO_ENCAP, slots, nullptr, mtu, 0, nullptr, wire_len, nullptr, nullptr};
         int crc;
-        if (coalesce_submit(ctx, rq, &crc)) return crc;
+        if (coalesce_submit(ctx, rq, &crc)) {
+            if (crc == BNK_OK) (void)tally_nonzero(ctx, TALLY_SEALED, wire_len, slots->n, BNK_MEM_HOST);
+            return crc;
+        }
     }
     Guard g(ctx);
     if (g.rc) return g.rc;
-    return wg_encap_impl(ctx, slots, mtu, wire_len, nullptr);
+    const int rc = wg_encap_impl(ctx, slots, mtu, wire_len, nullptr);
+    if (rc == BNK_OK) return tally_nonzero(ctx, TALLY_SEALED, wire_len, slots->n, slots->mem);
+    return rc;
     BNK_API_CATCH(ctx)
 }
 
@@ -577,11 +582,16 @@ extern "C" int bnk_wg_note_encap_batch(bnk_ctx *ctx, const bnk_batch *slots, uin
     {
         CoRequest rq{CO_NOTE_ENCAP, slots, nullptr, mtu, now_ns, nullptr, wire_len, nullptr, nullptr};
         int crc;
-        if (coalesce_submit(ctx, rq, &crc)) return crc;
+        if (coalesce_submit(ctx, rq, &crc)) {
+            if (crc == BNK_OK) (void)tally_nonzero(ctx, TALLY_SEALED, wire_len, slots->n, BNK_MEM_HOST);
+            return crc;
+        }
     }
     Guard g(ctx);
     if (g.rc) return g.rc;
-    return wg_encap_impl(ctx, slots, mtu, wire_len, &now_ns);
+    const int rc = wg_encap_impl(ctx, slots, mtu, wire_len, &now_ns);
+    if (rc == BNK_OK) return tally_nonzero(ctx, TALLY_SEALED, wire_len, slots->n, slots->mem);
+    return rc;
     BNK_API_CATCH(ctx)
 }
 
@@ -983,11 +993,16 @@ extern "C" int bnk_wg_decap_batch(bnk_ctx *ctx, const bnk_batch *wire, const bnk
     {
         CoRequest rq{CO_DECAP, wire, out, 0, 0, result, out_len, peer, counter};
         int crc;
-        if (coalesce_submit(ctx, rq, &crc)) return crc;
+        if (coalesce_submit(ctx, rq, &crc)) {
+            if (crc == BNK_OK) (void)tally_results(ctx, TALLY_DECAP, result, wire->n, BNK_MEM_HOST);
+            return crc;
+        }
     }
     Guard g(ctx);
     if (g.rc) return g.rc;
-    return wg_decap_impl(ctx, wire, out, result, out_len, peer, counter, nullptr);
+    const int rc = wg_decap_impl(ctx, wire, out, result, out_len, peer, counter, nullptr);
+    if (rc == BNK_OK) return tally_results(ctx, TALLY_DECAP, result, wire->n, wire->mem);
+    return rc;
     BNK_API_CATCH(ctx)
 }
 
@@ -999,10 +1014,15 @@ extern "C" int bnk_wg_decap_filter_batch(bnk_ctx *ctx, const bnk_batch *wire, co
     {
         CoRequest rq{CO_DECAP_FILTER, wire, out, 0, now_ns, result, out_len, peer, counter};
         int crc;
-        if (coalesce_submit(ctx, rq, &crc)) return crc;
+        if (coalesce_submit(ctx, rq, &crc)) {
+            if (crc == BNK_OK) (void)tally_results(ctx, TALLY_DECAP_CHECK, result, wire->n, BNK_MEM_HOST);
+            return crc;
+        }
     }
     Guard g(ctx);
     if (g.rc) return g.rc;
-    return wg_decap_impl(ctx, wire, out, result, out_len, peer, counter, &now_ns);
+    const int rc = wg_decap_impl(ctx, wire, out, result, out_len, peer, counter, &now_ns);
+    if (rc == BNK_OK) return tally_results(ctx, TALLY_DECAP_CHECK, result, wire->n, wire->mem);
+    return rc;
     BNK_API_CATCH(ctx)
 }

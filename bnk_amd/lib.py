@@ -61,6 +61,16 @@ class CoalesceStats(C.Structure):
         return {k: int(getattr(self, k)) for k, _ in self._fields_}
 
 
+class Counters(C.Structure):
+    """struct bnk_counters"""
+    _fields_ = [(k, C.c_uint64) for k in ("sealed", "opened", "rejected", "allowed", "denied", "delivered",
+                                          "keepalive", "replayed", "bad_header", "unknown_index", "bad_ip",
+                                          "not_allowed", "relayed")]
+
+    def as_dict(self) -> dict:
+        return {k: int(getattr(self, k)) for k, _ in self._fields_}
+
+
 _lib = None
 
 
@@ -232,6 +242,15 @@ class Context:
         st = CoalesceStats()
         self._chk(self._lib.bnk_coalesce_stats_get(self._h, C.byref(st)))
         return st.as_dict()
+
+    def counters(self) -> dict:
+        """Packets by outcome since the context was made or the counters were reset."""
+        c = Counters()
+        self._chk(self._lib.bnk_counters_get(self._h, C.byref(c)))
+        return c.as_dict()
+
+    def counters_reset(self) -> None:
+        self._chk(self._lib.bnk_counters_reset(self._h))
 
     def set_spread_max_packets(self, max_packets: int) -> None:
         """Batches of at most this many packets run one wave per packet

@@ -199,6 +199,35 @@ typedef struct bnk_coalesce_stats {
 } bnk_coalesce_stats;
 int bnk_coalesce_stats_get(bnk_ctx *ctx, bnk_coalesce_stats *out);
 
+/* ---- hot-path counters -------------------------------------------------- */
+
+/* Packets by outcome since bnk_init (or the last reset), over every entry point
+ * of this context.  An addition: the reference keeps no such counts (its
+ * filter drops without counting, internal/filter/filter.go:100-145, and
+ * wireguard-go counts bytes per peer only).  They are a histogram of the
+ * result bytes every call already leaves per packet, taken on the host for a
+ * host batch and by one small launch behind a device-resident batch; a call
+ * that returns an error counts nothing.
+ *   sealed         bnk_aead_seal_batch(_noalloc), packets bnk_wg_(note_)encap_batch
+ *                  gave a wire length other than 0
+ *   opened         bnk_aead_open_batch, verdict 1
+ *   rejected       a tag that did not verify: bnk_aead_open_batch verdict 0,
+ *                  BNK_WG_AUTH_FAIL, BNK_RELAY_FORGED
+ *   allowed/denied CheckInbound: bnk_filter_check_inbound_* verdict 1 / 0;
+ *                  bnk_wg_decap_filter_batch BNK_WG_OK / BNK_WG_FILTERED;
+ *                  BNK_RELAY_DENIED
+ *   delivered      BNK_WG_OK of the decapsulating calls
+ *   keepalive, replayed, bad_header, unknown_index, bad_ip, not_allowed
+ *                  the BNK_WG_* results of those names
+ *   relayed        BNK_RELAY_OK (opened and re-sealed)
+ * bnk_counters_get waits for the context's stream. */
+typedef struct bnk_counters {
+    uint64_t sealed, opened, rejected, allowed, denied, delivered, keepalive, replayed, bad_header,
+        unknown_index, bad_ip, not_allowed, relayed;
+} bnk_counters;
+int bnk_counters_get(bnk_ctx *ctx, bnk_counters *out);
+int bnk_counters_reset(bnk_ctx *ctx);
+
 /* ---- transport AEAD ---------------------------------------------------- */
 
 /* Loads n_peers 32-byte ChaCha20-Poly1305 keys (host memory) into key table

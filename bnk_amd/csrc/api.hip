@@ -385,17 +385,21 @@ uint32_t read_status_words(bnk_ctx *ctx)
 {
     volatile uint32_t *h = ctx->h_status;
     const uint32_t status = (h[STATUS_PEER_RANGE] ? STATUS_PEER_RANGE : 0u) |
-                            (h[STATUS_FLOWS_FULL] ? STATUS_FLOWS_FULL : 0u) | (h[STATUS_BOUNDS] ? STATUS_BOUNDS : 0u);
+                            (h[STATUS_FLOWS_FULL] ? STATUS_FLOWS_FULL : 0u) | (h[STATUS_BOUNDS] ? STATUS_BOUNDS : 0u) |
+                            (h[STATUS_INTERNAL] ? STATUS_INTERNAL : 0u);
     if (status) {
         h[STATUS_PEER_RANGE] = 0;
         h[STATUS_FLOWS_FULL] = 0;
         h[STATUS_BOUNDS] = 0;
+        h[STATUS_INTERNAL] = 0;
     }
     return status;
 }
 
 int status_to_rc(bnk_ctx *ctx, uint32_t status)
 {
+    if (status & STATUS_INTERNAL)
+        return fail(ctx, BNK_E_HIP, "a launch for short packets met a packet it does not handle (packets were skipped)");
     if (status & STATUS_BOUNDS)
         return fail(ctx, BNK_E_INVAL, "a packet of a device-resident batch reaches beyond its arena (it was skipped)");
     if (status & STATUS_PEER_RANGE) return fail(ctx, BNK_E_RANGE, "peer index beyond the key table");

@@ -121,7 +121,7 @@ constexpr uint32_t SPREAD_MAX_PACKETS = 4096;
 // plain store of 1 (the same store from every lane that has the news, so no
 // atomic is needed), and read by the host after it has waited for the stream,
 // with no copy.
-enum : uint32_t { STATUS_PEER_RANGE = 1u, STATUS_FLOWS_FULL = 2u, STATUS_BOUNDS = 4u };
+enum : uint32_t { STATUS_PEER_RANGE = 1u, STATUS_FLOWS_FULL = 2u, STATUS_BOUNDS = 4u, STATUS_INTERNAL = 8u };
 constexpr uint32_t STATUS_WORDS = 8; // word [bit value] holds that condition
 // Word 7 of the same block is no condition: a one-thread launch writes the number of the
 // wait it ends there, for the host to watch (wait_stream in api.hip).

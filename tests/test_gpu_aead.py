@@ -639,3 +639,60 @@ def test_concurrent_callers_share_one_context(ctx):
     for t in threads:
         t.join()
     assert not errors, errors[:3]
+
+
+@pytest.mark.parametrize("length", [0, 1, 15, 16, 17, 60, 63, 64, 65, 100, 127, 128, 129])
+@pytest.mark.parametrize("stride,shift", [(256, 0), (160, 16), (176, 48)])
+def test_uniform_short_device_batches_against_the_oracle(ctx, length, stride, shift):
+    """Device-resident batches of one common length up to 128 bytes with every
+    packet 16-byte aligned at the same place of a line in both arenas run in a
+    launch of their own (more waves per SIMD); 129 bytes and the strides that
+    put packets across two lines take the other paths.  Every ciphertext and
+    tag against the oracle, the round trip, and a forged tag's zero-fill."""
+    import torch
+    from bnk_amd import lib
+    from oracle import binding as O
+    n = 40000 + 37  # beyond the wave-per-packet launches, and not a whole number of waves
+    rng = np.random.default_rng(1000 + length)
+    keys = rng.integers(0, 256, (3, 32), dtype=np.uint8)
+    ctx.keys_set(lib.KEYS_SEND, keys)
+    ctx.keys_set(lib.KEYS_RECV, keys)
+    peer = rng.integers(0, 3, n).astype(np.uint32)
+    ctr = rng.integers(0, 1 << 62, n).astype(np.uint64)
+    nb = n * stride + shift + 64
+    plain = rng.integers(0, 256, nb, dtype=np.uint8)
+    off = (np.arange(n, dtype=np.uint64) * np.uint64(stride)) + np.uint64(shift)
+    want = np.zeros(nb, np.uint8)
+    O.seal_batch(keys, peer, ctr, plain, off, np.full(n, length, np.uint32), want, off, 4)
+    d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to("cuda:0")  # noqa: E731
+    d_plain, d_ct = d(plain), torch.zeros(nb, dtype=torch.uint8, device="cuda:0")
+    d_back = torch.full((nb,), 0xEE, dtype=torch.uint8, device="cuda:0")
+    d_peer, d_ctr = d(peer.astype(np.int32)), d(ctr.astype(np.int64))
+    verdict = torch.zeros(n, dtype=torch.uint8, device="cuda:0")
+    torch.cuda.synchronize()
+    view = lambda t: t[shift:]  # noqa: E731  (the batch starts `shift` bytes into the allocation)
+    ctx.seal(lib.make_batch(view(d_plain), nb - shift, n, lib.MEM_DEVICE, stride=stride, length=length, peer=d_peer,
+                            counters=d_ctr),
+             lib.make_batch(view(d_ct), nb - shift, n, lib.MEM_DEVICE, stride=stride))
+    ctx.sync()
+    got = d_ct.cpu().numpy()
+    assert np.array_equal(got, want)  # nothing between or beyond the packets was written either
+    forged = rng.choice(n, 9, replace=False)
+    got2 = got.copy()
+    got2[(off[forged] + np.uint64(length + 5)).astype(np.int64)] ^= 0x40
+    d_ct2 = d(got2)
+    torch.cuda.synchronize()
+    ctx.open(lib.make_batch(view(d_ct2), nb - shift, n, lib.MEM_DEVICE, stride=stride, length=length + 16,
+                            peer=d_peer, counters=d_ctr),
+             lib.make_batch(view(d_back), nb - shift, n, lib.MEM_DEVICE, stride=stride), verdict)
+    ctx.sync()
+    v = verdict.cpu().numpy()
+    expect_v = np.ones(n, np.uint8)
+    expect_v[forged] = 0
+    assert np.array_equal(v, expect_v)
+    back = d_back.cpu().numpy()
+    expect = np.full(nb, 0xEE, np.uint8)
+    for i in range(n):
+        o = int(off[i])
+        expect[o:o + length] = 0 if v[i] == 0 else plain[o:o + length]
+    assert np.array_equal(back, expect)

@@ -703,8 +703,9 @@ BNK_DEV void body_short(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
 
 // Tag and verdict of each lane's packet once its bytes have gone through the
 // MAC, and the zero-fill of rejected plaintexts.
+// Returns whether the lane's packet was rejected.
 template <bool OPEN>
-BNK_DEV void lane_finish(const AeadArgs &a, uint32_t lane, bool have, uint32_t i, uint32_t len,
+BNK_DEV bool lane_finish(const AeadArgs &a, uint32_t lane, bool have, uint32_t i, uint32_t len,
                          const uint8_t *src, uint8_t *dst, Poly32 &mac, const Head &head, uint8_t *record,
                          bool decap = false, uint32_t pr = 0)
 {
@@ -783,6 +784,7 @@ BNK_DEV void lane_finish(const AeadArgs &a, uint32_t lane, bool have, uint32_t i
             }
         }
     }
+    return reject;
 }
 
 // A lane per packet.  SHORT_ONLY: the launch for batches in which every wave
@@ -940,8 +942,18 @@ BNK_DEV void wave_main(const AeadArgs &a, uint8_t *tile)
     }
     else body_lines<OPEN, true>(tile, lane, src, dst, len, len_in, safe, k, n1, n2, mac, x, head);
 
-    lane_finish<OPEN>(a, lane, have, i, len, src, dst, mac, head, in_batch && a.heads ? a.heads + 32ull * t : nullptr,
-                      decap && in_batch && wg_res == BNK_WG_OK, pr);
+    const bool reject = lane_finish<OPEN>(a, lane, have, i, len, src, dst, mac, head,
+                                          in_batch && a.heads ? a.heads + 32ull * t : nullptr,
+                                          decap && in_batch && wg_res == BNK_WG_OK, pr);
+    if (OPEN && a.tally) {
+        // a plain open counting its own verdicts: verdict 1 exactly where the lane had a packet
+        // whose tag verified
+        const unsigned long long ok = __ballot(have && !reject), all = __ballot(in_batch);
+        if (lane == 0u) {
+            tally_bump(a.tally, TALLY_OPENED, (uint32_t)__popcll(ok));
+            tally_bump(a.tally, TALLY_REJECTED, (uint32_t)__popcll(all & ~ok));
+        }
+    }
 }
 
 template <bool OPEN>

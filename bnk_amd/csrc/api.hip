@@ -251,7 +251,12 @@ int aead_batch(bnk_ctx *ctx, bool open, const bnk_batch *in, const bnk_batch *ou
             rc = maybe_sort(ctx, &a, open ? 16 : 0);
             if (rc) return rc;
         }
+        // the verdicts are counted by the launch itself where a lane has a packet, else by a
+        // launch behind it
+        const bool count = open && ctx->tally_on.load(std::memory_order_relaxed);
+        if (count && !aead_runs_spread(a)) a.tally = reinterpret_cast<unsigned long long *>(ctx->d_tally);
         HIPCHK(ctx, open ? launch_aead_open(a, ctx->stream) : launch_aead_seal(a, ctx->stream));
+        if (count && !a.tally) return tally_results(ctx, TALLY_OPEN, verdict, n, BNK_MEM_DEVICE);
         return BNK_OK;
     }
     if (sort_scratch) return fail(ctx, BNK_E_INVAL, "this entry point takes device-resident batches only");
@@ -444,8 +449,9 @@ int bnk_init(int device_ordinal, bnk_ctx **out)
     if ((e = hipEventCreate(&ctx->ev0)) != hipSuccess) return bail("hipEventCreate", e);
     if ((e = hipEventCreate(&ctx->ev1)) != hipSuccess) return bail("hipEventCreate", e);
     for (auto &t : ctx->tally_host) t.store(0, std::memory_order_relaxed);
-    if ((e = hipMalloc((void **)&ctx->d_tally, TALLY_SLOTS * 8)) != hipSuccess) return bail("hipMalloc", e);
-    if ((e = hipMemset(ctx->d_tally, 0, TALLY_SLOTS * 8)) != hipSuccess) return bail("hipMemset", e);
+    if ((e = hipMalloc((void **)&ctx->d_tally, TALLY_SLOTS * TALLY_LANES * 8)) != hipSuccess)
+        return bail("hipMalloc", e);
+    if ((e = hipMemset(ctx->d_tally, 0, TALLY_SLOTS * TALLY_LANES * 8)) != hipSuccess) return bail("hipMemset", e);
     if ((e = hipEventCreateWithFlags(&ctx->ev_noalloc, hipEventDisableTiming)) != hipSuccess)
         return bail("hipEventCreate", e);
     if ((e = hipHostMalloc((void **)&ctx->h_status, 64, hipHostMallocDefault)) != hipSuccess)
@@ -712,7 +718,8 @@ int bnk_aead_open_batch(bnk_ctx *ctx, const bnk_batch *in, const bnk_batch *out,
     Guard g(ctx);
     if (g.rc) return g.rc;
     const int rc = aead_batch(ctx, true, in, out, verdict, nullptr);
-    if (rc == BNK_OK) return tally_results(ctx, TALLY_OPEN, verdict, in->n, in->mem);
+    // (a device-resident batch has been counted on the device)
+    if (rc == BNK_OK && in->mem == BNK_MEM_HOST) return tally_results(ctx, TALLY_OPEN, verdict, in->n, BNK_MEM_HOST);
     return rc;
     BNK_API_CATCH(ctx)
 }

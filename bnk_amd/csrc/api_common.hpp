@@ -78,11 +78,6 @@ struct Guard {
 // Hot-path counters (tally.hip).  A host batch's result bytes are counted on the
 // host, a device-resident batch's by a launch behind the batch on ctx->stream
 // (the caller holds the context's lock, as for every launch).
-enum TallySlot {
-    TALLY_SEALED, TALLY_OPENED, TALLY_REJECTED, TALLY_ALLOWED, TALLY_DENIED, TALLY_DELIVERED, TALLY_KEEPALIVE,
-    TALLY_REPLAYED, TALLY_BAD_HEADER, TALLY_UNKNOWN_INDEX, TALLY_BAD_IP, TALLY_NOT_ALLOWED, TALLY_RELAYED
-};
-static_assert(TALLY_RELAYED < TALLY_SLOTS, "slots");
 enum TallyKind { TALLY_OPEN, TALLY_CHECK, TALLY_DECAP, TALLY_DECAP_CHECK, TALLY_RELAY };
 void tally_add(bnk_ctx *ctx, TallySlot slot, uint64_t k);
 int tally_results(bnk_ctx *ctx, TallyKind kind, const uint8_t *res, uint32_t n, int mem);

@@ -99,7 +99,6 @@ struct HostStage {
     std::atomic<bool> busy{false}; // taken by a window's leader until it has copied its results out
 };
 constexpr uint32_t HOST_STAGES = 4;
-constexpr int TALLY_SLOTS = 16; // hot-path counters (tally.hip)
 
 } // namespace bnk
 
@@ -109,9 +108,10 @@ struct bnk_ctx {
     int device = -1;
     hipStream_t stream = nullptr;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
-    // hot-path counters: [slot], what launches counted and what the host counted
+    // hot-path counters: what launches counted ([slot][TALLY_LANES]) and what the host counted ([slot])
     uint64_t *d_tally = nullptr;
     std::atomic<uint64_t> tally_host[bnk::TALLY_SLOTS];
+    std::atomic<bool> tally_on{true};
     hipEvent_t ev_noalloc = nullptr; // recorded behind every bnk_aead_seal_batch_noalloc of this context
     // chunked host batches: upload and download streams, one event pair per chunk
     hipStream_t s_up = nullptr, s_down = nullptr;

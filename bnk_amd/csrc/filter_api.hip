@@ -231,7 +231,9 @@ int check_device_layout(bnk_ctx *ctx, const bnk_batch *b)
     return BNK_OK;
 }
 
-int filter_batch(bnk_ctx *ctx, bool check, const bnk_batch *pkts, int64_t now_ns, uint8_t *verdict)
+// *counted (check only): the launch has counted its own verdicts (bnk_counters_get)
+int filter_batch(bnk_ctx *ctx, bool check, const bnk_batch *pkts, int64_t now_ns, uint8_t *verdict,
+                 bool *counted = nullptr)
 {
     int rc = check_batch_common(ctx, pkts, "pkts");
     if (rc) return rc;
@@ -262,6 +264,10 @@ int filter_batch(bnk_ctx *ctx, bool check, const bnk_batch *pkts, int64_t now_ns
         a.len = pkts->len;
         a.verdict = verdict;
         if (pkts->offsets || pkts->lens) a.limit = pkts->bytes; // the lanes check what the host cannot read
+        if (check && counted && ctx->tally_on.load(std::memory_order_relaxed)) {
+            a.tally = reinterpret_cast<unsigned long long *>(ctx->d_tally);
+            *counted = true;
+        }
         HIPCHK(ctx, check ? launch_filter_check(a, f->max_blocks, ctx->stream)
                           : launch_filter_note(a, f->max_blocks, f->claimed_upper > 4096, ctx->stream));
         return BNK_OK;
@@ -404,8 +410,9 @@ int bnk_filter_check_inbound_batch(bnk_ctx *ctx, const bnk_batch *pkts, int64_t 
     BNK_API_TRY
     Guard g(ctx);
     if (g.rc) return g.rc;
-    const int rc = filter_batch(ctx, true, pkts, now_ns, verdict);
-    if (rc == BNK_OK && pkts) return tally_results(ctx, TALLY_CHECK, verdict, pkts->n, pkts->mem);
+    bool counted = false;
+    const int rc = filter_batch(ctx, true, pkts, now_ns, verdict, &counted);
+    if (rc == BNK_OK && pkts && !counted) return tally_results(ctx, TALLY_CHECK, verdict, pkts->n, pkts->mem);
     return rc;
     BNK_API_CATCH(ctx)
 }

@@ -75,6 +75,8 @@ struct FilterArgs {
     uint8_t *verdict;     // check only
     uint8_t *wg_result;   // check only, or nullptr: the BNK_WG_* results of the decapsulation that
                           // delivered these packets; a denied packet's BNK_WG_OK becomes BNK_WG_FILTERED
+    unsigned long long *tally; // check only, or nullptr: the launch counts its verdicts here
+                          // (TALLY_ALLOWED / TALLY_DENIED, see tally_bump)
     uint32_t *status;
     int64_t now;
     uint32_t n, stride, len;

@@ -292,6 +292,7 @@ __global__ __launch_bounds__(FILTER_THREADS, 8) void filter_check_kernel(FilterA
     __syncthreads();
     const uint32_t stride = gridDim.x * FILTER_THREADS;
     const uint32_t lane = threadIdx.x & 63u;
+    uint32_t n_pass = 0, n_drop = 0; // this wave's verdicts (the same in every lane)
     // whole waves stay in the loop together: the rule lookup is a joint effort
     for (uint32_t i0 = blockIdx.x * FILTER_THREADS + (threadIdx.x & ~63u); i0 < a.n; i0 += stride) {
         // t: this lane's place in the sweep; i: the packet it answers for
@@ -388,6 +389,15 @@ __global__ __launch_bounds__(FILTER_THREADS, 8) void filter_check_kernel(FilterA
             // a packet WireGuard delivered and this filter denied (BNK_WG_OK is 0)
             if (a.wg_result && !pass && a.wg_result[i] == 0) a.wg_result[i] = BNK_WG_FILTERED;
         }
+        if (a.tally) {
+            const unsigned long long in = __ballot(t < a.n), ok = __ballot(t < a.n && pass != 0);
+            n_pass += (uint32_t)__popcll(ok);
+            n_drop += (uint32_t)__popcll(in & ~ok);
+        }
+    }
+    if (a.tally && lane == 0u) {
+        tally_bump(a.tally, TALLY_ALLOWED, n_pass);
+        tally_bump(a.tally, TALLY_DENIED, n_drop);
     }
 }
 

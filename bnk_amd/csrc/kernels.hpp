@@ -109,6 +109,8 @@ struct AeadArgs {
                                // has checked the layout
     uint32_t first;            // the launch covers packets first .. first+n-1; order[] is relative to first
     uint32_t spread_max;       // launches of at most this many packets run one wave per packet
+    unsigned long long *tally; // open, a lane per packet, or nullptr: the launch counts its own verdicts
+                               // here (TALLY_OPENED / TALLY_REJECTED, see tally_bump)
     WgFuse wg;                 // only with aead_runs_spread(); mode 0: plain AEAD
 };
 
@@ -121,6 +123,23 @@ constexpr uint32_t SPREAD_MAX_PACKETS = 4096;
 // plain store of 1 (the same store from every lane that has the news, so no
 // atomic is needed), and read by the host after it has waited for the stream,
 // with no copy.
+// Hot-path counters (tally.hip): TALLY_LANES words per counter, summed when they
+// are read, so that the waves of a launch that counts for itself spread their
+// additions.
+enum TallySlot {
+    TALLY_SEALED, TALLY_OPENED, TALLY_REJECTED, TALLY_ALLOWED, TALLY_DENIED, TALLY_DELIVERED, TALLY_KEEPALIVE,
+    TALLY_REPLAYED, TALLY_BAD_HEADER, TALLY_UNKNOWN_INDEX, TALLY_BAD_IP, TALLY_NOT_ALLOWED, TALLY_RELAYED
+};
+constexpr int TALLY_SLOTS = 16;
+constexpr uint32_t TALLY_LANES = 64;
+static_assert(TALLY_RELAYED < TALLY_SLOTS, "slots");
+#if defined(__HIPCC__)
+__device__ inline void tally_bump(unsigned long long *tally, uint32_t slot, uint32_t k)
+{
+    if (k != 0u) atomicAdd(&tally[slot * TALLY_LANES + (blockIdx.x & (TALLY_LANES - 1u))], (unsigned long long)k);
+}
+#endif
+
 enum : uint32_t { STATUS_PEER_RANGE = 1u, STATUS_FLOWS_FULL = 2u, STATUS_BOUNDS = 4u, STATUS_INTERNAL = 8u };
 constexpr uint32_t STATUS_WORDS = 8; // word [bit value] holds that condition
 // Word 7 of the same block is no condition: a one-thread launch writes the number of the

@@ -3,11 +3,14 @@
 // counters, internal/filter/filter.go:100-145; wireguard-go counts bytes per
 // peer only), so these are an addition, read through bnk_counters_get.
 //
-// Nothing in the packet kernels changes for them: every entry point already
-// leaves one result byte per packet (verdict / result), and the counts are a
-// histogram of those bytes, taken where they lie -- on the host for a host
-// batch (the bytes have just come back), by one small launch behind the batch's
-// own work for a device-resident one.
+// Every entry point already leaves one result byte per packet (verdict /
+// result), and the counts are a histogram of those bytes, taken where they lie:
+// on the host for a host batch (the bytes have just come back); for a
+// device-resident one by the launch that writes them where it is the last to
+// touch them (a plain open, a CheckInbound on its own: a vote per wave and two
+// atomics, see tally_bump), else by one small launch behind the batch's own work
+// (the framing calls, whose results the window pass and the filter still change,
+// and the relay).
 #include "api_common.hpp"
 #include "kernels.hpp"
 
@@ -63,30 +66,52 @@ TallyMap map_of(TallyKind kind)
     return m;
 }
 
-// One count per result value per block in LDS, then one atomic per value that
-// occurred: a few hundred atomics for a batch of a million.
+// A thread takes 16 consecutive result bytes (one load where they are aligned).
+// Within a wave the lanes vote per distinct value and lane v keeps value v's
+// count in a register, so nothing is contended; lanes 0-15 of every wave then
+// add into the block's 16 LDS words, and the block issues one global atomic per
+// value that occurred: a few hundred atomics for a batch of a million.
 constexpr uint32_t TALLY_PER_THREAD = 16;
+
+__device__ __forceinline__ void tally_vote(uint32_t v, bool valid, uint32_t lane, uint32_t &mine)
+{
+    unsigned long long todo = __ballot(valid && v < 16u);
+    while (todo != 0ull) {
+        const int leader = __ffsll((long long)todo) - 1;
+        const uint32_t lv = (uint32_t)__builtin_amdgcn_readlane((int)v, leader);
+        const unsigned long long same = __ballot(valid && v == lv);
+        if (lane == lv) mine += (uint32_t)__popcll(same);
+        todo &= ~same;
+    }
+}
+
 __global__ __launch_bounds__(256) void tally_kernel(const uint8_t *res, uint32_t n, TallyMap map,
                                                     unsigned long long *counters)
 {
     __shared__ uint32_t hist[16];
     if (threadIdx.x < 16u) hist[threadIdx.x] = 0u;
     __syncthreads();
-    const uint32_t first = blockIdx.x * (256u * TALLY_PER_THREAD);
-#pragma unroll 4
-    for (uint32_t k = 0; k < TALLY_PER_THREAD; k++) {
-        const uint32_t i = first + k * 256u + threadIdx.x;
-        if (i < n) {
-            const uint8_t v = res[i];
-            if (v < 16u) atomicAdd(&hist[v], 1u);
-        }
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint64_t first = ((uint64_t)blockIdx.x * 256u + threadIdx.x) * TALLY_PER_THREAD;
+    uint32_t w[4] = {0, 0, 0, 0};
+    const bool whole = first + TALLY_PER_THREAD <= n && (((uintptr_t)(res + first)) & 15u) == 0;
+    if (whole) {
+        const uint4 q = *reinterpret_cast<const uint4 *>(res + first);
+        w[0] = q.x; w[1] = q.y; w[2] = q.z; w[3] = q.w;
+    } else {
+        for (uint32_t k = 0; k < TALLY_PER_THREAD; k++)
+            if (first + k < n) w[k >> 2] |= (uint32_t)res[first + k] << (8u * (k & 3u));
     }
+    uint32_t mine = 0; // lane v: how often value v occurred in this wave
+#pragma unroll
+    for (uint32_t k = 0; k < TALLY_PER_THREAD; k++)
+        tally_vote((w[k >> 2] >> (8u * (k & 3u))) & 0xFFu, first + k < n, lane, mine);
+    if (lane < 16u && mine != 0u) atomicAdd(&hist[lane], mine);
     __syncthreads();
     if (threadIdx.x < 16u && hist[threadIdx.x] != 0u) {
         if (map.slot[threadIdx.x] != NONE)
-            atomicAdd(&counters[map.slot[threadIdx.x]], (unsigned long long)hist[threadIdx.x]);
-        if (map.also[threadIdx.x] != NONE)
-            atomicAdd(&counters[map.also[threadIdx.x]], (unsigned long long)hist[threadIdx.x]);
+            tally_bump(counters, map.slot[threadIdx.x], hist[threadIdx.x]);
+        if (map.also[threadIdx.x] != NONE) tally_bump(counters, map.also[threadIdx.x], hist[threadIdx.x]);
     }
 }
 
@@ -97,28 +122,35 @@ __global__ __launch_bounds__(256) void tally_nonzero_kernel(const uint32_t *word
     __shared__ uint32_t count;
     if (threadIdx.x == 0u) count = 0u;
     __syncthreads();
-    const uint32_t first = blockIdx.x * (256u * TALLY_PER_THREAD);
-    uint32_t mine = 0;
-#pragma unroll 4
+    // (consecutive lanes read consecutive words)
+    const uint64_t first = (uint64_t)blockIdx.x * (256u * TALLY_PER_THREAD) + threadIdx.x;
+    uint32_t w[TALLY_PER_THREAD];
+#pragma unroll
     for (uint32_t k = 0; k < TALLY_PER_THREAD; k++) {
-        const uint32_t i = first + k * 256u + threadIdx.x;
-        if (i < n && words[i] != 0u) mine++;
+        const uint64_t i = first + (uint64_t)k * 256u;
+        w[k] = i < n ? words[i] : 0u;
     }
-    if (mine) atomicAdd(&count, mine);
+    uint32_t mine = 0;
+#pragma unroll
+    for (uint32_t k = 0; k < TALLY_PER_THREAD; k++) mine += w[k] != 0u ? 1u : 0u;
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) mine += (uint32_t)__shfl_xor((int)mine, off, 64);
+    if ((threadIdx.x & 63u) == 0u && mine != 0u) atomicAdd(&count, mine);
     __syncthreads();
-    if (threadIdx.x == 0u && count != 0u) atomicAdd(&counters[slot], (unsigned long long)count);
+    if (threadIdx.x == 0u) tally_bump(counters, slot, count);
 }
 
 } // namespace
 
 void tally_add(bnk_ctx *ctx, TallySlot slot, uint64_t k)
 {
+    if (!ctx->tally_on.load(std::memory_order_relaxed)) return;
     ctx->tally_host[slot].fetch_add(k, std::memory_order_relaxed);
 }
 
 int tally_results(bnk_ctx *ctx, TallyKind kind, const uint8_t *res, uint32_t n, int mem)
 {
-    if (!res || n == 0) return BNK_OK;
+    if (!res || n == 0 || !ctx->tally_on.load(std::memory_order_relaxed)) return BNK_OK;
     const TallyMap map = map_of(kind);
     if (mem == BNK_MEM_HOST) {
         uint64_t hist[16] = {0};
@@ -139,7 +171,7 @@ int tally_results(bnk_ctx *ctx, TallyKind kind, const uint8_t *res, uint32_t n, 
 
 int tally_nonzero(bnk_ctx *ctx, TallySlot slot, const uint32_t *words, uint32_t n, int mem)
 {
-    if (!words || n == 0) return BNK_OK;
+    if (!words || n == 0 || !ctx->tally_on.load(std::memory_order_relaxed)) return BNK_OK;
     if (mem == BNK_MEM_HOST) {
         uint64_t k = 0;
         for (uint32_t i = 0; i < n; i++) k += words[i] != 0u;
@@ -163,11 +195,14 @@ extern "C" int bnk_counters_get(bnk_ctx *ctx, bnk_counters *out)
     if (!out) return ctx ? fail(ctx, BNK_E_INVAL, "null argument") : BNK_E_INVAL;
     Guard g(ctx);
     if (g.rc) return g.rc;
-    uint64_t dev[TALLY_SLOTS];
+    static thread_local uint64_t dev[TALLY_SLOTS * TALLY_LANES];
     HIPCHK(ctx, hipMemcpyAsync(dev, ctx->d_tally, sizeof(dev), hipMemcpyDeviceToHost, ctx->stream));
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
     uint64_t v[TALLY_SLOTS];
-    for (int s = 0; s < TALLY_SLOTS; s++) v[s] = dev[s] + ctx->tally_host[s].load(std::memory_order_relaxed);
+    for (int s = 0; s < TALLY_SLOTS; s++) {
+        v[s] = ctx->tally_host[s].load(std::memory_order_relaxed);
+        for (uint32_t l = 0; l < TALLY_LANES; l++) v[s] += dev[s * TALLY_LANES + l];
+    }
     out->sealed = v[TALLY_SEALED];
     out->opened = v[TALLY_OPENED];
     out->rejected = v[TALLY_REJECTED];
@@ -190,9 +225,19 @@ extern "C" int bnk_counters_reset(bnk_ctx *ctx)
     BNK_API_TRY
     Guard g(ctx);
     if (g.rc) return g.rc;
-    HIPCHK(ctx, hipMemsetAsync(ctx->d_tally, 0, TALLY_SLOTS * 8, ctx->stream));
+    HIPCHK(ctx, hipMemsetAsync(ctx->d_tally, 0, TALLY_SLOTS * TALLY_LANES * 8, ctx->stream));
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
     for (int s = 0; s < TALLY_SLOTS; s++) ctx->tally_host[s].store(0, std::memory_order_relaxed);
+    return BNK_OK;
+    BNK_API_CATCH(ctx)
+}
+
+extern "C" int bnk_counters_enable(bnk_ctx *ctx, int on)
+{
+    BNK_API_TRY
+    Guard g(ctx);
+    if (g.rc) return g.rc;
+    ctx->tally_on.store(on != 0, std::memory_order_relaxed);
     return BNK_OK;
     BNK_API_CATCH(ctx)
 }

@@ -252,6 +252,9 @@ class Context:
     def counters_reset(self) -> None:
         self._chk(self._lib.bnk_counters_reset(self._h))
 
+    def counters_enable(self, on: bool) -> None:
+        self._chk(self._lib.bnk_counters_enable(self._h, C.c_int(1 if on else 0)))
+
     def set_spread_max_packets(self, max_packets: int) -> None:
         """Batches of at most this many packets run one wave per packet
         (0: always one lane per packet).  A tuning knob, results are the same."""

@@ -205,9 +205,11 @@ int bnk_coalesce_stats_get(bnk_ctx *ctx, bnk_coalesce_stats *out);
  * of this context.  An addition: the reference keeps no such counts (its
  * filter drops without counting, internal/filter/filter.go:100-145, and
  * wireguard-go counts bytes per peer only).  They are a histogram of the
- * result bytes every call already leaves per packet, taken on the host for a
- * host batch and by one small launch behind a device-resident batch; a call
- * that returns an error counts nothing.
+ * result bytes every call already leaves per packet.  A host batch is counted
+ * on the host once the call has succeeded (a call that returns an error counts
+ * nothing).  A device-resident batch is counted on the device as it runs: by
+ * the opening launch and by the CheckInbound launch themselves, elsewhere by
+ * one small launch behind the call's own.
  *   sealed         bnk_aead_seal_batch(_noalloc), packets bnk_wg_(note_)encap_batch
  *                  gave a wire length other than 0
  *   opened         bnk_aead_open_batch, verdict 1
@@ -227,6 +229,11 @@ typedef struct bnk_counters {
 } bnk_counters;
 int bnk_counters_get(bnk_ctx *ctx, bnk_counters *out);
 int bnk_counters_reset(bnk_ctx *ctx);
+/* Counting is on from bnk_init.  Where a device-resident batch needs a launch
+ * of its own for it (the framing calls and the relay) that costs about 8 us
+ * per 2^20 packets; on = 0 leaves the counting out, and calls made meanwhile
+ * are not counted. */
+int bnk_counters_enable(bnk_ctx *ctx, int on);
 
 /* ---- transport AEAD ---------------------------------------------------- */
 

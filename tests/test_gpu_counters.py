@@ -65,6 +65,19 @@ def test_seal_open_counts_host_and_device_and_reset():
         assert ctx.counters()["sealed"] == n
         ctx.counters_reset()
         assert ctx.counters() == ZERO
+        # switched off, calls are not counted (and a device-resident one launches nothing more)
+        ctx.counters_enable(False)
+        ctx.open(lib.make_batch(d_sealed, sealed.nbytes, n, lib.MEM_DEVICE, stride=stride, length=length + 16,
+                                peer=d_peer, counters=d_ctr),
+                 lib.make_batch(d_back, back.nbytes, n, lib.MEM_DEVICE, stride=stride), d_verdict)
+        assert ctx.counters() == ZERO
+        ctx.counters_enable(True)
+        # a result array that does not start on a 16-byte boundary, and not a multiple of 16 long
+        ctx.open(lib.make_batch(d_sealed, sealed.nbytes, n - 8, lib.MEM_DEVICE, stride=stride, length=length + 16,
+                                peer=d_peer, counters=d_ctr),
+                 lib.make_batch(d_back, back.nbytes, n - 8, lib.MEM_DEVICE, stride=stride), d_verdict[5:])
+        late = int((forged >= n - 8).sum())
+        assert ctx.counters() == {**ZERO, "opened": n - 8 - (7 - late), "rejected": 7 - late}
 
 
 def test_merged_calls_count_once_each():

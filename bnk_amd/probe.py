@@ -75,3 +75,15 @@ def aead_compute(paired: bool, waves_per_simd: int, data_blocks: int = 48, devic
     if rc != 0:
         raise RuntimeError(f"bnkp_aead_compute failed: {rc}")
     return float(r.value)
+
+
+def line_copy(packets: int = 1 << 20, stride: int = 1440, length: int = 1420, waves_per_simd: int = 2,
+              depth: int = 1, spin: int = 0, iters: int = 20, device: int = 0) -> float:
+    """Milliseconds per launch of the AEAD kernel's packet movement alone (see bnkprobe.h)."""
+    r = C.c_double(0)
+    rc = load().bnkp_line_copy(C.c_int(device), C.c_uint32(packets), C.c_uint32(stride), C.c_uint32(length),
+                               C.c_int(waves_per_simd), C.c_int(depth), C.c_uint32(spin), C.c_uint32(iters),
+                               C.byref(r))
+    if rc:
+        raise RuntimeError(f"bnkp_line_copy failed: {rc}")
+    return r.value

@@ -24,6 +24,17 @@ int bnkp_valu(int device, int op, uint32_t iters, double *ops_per_sec);
  * times (copy_kernel) and reports bytes read plus bytes written per second. */
 int bnkp_copy(int device, size_t bytes, uint32_t iters, double *bytes_per_sec);
 
+/* The AEAD kernel's way of moving packets with nothing (or a stand-in) to
+ * compute: `packets` slots `stride` bytes apart (a multiple of 16), `len` bytes
+ * each, copied from one device arena to the same place of another, a lane per
+ * packet, eight adjacent lanes per aligned 128-byte line, a wave walking its 64
+ * packets line by line with each line held in registers for `depth` (1 or 2)
+ * steps; `spin` dependent VALU instructions per line stand for the arithmetic;
+ * `waves_per_simd` (1..4) waves resident per SIMD.  Reports milliseconds per
+ * launch. */
+int bnkp_line_copy(int device, uint32_t packets, uint32_t stride, uint32_t len, int waves_per_simd,
+                   int depth, uint32_t spin, uint32_t iters, double *ms_per_launch);
+
 /* Two instruction streams sharing each SIMD: one workgroup of eight waves per
  * CU, waves 0-3 run kind_a and waves 4-7 (one on each SIMD beside the first
  * four) kind_b, or nothing with kind_b = -1.  Kinds: 0 v_add_u32, 1 v_xor_b32,

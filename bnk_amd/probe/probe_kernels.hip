@@ -95,6 +95,69 @@ static hipError_t launch_copy(const void *src, void *dst, size_t bytes, uint32_t
     return hipGetLastError();
 }
 
+// The AEAD kernel's way of moving packets, with nothing to compute: a lane per
+// packet for the bookkeeping, eight adjacent lanes per aligned 128-byte line, so
+// that one load instruction of a wave fetches one line from each of eight
+// packets (`stride` bytes apart) and a wave walks its 64 packets line by line,
+// each line held in registers for `depth` steps before it is stored to the same
+// place of the other arena.  `spin` dependent VALU instructions per step stand
+// for the arithmetic (0: none).  Dynamic LDS sets how many waves a SIMD holds.
+template <int DEPTH>
+__global__ __launch_bounds__(256) void line_copy_kernel(const uint8_t *src, uint8_t *dst, uint32_t packets,
+                                                        uint32_t stride, uint32_t len, uint32_t spin, uint32_t *sink)
+{
+    extern __shared__ uint32_t occupancy_pad[];
+    const uint32_t lane = threadIdx.x & 63u, sub = lane & 7u, g = lane >> 3;
+    const uint32_t wave_first = (blockIdx.x * 256u + (threadIdx.x & ~63u));
+    if (wave_first >= packets) return;
+    // the (packet, cell-of-line) positions this lane moves per line: packet 8 q + g of the wave
+    uint64_t at[8];
+    uint32_t lines = 0;
+#pragma unroll
+    for (int q = 0; q < 8; q++) {
+        const uint32_t p = min(wave_first + 8u * q + g, packets - 1u);
+        const uint64_t start = (uint64_t)p * stride;
+        at[q] = (start & ~127ull) + 16u * sub;
+        const uint32_t n = (uint32_t)((start & 127u) + len + 127u) >> 7;
+        lines = n > lines ? n : lines;
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        const uint32_t o = (uint32_t)__shfl_xor((int)lines, off, 64);
+        lines = o > lines ? o : lines;
+    }
+    lines = __builtin_amdgcn_readfirstlane(lines);
+    uint4 buf[DEPTH][8];
+    uint32_t acc = lane;
+    for (int d = 0; d < DEPTH; d++) {
+#pragma unroll
+        for (int q = 0; q < 8; q++) buf[d][q] = make_uint4(0, 0, 0, 0);
+    }
+    // step m: line m comes in, line m - DEPTH goes out
+    for (uint32_t m = 0; m < lines + DEPTH; m++) {
+        uint4 out[8];
+#pragma unroll
+        for (int q = 0; q < 8; q++) out[q] = buf[DEPTH - 1][q];
+#pragma unroll
+        for (int d = DEPTH - 1; d > 0; d--) {
+#pragma unroll
+            for (int q = 0; q < 8; q++) buf[d][q] = buf[d - 1][q];
+        }
+        if (m < lines) {
+#pragma unroll
+            for (int q = 0; q < 8; q++)
+                buf[0][q] = *reinterpret_cast<const uint4 *>(src + at[q] + 128ull * m);
+        }
+        if (m >= (uint32_t)DEPTH) {
+#pragma unroll
+            for (int q = 0; q < 8; q++)
+                *reinterpret_cast<uint4 *>(dst + at[q] + 128ull * (m - DEPTH)) = out[q];
+        }
+        for (uint32_t k = 0; k < spin; k++) asm volatile("v_add_u32 %0, %0, %0" : "+v"(acc));
+    }
+    if (acc == 0x12345u) sink[0] = acc; // keeps the spin alive
+}
+
 // ---------------------------------------------------------------------------
 // How a SIMD shares its issue between two waves.
 //
@@ -337,6 +400,59 @@ extern "C" int bnkp_copy(int device, size_t bytes, uint32_t iters, double *bytes
 fail:
     if (src) (void)hipFree(src);
     if (dst) (void)hipFree(dst);
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    if (s) (void)hipStreamDestroy(s);
+    return rc;
+}
+
+extern "C" int bnkp_line_copy(int device, uint32_t packets, uint32_t stride, uint32_t len, int waves_per_simd,
+                              int depth, uint32_t spin, uint32_t iters, double *ms_per_launch)
+{
+    if (!ms_per_launch || iters == 0 || packets == 0 || (stride & 15u) || len == 0 || len > stride ||
+        waves_per_simd < 1 || waves_per_simd > 4 || depth < 1 || depth > 2)
+        return -1;
+    hipStream_t s = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    uint8_t *src = nullptr, *dst = nullptr;
+    uint32_t *sink = nullptr;
+    float ms = 0;
+    int rc = -3;
+    const size_t bytes = (size_t)packets * stride + 256;
+    // a workgroup is four waves, one per SIMD: 160 KB of LDS / waves_per_simd workgroups
+    const size_t lds = (size_t)(160u * 1024u) / (size_t)waves_per_simd - 1024u;
+    const dim3 grid((packets + 255u) / 256u);
+    auto launch = [&]() -> hipError_t {
+        if (depth == 1)
+            hipLaunchKernelGGL(line_copy_kernel<1>, grid, dim3(256), lds, s, src, dst, packets, stride, len, spin, sink);
+        else
+            hipLaunchKernelGGL(line_copy_kernel<2>, grid, dim3(256), lds, s, src, dst, packets, stride, len, spin, sink);
+        return hipGetLastError();
+    };
+    PROBE_CHK(hipSetDevice(device));
+    PROBE_CHK(hipFuncSetAttribute(reinterpret_cast<const void *>(line_copy_kernel<1>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    PROBE_CHK(hipFuncSetAttribute(reinterpret_cast<const void *>(line_copy_kernel<2>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    PROBE_CHK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    PROBE_CHK(hipEventCreate(&e0));
+    PROBE_CHK(hipEventCreate(&e1));
+    PROBE_CHK(hipMalloc((void **)&src, bytes));
+    PROBE_CHK(hipMalloc((void **)&dst, bytes));
+    PROBE_CHK(hipMalloc((void **)&sink, 64));
+    PROBE_CHK(hipMemsetAsync(src, 0x5a, bytes, s));
+    for (int w = 0; w < 3; w++) PROBE_CHK(launch()); // warm-up
+    PROBE_CHK(hipEventRecord(e0, s));
+    for (uint32_t i = 0; i < iters; i++) PROBE_CHK(launch());
+    PROBE_CHK(hipEventRecord(e1, s));
+    PROBE_CHK(hipEventSynchronize(e1));
+    PROBE_CHK(hipEventElapsedTime(&ms, e0, e1));
+    *ms_per_launch = (double)ms / iters;
+    rc = 0;
+fail:
+    if (src) (void)hipFree(src);
+    if (dst) (void)hipFree(dst);
+    if (sink) (void)hipFree(sink);
     if (e0) (void)hipEventDestroy(e0);
     if (e1) (void)hipEventDestroy(e1);
     if (s) (void)hipStreamDestroy(s);

@@ -20,7 +20,7 @@ def test_probe_library_exports_every_declared_symbol():
     from bnk_amd import probe
     so = probe.load()
     names = _declared()
-    assert {"bnkp_valu", "bnkp_copy", "bnkp_pair", "bnkp_mix", "bnkp_aead_compute"} <= set(names)
+    assert {"bnkp_valu", "bnkp_copy", "bnkp_pair", "bnkp_mix", "bnkp_aead_compute", "bnkp_line_copy"} <= set(names)
     for name in names:
         assert hasattr(so, name), f"{name} is declared in bnkprobe.h but not exported"
 
@@ -36,6 +36,8 @@ def test_probe_rejects_bad_arguments_without_a_gpu_call():
     assert so.bnkp_copy(0, 100, 1, C.byref(r)) == -1
     assert so.bnkp_aead_compute(0, 1, 5, 48, C.byref(r)) == -1   # at most four waves per SIMD
     assert so.bnkp_aead_compute(0, 1, 2, 47, C.byref(r)) == -1   # blocks come in pairs
+    assert so.bnkp_line_copy(0, 1024, 1441, 1420, 2, 1, 0, 1, C.byref(r)) == -1  # stride not a multiple of 16
+    assert so.bnkp_line_copy(0, 1024, 1440, 1420, 2, 3, 0, 1, C.byref(r)) == -1  # a line is held one or two steps
 
 
 @pytest.mark.gpu

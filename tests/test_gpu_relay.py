@@ -210,6 +210,9 @@ def test_relay_full_size_device_resident_properties():
     expect = np.where(forged, 1, np.where(w.denied, 2, 0))
     assert np.array_equal(v, expect)
     assert abs((v == 2).mean() - 0.05) < 0.002 and (v == 1).sum() == k
+    # the verdicts are counted for bnk_counters_get by a launch behind the relay's own
+    got = ctx.counters()
+    assert (got["relayed"], got["rejected"], got["denied"]) == (int((v == 0).sum()), k, int((v == 2).sum()))
     # counters: base + rank among the same peer's survivors, batch order
     ok = v == 0
     surv = np.flatnonzero(ok)

@@ -47,9 +47,9 @@ VALU_SINGLE_ISSUE_TOPS = 39.3
 # Counter readings for one launch of aead_wave_kernel over 2^20 packets x 1420 B (mean of
 # seal and open), taken with rocprofv3 --pmc and kept in profiles/aead_wave_kernel_cfg2.md;
 # they change only when the kernel does.
-VALU_LANE_INSTR_PER_PACKET = 27700   # SQ_INSTS_VALU x 64 / 2^20
+VALU_LANE_INSTR_PER_PACKET = 27697   # SQ_INSTS_VALU x 64 / 2^20
 VALU_SINGLE_ISSUE_SHARE = 0.40       # of them: v_alignbit_b32, v_mad_u64_u32, v_add_co/v_addc_co (counted in the kernel's loops)
-TRAFFIC_BYTES_PER_LAUNCH = 3.1776e9   # FETCH_SIZE + WRITE_SIZE, scaled by copy_kernel
+TRAFFIC_BYTES_PER_LAUNCH = 3.1783e9   # FETCH_SIZE + WRITE_SIZE, scaled by copy_kernel
 # the same for filter_check_kernel over 2^22 headers (profiles/filter_check_kernel_cfg4.md)
 FILTER_TRAFFIC_BYTES_PER_LAUNCH = 192.0e6
 # The counter readings above describe the kernel sources as they were when the readings
@@ -58,7 +58,7 @@ FILTER_TRAFFIC_BYTES_PER_LAUNCH = 192.0e6
 # them, until the profile is taken again and the hash here replaced
 # (`python bench.py --source-hashes` prints the current ones).
 AEAD_COUNTER_SOURCES = ("bnk_amd/csrc/aead_kernels.hip", "bnk_amd/csrc/aead_lane.hpp", "bnk_amd/csrc/kernels.hpp")
-AEAD_COUNTERS_TAKEN_ON = "621e8c1d5e4d18f7"
+AEAD_COUNTERS_TAKEN_ON = "7e771221c05eec4d"
 FILTER_COUNTER_SOURCES = ("bnk_amd/csrc/filter_kernels.hip", "bnk_amd/csrc/filter_dev.hpp")
 FILTER_COUNTERS_TAKEN_ON = "f5d0b5f0eddaea31"
 

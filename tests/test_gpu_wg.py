@@ -1327,3 +1327,80 @@ def test_full_size_tunnel_round_trips_device_resident():
     assert np.array_equal(d_res.cpu().numpy(), want_res)
     assert bool((d_olen == 0).all())
     ctx.close()
+
+
+@pytest.mark.parametrize("plen", [20, 40, 60, 100, 113])
+def test_short_uniform_tunnel_batches_device_resident(plen):
+    """Device-resident batches of short packets of one common length: the
+    launches in which every wave takes the short path (three waves per SIMD)
+    also do the framing -- header, padding as implied zeros, wire lengths on the
+    way out; header checks, index lookup and the checks on the inner header on
+    the way in.  Every datagram against the oracle, then decapsulated in line
+    with the ciphertext, a forged one and a repeat among them."""
+    import torch
+    from bnk_amd import lib
+    from oracle import binding as O
+    dev = torch.device("cuda:0")
+    n, n_peers, stride = 20000 + 13, 37, 256
+    rng = np.random.default_rng(900 + plen)
+    keys = rng.integers(0, 256, (n_peers, 32), dtype=np.uint8)
+    idx_a = (np.arange(n_peers, dtype=np.uint32) * 7919 + 3).astype(np.uint32)
+    idx_b = (np.arange(n_peers, dtype=np.uint32) * 104729 + 11).astype(np.uint32)
+    addr = (0x64400000 + np.arange(n_peers, dtype=np.uint32)).astype(np.uint32)
+    full = np.full(n_peers, 0xFFFFFFFF, np.uint32)
+    side_a = np.stack([idx_a, idx_b, addr, full], 1)
+    side_b = np.stack([idx_b, idx_a, addr, full], 1)
+    peer = rng.integers(0, n_peers, n).astype(np.uint32)
+    h_arena = rng.integers(0, 256, (n, stride), dtype=np.uint8)
+    h_arena[:, 16] = 0x45
+    h_arena[:, 18], h_arena[:, 19] = plen >> 8, plen & 0xFF
+    h_arena[:, 28:32] = addr[peer].astype(">u4").view(np.uint8).reshape(n, 4)
+    plain = h_arena[:, 16:16 + plen].copy()
+    arena = torch.from_numpy(h_arena).to(dev)
+    d_peer = torch.from_numpy(peer.astype(np.int32)).to(dev)
+    d_wl = torch.zeros(n, dtype=torch.int32, device=dev)
+    torch.cuda.synchronize()
+    padded = (plen + 15) & ~15
+    with lib.Context(0) as tx, lib.Context(0) as rx:
+        tx.keys_set(lib.KEYS_SEND, keys)
+        tx.wg_peers_set(side_a)
+        tx.wg_encap(lib.make_batch(arena, arena.numel(), n, lib.MEM_DEVICE, stride=stride, length=plen, peer=d_peer),
+                    MTU, d_wl)
+        tx.sync()
+        assert bool((d_wl == 16 + padded + 16).all())
+        rank, seen = np.zeros(n, np.uint64), np.zeros(n_peers, np.uint64)
+        for i in range(n):
+            rank[i] = seen[peer[i]]
+            seen[peer[i]] += 1
+        wire = arena.cpu().numpy()
+        for i in range(n):
+            p = int(peer[i])
+            w = O.wg_encap(plain[i].tobytes(), MTU, keys[p].tobytes(), int(idx_b[p]), int(rank[i]))
+            assert wire[i, :len(w)].tobytes() == w, i
+            assert np.array_equal(wire[i, len(w):], h_arena[i, len(w):]), i  # nothing beyond the datagram written
+        # receive: packet 5 forged, packet 9 a copy of packet 8's datagram (a repeat)
+        wire[5, 16 + 3] ^= 0x80
+        wire[9] = wire[8]
+        d_wire = torch.from_numpy(wire).to(dev)
+        rx.keys_set(lib.KEYS_RECV, keys)
+        rx.wg_peers_set(side_b)
+        d_res = torch.full((n,), 99, dtype=torch.uint8, device=dev)
+        d_olen = torch.zeros(n, dtype=torch.int32, device=dev)
+        d_gp = torch.zeros(n, dtype=torch.int32, device=dev)
+        d_gc = torch.zeros(n, dtype=torch.int64, device=dev)
+        torch.cuda.synchronize()
+        flat = d_wire.view(-1)
+        rx.wg_decap(lib.make_batch(flat, flat.numel(), n, lib.MEM_DEVICE, stride=stride, length=16 + padded + 16),
+                    lib.make_batch(flat[16:], flat.numel() - 16, n, lib.MEM_DEVICE, stride=stride),
+                    d_res, d_olen, d_gp, d_gc)
+        rx.sync()
+        res = d_res.cpu().numpy()
+        want = np.zeros(n, np.uint8)
+        want[5], want[9] = lib.WG_AUTH_FAIL, lib.WG_REPLAY
+        assert np.array_equal(res, want)
+        olen = d_olen.cpu().numpy()
+        assert (olen[want == 0] == plen).all() and olen[5] == 0 and olen[9] == 0
+        got = d_wire.cpu().numpy()
+        ok = np.flatnonzero(want == 0)
+        assert np.array_equal(got[ok, 16:16 + plen], plain[ok])
+        assert not got[5, 16:16 + padded].any()  # a rejected packet's plaintext is cleared

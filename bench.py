@@ -760,6 +760,46 @@ def bench_callers(args) -> dict:
                     "windows": batches,
                     "windows_that_waited_in_vain": s1["timed_out"] - s0["timed_out"],
                 })
+    # Peers are independent of each other (keys, counters, windows, and a peer's flows are its
+    # own), so they can be sharded over contexts: the same 16 callers, eight on each of two
+    # contexts, whose streams run beside each other.
+    import threading
+    ctx2 = lib.Context(0)
+    ctx2.keys_set(lib.KEYS_SEND, keys)
+    ctx2.keys_set(lib.KEYS_RECV, keys)
+    ctx2.wg_peers_set([(0x1000 + 37 * t, 0x1000 + 37 * t, W.CGNAT_BASE + t, 0xFFFFFFFF) for t in range(t_max)])
+    ctx2.filter_set_rules([([(W.CGNAT_BASE, 10)], "tcp", [(8000, 8000)])])
+    for c in (ctx, ctx2):
+        c.set_coalesce(window_packets, wait_us)
+    for workload, name, legs in ((0, "seal + open", ("seal", "open")),
+                                 (1, "NoteOutbound + encapsulate, decapsulate + CheckInbound",
+                                  ("note_encap", "decap_filter"))):
+        res = [Result(), Result()]
+        rcs = [0, 0]
+
+        def half(k, c):
+            rcs[k] = so.bnkc_run(C.c_void_p(c._h.value), C.c_int(workload), C.c_uint32(t_max // 2),
+                                 C.c_uint32(per_call), C.c_uint32(L), C.c_uint32(rounds), C.c_uint32(warm),
+                                 C.c_int64(now), C.byref(res[k]))
+
+        th = [threading.Thread(target=half, args=(k, c)) for k, c in enumerate((ctx, ctx2))]
+        for t in th:
+            t.start()
+        for t in th:
+            t.join()
+        if any(rcs) or any(r.mismatches for r in res):
+            raise RuntimeError("callers workload on two contexts failed: %r" % (rcs,))
+        rate = sum(r.plaintext_bytes * 8e-9 / r.seconds for r in res)
+        rows.append({
+            "calls": name, "threads": t_max, "mode": "merged, two contexts of 8 callers each",
+            "gbit_per_s_round_trip": round(rate, 1), "gbit_per_s_per_direction": round(2 * rate, 1),
+            "us_per_call": {legs[0]: {"p50": round(max(r.out_p50_us for r in res), 1),
+                                      "p99": round(max(r.out_p99_us for r in res), 1)},
+                            legs[1]: {"p50": round(max(r.in_p50_us for r in res), 1),
+                                      "p99": round(max(r.in_p99_us for r in res), 1)}},
+        })
+    ctx2.set_coalesce(0)
+    ctx2.close()
     ctx.set_coalesce(0)
     ctx.close()
     best = max((x for x in rows if x["threads"] == 16 and x["mode"] == "merged" and x["calls"] == "seal + open"),

@@ -389,3 +389,44 @@ def test_window_pass_where_one_peer_fills_more_blocks_than_one_look_back_reads()
                      lib.make_batch(d_out, wire.nbytes, n_total, lib.MEM_DEVICE, stride=stride), res, olen, gp, gc)
         rxc.sync()
         assert (res.cpu().numpy() == lib.WG_REPLAY).all()
+
+
+@pytest.mark.parametrize("peers", [1, 2, 40])
+def test_window_pass_with_few_and_many_senders(peers, monkeypatch):
+    """The same walk as above, device resident, with one sender (every run spans
+    several blocks of the pass, so repeats are looked for across blocks and a
+    block's running maximum comes from the blocks before it), two, and forty
+    (short runs, several to a block), per packet against the sequential filter."""
+    import torch
+    import sys
+    from bnk_amd import lib
+    from oracle import binding as O
+    monkeypatch.setattr(sys.modules[__name__], "P", peers)
+    rng = np.random.default_rng(300 + peers)
+    tx, rx = _peers()
+    keys = rng.integers(0, 256, (peers, 32), dtype=np.uint8)
+    filters = [O.ReplayFilter() for _ in range(peers)]
+    last = [0] * peers
+    with lib.Context(0) as ctx:
+        ctx.keys_set(lib.KEYS_RECV, keys)
+        ctx.wg_peers_set(rx)
+        for b, n in enumerate([3000, 1100, 6000, 2500]):
+            arena, offs, lens, wires, last = _batch(rng, tx, keys, n, last, near_limit=(b == 1))
+            want = _expect(wires, rx, keys, filters)
+            total = arena.nbytes
+            d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to("cuda:0")  # noqa: E731
+            d_arena, d_out = d(arena), torch.zeros(total, dtype=torch.uint8, device="cuda:0")
+            res = torch.zeros(n, dtype=torch.uint8, device="cuda:0")
+            olen = torch.zeros(n, dtype=torch.int32, device="cuda:0")
+            gp = torch.zeros(n, dtype=torch.int32, device="cuda:0")
+            gc = torch.zeros(n, dtype=torch.int64, device="cuda:0")
+            d_off, d_len = d(offs.astype(np.int64)), d(lens.astype(np.int32))
+            torch.cuda.synchronize()
+            ctx.wg_decap(lib.make_batch(d_arena, total, n, lib.MEM_DEVICE, offsets=d_off, lens=d_len),
+                         lib.make_batch(d_out, total, n, lib.MEM_DEVICE, offsets=d_off), res, olen, gp, gc)
+            ctx.sync()
+            got = res.cpu().numpy()
+            bad = np.flatnonzero(got != want[0])
+            assert bad.size == 0, f"batch {b}: result differs at {bad[:5]}: got {got[bad[:5]]} want {want[0][bad[:5]]}"
+            assert np.array_equal(olen.cpu().numpy().astype(np.uint32), want[1])
+            assert (want[0] == lib.WG_REPLAY).sum() > 50

@@ -201,7 +201,8 @@ class Filter:
         self._f = C.c_void_p(_lib.bnko_filter_new())
 
     def __del__(self):
-        if getattr(self, "_f", None):
+        # (at interpreter exit the module's globals may be gone before the object is)
+        if getattr(self, "_f", None) and _lib is not None:
             _lib.bnko_filter_free(self._f)
             self._f = None
 

@@ -834,15 +834,17 @@ def bench_sizes(args) -> dict:
     per = {}
     for length in [int(x) for x in args.sizes.split(",")]:
         stride = (length + 16 + 15) // 16 * 16
-        plain = W.rand_bytes_torch(W.stream_seed(2, 50), n * stride, dev).clone()
-        sealed = torch.zeros_like(plain)
+        # --packed: the packets back to back on either side, no slot aligned
+        ps, ss = (length, length + 16) if args.packed else (stride, stride)
+        plain = W.rand_bytes_torch(W.stream_seed(2, 50), n * ps, dev).clone()
+        sealed = torch.zeros(n * ss, dtype=torch.uint8, device=dev)
         back = torch.zeros_like(plain)
         v = torch.zeros(n, dtype=torch.uint8, device=dev)
         torch.cuda.synchronize()
-        bi = lib.make_batch(plain, n * stride, n, lib.MEM_DEVICE, stride=stride, length=length)
-        bs = lib.make_batch(sealed, n * stride, n, lib.MEM_DEVICE, stride=stride)
-        bc = lib.make_batch(sealed, n * stride, n, lib.MEM_DEVICE, stride=stride, length=length + 16)
-        bb = lib.make_batch(back, n * stride, n, lib.MEM_DEVICE, stride=stride)
+        bi = lib.make_batch(plain, n * ps, n, lib.MEM_DEVICE, stride=ps, length=length)
+        bs = lib.make_batch(sealed, n * ss, n, lib.MEM_DEVICE, stride=ss)
+        bc = lib.make_batch(sealed, n * ss, n, lib.MEM_DEVICE, stride=ss, length=length + 16)
+        bb = lib.make_batch(back, n * ps, n, lib.MEM_DEVICE, stride=ps)
         for _ in range(args.warmup):
             ctx.seal(bi, bs)
             ctx.open(bc, bb, v)
@@ -858,7 +860,7 @@ def bench_sizes(args) -> dict:
         torch.cuda.synchronize()
         seal_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / args.steps
         open_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / args.steps
-        assert bool(v.all()) and torch.equal(back.view(n, stride)[:, :length], plain.view(n, stride)[:, :length])
+        assert bool(v.all()) and torch.equal(back.view(n, ps)[:, :length], plain.view(n, ps)[:, :length])
         ops = n * ops_aead(length)
         per[str(length)] = {
             "seal_us": round(seal_ms * 1e3, 1), "open_us": round(open_ms * 1e3, 1),
@@ -872,7 +874,9 @@ def bench_sizes(args) -> dict:
             "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": False,
             "dtype": "u32", "data": "synthetic",
             "config": {"workload": "seal and open of %d packets of one common length, device resident, "
-                                   "HIP events around each launch" % n, "lengths": args.sizes},
+                                   "HIP events around each launch" % n, "lengths": args.sizes,
+                       "layout": "back to back (plaintext stride = length, sealed stride = length + 16)"
+                       if args.packed else "slots of the next multiple of 16 above length + 16"},
             "per_length": per}
 
 
@@ -926,6 +930,8 @@ def main() -> int:
                     help="aead (default, the headline line, with the ACL filter rate as an extra); "
                          "filter / imix / relay / wg / host / latency / copy print one line for that workload alone")
     ap.add_argument("--sizes", default="60,576,1420", help="sizes: packet lengths, comma separated")
+    ap.add_argument("--packed", action="store_true",
+                    help="sizes: packets back to back on either side (no slot aligned) instead of 16-byte aligned slots")
     ap.add_argument("--slot-align", type=int, default=128, choices=[16, 32, 64, 128],
                     help="imix, relay: packets lie back to back, each starting at a multiple of this "
                          "(128: every packet in 128-byte lines of its own, as in a ring of buffers; "

@@ -760,6 +760,36 @@ def bench_callers(args) -> dict:
                     "windows": batches,
                     "windows_that_waited_in_vain": s1["timed_out"] - s0["timed_out"],
                 })
+    # The same 16 callers under an offered load (every caller's rounds due at fixed intervals,
+    # the callers' phases spread over an interval) instead of back to back: what a call costs
+    # when the library is not saturated.  Offered: a quarter, half and three quarters of what
+    # the merged calls carried above.  The outbound call's time counts from when it was due.
+    so.bnkc_run_paced.restype = C.c_int
+    for workload, name, legs in ((0, "seal + open", ("seal", "open")),
+                                 (1, "NoteOutbound + encapsulate, decapsulate + CheckInbound",
+                                  ("note_encap", "decap_filter"))):
+        full = max(x["gbit_per_s_per_direction"] for x in rows
+                   if x["calls"] == name and x["threads"] == t_max and x["mode"] == "merged") / 2.0
+        for share in (0.25, 0.5, 0.75):
+            for merged in (False, True):
+                ctx.set_coalesce(window_packets if merged else 0, wait_us)
+                s0 = ctx.coalesce_stats()
+                r = Result()
+                rc = so.bnkc_run_paced(C.c_void_p(ctx._h.value), C.c_int(workload), C.c_uint32(t_max),
+                                       C.c_uint32(per_call), C.c_uint32(L), C.c_uint32(rounds), C.c_uint32(warm),
+                                       C.c_int64(now), C.c_double(share * full), C.byref(r))
+                if rc != 0 or r.mismatches:
+                    raise RuntimeError("paced callers workload failed: rc %d, %d mismatches" % (rc, r.mismatches))
+                s1 = ctx.coalesce_stats()
+                calls, batches = s1["calls"] - s0["calls"], s1["batches"] - s0["batches"]
+                rows.append({
+                    "calls": name, "threads": t_max, "mode": ("merged" if merged else "direct") + ", offered load",
+                    "offered_gbit_per_s_each_way": round(share * full, 1),
+                    "carried_gbit_per_s_each_way": round(r.plaintext_bytes * 8e-9 / r.seconds, 1),
+                    "us_per_call": {legs[0]: {"p50": round(r.out_p50_us, 1), "p99": round(r.out_p99_us, 1)},
+                                    legs[1]: {"p50": round(r.in_p50_us, 1), "p99": round(r.in_p99_us, 1)}},
+                    "calls_per_launch": round(calls / batches, 2) if batches else 1.0,
+                })
     # Peers are independent of each other (keys, counters, windows, and a peer's flows are its
     # own), so they can be sharded over contexts: the same 16 callers, eight on each of two
     # contexts, whose streams run beside each other.

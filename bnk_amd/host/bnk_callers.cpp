@@ -74,10 +74,23 @@ void inner_packet(uint8_t *p, uint32_t len, uint32_t t, uint32_t i, uint32_t see
     p[23] = (uint8_t)dport;
 }
 
-} // namespace
+// Waits for a point in time: sleeping while it is far, yielding when it is near.
+void wait_until(Clock::time_point when)
+{
+    for (;;) {
+        const auto left = when - Clock::now();
+        if (left <= std::chrono::nanoseconds(0)) return;
+        if (left > std::chrono::microseconds(300)) std::this_thread::sleep_for(left - std::chrono::microseconds(200));
+        else std::this_thread::yield();
+    }
+}
 
-extern "C" int bnkc_run(bnk_ctx *ctx, int workload, uint32_t threads, uint32_t packets_per_call, uint32_t payload,
-                        uint32_t rounds, uint32_t warmup, int64_t now_ns, bnkc_result *out)
+// interval_us > 0: every thread starts its timed round r at a fixed time, r intervals
+// after its first (the threads' first rounds spread evenly over one interval), whether
+// or not the round before has returned: offered load instead of back-to-back calls.  A
+// call's time then counts from when its round was due.
+int run(bnk_ctx *ctx, int workload, uint32_t threads, uint32_t packets_per_call, uint32_t payload, uint32_t rounds,
+        uint32_t warmup, int64_t now_ns, double interval_us, bnkc_result *out)
 {
     if (!ctx || !out || threads == 0 || packets_per_call == 0 || rounds == 0) return BNK_E_INVAL;
     if (workload != BNKC_AEAD && workload != BNKC_TUNNEL) return BNK_E_INVAL;
@@ -135,6 +148,12 @@ extern "C" int bnkc_run(bnk_ctx *ctx, int workload, uint32_t threads, uint32_t p
             int rc;
             bool second = false;
             Clock::time_point c0, c1, c2;
+            Clock::time_point due{};
+            if (interval_us > 0 && r >= warmup) {
+                due = t_begin[t] + std::chrono::duration_cast<Clock::duration>(std::chrono::duration<double, std::micro>(
+                                       interval_us * ((double)(r - warmup) + (double)t / (double)threads)));
+                wait_until(due);
+            }
             if (workload == BNKC_AEAD) {
                 a.base = X + 16;
                 a.bytes = b.bytes = per_thread - 16;
@@ -194,6 +213,7 @@ extern "C" int bnkc_run(bnk_ctx *ctx, int workload, uint32_t threads, uint32_t p
                 break;
             }
             if (r >= warmup) {
+                if (interval_us > 0) c0 = due;
                 lat_out[t].push_back(std::chrono::duration<float, std::micro>(c1 - c0).count());
                 lat_in[t].push_back(std::chrono::duration<float, std::micro>(c2 - c1).count());
             }
@@ -240,4 +260,22 @@ extern "C" int bnkc_run(bnk_ctx *ctx, int workload, uint32_t threads, uint32_t p
     out->filtered = filtered.load();
     bnk_ring_free(ctx, ring[0]);
     return out->rc;
+}
+
+} // namespace
+
+extern "C" int bnkc_run(bnk_ctx *ctx, int workload, uint32_t threads, uint32_t packets_per_call, uint32_t payload,
+                        uint32_t rounds, uint32_t warmup, int64_t now_ns, bnkc_result *out)
+{
+    return run(ctx, workload, threads, packets_per_call, payload, rounds, warmup, now_ns, 0.0, out);
+}
+
+extern "C" int bnkc_run_paced(bnk_ctx *ctx, int workload, uint32_t threads, uint32_t packets_per_call,
+                              uint32_t payload, uint32_t rounds, uint32_t warmup, int64_t now_ns,
+                              double gbit_per_s_per_direction, bnkc_result *out)
+{
+    if (!(gbit_per_s_per_direction > 0)) return BNK_E_INVAL;
+    // one round of every thread carries threads x packets x payload bytes each way
+    const double interval_us = (double)threads * packets_per_call * payload * 8.0 / (gbit_per_s_per_direction * 1e3);
+    return run(ctx, workload, threads, packets_per_call, payload, rounds, warmup, now_ns, interval_us, out);
 }

@@ -37,6 +37,17 @@ typedef struct bnkc_result {
 int bnkc_run(bnk_ctx *ctx, int workload, uint32_t threads, uint32_t packets_per_call, uint32_t payload,
              uint32_t rounds, uint32_t warmup, int64_t now_ns, bnkc_result *out);
 
+/* The same under an offered load instead of back-to-back calls: the threads
+ * together offer gbit_per_s_per_direction of plaintext each way, every thread
+ * starting its timed rounds at fixed intervals (first rounds spread evenly over
+ * one interval) whether or not the round before has returned.  The outbound
+ * call's time counts from when its round was due, so a thread that has fallen
+ * behind shows it; `seconds` against the offered rate tells whether the load
+ * was carried. */
+int bnkc_run_paced(bnk_ctx *ctx, int workload, uint32_t threads, uint32_t packets_per_call, uint32_t payload,
+                   uint32_t rounds, uint32_t warmup, int64_t now_ns, double gbit_per_s_per_direction,
+                   bnkc_result *out);
+
 #ifdef __cplusplus
 }
 #endif

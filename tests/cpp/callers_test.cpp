@@ -114,6 +114,17 @@ int main()
     CHECK(bnk_coalesce_stats_get(ctx, &s1) == 0);
     CHECK(r.mismatches == 0 && s1.batches - s0.batches == s1.calls - s0.calls && s1.timed_out == s0.timed_out);
     printf("one caller, merging on: out p50 %.1f us, in p50 %.1f us\n", r.out_p50_us, r.in_p50_us);
+    // the same callers under an offered load well below what they carry back to back: every
+    // round's results right, and the load carried (the rounds take the time they were spread over)
+    for (int workload : {BNKC_AEAD, BNKC_TUNNEL}) {
+        bnkc_result p{};
+        const double offered = workload == BNKC_AEAD ? 8.0 : 5.0;
+        CHECK(bnkc_run_paced(ctx, workload, 8, 128, 1420, 60, 3, now, offered, &p) == 0);
+        const double carried = (double)p.plaintext_bytes * 8e-9 / p.seconds;
+        printf("8 callers offering %.1f Gbit/s each way, merging on: carried %.1f, out p50 %.1f p99 %.1f us\n", offered,
+               carried, p.out_p50_us, p.out_p99_us);
+        CHECK(p.mismatches == 0 && carried > 0.8 * offered && carried < 1.1 * offered);
+    }
     bnk_shutdown(ctx);
     printf("callers_test ok\n");
     return 0;

@@ -156,7 +156,7 @@ BNK_DEV void wave_sync()
 // batches): 64 bytes per packet per step, four adjacent lanes per packet, any
 // byte alignment.
 constexpr uint32_t LDS_ROW = 80;    // generic: 64 data bytes + 16 pad
-constexpr uint32_t RING_ROW = 272;  // line path: 2 x 128-byte lines + 16 pad
+constexpr uint32_t RING_ROW = 272;  // line path: 2 x 128-byte lines + 16 pad (where the shifted output keeps a copy of the first cell)
 constexpr uint32_t WAVES_PER_BLOCK = 4;
 // The lane-per-packet launches run workgroups of one wave: their waves share nothing, and a
 // wave that has finished gives its place to the next at once instead of waiting for the
@@ -336,9 +336,10 @@ BNK_DEV void body_generic(uint8_t *tile, uint32_t lane, const uint8_t *src, uint
 // SHIFT (not ALIGNED, every destination of the wave 4-byte aligned): the input
 // comes in as such pieces, but the output leaves as whole aligned 16-byte cells
 // of the destination's own 128-byte lines.  A lane that moves such a cell reads
-// the two ring cells it straddles and picks its four words from their eight;
-// the first and the last cell of a packet, which it shares with its neighbours,
-// leave word by word.  (Misaligned 16-byte stores run at half rate and leave
+// its four words from where they lie in the ring, a multiple of 4 bytes into a
+// ring cell (the 16 bytes behind a row's ring repeat its first cell, so that
+// such a read never wraps); the first and the last cell of a packet, which it
+// shares with its neighbours, leave word by word.  (Misaligned 16-byte stores run at half rate and leave
 // every line in two parts.)  A destination line lags the packet's pieces by up to
 // 124 bytes, so a piece enters the ring one step later than otherwise: just
 // before it is needed, after the line that still holds the end of the piece
@@ -367,7 +368,6 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
     uint32_t cfirst[8], cend[8], cend_ld[8];
     int32_t pofs[8];
     uint32_t whole[8];
-    bool odd1[8], odd2[8];
 #pragma unroll
     for (int q = 0; q < 8; q++) {
         const int owner = 8 * q + (int)(lane >> 3);
@@ -385,8 +385,6 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
             cdst[q] = reinterpret_cast<uint8_t *>(od - skd) + 16u * sub; // my cell of the line holding the packet's first byte
             pofs[q] = (int32_t)(16u * sub) - (int32_t)skd;               // where that cell starts within the packet
             whole[q] = olen & ~15u;                                      // bytes of it that go through the ring
-            odd1[q] = (pofs[q] & 4) != 0;
-            odd2[q] = (pofs[q] & 8) != 0;
         }
     }
     uint32_t maxsteps = steps;
@@ -441,19 +439,13 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
 #define BNK_PUT(q, m) if (BNK_INSIDE(q, m)) BNK_ST(cdst[q] + 128u * (m), out##q)
 #define BNK_PUT_ALL(q, m) BNK_ST(cdst[q] + 128u * (m), out##q)
     // SHIFT: my cell of destination line m starts pofs[q] + 128 m bytes into the packet
-    // (before it when negative), a multiple of 4: ring cells at and after that place,
-    // and of their eight words the four from word (offset / 4) % 4 on
+    // (before it when negative), a multiple of 4: its four words from that place of the ring
+    // on, running into the copy of the ring's first cell behind its end where they would wrap
 #define BNK_TAKE_SHIFT(q, m)                                                                \
     do {                                                                                    \
-        const int32_t at_##q = pofs[q] + (int32_t)(128u * (m));                             \
-        const uint32_t cl_##q = (uint32_t)(at_##q >> 4);                                    \
-        const uint4 lo_##q = *reinterpret_cast<const uint4 *>(mycell + 8u * q * RING_ROW + ((cl_##q & 15u) << 4));        \
-        const uint4 hi_##q = *reinterpret_cast<const uint4 *>(mycell + 8u * q * RING_ROW + (((cl_##q + 1u) & 15u) << 4)); \
-        const uint32_t u0_##q = odd1[q] ? lo_##q.y : lo_##q.x, u1_##q = odd1[q] ? lo_##q.z : lo_##q.y;                    \
-        const uint32_t u2_##q = odd1[q] ? lo_##q.w : lo_##q.z, u3_##q = odd1[q] ? hi_##q.x : lo_##q.w;                    \
-        const uint32_t u4_##q = odd1[q] ? hi_##q.y : hi_##q.x, u5_##q = odd1[q] ? hi_##q.z : hi_##q.y;                    \
-        out##q = make_uint4(odd2[q] ? u2_##q : u0_##q, odd2[q] ? u3_##q : u1_##q, odd2[q] ? u4_##q : u2_##q,             \
-                            odd2[q] ? u5_##q : u3_##q);                                     \
+        const uint32_t at_##q = (uint32_t)(pofs[q] + (int32_t)(128u * (m))) & 255u;         \
+        const uint32_t *const w_##q = reinterpret_cast<const uint32_t *>(mycell + 8u * q * RING_ROW + at_##q); \
+        out##q = make_uint4(w_##q[0], w_##q[1], w_##q[2], w_##q[3]);                        \
     } while (0)
 #define BNK_PUT_SHIFT(q, m)                                                                 \
     do {                                                                                    \
@@ -562,6 +554,11 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
                 }
             }
             if (OPEN && s == 0) capture_head(head, row + (c0 << 4), row + (((c0 + 1u) & 15u) << 4));
+            // SHIFT: a step that has written the ring's first cell (every second one: the ring
+            // holds a packet from its first byte) repeats it behind the ring's end
+            static_assert(!SHIFT || RING_ROW >= 256u + 16u, "no room behind the ring for the copy of its first cell");
+            if (SHIFT && (s & 1u) == 0u)
+                *reinterpret_cast<uint4 *>(row + 256) = *reinterpret_cast<const uint4 *>(row);
         }
         wave_sync();
     }

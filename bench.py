@@ -1295,12 +1295,17 @@ def main() -> int:
     # workload (their full lines: --workload imix | relay | wg)
     others = {}
     oargs = argparse.Namespace(**vars(args))
-    oargs.steps, oargs.warmup, oargs.no_cpu_baseline, oargs.no_extras = 20, 20, True, True
-    for name, fn in (("cfg3_imix", bench_imix), ("cfg5_relay", bench_relay), ("transport_framing", bench_wg)):
+    oargs.no_cpu_baseline, oargs.no_extras = True, True
+    # (warm-up by time rather than by count: some 60 ms of work, which is what a chip that has
+    # idled through the host-side legs above needs to reach the clocks it then holds)
+    for name, fn, steps, warm in (("cfg3_imix", bench_imix, 40, 110), ("cfg5_relay", bench_relay, 20, 30),
+                                  ("transport_framing", bench_wg, 20, 35)):
         try:
+            oargs.steps, oargs.warmup = steps, warm
             r = fn(oargs)
             others[name] = {"metric": r["metric"], "value": r["value"], "unit": r["unit"],
-                            "ms_per_step": r["ms_per_step"], "workload": r["config"]["workload"]}
+                            "ms_per_step": r["ms_per_step"], "steps": steps, "warmup": warm,
+                            "workload": r["config"]["workload"]}
         except Exception as e:  # a side measurement must not take the headline line with it
             others[name] = {"error": "%s: %s" % (type(e).__name__, e)}
     out["extra"]["other_configurations"] = others

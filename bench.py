@@ -952,9 +952,10 @@ def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=30,
+    ap.add_argument("--warmup", type=int, default=None,
                     help="untimed steps first: a chip that was idle needs some 50 ms of work to reach the "
-                         "clocks it then holds (the first 20 steps run about 5 %% slower)")
+                         "clocks it then holds (the first 20 steps run about 5 %% slower); default 30, "
+                         "110 for imix and 35 for wg, whose steps are shorter")
     ap.add_argument("--packets", type=int, default=1 << 20)
     ap.add_argument("--workload", default="aead", choices=["aead", "filter", "imix", "relay", "wg", "host", "latency", "callers", "copy", "sizes", "issue"],
                     help="aead (default, the headline line, with the ACL filter rate as an extra); "
@@ -975,6 +976,8 @@ def main() -> int:
     ap.add_argument("--source-hashes", action="store_true",
                     help="print the hashes of the kernel sources the pasted counter readings belong to, and exit")
     args = ap.parse_args()
+    if args.warmup is None:
+        args.warmup = {"imix": 110, "wg": 35}.get(args.workload, 30)
     if args.source_hashes:
         print(json.dumps({"AEAD_COUNTERS_TAKEN_ON": source_hash(AEAD_COUNTER_SOURCES),
                           "FILTER_COUNTERS_TAKEN_ON": source_hash(FILTER_COUNTER_SOURCES)}))

@@ -497,6 +497,15 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
         }
         wave_sync();
         BNK_COMMIT_LINE(s + AHEAD);
+        // Sealing: nothing of the wave's is in flight here but the stores of the line that left
+        // a step ago.  Waiting for them by hand tells the compiler that the registers the next
+        // loads fill are free: otherwise it protects them with a wait of its own, for
+        // everything, which lands behind the first seven of those loads (the eighth is shared
+        // by the two forms of the line and issued after them) and makes the wave sit out their
+        // whole way to memory and back in every step: 5 % of a sealing launch.  (The opening
+        // code comes out without that wait, and with this one it is 1 % slower.
+        // tests/test_kernel_isa.py looks for the pattern in both.)
+        if (!OPEN) __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
         if (s + AHEAD + 1u <= maxsteps) BNK_ISSUE_LINE(s + AHEAD + 1u);
         if (s >= 1) {
             if (SHIFT) {

@@ -522,22 +522,20 @@ BNK_DEV void body_lines(uint8_t *tile, uint32_t lane, const uint8_t *src, uint8_
                 // keystream blocks side by side
                 uint32_t y[16];
                 const uint32_t r0 = c0 + 8u * s;
-                if (OPEN) {
-                    // (open has no registers for reading cells ahead of the keystream)
-                    chacha_block2_shared(k, shared, 2u * s + 1u, n1, n2, x, y);
+                // The step's first cell leaves LDS while the keystream is computed, every other
+                // one while the cell before it goes through the cipher and the MAC (a read
+                // where the cell is used costs open 1 %; reading four ahead of the keystream,
+                // which seal had registers for, is no faster than this).
+                uint4 cur = *reinterpret_cast<const uint4 *>(row + ((r0 & 15u) << 4));
+                chacha_block2_shared(k, shared, 2u * s + 1u, n1, n2, x, y);
 #pragma unroll
-                    for (int j = 0; j < 4; j++) crypt_cell<OPEN>(mac, x, j, row + (((r0 + j) & 15u) << 4));
-                } else {
-                    // the first block's cells leave LDS while the keystream is computed
-                    uint4 v[4];
-#pragma unroll
-                    for (int j = 0; j < 4; j++) v[j] = *reinterpret_cast<const uint4 *>(row + (((r0 + j) & 15u) << 4));
-                    chacha_block2_shared(k, shared, 2u * s + 1u, n1, n2, x, y);
-#pragma unroll
-                    for (int j = 0; j < 4; j++) crypt_cell_v<OPEN>(mac, x, j, v[j], row + (((r0 + j) & 15u) << 4));
+                for (int j = 0; j < 8; j++) {
+                    uint4 nxt = cur;
+                    if (j < 7) nxt = *reinterpret_cast<const uint4 *>(row + (((r0 + j + 1u) & 15u) << 4));
+                    if (j < 4) crypt_cell_v<OPEN>(mac, x, j, cur, row + (((r0 + j) & 15u) << 4));
+                    else crypt_cell_v<OPEN>(mac, y, j - 4, cur, row + (((r0 + j) & 15u) << 4));
+                    cur = nxt;
                 }
-#pragma unroll
-                for (int j = 0; j < 4; j++) crypt_cell<OPEN>(mac, y, j, row + (((r0 + 4u + j) & 15u) << 4));
             } else {
 #pragma unroll 1
                 for (uint32_t h = 0; h < 2; h++) {

@@ -58,7 +58,7 @@ FILTER_TRAFFIC_BYTES_PER_LAUNCH = 192.0e6
 # them, until the profile is taken again and the hash here replaced
 # (`python bench.py --source-hashes` prints the current ones).
 AEAD_COUNTER_SOURCES = ("bnk_amd/csrc/aead_kernels.hip", "bnk_amd/csrc/aead_lane.hpp", "bnk_amd/csrc/kernels.hpp")
-AEAD_COUNTERS_TAKEN_ON = "114cd99af993fe0e"
+AEAD_COUNTERS_TAKEN_ON = "1f5676f98fa92181"
 FILTER_COUNTER_SOURCES = ("bnk_amd/csrc/filter_kernels.hip", "bnk_amd/csrc/filter_dev.hpp")
 FILTER_COUNTERS_TAKEN_ON = "f5d0b5f0eddaea31"
 

@@ -89,6 +89,31 @@ BNK_DEV uint4 ld_partial(const uint8_t *p, uint32_t m)
     return make_uint4(w[0], w[1], w[2], w[3]);
 }
 
+// The same with every load issued whatever m is (from `safe`, 4 readable bytes at an even
+// address, where the packet has nothing there), for a caller whose other loads should not
+// queue behind a branch: m may be 0, the result is then zero.
+BNK_DEV uint4 ld_partial_flat(const uint8_t *p, uint32_t m, const uint8_t *safe)
+{
+    const uint32_t nd = m >> 2;
+    uint32_t w[4];
+#pragma unroll
+    for (int q = 0; q < 3; q++)
+        w[q] = *reinterpret_cast<const BNK_GLOBAL u32_unaligned *>((uintptr_t)((uint32_t)q < nd ? p + 4 * q : safe));
+    const uint32_t half = *reinterpret_cast<const BNK_GLOBAL u16_unaligned *>((uintptr_t)((m & 2u) ? p + 4u * nd : safe));
+    const uint32_t byte = ld8((m & 1u) ? p + 4u * nd + (m & 2u) : safe);
+#pragma unroll
+    for (int q = 0; q < 3; q++)
+        if ((uint32_t)q >= nd) w[q] = 0;
+    w[3] = 0;
+    uint32_t last = (m & 2u) ? half : 0u;
+    if (m & 1u) last |= byte << (8u * (m & 2u));
+    if (nd == 0) w[0] = last;
+    else if (nd == 1) w[1] = last;
+    else if (nd == 2) w[2] = last;
+    else w[3] = last;
+    return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
 BNK_DEV void st_partial(uint8_t *p, uint4 v, uint32_t m)
 {
     const uint32_t w[4] = {v.x, v.y, v.z, v.w};
@@ -1015,11 +1040,25 @@ __global__ __launch_bounds__(256) void aead_spread_kernel(AeadArgs a)
     if (w >= a.n) return;
     // everything up to the per-lane work below is uniform across the wave
     const uint32_t i = a.first + w;
-    uint32_t len = a.lens ? a.lens[i] : a.len;
+    // The packet's entries in the per-packet arrays, every one loaded whether or not the
+    // array is there (from the key table where it is not): a load under a branch is waited
+    // for where the branch closes, and a host batch's arrays lie in host memory, a trip over
+    // the link for each wait.
+    const uint8_t *const safe = reinterpret_cast<const uint8_t *>(a.keys);
+    const uint32_t *const safe32 = a.keys;
+    const uint64_t *const safe64 = reinterpret_cast<const uint64_t *>(a.keys);
+    const uint32_t len_ld = *(a.lens ? a.lens + i : safe32);
+    const uint32_t peer_ld = *(a.peer ? a.peer + i : safe32);
+    const uint64_t in_off_ld = *(a.in_off ? a.in_off + i : safe64);
+    const uint64_t out_off_ld = *(a.out_off ? a.out_off + i : safe64);
+    const uint64_t ctr_ld = *(a.counters ? a.counters + i : safe64);
+    const uint8_t skip_ld = *(a.skip ? a.skip + i : safe);
+    uint32_t len = a.lens ? len_ld : a.len;
     if (!OPEN) len = len >= a.trim ? len - a.trim : 0u;
-    uint32_t pr = a.peer ? a.peer[i] : 0u;
-    const uint8_t *src = a.in + (a.in_off ? a.in_off[i] : (uint64_t)i * a.in_stride) + a.in_skip;
-    uint8_t *dst = a.out + (a.out_off ? a.out_off[i] : (uint64_t)i * a.out_stride) + a.out_skip;
+    uint32_t pr = a.peer ? peer_ld : 0u;
+    const uint8_t *src = a.in + (a.in_off ? in_off_ld : (uint64_t)i * a.in_stride) + a.in_skip;
+    uint8_t *dst = a.out + (a.out_off ? out_off_ld : (uint64_t)i * a.out_stride) + a.out_skip;
+    const bool skipped = a.skip != nullptr && skip_ld != 0;
     uint64_t ctr = 0;
     if (!WG) {
         // (framing launches only run on layouts the host has checked)
@@ -1028,7 +1067,7 @@ __global__ __launch_bounds__(256) void aead_spread_kernel(AeadArgs a)
         if (beyond_arena(in_at, len, a.in_limit) ||
             beyond_arena(out_at, OPEN ? (short_ct ? 0u : len - 16u) : (uint64_t)len + 16u, a.out_limit) ||
             (len > MAX_PACKET_BYTES && (a.in_limit | a.out_limit) != 0)) {
-            if (lane == 0 && !(a.skip && a.skip[i] != 0)) {
+            if (lane == 0 && !skipped) {
                 status_raise(a.status, STATUS_BOUNDS);
                 if (OPEN) a.verdict[i] = 0;
             }
@@ -1064,23 +1103,41 @@ __global__ __launch_bounds__(256) void aead_spread_kernel(AeadArgs a)
     // fetching its own block reads 16 bytes every 64: sixty-four small requests
     // an instruction, which a packet that lies in host memory pays for with a
     // read of its own over the link for each.)
+    // What the packet's bytes wait for goes out ahead of them, so that a wait for it does
+    // not wait for them as well (a wave's loads complete in the order they were issued): the
+    // sender's key where the sender is known by now, with the receiver's index for the
+    // header on the way out; on the way in the header, which names the sender.
+    uint4 key_lo = make_uint4(0, 0, 0, 0), key_hi = key_lo, wg_head = key_lo;
+    uint32_t wg_remote = 0;
+    if (!(WG && OPEN)) {
+        const uint32_t known = pr < (WG ? a.wg.n_peers : a.n_peers) ? pr : 0u; // (the table has a row 0)
+        const uint4 *kp = reinterpret_cast<const uint4 *>(a.keys + 8u * known);
+        key_lo = kp[0];
+        key_hi = kp[1];
+        if (WG) wg_remote = a.wg.remote_index[known];
+    } else {
+        wg_head = ld16(len >= 32u && len - 32u <= WG_FUSE_MAX_LEN ? src : safe);
+    }
+    // Every load below is issued whatever the lane's share is (from the key table where it
+    // has none), so that they are all in flight together: the pieces, the last 1-15 bytes of
+    // the packet (one lane's, by words, a halfword and a byte: nothing beyond the packet is
+    // touched), and the tag.
     uint4 pre[4];
 #pragma unroll
     for (int j = 0; j < 4; j++) {
         const uint32_t off = 1024u * j + 16u * lane;
-        uint4 v = make_uint4(0, 0, 0, 0);
-        if (1024u * j < data_there) { // (the same for the whole wave)
-            if (off + 16u <= data_there) v = ld16(data + off);
-            else if (off < data_there) v = ld_partial(data + off, data_there - off);
-        }
-        pre[j] = v;
+        pre[j] = ld16(off + 16u <= data_there ? data + off : safe);
     }
-    uint4 want_tag = make_uint4(0, 0, 0, 0);
-    if (OPEN && (WG ? len >= 32u && len - 32u <= WG_FUSE_MAX_LEN : len >= 16u && data_len <= SPREAD_MAX_LEN))
-        want_tag = ld16(data + data_len);
+    const uint32_t odd = data_there & 15u, odd_at = data_there & ~15u; // the packet's last, partial cell
+    const bool odd_mine = odd != 0u && ((odd_at >> 4) & 63u) == lane;
+    const uint4 odd_cell = ld_partial_flat(data + odd_at, odd_mine ? odd : 0u, safe);
+    const bool tagged = OPEN && (WG ? len >= 32u && len - 32u <= WG_FUSE_MAX_LEN : len >= 16u && data_len <= SPREAD_MAX_LEN);
+    uint4 want_tag = ld16(tagged ? data + data_len : safe);
+    // (what the lanes without a share have fetched is set aside where the pieces are used,
+    // further down: looking at it here would make the key wait for the packet)
 
     if (!WG) {
-        if (a.skip && a.skip[i] != 0) return;
+        if (skipped) return;
         if (pr >= a.n_peers) {
             if (lane == 0) {
                 status_raise(a.status, STATUS_PEER_RANGE);
@@ -1093,21 +1150,21 @@ __global__ __launch_bounds__(256) void aead_spread_kernel(AeadArgs a)
             return;
         }
         if (OPEN) len -= 16u;
-        ctr = a.counters ? a.counters[i] : a.counter0 + i;
+        ctr = a.counters ? ctr_ld : a.counter0 + i;
     } else if (!OPEN) {
         // ---- encapsulate: header into the headroom, padding as implied zeros ----
         if (pr >= a.wg.n_peers || len + 15u > WG_FUSE_MAX_LEN) {
             if (lane == 0) a.wg.wire_len[i] = 0;
             return;
         }
-        ctr = a.counters[i];
+        ctr = ctr_ld;
         if (ctr >= WG_REJECT_AFTER_MESSAGES) { // the keypair has used up its nonces
             if (lane == 0) a.wg.wire_len[i] = 0;
             return;
         }
         len += wg_padding(len, a.wg.mtu);
         if (lane == 0) {
-            st16(dst, make_uint4(4u, a.wg.remote_index[pr], (uint32_t)ctr, (uint32_t)(ctr >> 32)));
+            st16(dst, make_uint4(4u, wg_remote, (uint32_t)ctr, (uint32_t)(ctr >> 32)));
             a.wg.wire_len[i] = 16u + len + 16u;
         }
         src += 16;
@@ -1117,7 +1174,7 @@ __global__ __launch_bounds__(256) void aead_spread_kernel(AeadArgs a)
         uint8_t res = BNK_WG_OK;
         uint4 h = make_uint4(0, 0, 0, 0);
         if (len < 32u || len - 32u > WG_FUSE_MAX_LEN) res = BNK_WG_BAD_HEADER;
-        else h = ld16(src);
+        else h = wg_head;
         if (res == BNK_WG_OK && h.x != 4u) res = BNK_WG_BAD_HEADER;
         if (res == BNK_WG_OK) {
             // narrow [lo, hi) to at most 64 entries, 64 probes at a time
@@ -1156,10 +1213,13 @@ __global__ __launch_bounds__(256) void aead_spread_kernel(AeadArgs a)
     }
     uint32_t k[8];
     {
-        const uint4 *kp = reinterpret_cast<const uint4 *>(a.keys + 8u * pr);
-        const uint4 k0 = kp[0], k1 = kp[1];
-        k[0] = k0.x; k[1] = k0.y; k[2] = k0.z; k[3] = k0.w;
-        k[4] = k1.x; k[5] = k1.y; k[6] = k1.z; k[7] = k1.w;
+        if (WG && OPEN) { // (the sender has only now been found)
+            const uint4 *kp = reinterpret_cast<const uint4 *>(a.keys + 8u * pr);
+            key_lo = kp[0];
+            key_hi = kp[1];
+        }
+        k[0] = key_lo.x; k[1] = key_lo.y; k[2] = key_lo.z; k[3] = key_lo.w;
+        k[4] = key_hi.x; k[5] = key_hi.y; k[6] = key_hi.z; k[7] = key_hi.w;
     }
     const uint32_t n1 = (uint32_t)ctr, n2 = (uint32_t)(ctr >> 32);
     uint32_t x[16];
@@ -1180,10 +1240,16 @@ __global__ __launch_bounds__(256) void aead_spread_kernel(AeadArgs a)
     // Block b of the packet lies at stage + 80 b (rows padded against bank
     // conflicts): written in the order the pieces came in, read a block per lane.
     uint8_t *stage = tile_all[threadIdx.x >> 6];
+    if (!tagged) want_tag = make_uint4(0, 0, 0, 0);
 #pragma unroll
-    for (int j = 0; j < 4; j++)
+    for (int j = 0; j < 4; j++) {
+        const uint32_t off = 1024u * j + 16u * lane;
+        // a cell beyond the packet's whole cells is zeros, but for its last 1-15 bytes
+        if (off + 16u > data_there) pre[j] = make_uint4(0, 0, 0, 0);
+        if (odd_mine && (odd_at >> 10) == (uint32_t)j) pre[j] = odd_cell;
         if (1024u * j < data_there)
             *reinterpret_cast<uint4 *>(stage + (16u * j + (lane >> 2)) * LDS_ROW + 16u * (lane & 3u)) = pre[j];
+    }
     wave_sync();
     uint32_t m[16];
 #pragma unroll
